@@ -1,0 +1,239 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged-attention hot path on one MI355X.
+
+Prints ONE JSON line.  The headline (`metric`/`value`) is BASELINE config 3:
+paged-attention decode, batch 256, context lengths log-uniform in [128, 32768],
+32 query heads / 8 KV heads / head_dim 128, bf16 cache, block_size 16, reported
+as algorithmic HBM GB/s.  A "step" is one decode call over the whole batch with
+all inputs resident in HBM.  `extra` carries the other measured workloads
+(decode at block_size 256, varlen prefill TFLOP/s and store_kvcache GB/s on
+config 2).  `cpu_baseline` times the CPU oracle's naive decode on a bounded
+subset of the same batch on the host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
+    ap.add_argument("--only", default="", help="comma list out of decode,decode256,prefill,store,cpu to restrict the run")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    return ap.parse_args()
+
+
+def time_steps(fn, steps, warmup):
+    """W untimed calls, then K calls timed by wall clock (synchronised both sides) and by HIP events on the
+    current torch stream (the stream the kernels are launched on).  Returns (wall ms/step, event ms/step)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, start.elapsed_time(stop) / steps
+
+
+def decode_bytes(ctx, block_size, num_heads, num_kv_heads, head_dim, kv_elem, q_elem, ctx_elem, int8_scales=False):
+    """Algorithmic HBM bytes of one decode call: every live K/V element once, q read + out written once,
+    one table entry per live block, one context length per sequence.  Split-K scratch is not counted."""
+    tokens = int(ctx.sum())
+    blocks = int(((ctx + block_size - 1) // block_size).sum())
+    b = ctx.numel()
+    total = tokens * num_kv_heads * head_dim * 2 * kv_elem
+    if int8_scales:
+        total += tokens * num_kv_heads * 2 * 4
+    total += 2 * b * num_heads * head_dim * q_elem + 4 * blocks + ctx_elem * b
+    return total
+
+
+def bench_decode(args, block_size, want_cpu):
+    import torch
+    from helpers import extract_sequence, make_paged_case_on_device
+    from minivllm_amd.layers.attention import paged_attention_decode
+
+    dev = "cuda:0"
+    hq, hkv, d, batch = 32, 8, 128, 256
+    q, kc, vc, tables, ctx = make_paged_case_on_device(args.seed, dev, batch, 128, 32768, hq, hkv, d, block_size)
+    scale = 1.0 / math.sqrt(d)
+    td, cd = tables.to(dev), ctx.to(dev)
+
+    def step():
+        return paged_attention_decode(q, kc, vc, td, cd, scale, hq, hkv, d, block_size)
+
+    wall_ms, event_ms = time_steps(step, args.steps, args.warmup)
+    nbytes = decode_bytes(ctx, block_size, hq, hkv, d, 2, 2, 8)
+    res = {
+        "workload": f"decode B256 ctx~logU[128,32768] Hq32 Hkv8 D128 bf16 block_size {block_size}",
+        "tokens": int(ctx.sum()), "algorithmic_bytes": nbytes,
+        "ms_per_step": wall_ms, "event_ms_per_step": event_ms,
+        "gbs": nbytes / (wall_ms * 1e-3) / 1e9, "gbs_event": nbytes / (event_ms * 1e-3) / 1e9,
+    }
+    cpu = None
+    if want_cpu:
+        import oracle
+        # bounded sample: the first sequences of the same batch up to ~24k context tokens in total
+        picked, tok = [], 0
+        for b in range(batch):
+            if picked and tok + int(ctx[b]) > 24576:
+                break
+            picked.append(b)
+            tok += int(ctx[b])
+        parts = [extract_sequence(kc, vc, tables, ctx, b, block_size) for b in picked]
+        # one compact CPU cache with per-sequence tables (block ids shifted)
+        ks, vs, rows, at = [], [], [], 0
+        width = max(p[2].shape[1] for p in parts)
+        for k1, v1, t1, _ in parts:
+            ks.append(k1.float())
+            vs.append(v1.float())
+            row = torch.full((width,), -1, dtype=torch.int32)
+            row[:t1.shape[1]] = t1[0] + at
+            rows.append(row)
+            at += k1.shape[0]
+        kcpu, vcpu, tcpu = torch.cat(ks), torch.cat(vs), torch.stack(rows)
+        qcpu, ccpu = q[picked].float().cpu(), ctx[picked]
+        oracle.decode_naive_oracle(qcpu[:1], kcpu, vcpu, tcpu[:1], ccpu[:1], scale, hq, hkv, d, block_size)
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            ref = oracle.decode_naive_oracle(qcpu, kcpu, vcpu, tcpu, ccpu, scale, hq, hkv, d, block_size)
+            reps += 1
+            if time.perf_counter() - t0 > 10.0 or reps >= 20:
+                break
+        cpu_s = (time.perf_counter() - t0) / reps
+        sub_bytes = decode_bytes(ccpu, block_size, hq, hkv, d, 2, 2, 8)
+        got = step()[picked].float().cpu()
+        cpu = {
+            "value": sub_bytes / cpu_s / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle naive decode (fp32, torch-CPU) on the first {len(picked)} sequences of the same "
+                      f"batch ({tok} context tokens), {reps} reps, {cpu_s * 1e3:.1f} ms each; bf16-equivalent "
+                      f"algorithmic bytes",
+            "host_cpu_count": os.cpu_count(),
+            "gpu_vs_oracle_max_abs": (got - ref).abs().max().item(),
+        }
+    del kc, vc
+    torch.cuda.empty_cache()
+    return res, cpu
+
+
+def bench_prefill_store(args, which):
+    """BASELINE config 2: 16 prompts L~U[64,2048], Hq32/Hkv8/D128 bf16; store into a block-256 paged cache."""
+    import torch
+    from helpers import make_slot_mapping
+    from minivllm_amd.layers.attention import flash_attention_prefill, store_kvcache
+
+    dev = "cuda:0"
+    hq, hkv, d, bs = 32, 8, 128, 256
+    g = torch.Generator().manual_seed(args.seed)
+    lengths = torch.randint(64, 2049, (16,), generator=g).tolist()
+    total = sum(lengths)
+    dg = torch.Generator(device=dev).manual_seed(args.seed + 1)
+    q = torch.randn(total, hq, d, generator=dg, device=dev).to(torch.bfloat16)
+    k = torch.randn(total, hkv, d, generator=dg, device=dev).to(torch.bfloat16)
+    v = torch.randn(total, hkv, d, generator=dg, device=dev).to(torch.bfloat16)
+    cu = torch.zeros(17, dtype=torch.int32)
+    cu[1:] = torch.tensor(lengths).cumsum(0)
+    cu = cu.to(dev)
+    out = {}
+    if "prefill" in which:
+        scale = 1.0 / math.sqrt(d)
+        wall_ms, event_ms = time_steps(lambda: flash_attention_prefill(q, k, v, cu, scale, hq, hkv, d),
+                                       max(3, args.steps // 3), max(1, args.warmup // 2))
+        flops = 4 * hq * d * sum(n * (n + 1) // 2 for n in lengths)
+        out["prefill"] = {
+            "workload": "varlen causal prefill, 16 prompts L~U[64,2048], Hq32 Hkv8 D128 bf16",
+            "tokens": total, "algorithmic_flops": flops, "ms_per_step": wall_ms, "event_ms_per_step": event_ms,
+            "tflops": flops / (event_ms * 1e-3) / 1e12,
+            "frac_of_bf16_mfma_peak": flops / (event_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        }
+    if "store" in which:
+        slots, _, nb = make_slot_mapping(args.seed + 2, lengths, bs)
+        kc = torch.zeros(nb, bs, hkv, d, dtype=torch.bfloat16, device=dev)
+        vc = torch.zeros_like(kc)
+        sl = slots.to(dev)
+        wall_ms, event_ms = time_steps(lambda: store_kvcache(k, v, kc, vc, sl, bs), args.steps, args.warmup)
+        nbytes = 2 * total * hkv * d * (2 + 2) + 8 * total
+        out["store"] = {
+            "workload": "store_kvcache of the same batch into a block-256 bf16 cache, shuffled blocks",
+            "tokens": total, "algorithmic_bytes": nbytes, "ms_per_step": wall_ms, "event_ms_per_step": event_ms,
+            "gbs": nbytes / (event_ms * 1e-3) / 1e9,
+        }
+    return out
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (no collectives or sharding are part of it); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the hot path has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    from minivllm_amd import _C
+    _C.load()
+
+    only = set(x for x in args.only.split(",") if x)
+    want = lambda name: not only or name in only
+    extra = {}
+    head, cpu = bench_decode(args, args.block_size, want_cpu=not args.no_cpu and want("cpu"))
+    if want("decode256") and args.block_size != 256:
+        extra["decode_block256"], _ = bench_decode(args, 256, want_cpu=False)
+    which = [n for n in ("prefill", "store") if want(n)]
+    if which:
+        extra.update(bench_prefill_store(args, which))
+
+    line = {
+        "metric": "decode-attn HBM GB/s (% peak); prefill TFLOP/s (% MFMA); engine out tok/s",
+        "value": head["gbs"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic (seeded N(0,1) q/K/V, random disjoint block tables, seed %d)" % args.seed,
+        "config": {"workload": head["workload"], "tokens": head["tokens"], "algorithmic_bytes": head["algorithmic_bytes"]},
+        "roofline": {
+            "bound": "hbm",
+            "achieved": head["gbs_event"],
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": head["gbs_event"] / HBM_PEAK_GBS,
+            "traffic": None,
+            "kernel": "decode_mfma_kernel + decode_reduce_kernel (one decode call, HIP events on the launch stream)",
+        },
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,146 @@
+/*
+ * minivllm_amd.h -- C ABI of libminivllm_amd.so (gfx950 / MI355X).
+ *
+ * The reference (Wenyueh/MinivLLM) is pure Python + Triton and has no FFI;
+ * each entry point below replaces the Triton launch inside one of the
+ * reference's Python operators and is what a ctypes binding of that operator
+ * calls.  The reference location of the operator is cited per function.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - return value: 0 ok, <0 invalid argument / unsupported shape
+ *     (see mvllm_status_string), >0 a hipError_t from the launch;
+ *   - the library never allocates, frees or synchronises; outputs and
+ *     workspaces are caller-owned; launches have static grids derived from the
+ *     host arguments only, so every call is legal under hipGraph capture;
+ *   - tensors are dense row-major ("contiguous") in the stated shape.
+ */
+#ifndef MINIVLLM_AMD_H_
+#define MINIVLLM_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of q/k/v/out and of a non-quantised KV cache */
+enum mvllm_dtype {
+  MVLLM_F32 = 0,
+  MVLLM_BF16 = 1,
+  MVLLM_F16 = 2,
+};
+
+/* negative status codes */
+enum mvllm_status {
+  MVLLM_OK = 0,
+  MVLLM_ERR_NULL_POINTER = -1,
+  MVLLM_ERR_BAD_DTYPE = -2,
+  MVLLM_ERR_BAD_SHAPE = -3,      /* a size is <= 0 where it must be positive, or not divisible as required */
+  MVLLM_ERR_UNSUPPORTED = -4,    /* shape valid but no kernel is built for it */
+  MVLLM_ERR_WORKSPACE = -5,      /* workspace missing or smaller than *_workspace_bytes() */
+  MVLLM_ERR_MISALIGNED = -6,     /* pointer not aligned to 16 bytes */
+};
+
+/* ABI version: major*1000 + minor. */
+int mvllm_version(void);
+
+/* Static, human-readable text for a status returned by this library
+ * (negative codes only; positive codes are hipError_t). HOST pointer. */
+const char* mvllm_status_string(int status);
+
+/*
+ * store_kvcache -- src/myvllm/layers/attention.py:67-108 (kernel :7-64).
+ * For every token t with slot = slot_mapping[t]:
+ *     slot == -1 (or outside [0, num_slots))  -> nothing is written
+ *     else k_cache_flat[slot, :, :] = key[t, :, :], same for value,
+ * where *_cache_flat is the [num_slots = num_blocks*block_size, Hkv, D] view of
+ * the [num_blocks, block_size, Hkv, D] cache.  key/value: [T, Hkv, D], same
+ * dtype as the caches (a bit-exact copy).  slot_mapping: int64 [T].
+ */
+int mvllm_store_kvcache(const void* key, const void* value,
+                        void* k_cache, void* v_cache,
+                        const int64_t* slot_mapping,
+                        int64_t num_tokens, int64_t num_slots,
+                        int num_kv_heads, int head_dim,
+                        int dtype, void* stream);
+
+/*
+ * INT8 variant of store_kvcache (no counterpart in the reference; it serves
+ * the same call site, attention.py:510, when the cache is int8).
+ * Per (token, kv head): amax = max|x| in fp32, scale = amax / 127 (IEEE fp32
+ * divide), code = clamp(rint(x / scale), -127, 127) (round half to even);
+ * amax == 0 -> scale 0, codes 0.  Codes go to int8 caches [num_slots, Hkv, D],
+ * scales to fp32 [num_slots, Hkv].  `dtype` is the dtype of key/value.
+ */
+int mvllm_store_kvcache_int8(const void* key, const void* value,
+                             int8_t* k_cache, int8_t* v_cache,
+                             float* k_scale, float* v_scale,
+                             const int64_t* slot_mapping,
+                             int64_t num_tokens, int64_t num_slots,
+                             int num_kv_heads, int head_dim,
+                             int dtype, void* stream);
+
+/*
+ * Bytes of fp32 split-K workspace mvllm_paged_decode{,_int8} need for these
+ * static sizes (0 if the shape needs none).  Pure host arithmetic.
+ */
+size_t mvllm_paged_decode_workspace_bytes(int batch, int num_heads, int head_dim,
+                                          int max_num_blocks, int block_size);
+
+/*
+ * paged_attention_decode -- src/myvllm/layers/attention.py:418-473 (kernel :283-415).
+ * out[b,h,:] = softmax_t( scale * q[b,h,:] . K[b,t,g(h),:] ) V[b,t,g(h),:],
+ * t in [0, context_lens[b]), g(h) = h / (Hq/Hkv); token t of sequence b lives at
+ * cache[block_tables[b, t / block_size], t % block_size, g, :].
+ * Tokens whose table index is >= max_num_blocks, or whose entry is < 0 or
+ * >= num_blocks, contribute nothing; context_len <= 0 gives a row of zeros.
+ *   out, q        [batch, Hq, D]  `dtype`
+ *   k/v_cache     [num_blocks, block_size, Hkv, D]  `dtype`
+ *   block_tables  int32 [batch, max_num_blocks]
+ *   context_lens  int64 [batch] if ctx_is_i64 else int32 [batch]
+ *   workspace     >= mvllm_paged_decode_workspace_bytes(...) bytes, 16-byte aligned
+ */
+int mvllm_paged_decode(void* out, const void* q,
+                       const void* k_cache, const void* v_cache,
+                       const int32_t* block_tables, int max_num_blocks,
+                       const void* context_lens, int ctx_is_i64,
+                       int batch, int num_heads, int num_kv_heads, int head_dim,
+                       int block_size, int64_t num_blocks, float scale, int dtype,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * INT8-cache variant of paged decode (no counterpart in the reference).
+ * K/V rows are dequantised in-kernel as code * scale in fp32.
+ *   k/v_cache  int8 [num_blocks, block_size, Hkv, D]
+ *   k/v_scale  fp32 [num_blocks, block_size, Hkv]
+ *   `dtype` is the dtype of q and out.
+ */
+int mvllm_paged_decode_int8(void* out, const void* q,
+                            const int8_t* k_cache, const int8_t* v_cache,
+                            const float* k_scale, const float* v_scale,
+                            const int32_t* block_tables, int max_num_blocks,
+                            const void* context_lens, int ctx_is_i64,
+                            int batch, int num_heads, int num_kv_heads, int head_dim,
+                            int block_size, int64_t num_blocks, float scale, int dtype,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * flash_attention_prefill -- src/myvllm/layers/attention.py:212-280 (kernel :111-209).
+ * Packed ragged batch: sequence s owns rows [cu_seqlens[s], cu_seqlens[s+1]).
+ * out[i,h,:] = softmax_{j<=i, same sequence}( scale * q[i,h,:] . k[j,g(h),:] ) v[j,g(h),:].
+ *   out, q  [T, Hq, D];  k, v  [T, Hkv, D];  cu_seqlens int32 [num_seqs+1]
+ * Needs no maximum sequence length: the grid is sized from total_tokens and
+ * num_seqs (the reference synchronises with the host to find it, :263-264).
+ */
+int mvllm_prefill_varlen(void* out, const void* q, const void* k, const void* v,
+                         const int32_t* cu_seqlens, int num_seqs, int64_t total_tokens,
+                         int num_heads, int num_kv_heads, int head_dim,
+                         float scale, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MINIVLLM_AMD_H_ */

@@ -1,0 +1,68 @@
+"""Builds libminivllm_amd.so (gfx950) in-tree with hipcc.
+
+``python -m minivllm_amd._build`` or ``build_library()``.  The library is
+written next to the sources' package (minivllm_amd/libminivllm_amd.so).
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_PATH = os.path.join(PKG_DIR, "libminivllm_amd.so")
+SOURCES = ["capi.hip", "store_kvcache.hip", "paged_decode.hip", "prefill_varlen.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-fhip-fp32-correctly-rounded-divide-sqrt",   # INT8 scales/codes must match IEEE division
+    "-fno-fast-math",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; cannot build libminivllm_amd.so")
+    return exe
+
+
+def build_library(verbose: bool = True, jobs: int = 4) -> str:
+    hipcc = _hipcc()
+    obj_dir = os.path.join(PKG_DIR, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+
+    def compile_one(src):
+        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {src}:\n{err}")
+        if verbose and err.strip():
+            print(err, file=sys.stderr)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library())

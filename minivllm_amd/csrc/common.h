@@ -1,0 +1,111 @@
+// Shared device helpers for the gfx950 kernels of libminivllm_amd.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/minivllm_amd.h"
+
+namespace mvllm {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 v8bf16;
+typedef __attribute__((ext_vector_type(8))) _Float16 v8f16;
+typedef __attribute__((ext_vector_type(4))) float v4f;
+typedef __attribute__((ext_vector_type(16))) float v16f;
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---- element types ---------------------------------------------------------
+// Storage structs so templates can be instantiated per dtype without pulling in
+// the HIP bf16/half class headers.
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 v; };
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16_t x) { return __uint_as_float(((uint32_t)x.bits) << 16); }
+__device__ __forceinline__ float to_float(f16_t x) { return (float)x.v; }
+
+// round-to-nearest-even conversions from fp32
+template <typename T> __device__ __forceinline__ T from_float(float x);
+template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float x) {
+  uint32_t u = __float_as_uint(x);
+  bf16_t r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {  // NaN stays NaN
+    r.bits = (uint16_t)((u >> 16) | 0x0040u);
+  } else {
+    u += 0x7fffu + ((u >> 16) & 1u);
+    r.bits = (uint16_t)(u >> 16);
+  }
+  return r;
+}
+template <> __device__ __forceinline__ f16_t from_float<f16_t>(float x) {
+  f16_t r;
+  r.v = (_Float16)x;
+  return r;
+}
+
+// The two 16-bit halves of a 32-bit word as fp32 (bf16 / fp16 pairs).
+template <typename T> __device__ __forceinline__ float lo_to_float(uint32_t w);
+template <typename T> __device__ __forceinline__ float hi_to_float(uint32_t w);
+template <> __device__ __forceinline__ float lo_to_float<bf16_t>(uint32_t w) { return __uint_as_float(w << 16); }
+template <> __device__ __forceinline__ float hi_to_float<bf16_t>(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+template <> __device__ __forceinline__ float lo_to_float<f16_t>(uint32_t w) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+}
+template <> __device__ __forceinline__ float hi_to_float<f16_t>(uint32_t w) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+}
+
+// 16x16x32 MFMA on 8-element 16-bit fragments held as uint4.
+template <typename T> __device__ __forceinline__ v4f mfma16x16x32(uint4 a, uint4 b, v4f c);
+template <> __device__ __forceinline__ v4f mfma16x16x32<bf16_t>(uint4 a, uint4 b, v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf16, a), __builtin_bit_cast(v8bf16, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ v4f mfma16x16x32<f16_t>(uint4 a, uint4 b, v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, a), __builtin_bit_cast(v8f16, b), c, 0, 0, 0);
+}
+
+// 32x32x16 MFMA.
+template <typename T> __device__ __forceinline__ v16f mfma32x32x16(uint4 a, uint4 b, v16f c);
+template <> __device__ __forceinline__ v16f mfma32x32x16<bf16_t>(uint4 a, uint4 b, v16f c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf16, a), __builtin_bit_cast(v8bf16, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ v16f mfma32x32x16<f16_t>(uint4 a, uint4 b, v16f c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8f16, a), __builtin_bit_cast(v8f16, b), c, 0, 0, 0);
+}
+
+// ---- cross-lane helpers ----------------------------------------------------
+// Value held by lane (quad base + SRC) of the caller's 4-lane quad.
+template <int SRC> __device__ __forceinline__ float quad_bcast(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), SRC * 0x55, 0xf, 0xf, false));
+}
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+  return x;
+}
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+  return x;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---- host helpers ----------------------------------------------------------
+inline int dtype_size(int dtype) {
+  switch (dtype) {
+    case MVLLM_F32: return 4;
+    case MVLLM_BF16: return 2;
+    case MVLLM_F16: return 2;
+    default: return 0;
+  }
+}
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
+
+}  // namespace mvllm

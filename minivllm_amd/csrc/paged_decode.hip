@@ -1,0 +1,594 @@
+// Paged-attention decode for gfx950: split-K over fixed token partitions,
+// GQA-shared K/V reads, log-sum-exp merge in a second pass.
+// Replaces the Triton kernel of src/myvllm/layers/attention.py:283-415.
+//
+// Work decomposition (fast path, 16-bit cache, head_dim 128, block_size % 16 == 0)
+//   workgroup = (partition p, sequence b, group of <= 8 kv heads); wave w of the
+//   workgroup owns kv head g and all Hq/Hkv query heads that share it, so the
+//   waves of one workgroup stream whole contiguous [token, Hkv, D] rows.
+//   A wave walks its partition in tiles of 16 tokens:
+//     S[16 tok x 16 col]   = K_tile (A operand, straight from global in MFMA
+//                            layout) x Q^T (B operand, column n = head n%4)
+//                            -> lane l holds tokens 4*(l/16)+i, head l%4
+//     online softmax       per lane over its token class, base-2, lazy rescale
+//     O[head][8 dims]     += p * V  on the VALU; V rows are loaded fully
+//                            coalesced (lane l: token 4*(l/16)+i, dims 8*(l%16)..)
+//                            and p of head h comes from quad lane h via DPP.
+//   The four token classes are merged once per partition with xor-shuffles.
+// Everything is HBM-bound by construction: QK^T costs no VALU, PV costs
+// ~5 lane-ops per cache element.
+#include "common.h"
+
+namespace mvllm {
+
+constexpr int kTile = 16;            // tokens per MFMA tile
+constexpr int kMaxParts = 64;        // split-K partitions per sequence (upper bound)
+constexpr int kMinPartTokens = 256;  // smallest partition
+constexpr float kLazyRescale = 8.f;  // rescale accumulators only when the max grows by > 2^8
+
+struct DecodeArgs {
+  void* out;
+  const void* q;
+  const void* k_cache;
+  const void* v_cache;
+  const float* k_scale;   // INT8 only
+  const float* v_scale;   // INT8 only
+  const int32_t* block_tables;
+  const void* context_lens;
+  float* ws_acc;          // [B, NP, Hq, D]
+  float* ws_ml;           // [B, NP, Hq, 2]  (max in log2 units, sum)
+  int64_t num_blocks;
+  int ctx_is_i64;
+  int max_num_blocks;
+  int batch;
+  int num_heads;
+  int num_kv_heads;
+  int head_dim;
+  int block_size;
+  int part_tokens;
+  int num_parts;          // partitions per sequence in the grid / workspace
+  float scale_log2;       // scale * log2(e)
+};
+
+__host__ __device__ inline int partition_tokens_for(int64_t max_ctx) {
+  int64_t part = kMinPartTokens;
+  while ((max_ctx + part - 1) / part > kMaxParts) part *= 2;
+  return (int)part;
+}
+
+__device__ __forceinline__ int64_t load_ctx(const DecodeArgs& a, int b) {
+  int64_t c = a.ctx_is_i64 ? reinterpret_cast<const int64_t*>(a.context_lens)[b]
+                           : (int64_t) reinterpret_cast<const int32_t*>(a.context_lens)[b];
+  const int64_t cap = (int64_t)a.max_num_blocks * a.block_size;
+  if (c > cap) c = cap;   // tokens past the table contribute nothing
+  if (c < 0) c = 0;
+  return c;
+}
+
+__device__ __forceinline__ float safe_exp2_diff(float m_old, float m_new) {
+  // exp2(m_old - m_new) with -inf - -inf := 0 contribution
+  return (m_old == -INFINITY) ? 0.f : fast_exp2(m_old - m_new);
+}
+
+// ---------------------------------------------------------------------------
+// Fast path
+// ---------------------------------------------------------------------------
+template <typename T>
+struct KVTile {
+  uint4 k[4];
+  uint4 v[4];
+  int t0;
+  bool ok;
+};
+
+template <typename T, int NCH>
+struct DecodeWave {
+  // per-lane online-softmax state for head (lane%4) of chunk c, token class lane/16
+  float m[NCH];
+  float l[NCH];
+  float acc[NCH][4][8];
+  uint4 qf[NCH][4];
+
+  __device__ __forceinline__ void init() {
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      m[c] = -INFINITY;
+      l[c] = 0.f;
+#pragma unroll
+      for (int h = 0; h < 4; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[c][h][e] = 0.f;
+    }
+  }
+
+  template <int H>
+  __device__ __forceinline__ void scale_head(int c, float a) {
+    const float ah = quad_bcast<H>(a);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[c][H][e] *= ah;
+  }
+  template <int H>
+  __device__ __forceinline__ void fma_head(int c, float p, const float (&vf)[8]) {
+    const float ph = quad_bcast<H>(p);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[c][H][e] = fmaf(ph, vf[e], acc[c][H][e]);
+  }
+
+  __device__ __forceinline__ void consume(const KVTile<T>& t, int part_end, float scale_log2, int lane) {
+    const int tok_base = t.t0 + 4 * (lane >> 4);
+    const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
+    float p[NCH][4];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      v4f s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s = mfma16x16x32<T>(t.k[j], qf[c][j], s);
+      float s2[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s2[i] = s[i] * scale_log2;
+      if (partial) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (!t.ok || tok_base + i >= part_end) s2[i] = -INFINITY;
+      }
+      const float tile_max = fmaxf(fmaxf(s2[0], s2[1]), fmaxf(s2[2], s2[3]));
+      const bool grow = tile_max > m[c] + kLazyRescale || (m[c] == -INFINITY && tile_max > -INFINITY);
+      if (__any(grow)) {
+        const float m_new = grow ? tile_max : m[c];
+        const float a = (m_new == m[c]) ? 1.f : safe_exp2_diff(m[c], m_new);
+        l[c] *= a;
+        scale_head<0>(c, a);
+        scale_head<1>(c, a);
+        scale_head<2>(c, a);
+        scale_head<3>(c, a);
+        m[c] = m_new;
+      }
+      const float m_eff = (m[c] == -INFINITY) ? 0.f : m[c];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[c][i] = fast_exp2(s2[i] - m_eff);
+        l[c] += p[c][i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint4 w = t.v[i];
+      if (partial && (!t.ok || tok_base + i >= part_end)) w = make_uint4(0u, 0u, 0u, 0u);
+      float vf[8];
+      vf[0] = lo_to_float<T>(w.x); vf[1] = hi_to_float<T>(w.x);
+      vf[2] = lo_to_float<T>(w.y); vf[3] = hi_to_float<T>(w.y);
+      vf[4] = lo_to_float<T>(w.z); vf[5] = hi_to_float<T>(w.z);
+      vf[6] = lo_to_float<T>(w.w); vf[7] = hi_to_float<T>(w.w);
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        fma_head<0>(c, p[c][i], vf);
+        fma_head<1>(c, p[c][i], vf);
+        fma_head<2>(c, p[c][i], vf);
+        fma_head<3>(c, p[c][i], vf);
+      }
+    }
+  }
+
+  template <int H>
+  __device__ __forceinline__ void merge_head(int c, float a, float ao, int off) {
+    const float ah = quad_bcast<H>(a);
+    const float aoh = quad_bcast<H>(ao);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float other = __shfl_xor(acc[c][H][e], off, 64);
+      acc[c][H][e] = acc[c][H][e] * ah + other * aoh;
+    }
+  }
+
+  // Fold the four token classes (lane/16) together; afterwards every lane holds
+  // the statistics of the whole partition for its head / dims.
+  __device__ __forceinline__ void merge_token_classes() {
+#pragma unroll
+    for (int off = 16; off <= 32; off <<= 1) {
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const float mo = __shfl_xor(m[c], off, 64);
+        const float lo = __shfl_xor(l[c], off, 64);
+        const float mn = fmaxf(m[c], mo);
+        const float a = safe_exp2_diff(m[c], mn);
+        const float ao = safe_exp2_diff(mo, mn);
+        l[c] = l[c] * a + lo * ao;
+        m[c] = mn;
+        merge_head<0>(c, a, ao, off);
+        merge_head<1>(c, a, ao, off);
+        merge_head<2>(c, a, ao, off);
+        merge_head<3>(c, a, ao, off);
+      }
+    }
+  }
+};
+
+template <typename T, int NCH>
+__global__ __launch_bounds__(512) void decode_mfma_kernel(const DecodeArgs a) {
+  constexpr int D = 128;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int waves_per_block = blockDim.x >> 6;
+  const int p = blockIdx.x;
+  const int b = blockIdx.y;
+  const int g = blockIdx.z * waves_per_block + wave;   // kv head
+  const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head
+  const bool direct = (a.num_parts == 1);
+
+  const int ctx = (int)load_ctx(a, b);
+  const int part_start = p * a.part_tokens;
+  if (part_start >= ctx && !(direct && p == 0)) return;
+  const int part_end = min(ctx, part_start + a.part_tokens);
+  const int ntiles = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
+
+  DecodeWave<T, NCH> w;
+  w.init();
+
+  // Q fragments: B operand, column n = lane%16 -> head (n%4) of chunk c, k = 8*(lane/16)+32j
+  {
+    const T* q = reinterpret_cast<const T*>(a.q);
+    const int hq = lane & 3;
+    const int kq = lane >> 4;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int hl = c * 4 + hq;
+      const bool live = hl < group;
+      const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? hl : 0)) * D + kq * 8;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint4 x = *reinterpret_cast<const uint4*>(src + 32 * j);
+        w.qf[c][j] = live ? x : make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
+  }
+
+  const int bs = a.block_size;
+  const int64_t row = (int64_t)a.num_kv_heads * D;       // elements per token row
+  const T* kc = reinterpret_cast<const T*>(a.k_cache) + (int64_t)g * D;
+  const T* vc = reinterpret_cast<const T*>(a.v_cache) + (int64_t)g * D;
+  const int32_t* table = a.block_tables + (int64_t)b * a.max_num_blocks;
+
+  // Block-table window: lane i holds entry (win_base + i) of this sequence.
+  int bi = part_start / bs;          // logical block of the next tile to load
+  int off = part_start - bi * bs;    // token offset inside that block
+  int win_base = bi;
+  int win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
+
+  const int k_lane_off = (lane & 15) * (int)row + (lane >> 4) * 8;   // token lane%16, dims 8*(lane/16)
+  const int v_lane_off = 4 * (lane >> 4) * (int)row + (lane & 15) * 8;  // token 4*(lane/16), dims 8*(lane%16)
+
+  auto load_tile = [&](KVTile<T>& t, int tile) {
+    t.t0 = part_start + tile * kTile;
+    if (bi - win_base >= 64) {
+      win_base = bi;
+      win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
+    }
+    const int phys = __builtin_amdgcn_readlane(win, bi - win_base);
+    t.ok = (bi < a.max_num_blocks) && phys >= 0 && (int64_t)phys < a.num_blocks;
+    if (t.ok) {
+      const int64_t base = ((int64_t)phys * bs + off) * row;
+      const T* kp = kc + base + k_lane_off;
+      const T* vp = vc + base + v_lane_off;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.v[i] = *reinterpret_cast<const uint4*>(vp + (int64_t)i * row);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    off += kTile;
+    if (off >= bs) { off = 0; ++bi; }
+  };
+
+  KVTile<T> ta, tb;
+  if (ntiles > 0) load_tile(ta, 0);
+  int tile = 0;
+  while (tile < ntiles) {
+    if (tile + 1 < ntiles) load_tile(tb, tile + 1);
+    w.consume(ta, part_end, a.scale_log2, lane);
+    ++tile;
+    if (tile >= ntiles) break;
+    if (tile + 1 < ntiles) load_tile(ta, tile + 1);
+    w.consume(tb, part_end, a.scale_log2, lane);
+    ++tile;
+  }
+
+  w.merge_token_classes();
+
+  // Lanes 0..15 (token class 0) now hold dims 8*lane.. for heads 0..3 of every chunk.
+  if (lane < 16) {
+    const int head0 = g * group;
+    if (direct) {
+      T* out = reinterpret_cast<T*>(a.out);
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const float linv = w.l[c] > 0.f ? 1.f / w.l[c] : 0.f;
+        const float li[4] = {quad_bcast<0>(linv), quad_bcast<1>(linv), quad_bcast<2>(linv), quad_bcast<3>(linv)};
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          if (c * 4 + h < group) {
+            T* dst = out + ((int64_t)b * a.num_heads + head0 + c * 4 + h) * D + lane * 8;
+            T o[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = from_float<T>(w.acc[c][h][e] * li[h]);
+            *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(o);
+          }
+        }
+      }
+    } else {
+      const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          if (c * 4 + h < group) {
+            float* dst = a.ws_acc + (slot + c * 4 + h) * D + lane * 8;
+            *reinterpret_cast<float4*>(dst) = make_float4(w.acc[c][h][0], w.acc[c][h][1], w.acc[c][h][2], w.acc[c][h][3]);
+            *reinterpret_cast<float4*>(dst + 4) = make_float4(w.acc[c][h][4], w.acc[c][h][5], w.acc[c][h][6], w.acc[c][h][7]);
+          }
+        }
+        if (lane < 4 && c * 4 + lane < group) {
+          float* ml = a.ws_ml + (slot + c * 4 + lane) * 2;
+          *reinterpret_cast<float2*>(ml) = make_float2(w.m[c], w.l[c]);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Generic path: any element type (fp32 included), head_dim <= 512, any
+// block_size and group size.  One wave per (partition, sequence, q head);
+// lanes split head_dim, one token per step.  Correctness path for shapes the
+// MFMA kernel is not built for.
+// ---------------------------------------------------------------------------
+constexpr int kGenericMaxR = 8;  // head_dim <= 64 * 8
+
+template <typename T, bool INT8>
+__global__ __launch_bounds__(64) void decode_generic_kernel(const DecodeArgs a) {
+  const int lane = threadIdx.x;
+  const int p = blockIdx.x;
+  const int b = blockIdx.y;
+  const int h = blockIdx.z;
+  const int D = a.head_dim;
+  const int group = a.num_heads / a.num_kv_heads;
+  const int g = h / group;
+  const bool direct = (a.num_parts == 1);
+
+  const int ctx = (int)load_ctx(a, b);
+  const int part_start = p * a.part_tokens;
+  if (part_start >= ctx && !(direct && p == 0)) return;
+  const int part_end = min(ctx, part_start + a.part_tokens);
+
+  float qv[kGenericMaxR], acc[kGenericMaxR];
+  const T* q = reinterpret_cast<const T*>(a.q) + ((int64_t)b * a.num_heads + h) * D;
+#pragma unroll
+  for (int r = 0; r < kGenericMaxR; ++r) {
+    const int d = lane + 64 * r;
+    qv[r] = d < D ? to_float(q[d]) : 0.f;
+    acc[r] = 0.f;
+  }
+  float m = -INFINITY, l = 0.f;
+  const int bs = a.block_size;
+  const int32_t* table = a.block_tables + (int64_t)b * a.max_num_blocks;
+  const int64_t row = (int64_t)a.num_kv_heads * D;
+
+  for (int t = part_start; t < part_end; ++t) {
+    const int bi = t / bs;
+    if (bi >= a.max_num_blocks) break;
+    const int phys = table[bi];
+    if (phys < 0 || (int64_t)phys >= a.num_blocks) continue;
+    const int64_t tok = (int64_t)phys * bs + (t - bi * bs);
+    const int64_t base = tok * row + (int64_t)g * D;
+    float kscale = 1.f, vscale = 1.f;
+    if (INT8) {
+      kscale = a.k_scale[tok * a.num_kv_heads + g];
+      vscale = a.v_scale[tok * a.num_kv_heads + g];
+    }
+    float kv[kGenericMaxR], vv[kGenericMaxR];
+    float dot = 0.f;
+#pragma unroll
+    for (int r = 0; r < kGenericMaxR; ++r) {
+      const int d = lane + 64 * r;
+      if (d < D) {
+        if (INT8) {
+          kv[r] = (float)reinterpret_cast<const int8_t*>(a.k_cache)[base + d] * kscale;
+          vv[r] = (float)reinterpret_cast<const int8_t*>(a.v_cache)[base + d] * vscale;
+        } else {
+          kv[r] = to_float(reinterpret_cast<const T*>(a.k_cache)[base + d]);
+          vv[r] = to_float(reinterpret_cast<const T*>(a.v_cache)[base + d]);
+        }
+        dot = fmaf(qv[r], kv[r], dot);
+      } else {
+        vv[r] = 0.f;
+      }
+    }
+    const float s2 = wave_sum(dot) * a.scale_log2;
+    const float m_new = fmaxf(m, s2);
+    const float alpha = safe_exp2_diff(m, m_new);
+    const float pr = fast_exp2(s2 - m_new);
+    l = l * alpha + pr;
+#pragma unroll
+    for (int r = 0; r < kGenericMaxR; ++r) acc[r] = fmaf(pr, vv[r], acc[r] * alpha);
+    m = m_new;
+  }
+
+  if (direct) {
+    T* out = reinterpret_cast<T*>(a.out) + ((int64_t)b * a.num_heads + h) * D;
+    const float linv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+    for (int r = 0; r < kGenericMaxR; ++r) {
+      const int d = lane + 64 * r;
+      if (d < D) out[d] = from_float<T>(acc[r] * linv);
+    }
+  } else {
+    const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + h;
+#pragma unroll
+    for (int r = 0; r < kGenericMaxR; ++r) {
+      const int d = lane + 64 * r;
+      if (d < D) a.ws_acc[slot * D + d] = acc[r];
+    }
+    if (lane == 0) {
+      a.ws_ml[slot * 2] = m;
+      a.ws_ml[slot * 2 + 1] = l;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Second pass: merge the per-partition partials of one (sequence, q head).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(128) void decode_reduce_kernel(const DecodeArgs a) {
+  const int h = blockIdx.x;
+  const int b = blockIdx.y;
+  const int D = a.head_dim;
+  const int ctx = (int)load_ctx(a, b);
+  int np = (ctx + a.part_tokens - 1) / a.part_tokens;
+  if (np > a.num_parts) np = a.num_parts;
+  const int64_t slot0 = ((int64_t)b * a.num_parts) * a.num_heads + h;
+  const int64_t stride = a.num_heads;
+  float mx = -INFINITY;
+  for (int p = 0; p < np; ++p) mx = fmaxf(mx, a.ws_ml[(slot0 + p * stride) * 2]);
+  T* out = reinterpret_cast<T*>(a.out) + ((int64_t)b * a.num_heads + h) * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float o = 0.f, lsum = 0.f;
+    for (int p = 0; p < np; ++p) {
+      const int64_t s = slot0 + p * stride;
+      const float wgt = safe_exp2_diff(a.ws_ml[s * 2], mx);
+      lsum = fmaf(wgt, a.ws_ml[s * 2 + 1], lsum);
+      o = fmaf(wgt, a.ws_acc[s * D + d], o);
+    }
+    out[d] = from_float<T>(lsum > 0.f ? o / lsum : 0.f);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+static int largest_divisor_le(int n, int cap) {
+  for (int d = cap; d >= 1; --d)
+    if (n % d == 0) return d;
+  return 1;
+}
+
+static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int max_num_blocks, int block_size) {
+  if (batch <= 0 || num_heads <= 0 || head_dim <= 0 || max_num_blocks <= 0 || block_size <= 0) return 0;
+  const int64_t max_ctx = (int64_t)max_num_blocks * block_size;
+  const int part = partition_tokens_for(max_ctx);
+  const int64_t np = (max_ctx + part - 1) / part;
+  if (np <= 1) return 0;
+  return (size_t)batch * (size_t)np * (size_t)num_heads * (size_t)(head_dim + 2) * sizeof(float);
+}
+
+template <typename T> struct IsSixteenBit { static constexpr bool value = true; };
+template <> struct IsSixteenBit<float> { static constexpr bool value = false; };
+
+template <typename T>
+static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stream) {
+  const int group = a.num_heads / a.num_kv_heads;
+  bool launched = false;
+  if constexpr (IsSixteenBit<T>::value) {
+    if (fast_ok && !int8) {
+      const int wpb = largest_divisor_le(a.num_kv_heads, 8);
+      dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, (unsigned)(a.num_kv_heads / wpb));
+      dim3 block(64 * wpb);
+      if (group <= 4) decode_mfma_kernel<T, 1><<<grid, block, 0, stream>>>(a);
+      else decode_mfma_kernel<T, 2><<<grid, block, 0, stream>>>(a);
+      launched = true;
+    }
+  }
+  if (!launched) {
+    dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, (unsigned)a.num_heads);
+    if (int8) decode_generic_kernel<T, true><<<grid, dim3(64), 0, stream>>>(a);
+    else decode_generic_kernel<T, false><<<grid, dim3(64), 0, stream>>>(a);
+  }
+  int st = launch_status();
+  if (st != 0) return st;
+  if (a.num_parts > 1) {
+    decode_reduce_kernel<T><<<dim3((unsigned)a.num_heads, (unsigned)a.batch), dim3(128), 0, stream>>>(a);
+    st = launch_status();
+  }
+  return st;
+}
+
+static int decode_entry(void* out, const void* q, const void* k_cache, const void* v_cache,
+                        const float* k_scale, const float* v_scale, bool int8,
+                        const int32_t* block_tables, int max_num_blocks, const void* context_lens,
+                        int ctx_is_i64, int batch, int num_heads, int num_kv_heads, int head_dim,
+                        int block_size, int64_t num_blocks, float scale, int dtype, void* workspace,
+                        size_t workspace_bytes, void* stream) {
+  if (dtype_size(dtype) == 0) return MVLLM_ERR_BAD_DTYPE;
+  if (batch < 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 ||
+      max_num_blocks <= 0 || num_blocks < 0)
+    return MVLLM_ERR_BAD_SHAPE;
+  if (num_heads % num_kv_heads != 0) return MVLLM_ERR_BAD_SHAPE;
+  if (batch == 0) return MVLLM_OK;
+  if (!out || !q || !k_cache || !v_cache || !block_tables || !context_lens) return MVLLM_ERR_NULL_POINTER;
+  if (int8 && (!k_scale || !v_scale)) return MVLLM_ERR_NULL_POINTER;
+  if (head_dim > 64 * kGenericMaxR) return MVLLM_ERR_UNSUPPORTED;
+  if ((int64_t)max_num_blocks * block_size > (int64_t)1 << 30) return MVLLM_ERR_UNSUPPORTED;
+  if (batch > 65535 || num_heads > 65535) return MVLLM_ERR_UNSUPPORTED;
+
+  DecodeArgs a;
+  a.out = out; a.q = q; a.k_cache = k_cache; a.v_cache = v_cache;
+  a.k_scale = k_scale; a.v_scale = v_scale;
+  a.block_tables = block_tables; a.context_lens = context_lens;
+  a.num_blocks = num_blocks; a.ctx_is_i64 = ctx_is_i64; a.max_num_blocks = max_num_blocks;
+  a.batch = batch; a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.head_dim = head_dim;
+  a.block_size = block_size;
+  const int64_t max_ctx = (int64_t)max_num_blocks * block_size;
+  a.part_tokens = partition_tokens_for(max_ctx);
+  a.num_parts = (int)((max_ctx + a.part_tokens - 1) / a.part_tokens);
+  a.scale_log2 = scale * kLog2e;
+  a.ws_acc = nullptr; a.ws_ml = nullptr;
+  if (a.num_parts > 1) {
+    const size_t need = workspace_bytes_for(batch, num_heads, head_dim, max_num_blocks, block_size);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MVLLM_ERR_WORKSPACE;
+    a.ws_acc = reinterpret_cast<float*>(workspace);
+    a.ws_ml = a.ws_acc + (size_t)batch * a.num_parts * num_heads * head_dim;
+  }
+  const int group = num_heads / num_kv_heads;
+  const bool fast_ok = dtype != MVLLM_F32 && head_dim == 128 && block_size % kTile == 0 && group <= 8 &&
+                       aligned16(q) && aligned16(out) && aligned16(k_cache) && aligned16(v_cache) &&
+                       (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case MVLLM_F32: return launch_decode<float>(a, int8, false, s);
+    case MVLLM_BF16: return launch_decode<bf16_t>(a, int8, fast_ok, s);
+    default: return launch_decode<f16_t>(a, int8, fast_ok, s);
+  }
+}
+
+}  // namespace mvllm
+
+using namespace mvllm;
+
+extern "C" size_t mvllm_paged_decode_workspace_bytes(int batch, int num_heads, int head_dim,
+                                                     int max_num_blocks, int block_size) {
+  return workspace_bytes_for(batch, num_heads, head_dim, max_num_blocks, block_size);
+}
+
+extern "C" int mvllm_paged_decode(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                  const int32_t* block_tables, int max_num_blocks, const void* context_lens,
+                                  int ctx_is_i64, int batch, int num_heads, int num_kv_heads, int head_dim,
+                                  int block_size, int64_t num_blocks, float scale, int dtype, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  return decode_entry(out, q, k_cache, v_cache, nullptr, nullptr, false, block_tables, max_num_blocks,
+                      context_lens, ctx_is_i64, batch, num_heads, num_kv_heads, head_dim, block_size,
+                      num_blocks, scale, dtype, workspace, workspace_bytes, stream);
+}
+
+extern "C" int mvllm_paged_decode_int8(void* out, const void* q, const int8_t* k_cache, const int8_t* v_cache,
+                                       const float* k_scale, const float* v_scale, const int32_t* block_tables,
+                                       int max_num_blocks, const void* context_lens, int ctx_is_i64, int batch,
+                                       int num_heads, int num_kv_heads, int head_dim, int block_size,
+                                       int64_t num_blocks, float scale, int dtype, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  return decode_entry(out, q, k_cache, v_cache, k_scale, v_scale, true, block_tables, max_num_blocks,
+                      context_lens, ctx_is_i64, batch, num_heads, num_kv_heads, head_dim, block_size,
+                      num_blocks, scale, dtype, workspace, workspace_bytes, stream);
+}

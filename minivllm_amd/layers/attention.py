@@ -1,0 +1,304 @@
+"""Attention operator layer: the reference's Python surface over gfx950 HIP kernels.
+
+Same public names, argument order, shapes and return conventions as
+src/myvllm/layers/attention.py: ``store_kvcache`` (:67-108),
+``flash_attention_prefill`` (:212-280), ``paged_attention_decode`` (:418-473)
+and the ``Attention`` module (:476-557).  Every operator calls
+libminivllm_amd.so through ctypes on the current torch stream; there is no
+Triton, no PyTorch fallback and no CPU path.
+
+Additions with no counterpart in the reference: the INT8 KV-cache operators
+``store_kvcache_int8`` / ``paged_attention_decode_int8`` and the
+``kv_cache_dtype="int8"`` mode of ``Attention``.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from minivllm_amd import _C
+from minivllm_amd.utils.context import get_context
+
+__all__ = [
+    "store_kvcache", "store_kvcache_int8", "flash_attention_prefill",
+    "paged_attention_decode", "paged_attention_decode_int8", "Attention",
+]
+
+_workspaces: dict = {}   # device index -> uint8 tensor reused by every decode call on that device
+
+
+def _decode_workspace(device: torch.device, nbytes: int):
+    """Split-K scratch for paged decode: grown on demand, never shrunk, one per device."""
+    if nbytes == 0:
+        return None
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _check_cache(name, cache, num_kv_heads, head_dim):
+    if cache.dim() != 4 or cache.shape[2] != num_kv_heads or cache.shape[3] != head_dim:
+        raise ValueError(f"{name} must be [num_blocks, block_size, {num_kv_heads}, {head_dim}], got "
+                         f"{tuple(cache.shape)}")
+    if not cache.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def _slots(slot_mapping):
+    if slot_mapping.dtype != torch.int64:
+        slot_mapping = slot_mapping.to(torch.int64)
+    return slot_mapping.contiguous()
+
+
+def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  slot_mapping: torch.Tensor, block_size: int) -> None:
+    """Scatter K/V token rows into the paged caches (in place).
+
+    key/value: (num_tokens, num_kv_heads, head_dim); k/v_cache:
+    (num_blocks, block_size, num_kv_heads, head_dim); slot_mapping:
+    (num_tokens,) flat slot per token, -1 = skip.  Reference: attention.py:67-108.
+    """
+    num_tokens, num_kv_heads, head_dim = key.shape
+    assert k_cache.shape == v_cache.shape, "K and V cache shapes must match"
+    assert slot_mapping.numel() == num_tokens, "Slot mapping size must match number of tokens"
+    _C.require_cuda(key, value, k_cache, v_cache, slot_mapping)
+    if value.shape != key.shape:
+        raise ValueError("key and value shapes must match")
+    if key.dtype != k_cache.dtype or value.dtype != v_cache.dtype:
+        raise ValueError(f"store_kvcache is a same-dtype copy: key {key.dtype}, cache {k_cache.dtype}")
+    _check_cache("k_cache", k_cache, num_kv_heads, head_dim)
+    _check_cache("v_cache", v_cache, num_kv_heads, head_dim)
+    key = key.contiguous()
+    value = value.contiguous()
+    slots = _slots(slot_mapping)
+    num_slots = k_cache.shape[0] * k_cache.shape[1]
+    lib = _C.load()
+    st = lib.mvllm_store_kvcache(_ptr(key), _ptr(value), _ptr(k_cache), _ptr(v_cache), _ptr(slots),
+                                 num_tokens, num_slots, num_kv_heads, head_dim,
+                                 _C.dtype_code(key.dtype), _C.current_stream_ptr(key.device))
+    _C.check(st, "store_kvcache")
+
+
+def store_kvcache_int8(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                       k_scale: torch.Tensor, v_scale: torch.Tensor, slot_mapping: torch.Tensor,
+                       block_size: int) -> None:
+    """Quantise each (token, kv head) vector to int8 (scale = absmax/127) and scatter.
+
+    k/v_cache: int8 (num_blocks, block_size, Hkv, D); k/v_scale: float32
+    (num_blocks, block_size, Hkv).  Otherwise as ``store_kvcache``.
+    """
+    num_tokens, num_kv_heads, head_dim = key.shape
+    assert k_cache.shape == v_cache.shape, "K and V cache shapes must match"
+    assert slot_mapping.numel() == num_tokens, "Slot mapping size must match number of tokens"
+    _C.require_cuda(key, value, k_cache, v_cache, k_scale, v_scale, slot_mapping)
+    if value.shape != key.shape or value.dtype != key.dtype:
+        raise ValueError("key and value must have the same shape and dtype")
+    if k_cache.dtype != torch.int8 or v_cache.dtype != torch.int8:
+        raise ValueError("int8 caches expected")
+    _check_cache("k_cache", k_cache, num_kv_heads, head_dim)
+    _check_cache("v_cache", v_cache, num_kv_heads, head_dim)
+    for name, s in (("k_scale", k_scale), ("v_scale", v_scale)):
+        if s.dtype != torch.float32 or tuple(s.shape) != tuple(k_cache.shape[:3]) or not s.is_contiguous():
+            raise ValueError(f"{name} must be contiguous float32 {tuple(k_cache.shape[:3])}")
+    key = key.contiguous()
+    value = value.contiguous()
+    slots = _slots(slot_mapping)
+    num_slots = k_cache.shape[0] * k_cache.shape[1]
+    lib = _C.load()
+    st = lib.mvllm_store_kvcache_int8(_ptr(key), _ptr(value), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale),
+                                      _ptr(v_scale), _ptr(slots), num_tokens, num_slots, num_kv_heads,
+                                      head_dim, _C.dtype_code(key.dtype), _C.current_stream_ptr(key.device))
+    _C.check(st, "store_kvcache_int8")
+
+
+def flash_attention_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor,
+                            scale: float, num_heads: int, num_kv_heads: int, head_dim: int) -> torch.Tensor:
+    """Causal attention over a packed ragged batch.  Reference: attention.py:212-280.
+
+    q: (total_tokens, num_heads, head_dim); k, v: (total_tokens, num_kv_heads,
+    head_dim); cu_seqlens: int32 (num_seqs + 1,).  Returns a tensor like q.
+    No device->host synchronisation happens here.
+    """
+    _C.require_cuda(q, k, v, cu_seqlens)
+    if q.dim() != 3 or tuple(q.shape[1:]) != (num_heads, head_dim):
+        raise ValueError(f"q must be (total_tokens, {num_heads}, {head_dim}), got {tuple(q.shape)}")
+    total = q.shape[0]
+    for name, t in (("k", k), ("v", v)):
+        if tuple(t.shape) != (total, num_kv_heads, head_dim):
+            raise ValueError(f"{name} must be ({total}, {num_kv_heads}, {head_dim}), got {tuple(t.shape)}")
+        if t.dtype != q.dtype:
+            raise ValueError("q, k and v must share one dtype")
+    q = q.contiguous()
+    k = k.contiguous()
+    v = v.contiguous()
+    if cu_seqlens.dtype != torch.int32:
+        cu_seqlens = cu_seqlens.to(torch.int32)
+    cu_seqlens = cu_seqlens.contiguous()
+    output = torch.empty_like(q)
+    num_seqs = cu_seqlens.shape[0] - 1
+    lib = _C.load()
+    st = lib.mvllm_prefill_varlen(_ptr(output), _ptr(q), _ptr(k), _ptr(v), _ptr(cu_seqlens), num_seqs, total,
+                                  num_heads, num_kv_heads, head_dim, float(scale), _C.dtype_code(q.dtype),
+                                  _C.current_stream_ptr(q.device))
+    _C.check(st, "flash_attention_prefill")
+    return output
+
+
+def _decode_common(query, k_cache, v_cache, block_tables, context_lens, num_heads, num_kv_heads, head_dim,
+                   block_size):
+    if query.dim() != 3 or tuple(query.shape[1:]) != (num_heads, head_dim):
+        raise ValueError(f"query must be (batch, {num_heads}, {head_dim}), got {tuple(query.shape)}")
+    _check_cache("k_cache", k_cache, num_kv_heads, head_dim)
+    _check_cache("v_cache", v_cache, num_kv_heads, head_dim)
+    if k_cache.shape != v_cache.shape:
+        raise ValueError("K and V cache shapes must match")
+    if k_cache.shape[1] != block_size:
+        raise ValueError(f"cache block dimension {k_cache.shape[1]} != block_size {block_size}")
+    batch = query.shape[0]
+    if block_tables is None or context_lens is None:
+        raise ValueError("block_tables and context_lens must be provided for paged decode")
+    if block_tables.dim() != 2 or block_tables.shape[0] != batch:
+        raise ValueError(f"block_tables must be ({batch}, max_num_blocks), got {tuple(block_tables.shape)}")
+    if context_lens.numel() != batch:
+        raise ValueError("context_lens must have one entry per sequence")
+    if block_tables.dtype != torch.int32:
+        block_tables = block_tables.to(torch.int32)
+    block_tables = block_tables.contiguous()
+    if context_lens.dtype not in (torch.int32, torch.int64):
+        context_lens = context_lens.to(torch.int64)
+    context_lens = context_lens.contiguous()
+    return query.contiguous(), block_tables, context_lens
+
+
+def paged_attention_decode(query: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                           block_tables: torch.Tensor, context_lens: torch.Tensor, scale: float,
+                           num_heads: int, num_kv_heads: int, head_dim: int, block_size: int) -> torch.Tensor:
+    """One query token per sequence over its paged KV.  Reference: attention.py:418-473.
+
+    query: (batch, num_heads, head_dim); caches (num_blocks, block_size, Hkv, D);
+    block_tables int32 (batch, max_num_blocks), -1 padded; context_lens int32 or
+    int64 (batch,).  Returns a tensor like query; rows with context_len 0 are zeros.
+    """
+    _C.require_cuda(query, k_cache, v_cache, block_tables, context_lens)
+    if k_cache.dtype != query.dtype or v_cache.dtype != query.dtype:
+        raise ValueError(f"query {query.dtype} and cache {k_cache.dtype} dtypes differ")
+    query, block_tables, context_lens = _decode_common(query, k_cache, v_cache, block_tables, context_lens,
+                                                       num_heads, num_kv_heads, head_dim, block_size)
+    batch, max_blocks = block_tables.shape
+    output = torch.empty_like(query)
+    if batch == 0:
+        return output
+    lib = _C.load()
+    nbytes = lib.mvllm_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks, block_size)
+    ws = _decode_workspace(query.device, nbytes)
+    st = lib.mvllm_paged_decode(_ptr(output), _ptr(query), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                max_blocks, _ptr(context_lens), int(context_lens.dtype == torch.int64), batch,
+                                num_heads, num_kv_heads, head_dim, block_size, k_cache.shape[0], float(scale),
+                                _C.dtype_code(query.dtype), _ptr(ws), 0 if ws is None else ws.numel(),
+                                _C.current_stream_ptr(query.device))
+    _C.check(st, "paged_attention_decode")
+    return output
+
+
+def paged_attention_decode_int8(query: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                                k_scale: torch.Tensor, v_scale: torch.Tensor, block_tables: torch.Tensor,
+                                context_lens: torch.Tensor, scale: float, num_heads: int, num_kv_heads: int,
+                                head_dim: int, block_size: int) -> torch.Tensor:
+    """Paged decode over an int8 cache written by ``store_kvcache_int8``."""
+    _C.require_cuda(query, k_cache, v_cache, k_scale, v_scale, block_tables, context_lens)
+    if k_cache.dtype != torch.int8 or v_cache.dtype != torch.int8:
+        raise ValueError("int8 caches expected")
+    query, block_tables, context_lens = _decode_common(query, k_cache, v_cache, block_tables, context_lens,
+                                                       num_heads, num_kv_heads, head_dim, block_size)
+    for name, s in (("k_scale", k_scale), ("v_scale", v_scale)):
+        if s.dtype != torch.float32 or tuple(s.shape) != tuple(k_cache.shape[:3]) or not s.is_contiguous():
+            raise ValueError(f"{name} must be contiguous float32 {tuple(k_cache.shape[:3])}")
+    batch, max_blocks = block_tables.shape
+    output = torch.empty_like(query)
+    if batch == 0:
+        return output
+    lib = _C.load()
+    nbytes = lib.mvllm_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks, block_size)
+    ws = _decode_workspace(query.device, nbytes)
+    st = lib.mvllm_paged_decode_int8(_ptr(output), _ptr(query), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale),
+                                     _ptr(v_scale), _ptr(block_tables), max_blocks, _ptr(context_lens),
+                                     int(context_lens.dtype == torch.int64), batch, num_heads, num_kv_heads,
+                                     head_dim, block_size, k_cache.shape[0], float(scale),
+                                     _C.dtype_code(query.dtype), _ptr(ws), 0 if ws is None else ws.numel(),
+                                     _C.current_stream_ptr(query.device))
+    _C.check(st, "paged_attention_decode_int8")
+    return output
+
+
+class Attention(nn.Module):
+    """Dispatches on the engine ``Context``: optional KV store, then varlen
+    prefill or paged decode.  Reference: attention.py:476-557.
+
+    ``k_cache`` / ``v_cache`` are assigned from outside (views of the engine's
+    pool, ``[num_blocks, block_size, Hkv, D]``); until then they are empty and
+    the store is skipped.  With ``kv_cache_dtype="int8"`` the caches are int8
+    and ``k_scale`` / ``v_scale`` (float32 ``[num_blocks, block_size, Hkv]``)
+    must be assigned too.
+    """
+
+    def __init__(self, num_heads: int, head_dim: int, scale: float = 1.0, num_kv_heads: int = None,
+                 block_size: int = 16, kv_cache_dtype: str = "auto"):
+        super().__init__()
+        self.num_heads = num_heads
+        self.head_dim = head_dim
+        self.scale = scale
+        self.num_kv_heads = num_kv_heads if num_kv_heads is not None else num_heads
+        self.block_size = block_size
+        if kv_cache_dtype not in ("auto", "int8"):
+            raise ValueError("kv_cache_dtype must be 'auto' or 'int8'")
+        self.kv_cache_dtype = kv_cache_dtype
+        self.k_cache = self.v_cache = torch.tensor([])
+        self.k_scale = self.v_scale = torch.tensor([])
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+        context = get_context()
+        k_cache, v_cache = self.k_cache, self.v_cache
+        int8 = self.kv_cache_dtype == "int8"
+
+        if k_cache.numel() > 0 and v_cache.numel() > 0 and context.slot_mapping is not None:
+            if k.dim() == 4:      # (B, N, Hkv, D) -> (B*N, Hkv, D)
+                k_rows = k.reshape(-1, k.shape[-2], k.shape[-1])
+                v_rows = v.reshape(-1, v.shape[-2], v.shape[-1])
+            else:
+                k_rows, v_rows = k, v
+            if int8:
+                store_kvcache_int8(k_rows, v_rows, k_cache, v_cache, self.k_scale, self.v_scale,
+                                   context.slot_mapping, self.block_size)
+            else:
+                store_kvcache(k_rows, v_rows, k_cache, v_cache, context.slot_mapping, self.block_size)
+
+        scale = self.scale / (self.head_dim ** 0.5)
+
+        if context.is_prefill:
+            if q.dim() != 3:
+                raise ValueError("prefill expects packed varlen q of shape (total_tokens, num_heads, head_dim); "
+                                 "batched 4-D prefill is not provided")
+            cu_seqlens = context.cu_seqlens_q
+            if cu_seqlens is None:
+                raise ValueError("cu_seqlens_q must be provided for varlen attention")
+            o = flash_attention_prefill(q, k, v, cu_seqlens, scale, self.num_heads, self.num_kv_heads,
+                                        self.head_dim)
+            return o.reshape(o.shape[0], self.num_heads * self.head_dim)
+
+        if q.dim() == 4:          # (B, 1, Hq, D) -> (B, Hq, D)
+            q = q.squeeze(1)
+        if int8:
+            o = paged_attention_decode_int8(q, k_cache, v_cache, self.k_scale, self.v_scale,
+                                            context.block_tables, context.context_lens, scale,
+                                            self.num_heads, self.num_kv_heads, self.head_dim, self.block_size)
+        else:
+            o = paged_attention_decode(q, k_cache, v_cache, context.block_tables, context.context_lens, scale,
+                                       self.num_heads, self.num_kv_heads, self.head_dim, self.block_size)
+        return o.reshape(o.shape[0], self.num_heads * self.head_dim)

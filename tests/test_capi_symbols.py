@@ -1,0 +1,69 @@
+"""The C-ABI library loads and exports every symbol include/minivllm_amd.h declares.
+No compute calls: there is no GPU here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "minivllm_amd.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mvllm_[a-z0-9_]+)\s*\(", text)))
+
+
+def _lib():
+    from minivllm_amd import _C
+    if not os.path.exists(_C.lib_path()):
+        from minivllm_amd._build import build_library
+        build_library(verbose=False)
+    return _C
+
+
+def test_header_declares_expected_entry_points():
+    names = _declared()
+    for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
+              "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_prefill_varlen",
+              "mvllm_version", "mvllm_status_string"]:
+        assert n in names
+
+
+def test_library_exports_every_declared_symbol():
+    _C = _lib()
+    raw = ctypes.CDLL(_C.lib_path())
+    for name in _declared():
+        assert hasattr(raw, name), f"{name} declared in the header but not exported"
+    assert set(_C.SIGNATURES) == set(_declared())
+
+
+def test_host_only_entry_points():
+    _C = _lib()
+    lib = _C.load()
+    assert lib.mvllm_version() >= 1000
+    assert lib.mvllm_status_string(-5).decode().startswith("workspace")
+    # pure host arithmetic: <= 64 partitions of >= 256 tokens, (D + 2) floats per (seq, part, head)
+    assert lib.mvllm_paged_decode_workspace_bytes(8, 16, 128, 16, 16) == 0          # 256 tokens: 1 partition
+    assert lib.mvllm_paged_decode_workspace_bytes(2, 4, 128, 64, 16) == 2 * 4 * 4 * 130 * 4
+    assert lib.mvllm_paged_decode_workspace_bytes(256, 32, 128, 2048, 16) == 256 * 64 * 32 * 130 * 4
+
+
+def test_argument_validation_without_gpu():
+    """Invalid arguments are rejected before any launch, so this is safe on CPU."""
+    _C = _lib()
+    lib = _C.load()
+    assert lib.mvllm_store_kvcache(0, 0, 0, 0, 0, 4, 16, 2, 8, 7, 0) == -2      # bad dtype
+    assert lib.mvllm_store_kvcache(0, 0, 0, 0, 0, 4, 16, 0, 8, 1, 0) == -3      # bad shape
+    assert lib.mvllm_store_kvcache(0, 0, 0, 0, 0, 4, 16, 2, 8, 1, 0) == -1      # null pointers
+    assert lib.mvllm_store_kvcache(0, 0, 0, 0, 0, 0, 16, 2, 8, 1, 0) == 0       # empty is a no-op
+    assert lib.mvllm_store_kvcache_int8(0, 0, 0, 0, 0, 0, 0, 4, 16, 2, 12, 1, 0) == -4   # D % 8 != 0
+    assert lib.mvllm_paged_decode(0, 0, 0, 0, 0, 4, 0, 1, 2, 6, 4, 128, 16, 8, 1.0, 1, 0, 0, 0) == -3  # Hq % Hkv
+    assert lib.mvllm_prefill_varlen(0, 0, 0, 0, 0, 0, 0, 4, 2, 128, 1.0, 1, 0) == 0      # empty batch
+    assert lib.mvllm_prefill_varlen(0, 0, 0, 0, 0, 1, 5, 4, 2, 128, 1.0, 1, 0) == -1
+    with pytest.raises(ValueError):
+        _C.check(-3, "x")
+    with pytest.raises(RuntimeError):
+        _C.check(700, "x")

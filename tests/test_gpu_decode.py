@@ -1,0 +1,189 @@
+"""paged_attention_decode on the GPU vs the CPU oracle.
+
+Tolerances (BASELINE north_star): bf16/fp16 outputs max-abs <= 2e-2 and
+mean-abs <= 2e-3 against the oracle evaluated in fp32 on the same (upcast)
+inputs; fp32 outputs max-abs <= 2e-4."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import error_stats, extract_sequence, make_paged_case, make_paged_case_on_device
+from minivllm_amd.layers.attention import Attention, paged_attention_decode
+from minivllm_amd.utils import reset_context, set_context
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+MAX_ABS_16, MEAN_ABS_16, MAX_ABS_32 = 2e-2, 2e-3, 2e-4
+
+
+def _run(q, kc, vc, tables, ctx, scale, hq, hkv, d, bs, ctx_dtype=torch.int32):
+    out = paged_attention_decode(q.to(DEV), kc.to(DEV), vc.to(DEV), tables.to(DEV), ctx.to(ctx_dtype).to(DEV),
+                                 scale, hq, hkv, d, bs)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def _oracle32(q, kc, vc, tables, ctx, scale, hq, hkv, d, bs):
+    return oracle.decode_naive_oracle(q.float(), kc.float(), vc.float(), tables, ctx, scale, hq, hkv, d, bs)
+
+
+def test_config1_fp32_elementwise():
+    """BASELINE config 1: B 8, ctx U[16,512], Hq16/Hkv8, D128, bs16, fp32 cache, shuffled tables."""
+    hq, hkv, d, bs = 16, 8, 128, 16
+    case = make_paged_case(31, 8, 16, 512, hq, hkv, d, bs)
+    scale = 1 / math.sqrt(d)
+    got = _run(*case, scale, hq, hkv, d, bs)
+    want = oracle.decode_naive_oracle(*case, scale, hq, hkv, d, bs)
+    want2 = oracle.decode_vectorised_oracle(*case, scale, hq, hkv, d, bs)
+    assert got.dtype == torch.float32 and got.shape == want.shape
+    assert error_stats(got, want)[0] <= MAX_ABS_32 and error_stats(got, want2)[0] <= MAX_ABS_32
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,bs,ctx_hi", [
+    (32, 8, 16, 700),      # GQA 4, multi-partition
+    (32, 8, 256, 1500),    # big blocks
+    (16, 8, 16, 255),      # GQA 2, single partition (direct output)
+    (8, 8, 32, 300),       # MHA
+    (32, 4, 16, 600),      # GQA 8 (two head chunks)
+    (6, 2, 48, 500),       # GQA 3, block size not a power of two
+])
+def test_fast_path_vs_oracle(dtype, hq, hkv, bs, ctx_hi):
+    d = 128
+    case = make_paged_case(32, 9, 1, ctx_hi, hq, hkv, d, bs, dtype=dtype)
+    scale = 1 / math.sqrt(d)
+    got = _run(*case, scale, hq, hkv, d, bs, ctx_dtype=torch.int64)
+    want = _oracle32(*case, scale, hq, hkv, d, bs)
+    mx, mean = error_stats(got, want)
+    assert got.dtype == dtype and mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
+@pytest.mark.parametrize("ctx_list", [[1, 2, 15, 16, 17], [255, 256, 257, 511, 512, 513], [31, 32, 33, 1024, 1025]])
+def test_context_length_boundaries(ctx_list):
+    hq, hkv, d, bs = 8, 2, 128, 16
+    case = make_paged_case(33, 0, 0, 0, hq, hkv, d, bs, dtype=torch.bfloat16, ctx_list=ctx_list)
+    got = _run(*case, 0.1, hq, hkv, d, bs)
+    want = _oracle32(*case, 0.1, hq, hkv, d, bs)
+    mx, mean = error_stats(got, want)
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
+@pytest.mark.parametrize("dtype,hq,hkv,d,bs", [
+    (torch.float32, 4, 2, 64, 4),       # generic kernel: fp32
+    (torch.bfloat16, 16, 16, 64, 256),  # head_dim 64 (the reference demo's shape)
+    (torch.float16, 6, 3, 80, 3),       # odd head_dim and block size
+    (torch.bfloat16, 4, 1, 256, 16),
+])
+def test_generic_path_vs_oracle(dtype, hq, hkv, d, bs):
+    case = make_paged_case(34, 5, 1, 400, hq, hkv, d, bs, dtype=dtype)
+    scale = 1 / math.sqrt(d)
+    got = _run(*case, scale, hq, hkv, d, bs)
+    want = _oracle32(*case, scale, hq, hkv, d, bs)
+    mx, mean = error_stats(got, want)
+    if dtype == torch.float32:
+        assert mx <= MAX_ABS_32, mx
+    else:
+        assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
+def test_padded_rows_zero_context_and_missing_blocks():
+    """Graph-replay padding (context_len 0, stale table rows) gives zero rows; tokens whose table entry is -1
+    contribute nothing (attention.py:350-355)."""
+    hq, hkv, d, bs = 8, 2, 128, 16
+    q, kc, vc, tables, ctx = make_paged_case(35, 0, 0, 0, hq, hkv, d, bs, dtype=torch.bfloat16,
+                                             ctx_list=[40, 0, 300, 64])
+    tables[1] = 0                       # stale entries on the padded row
+    got = _run(q, kc, vc, tables, ctx, 0.09, hq, hkv, d, bs)
+    assert torch.count_nonzero(got[1]) == 0 and torch.isfinite(got).all()
+    keep = [0, 2, 3]
+    want = _oracle32(q[keep], kc, vc, tables[keep], ctx[keep], 0.09, hq, hkv, d, bs)
+    assert error_stats(got[keep], want)[0] <= MAX_ABS_16
+    # knock out the 2nd block of sequence 2 (tokens 16..31): same as attending to the other tokens only
+    hole = tables.clone()
+    hole[2, 1] = -1
+    got2 = _run(q, kc, vc, hole, ctx, 0.09, hq, hkv, d, bs)
+    kf, vf = kc.float(), vc.float()
+    rows_k = oracle.gather_sequence_kv(kf, tables[2], 300, bs)
+    rows_v = oracle.gather_sequence_kv(vf, tables[2], 300, bs)
+    sel = torch.cat([torch.arange(0, 16), torch.arange(32, 300)])
+    for h in range(hq):
+        s = (rows_k[sel, h // 4] @ q[2, h].float()) * 0.09
+        want_h = torch.softmax(s, 0) @ rows_v[sel, h // 4]
+        assert (got2[2, h].float() - want_h).abs().max() <= MAX_ABS_16
+    # a sequence whose every block is missing: zeros
+    hole[0, :] = -1
+    got3 = _run(q, kc, vc, hole, ctx, 0.09, hq, hkv, d, bs)
+    assert torch.count_nonzero(got3[0]) == 0
+
+
+def test_block_permutation_and_batch_order_invariance():
+    hq, hkv, d, bs = 32, 8, 128, 16
+    q, kc, vc, tables, ctx = make_paged_case(36, 12, 1, 900, hq, hkv, d, bs, dtype=torch.bfloat16)
+    a = _run(q, kc, vc, tables, ctx, 0.088, hq, hkv, d, bs)
+    perm = torch.randperm(kc.shape[0], generator=torch.Generator().manual_seed(37))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(perm.numel())
+    t2 = torch.where(tables >= 0, inv[tables.clamp(min=0).long()].to(torch.int32), tables)
+    b = _run(q, kc[perm], vc[perm], t2, ctx, 0.088, hq, hkv, d, bs)
+    assert torch.equal(a, b)
+    order = torch.randperm(12, generator=torch.Generator().manual_seed(38))
+    c = _run(q[order], kc, vc, tables[order], ctx[order], 0.088, hq, hkv, d, bs)
+    assert torch.equal(a[order], c)
+
+
+def test_wider_table_same_result():
+    """Split-K invariance: a wider (more -1 padded) block table changes the partitioning, not the result."""
+    hq, hkv, d, bs = 32, 8, 128, 16
+    q, kc, vc, tables, ctx = make_paged_case(39, 6, 1, 1000, hq, hkv, d, bs, dtype=torch.bfloat16)
+    a = _run(q, kc, vc, tables, ctx, 0.088, hq, hkv, d, bs)
+    wide = torch.full((6, 2048), -1, dtype=torch.int32)
+    wide[:, :tables.shape[1]] = tables
+    b = _run(q, kc, vc, wide, ctx, 0.088, hq, hkv, d, bs)
+    want = _oracle32(q, kc, vc, tables, ctx, 0.088, hq, hkv, d, bs)
+    assert error_stats(a, want)[0] <= MAX_ABS_16 and error_stats(b, want)[0] <= MAX_ABS_16
+    assert (a.float() - b.float()).abs().max() <= 4e-3
+
+
+@pytest.mark.parametrize("bs", [16, 256])
+def test_config3_full_size_subset_vs_oracle(bs):
+    """BASELINE config 3: B 256, ctx log-uniform [128, 32768], Hq32/Hkv8/D128 bf16.  The oracle is evaluated on
+    a seeded subset of sequences (the padded formulation does not fit in host memory for all 256)."""
+    hq, hkv, d = 32, 8, 128
+    q, kd, vd, tables, ctx = make_paged_case_on_device(40, DEV, 256, 128, 32768, hq, hkv, d, bs)
+    scale = 1 / math.sqrt(d)
+    td, cd = tables.to(DEV), ctx.to(DEV)
+    got = paged_attention_decode(q, kd, vd, td, cd, scale, hq, hkv, d, bs).cpu()
+    assert torch.isfinite(got).all()
+    pick = [0, 1, 2, int(ctx.argmax()), int(ctx.argmin()), 100, 200, 255]
+    for b in pick:
+        kc, vc, table, c = extract_sequence(kd, vd, tables, ctx, b, bs)
+        want = _oracle32(q[b:b + 1].cpu(), kc, vc, table, c, scale, hq, hkv, d, bs)
+        mx, mean = error_stats(got[b:b + 1], want)
+        assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (b, int(ctx[b]), mx, mean)
+    # size-independent property at full size: linearity in V (attention weights do not depend on V)
+    vd *= 2
+    got2 = paged_attention_decode(q, kd, vd, td, cd, scale, hq, hkv, d, bs).cpu()
+    assert (got2.float() - 2 * got.float()).abs().max() <= 2e-2
+
+
+def test_attention_module_decode_dispatch():
+    hq, hkv, d, bs = 16, 8, 128, 256
+    q, kc, vc, tables, ctx = make_paged_case(41, 5, 1, 352, hq, hkv, d, bs, dtype=torch.bfloat16)
+    layer = Attention(hq, d, 1.0, hkv, bs)
+    layer.k_cache, layer.v_cache = kc.to(DEV), vc.to(DEV)
+    # the new token's K/V is stored first, then decode reads context_len tokens including it
+    g = torch.Generator().manual_seed(42)
+    k_new = torch.randn(5, hkv, d, generator=g).to(torch.bfloat16)
+    v_new = torch.randn(5, hkv, d, generator=g).to(torch.bfloat16)
+    slots = torch.tensor([int(tables[b, (int(ctx[b]) - 1) // bs]) * bs + (int(ctx[b]) - 1) % bs for b in range(5)])
+    set_context(False, slot_mapping=slots.to(DEV), context_lens=ctx.to(DEV), block_tables=tables.to(DEV))
+    out = layer(q.to(DEV), k_new.to(DEV), v_new.to(DEV))
+    reset_context()
+    kc2, vc2 = kc.clone(), vc.clone()
+    oracle.store_kvcache_oracle(k_new, v_new, kc2, vc2, slots, bs)
+    want = _oracle32(q, kc2, vc2, tables, ctx, 1 / math.sqrt(d), hq, hkv, d, bs).reshape(5, hq * d)
+    assert out.shape == (5, hq * d)
+    mx, mean = error_stats(out.cpu(), want)
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16

@@ -1,0 +1,99 @@
+"""flash_attention_prefill on the GPU vs the CPU oracle (tolerances as in test_gpu_decode)."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import error_stats, make_slot_mapping, make_varlen_case
+from minivllm_amd.layers.attention import Attention, flash_attention_prefill, paged_attention_decode
+from minivllm_amd.utils import reset_context, set_context
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+MAX_ABS_16, MEAN_ABS_16, MAX_ABS_32 = 2e-2, 2e-3, 2e-4
+
+
+def _run(q, k, v, cu, scale, hq, hkv, d):
+    out = flash_attention_prefill(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), scale, hq, hkv, d)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def _oracle32(q, k, v, cu, scale, hq, hkv, d):
+    return oracle.prefill_standard_oracle(q.float(), k.float(), v.float(), cu, scale, hq, hkv, d)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("hq,hkv,d,lengths", [
+    (32, 8, 128, [64, 1, 130, 257, 31]),
+    (16, 8, 128, [96, 33, 32, 128]),
+    (8, 8, 128, [200]),
+    (16, 16, 64, [60, 60]),             # the reference demo's head_dim
+    (6, 2, 80, [17, 5]),
+])
+def test_prefill_vs_oracle(dtype, hq, hkv, d, lengths):
+    case = make_varlen_case(51, lengths, hq, hkv, d, dtype=dtype)
+    scale = 1 / math.sqrt(d)
+    got = _run(*case, scale, hq, hkv, d)
+    want = _oracle32(*case, scale, hq, hkv, d)
+    mx, mean = error_stats(got, want)
+    assert got.dtype == dtype and got.shape == want.shape
+    if dtype == torch.float32:
+        assert mx <= MAX_ABS_32, mx
+    else:
+        assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
+def test_prefill_zero_length_sequences_and_independence():
+    hq, hkv, d = 8, 2, 128
+    lengths = [0, 70, 0, 0, 129, 0]
+    q, k, v, cu = make_varlen_case(52, lengths, hq, hkv, d, dtype=torch.bfloat16)
+    got = _run(q, k, v, cu, 0.09, hq, hkv, d)
+    want = _oracle32(q, k, v, cu, 0.09, hq, hkv, d)
+    assert error_stats(got, want)[0] <= MAX_ABS_16
+    # first row of each sequence is exactly its own V row (softmax over one element)
+    for start in (0, 70):
+        for h in range(hq):
+            assert torch.equal(got[start, h], v[start, h // 4])
+    # sequences are independent: changing the second prompt leaves the first bit-identical
+    k2, v2 = k.clone(), v.clone()
+    k2[70:] = 1.0
+    v2[70:] = -1.0
+    got2 = _run(q, k2, v2, cu, 0.09, hq, hkv, d)
+    assert torch.equal(got[:70], got2[:70])
+
+
+def test_config2_full_size():
+    """BASELINE config 2: 16 prompts L U[64,2048], Hq32/Hkv8/D128 bf16; store into block-256 cache; the last
+    row of each prompt must agree with a paged decode of that token over the stored cache."""
+    hq, hkv, d, bs = 32, 8, 128, 256
+    g = torch.Generator().manual_seed(53)
+    lengths = torch.randint(64, 2049, (16,), generator=g).tolist()
+    q, k, v, cu = make_varlen_case(54, lengths, hq, hkv, d, dtype=torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    slots, tables, nb = make_slot_mapping(55, lengths, bs)
+    layer = Attention(hq, d, 1.0, hkv, bs)
+    layer.k_cache = torch.zeros(nb, bs, hkv, d, dtype=torch.bfloat16, device=DEV)
+    layer.v_cache = torch.zeros_like(layer.k_cache)
+    set_context(True, cu.to(DEV), cu.to(DEV), max(lengths), max(lengths), slots.to(DEV), None, None)
+    out = layer(q.to(DEV), k.to(DEV), v.to(DEV))
+    reset_context()
+    assert out.shape == (sum(lengths), hq * d)
+    out = out.cpu().view(-1, hq, d)
+    # oracle on the three shortest and the longest prompt (O(L^2) on CPU)
+    order = sorted(range(16), key=lambda i: lengths[i])
+    for s in order[:3] + order[-1:]:
+        lo, hi = int(cu[s]), int(cu[s + 1])
+        sub_cu = torch.tensor([0, hi - lo], dtype=torch.int32)
+        want = _oracle32(q[lo:hi], k[lo:hi], v[lo:hi], sub_cu, scale, hq, hkv, d)
+        mx, mean = error_stats(out[lo:hi], want)
+        assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (s, hi - lo, mx, mean)
+    # size-independent cross-check over all prompts: last prefill row == decode over the stored cache
+    width = max(len(t) for t in tables)
+    bt = torch.tensor([t + [-1] * (width - len(t)) for t in tables], dtype=torch.int32, device=DEV)
+    last = (cu[1:] - 1).long()
+    dec = paged_attention_decode(q[last].to(DEV), layer.k_cache, layer.v_cache, bt,
+                                 torch.tensor(lengths, device=DEV), scale, hq, hkv, d, bs).cpu()
+    mx, mean = error_stats(dec, out[last])
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)

@@ -1,0 +1,311 @@
+"""Pins the CPU oracle against what the mathematics fixes (the reference has no
+tests, golden vectors or fixtures for this path).  Each check is chosen so a
+plausible slip (dropped scale, wrong GQA map, off-by-one in the causal mask or
+block arithmetic, transposed operand) fails it."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from helpers import make_paged_case, make_slot_mapping, make_varlen_case
+
+
+# ---------------------------------------------------------------- store -----
+def test_store_closed_form_on_poisoned_cache():
+    lengths = [5, 33, 16]
+    bs, hkv, d = 16, 2, 8
+    slots, _, nb = make_slot_mapping(1, lengths, bs)
+    t = sum(lengths)
+    g = torch.Generator().manual_seed(2)
+    key = torch.randn(t, hkv, d, generator=g)
+    val = torch.randn(t, hkv, d, generator=g)
+    slots[7] = -1                                    # a skipped token
+    kc = torch.full((nb, bs, hkv, d), 777.0)
+    vc = torch.full((nb, bs, hkv, d), -777.0)
+    oracle.store_kvcache_oracle(key, val, kc, vc, slots, bs)
+    flat_k, flat_v = kc.view(-1, hkv, d), vc.view(-1, hkv, d)
+    written = torch.zeros(nb * bs, dtype=torch.bool)
+    for i, s in enumerate(slots.tolist()):
+        if s < 0:
+            continue
+        written[s] = True
+        assert torch.equal(flat_k[s], key[i]) and torch.equal(flat_v[s], val[i])
+    assert (flat_k[~written] == 777.0).all() and (flat_v[~written] == -777.0).all()
+    assert written.sum().item() == t - 1
+
+
+def test_store_round_trip_through_block_table():
+    """Store with engine-style slots, gather back by block table: identity."""
+    lengths = [40, 7]
+    bs, hkv, d = 16, 2, 4
+    slots, tables, nb = make_slot_mapping(3, lengths, bs)
+    g = torch.Generator().manual_seed(4)
+    key = torch.randn(sum(lengths), hkv, d, generator=g)
+    val = torch.randn(sum(lengths), hkv, d, generator=g)
+    kc = torch.zeros(nb, bs, hkv, d)
+    vc = torch.zeros(nb, bs, hkv, d)
+    oracle.store_kvcache_oracle(key, val, kc, vc, slots, bs)
+    at = 0
+    for n, blocks in zip(lengths, tables):
+        row = torch.tensor(blocks, dtype=torch.int32)
+        assert torch.equal(oracle.gather_sequence_kv(kc, row, n, bs), key[at:at + n])
+        assert torch.equal(oracle.gather_sequence_kv(vc, row, n, bs), val[at:at + n])
+        at += n
+
+
+# --------------------------------------------------------------- decode -----
+def _brute_force_decode(q, kc, vc, tables, ctx, scale, hq, hkv, bs):
+    out = torch.zeros(q.shape, dtype=torch.float64)
+    rep = hq // hkv
+    for b in range(q.shape[0]):
+        for h in range(hq):
+            g = h // rep
+            scores, rows = [], []
+            for t in range(int(ctx[b])):
+                blk = int(tables[b, t // bs])
+                kvec = kc[blk, t % bs, g].double()
+                scores.append(float((q[b, h].double() * kvec).sum()) * scale)
+                rows.append(vc[blk, t % bs, g].double())
+            mx = max(scores)
+            w = [math.exp(s - mx) for s in scores]
+            tot = sum(w)
+            for wi, r in zip(w, rows):
+                out[b, h] += (wi / tot) * r
+    return out
+
+
+@pytest.mark.parametrize("fn", [oracle.decode_naive_oracle, oracle.decode_vectorised_oracle])
+def test_decode_matches_fp64_brute_force(fn):
+    hq, hkv, d, bs = 4, 2, 8, 4
+    q, kc, vc, tables, ctx = make_paged_case(5, 3, 1, 19, hq, hkv, d, bs)
+    scale = 0.37
+    got = fn(q, kc, vc, tables, ctx, scale, hq, hkv, d, bs)
+    want = _brute_force_decode(q, kc, vc, tables, ctx, scale, hq, hkv, bs)
+    assert torch.allclose(got.double(), want, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("fn", [oracle.decode_naive_oracle, oracle.decode_vectorised_oracle])
+def test_decode_special_cases(fn):
+    hq, hkv, d, bs = 4, 2, 8, 4
+    # ctx = 1 -> output is V[token 0] of the shared kv head, whatever q and scale are
+    q, kc, vc, tables, ctx = make_paged_case(6, 2, 1, 1, hq, hkv, d, bs)
+    got = fn(q, kc, vc, tables, ctx, 3.0, hq, hkv, d, bs)
+    for b in range(2):
+        for h in range(hq):
+            assert torch.allclose(got[b, h], vc[int(tables[b, 0]), 0, h // 2], atol=1e-6)
+    # all K rows equal -> uniform mean of the V rows
+    q, kc, vc, tables, ctx = make_paged_case(7, 2, 5, 11, hq, hkv, d, bs)
+    kc[:] = kc[0, 0, 0]
+    got = fn(q, kc, vc, tables, ctx, 1.0, hq, hkv, d, bs)
+    for b in range(2):
+        n = int(ctx[b])
+        rows = oracle.gather_sequence_kv(vc, tables[b], n, bs)
+        for h in range(hq):
+            assert torch.allclose(got[b, h], rows[:, h // 2].mean(0), atol=1e-5)
+
+
+def test_decode_identity_table_equals_dense_sdpa():
+    hq, hkv, d, bs, n = 4, 2, 16, 8, 24
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(2, hq, d, generator=g)
+    kc = torch.randn(6, bs, hkv, d, generator=g)
+    vc = torch.randn(6, bs, hkv, d, generator=g)
+    tables = torch.arange(6, dtype=torch.int32).reshape(2, 3)
+    ctx = torch.tensor([n, n])
+    scale = 1 / math.sqrt(d)
+    got = oracle.decode_naive_oracle(q, kc, vc, tables, ctx, scale, hq, hkv, d, bs)
+    kd = kc.reshape(2, n, hkv, d).repeat_interleave(2, dim=2).transpose(1, 2)
+    vd = vc.reshape(2, n, hkv, d).repeat_interleave(2, dim=2).transpose(1, 2)
+    want = F.scaled_dot_product_attention(q.unsqueeze(2), kd, vd, scale=scale).squeeze(2)
+    assert torch.allclose(got, want, atol=1e-5)
+
+
+def test_decode_block_permutation_invariance_and_agreement():
+    hq, hkv, d, bs = 8, 2, 16, 4
+    q, kc, vc, tables, ctx = make_paged_case(9, 4, 3, 30, hq, hkv, d, bs)
+    a = oracle.decode_naive_oracle(q, kc, vc, tables, ctx, 0.25, hq, hkv, d, bs)
+    b = oracle.decode_vectorised_oracle(q, kc, vc, tables, ctx, 0.25, hq, hkv, d, bs)
+    assert torch.allclose(a, b, atol=1e-6)
+    perm = torch.randperm(kc.shape[0], generator=torch.Generator().manual_seed(10))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(perm.numel())
+    kc2, vc2 = kc[perm], vc[perm]                      # new block j holds old block perm[j]
+    tables2 = torch.where(tables >= 0, inv[tables.clamp(min=0).long()].to(torch.int32), tables)
+    c = oracle.decode_naive_oracle(q, kc2, vc2, tables2, ctx, 0.25, hq, hkv, d, bs)
+    assert torch.equal(a, c)
+
+
+# -------------------------------------------------------------- prefill -----
+def test_prefill_matches_library_sdpa_and_row0():
+    hq, hkv, d = 4, 2, 16
+    lengths = [1, 7, 33, 12]
+    q, k, v, cu = make_varlen_case(11, lengths, hq, hkv, d)
+    scale = 1 / math.sqrt(d)
+    got = oracle.prefill_standard_oracle(q, k, v, cu, scale, hq, hkv, d)
+    at = 0
+    for n in lengths:
+        qs = q[at:at + n].transpose(0, 1).unsqueeze(0)
+        ks = k[at:at + n].transpose(0, 1).repeat_interleave(2, dim=0).unsqueeze(0)
+        vs = v[at:at + n].transpose(0, 1).repeat_interleave(2, dim=0).unsqueeze(0)
+        want = F.scaled_dot_product_attention(qs, ks, vs, is_causal=True, scale=scale)[0].transpose(0, 1)
+        assert torch.allclose(got[at:at + n], want, atol=1e-5)
+        # first row of a sequence sees only itself
+        for h in range(hq):
+            assert torch.allclose(got[at, h], v[at, h // 2], atol=1e-6)
+        at += n
+
+
+def test_prefill_fp64_brute_force_and_independence():
+    hq, hkv, d = 2, 1, 4
+    lengths = [3, 5]
+    q, k, v, cu = make_varlen_case(12, lengths, hq, hkv, d)
+    scale = 0.8
+    got = oracle.prefill_standard_oracle(q, k, v, cu, scale, hq, hkv, d)
+    at = 0
+    for n in lengths:
+        for i in range(n):
+            for h in range(hq):
+                s = [float((q[at + i, h].double() * k[at + j, 0].double()).sum()) * scale for j in range(i + 1)]
+                mx = max(s)
+                w = [math.exp(x - mx) for x in s]
+                want = sum(wj * v[at + j, 0].double() for j, wj in enumerate(w)) / sum(w)
+                assert torch.allclose(got[at + i, h].double(), want, atol=1e-6)
+        at += n
+    # changing the second prompt leaves the first prompt's rows bit-identical
+    k2, v2 = k.clone(), v.clone()
+    k2[3:] += 1.0
+    v2[3:] -= 2.0
+    got2 = oracle.prefill_standard_oracle(q, k2, v2, cu, scale, hq, hkv, d)
+    assert torch.equal(got[:3], got2[:3])
+
+
+def test_prefill_last_row_equals_decode_after_store():
+    hq, hkv, d, bs = 4, 2, 8, 4
+    lengths = [9, 4]
+    q, k, v, cu = make_varlen_case(13, lengths, hq, hkv, d)
+    slots, tables, nb = make_slot_mapping(14, lengths, bs)
+    kc = torch.zeros(nb, bs, hkv, d)
+    vc = torch.zeros(nb, bs, hkv, d)
+    oracle.store_kvcache_oracle(k, v, kc, vc, slots, bs)
+    width = max(len(t) for t in tables)
+    bt = torch.tensor([t + [-1] * (width - len(t)) for t in tables], dtype=torch.int32)
+    last = torch.tensor([8, 12])
+    pre = oracle.prefill_standard_oracle(q, k, v, cu, 0.5, hq, hkv, d)
+    dec = oracle.decode_naive_oracle(q[last], kc, vc, bt, torch.tensor(lengths), 0.5, hq, hkv, d, bs)
+    assert torch.allclose(pre[last], dec, atol=1e-6)
+
+
+# ----------------------------------------------------------------- int8 -----
+def test_int8_spec_invariants():
+    g = torch.Generator().manual_seed(15)
+    x = torch.randn(64, 4, 128, generator=g)
+    x[torch.rand(x.shape, generator=g) < 0.01] *= 8.0
+    x[3, 1] = 0.0                                      # an all-zero vector
+    codes, scale = oracle.quantize_int8_oracle(x)
+    assert codes.dtype == torch.int8 and scale.dtype == torch.float32
+    amax = x.abs().amax(-1)
+    assert torch.equal(scale, amax / torch.tensor(127.0))          # bit-equal fp32 division
+    assert codes.abs().max().item() <= 127
+    live = amax > 0
+    assert (codes.abs().amax(-1)[live] == 127).all()               # the absmax element maps to +-127
+    assert (codes[3, 1] == 0).all() and scale[3, 1] == 0
+    err = (x - codes.float() * scale.unsqueeze(-1)).abs()
+    assert (err <= scale.unsqueeze(-1) * 0.5 * (1 + 1e-5)).all()
+    # sign symmetry and round-half-even on exact ties
+    c2, s2 = oracle.quantize_int8_oracle(-x)
+    assert torch.equal(c2, -codes) and torch.equal(s2, scale)
+    t = torch.tensor([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5, 3.49, 0.0]])
+    ct, st = oracle.quantize_int8_oracle(t)
+    assert st.item() == 1.0 and ct.tolist() == [[127, 0, 2, 2, 0, -2, 3, 0]]
+
+
+def test_int8_store_then_decode_close_to_fp32():
+    hq, hkv, d, bs = 4, 2, 32, 4
+    lengths = [13, 6]
+    g = torch.Generator().manual_seed(16)
+    k = torch.randn(sum(lengths), hkv, d, generator=g)
+    v = torch.randn(sum(lengths), hkv, d, generator=g)
+    slots, tables, nb = make_slot_mapping(17, lengths, bs)
+    kc = torch.zeros(nb, bs, hkv, d, dtype=torch.int8)
+    vc = torch.zeros_like(kc)
+    ks = torch.zeros(nb, bs, hkv)
+    vs = torch.zeros_like(ks)
+    oracle.store_kvcache_int8_oracle(k, v, kc, vc, ks, vs, slots, bs)
+    kf = torch.zeros(nb, bs, hkv, d)
+    vf = torch.zeros_like(kf)
+    oracle.store_kvcache_oracle(k, v, kf, vf, slots, bs)
+    width = max(len(t) for t in tables)
+    bt = torch.tensor([t + [-1] * (width - len(t)) for t in tables], dtype=torch.int32)
+    q = torch.randn(2, hq, d, generator=g)
+    ctx = torch.tensor(lengths)
+    a = oracle.decode_int8_oracle(q, kc, vc, ks, vs, bt, ctx, 0.2, hq, hkv, d, bs)
+    b = oracle.decode_naive_oracle(q, kf, vf, bt, ctx, 0.2, hq, hkv, d, bs)
+    assert (a - b).abs().max().item() < 0.05
+    assert torch.equal(oracle.dequantize_cache_oracle(kc, ks).view(-1, hkv, d)[slots],
+                       oracle.quantize_int8_oracle(k)[0].float() * oracle.quantize_int8_oracle(k)[1].unsqueeze(-1))
+
+
+# ------------------------------------------------------------ producers -----
+def test_prefill_metadata_reference_example():
+    """model_runner.py:174-179: three prompts of 3, 2, 4 tokens -> cu_seqlens_q [0,3,5,9]."""
+    bs = 4
+    seqs = [dict(num_tokens=3, num_cached_tokens=0, block_table=[5]),
+            dict(num_tokens=2, num_cached_tokens=0, block_table=[2]),
+            dict(num_tokens=4, num_cached_tokens=0, block_table=[7])]
+    md = oracle.prefill_metadata_oracle(seqs, bs)
+    assert md["cu_seqlens_q"] == [0, 3, 5, 9] and md["cu_seqlens_k"] == [0, 3, 5, 9]
+    assert md["slot_mapping"] == [20, 21, 22, 8, 9, 28, 29, 30, 31]
+    assert md["max_seqlen_q"] == 4 and md["block_tables"] is None
+
+
+def test_prefill_metadata_with_cached_prefix():
+    bs = 4
+    seqs = [dict(num_tokens=10, num_cached_tokens=4, block_table=[3, 9, 1]),
+            dict(num_tokens=2, num_cached_tokens=0, block_table=[6])]
+    md = oracle.prefill_metadata_oracle(seqs, bs)
+    assert md["cu_seqlens_q"] == [0, 6, 8] and md["cu_seqlens_k"] == [0, 10, 12]
+    assert md["slot_mapping"] == [36, 37, 38, 39, 4, 5, 24, 25]
+    assert md["block_tables"] == [[3, 9, 1], [6, -1, -1]]
+    assert md["token_ranges"] == [(4, 10), (0, 2)]
+
+
+def test_decode_metadata_hand_worked():
+    bs = 4
+    seqs = [dict(num_tokens=5, block_table=[2, 8], last_token=11),     # 5th token -> block 8 offset 0
+            dict(num_tokens=4, block_table=[3], last_token=12),        # exact multiple -> block 3 offset 3
+            dict(num_tokens=11, block_table=[0, 1, 7], last_token=13)]
+    md = oracle.decode_metadata_oracle(seqs, bs)
+    assert md["slot_mapping"] == [32, 15, 30]
+    assert md["context_lens"] == [5, 4, 11] and md["input_ids"] == [11, 12, 13]
+    assert md["block_tables"] == [[2, 8, -1], [3, -1, -1], [0, 1, 7]]
+
+
+def test_metadata_slots_unique_and_owned():
+    from hypothesis import given, settings, strategies as st
+
+    @settings(max_examples=60, deadline=None)
+    @given(st.lists(st.integers(1, 70), min_size=1, max_size=6), st.sampled_from([1, 4, 16]))
+    def run(lengths, bs):
+        at, seqs = 0, []
+        for n in lengths:
+            nb = -(-n // bs)
+            seqs.append(dict(num_tokens=n, num_cached_tokens=0, block_table=list(range(at, at + nb)),
+                             last_token=0))
+            at += nb
+        md = oracle.prefill_metadata_oracle(seqs, bs)
+        slots = md["slot_mapping"]
+        assert len(slots) == sum(lengths) == md["cu_seqlens_q"][-1]
+        assert len(set(slots)) == len(slots)
+        pos = 0
+        for s in seqs:
+            for i in range(s["num_tokens"]):
+                assert slots[pos] == s["block_table"][i // bs] * bs + i % bs
+                pos += 1
+        dm = oracle.decode_metadata_oracle(seqs, bs)
+        for s, slot in zip(seqs, dm["slot_mapping"]):
+            n = s["num_tokens"]
+            assert slot == s["block_table"][(n - 1) // bs] * bs + (n - 1) % bs
+
+    run()
