@@ -36,6 +36,9 @@ def parse_args():
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
     ap.add_argument("--only", default="", help="comma list out of decode,decode256,prefill,store,cpu to restrict the run")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
+                         "--pmc run can scale FETCH_SIZE / WRITE_SIZE against a kernel of known traffic")
     return ap.parse_args()
 
 
@@ -196,6 +199,13 @@ def main():
     from minivllm_amd import _C
     _C.load()
 
+    if args.calib_copy:
+        src = torch.ones(1 << 30, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     only = set(x for x in args.only.split(",") if x)
     want = lambda name: not only or name in only
     extra = {}
