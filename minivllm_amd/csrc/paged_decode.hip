@@ -21,9 +21,20 @@
 
 namespace mvllm {
 
-constexpr int kTile = 16;            // tokens per MFMA tile
-constexpr int kMaxParts = 64;        // split-K partitions per sequence (upper bound)
-constexpr int kMinPartTokens = 256;  // smallest partition
+// Tuning constants (overridable at compile time for experiments).
+#ifndef MVLLM_DECODE_MAX_PARTS
+#define MVLLM_DECODE_MAX_PARTS 32
+#endif
+#ifndef MVLLM_DECODE_MIN_PART
+#define MVLLM_DECODE_MIN_PART 256
+#endif
+#ifndef MVLLM_DECODE_WAVES_PER_EU
+#define MVLLM_DECODE_WAVES_PER_EU 2
+#endif
+
+constexpr int kTile = 16;                                 // tokens per MFMA tile
+constexpr int kMaxParts = MVLLM_DECODE_MAX_PARTS;         // split-K partitions per sequence (upper bound)
+constexpr int kMinPartTokens = MVLLM_DECODE_MIN_PART;     // smallest partition
 constexpr float kLazyRescale = 8.f;  // rescale accumulators only when the max grows by > 2^8
 
 struct DecodeArgs {
@@ -204,13 +215,20 @@ struct DecodeWave {
 };
 
 template <typename T, int NCH>
-__global__ __launch_bounds__(512) void decode_mfma_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_kernel(const DecodeArgs a) {
   constexpr int D = 128;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int waves_per_block = blockDim.x >> 6;
-  const int p = blockIdx.x;
   const int b = blockIdx.y;
+  // Rotate the partition index by the sequence index: workgroups are dealt to the 8 XCDs
+  // round-robin by linear id, and without the rotation every short sequence (only partition 0
+  // live) would land on the same XCD.
+#ifndef MVLLM_DECODE_NO_SWIZZLE
+  const int p = (int)((blockIdx.x + (unsigned)b) % (unsigned)a.num_parts);
+#else
+  const int p = blockIdx.x;
+#endif
   const int g = blockIdx.z * waves_per_block + wave;   // kv head
   const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head
   const bool direct = (a.num_parts == 1);
@@ -350,8 +368,8 @@ constexpr int kGenericMaxR = 8;  // head_dim <= 64 * 8
 template <typename T, bool INT8>
 __global__ __launch_bounds__(64) void decode_generic_kernel(const DecodeArgs a) {
   const int lane = threadIdx.x;
-  const int p = blockIdx.x;
   const int b = blockIdx.y;
+  const int p = (int)((blockIdx.x + (unsigned)b) % (unsigned)a.num_parts);   // see decode_mfma_kernel
   const int h = blockIdx.z;
   const int D = a.head_dim;
   const int group = a.num_heads / a.num_kv_heads;
@@ -442,27 +460,56 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(const DecodeArgs a) 
 // Second pass: merge the per-partition partials of one (sequence, q head).
 // ---------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(128) void decode_reduce_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(256) void decode_reduce_kernel(const DecodeArgs a) {
+  __shared__ float s_max[4];
+  __shared__ float s_l[4];
+  __shared__ float s_acc[4][64 * kGenericMaxR];
   const int h = blockIdx.x;
   const int b = blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
   const int D = a.head_dim;
   const int ctx = (int)load_ctx(a, b);
   int np = (ctx + a.part_tokens - 1) / a.part_tokens;
   if (np > a.num_parts) np = a.num_parts;
   const int64_t slot0 = ((int64_t)b * a.num_parts) * a.num_heads + h;
   const int64_t stride = a.num_heads;
-  float mx = -INFINITY;
-  for (int p = 0; p < np; ++p) mx = fmaxf(mx, a.ws_ml[(slot0 + p * stride) * 2]);
-  T* out = reinterpret_cast<T*>(a.out) + ((int64_t)b * a.num_heads + h) * D;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float o = 0.f, lsum = 0.f;
-    for (int p = 0; p < np; ++p) {
-      const int64_t s = slot0 + p * stride;
-      const float wgt = safe_exp2_diff(a.ws_ml[s * 2], mx);
-      lsum = fmaf(wgt, a.ws_ml[s * 2 + 1], lsum);
-      o = fmaf(wgt, a.ws_acc[s * D + d], o);
+
+  // global max over the partitions
+  float mloc = -INFINITY;
+  for (int p = threadIdx.x; p < np; p += 256) mloc = fmaxf(mloc, a.ws_ml[(slot0 + p * stride) * 2]);
+  mloc = wave_max(mloc);
+  if (lane == 0) s_max[wave] = mloc;
+  __syncthreads();
+  const float mx = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+
+  // wave w folds partitions w, w+4, ...; lane owns dims lane + 64 r
+  float acc[kGenericMaxR];
+#pragma unroll
+  for (int r = 0; r < kGenericMaxR; ++r) acc[r] = 0.f;
+  float lsum = 0.f;
+#pragma unroll 4
+  for (int p = wave; p < np; p += 4) {
+    const int64_t s = slot0 + p * stride;
+    const float2 ml = *reinterpret_cast<const float2*>(a.ws_ml + s * 2);
+    const float wgt = safe_exp2_diff(ml.x, mx);
+    lsum = fmaf(wgt, ml.y, lsum);
+#pragma unroll
+    for (int r = 0; r < kGenericMaxR; ++r) {
+      const int d = lane + 64 * r;
+      if (d < D) acc[r] = fmaf(wgt, a.ws_acc[s * D + d], acc[r]);
     }
-    out[d] = from_float<T>(lsum > 0.f ? o / lsum : 0.f);
+  }
+#pragma unroll
+  for (int r = 0; r < kGenericMaxR; ++r) s_acc[wave][lane + 64 * r] = acc[r];
+  if (lane == 0) s_l[wave] = lsum;
+  __syncthreads();
+  T* out = reinterpret_cast<T*>(a.out) + ((int64_t)b * a.num_heads + h) * D;
+  const float ltot = s_l[0] + s_l[1] + s_l[2] + s_l[3];
+  const float linv = ltot > 0.f ? 1.f / ltot : 0.f;
+  for (int d = threadIdx.x; d < D; d += 256) {
+    const float o = s_acc[0][d] + s_acc[1][d] + s_acc[2][d] + s_acc[3][d];
+    out[d] = from_float<T>(o * linv);
   }
 }
 
@@ -509,7 +556,7 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stre
   int st = launch_status();
   if (st != 0) return st;
   if (a.num_parts > 1) {
-    decode_reduce_kernel<T><<<dim3((unsigned)a.num_heads, (unsigned)a.batch), dim3(128), 0, stream>>>(a);
+    decode_reduce_kernel<T><<<dim3((unsigned)a.num_heads, (unsigned)a.batch), dim3(256), 0, stream>>>(a);
     st = launch_status();
   }
   return st;

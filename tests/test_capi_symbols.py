@@ -45,10 +45,10 @@ def test_host_only_entry_points():
     lib = _C.load()
     assert lib.mvllm_version() >= 1000
     assert lib.mvllm_status_string(-5).decode().startswith("workspace")
-    # pure host arithmetic: <= 64 partitions of >= 256 tokens, (D + 2) floats per (seq, part, head)
+    # pure host arithmetic: <= 32 partitions of >= 256 tokens, (D + 2) floats per (seq, part, head)
     assert lib.mvllm_paged_decode_workspace_bytes(8, 16, 128, 16, 16) == 0          # 256 tokens: 1 partition
     assert lib.mvllm_paged_decode_workspace_bytes(2, 4, 128, 64, 16) == 2 * 4 * 4 * 130 * 4
-    assert lib.mvllm_paged_decode_workspace_bytes(256, 32, 128, 2048, 16) == 256 * 64 * 32 * 130 * 4
+    assert lib.mvllm_paged_decode_workspace_bytes(256, 32, 128, 2048, 16) == 256 * 32 * 32 * 130 * 4
 
 
 def test_argument_validation_without_gpu():
