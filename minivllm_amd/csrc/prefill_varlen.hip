@@ -112,6 +112,264 @@ __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs 
   }
 }
 
+// ---------------------------------------------------------------------------
+// MFMA path: 16-bit inputs, head_dim 128.
+//
+// Workgroup = 4 waves = (one kv head, HPW of the query heads that share it,
+// 4/HPW consecutive 64-row query tiles); every wave owns 64 query rows of one
+// head.  All waves walk the same 64-row K/V tiles, which are DMA'd from global
+// into LDS once per workgroup (global_load_lds, 16 B per lane, double
+// buffered), so K/V traffic is shared by the GQA group inside the tile.
+//
+// Per wave and K/V tile (all MFMA 32x32x16):
+//   S^T[kv][q]  = K (A operand, ds_read_b128 from LDS) x Q^T (B operand, registers)
+//                 -> lane l holds query row l%32, kv rows 8*(r/4) + 4*(l/32) + r%4
+//   softmax       one query row per lane: no cross-lane work except one
+//                 xor-32 max; base-2, lazy rescale
+//   O^T[d][q]  += V^T (A operand, ds_read_b64_tr_b16 transposing loads) x P^T
+//                 (B operand = the S^T accumulators packed to 16 bit in place)
+// The contraction index of the second product is permuted so that P needs no
+// data movement: k-slot (l/32, e) of step s is kv = 16 s + 8 (e/4) + 4 (l/32) + e%4.
+// LDS rows are 256 B; 16-byte chunks are xor-swizzled (K: by row%16, V: by
+// 4*(row%4)) so both access patterns spread over all banks.  Causal tiles past
+// the diagonal are never visited; only the diagonal tile is masked.
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(4))) short v4s;
+typedef __attribute__((ext_vector_type(2))) float v2f;
+typedef __attribute__((ext_vector_type(2))) __bf16 v2bf16;
+typedef __attribute__((ext_vector_type(2))) _Float16 v2f16;
+
+constexpr int kBN = 64;                 // K/V rows per LDS tile
+constexpr int kWaveRows = 64;           // query rows per wave
+constexpr int kTileBytes = kBN * 256;   // one K (or V) tile, head_dim 128 x 2 B
+
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
+  v2f x = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, v2bf16));
+}
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
+  v2f x = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, v2f16));
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+template <typename T, int HPW>
+__global__ __launch_bounds__(256, 1) void prefill_mfma_kernel(const PrefillArgs a) {
+  constexpr int D = 128;
+  constexpr int ROW_TILES = 4 / HPW;            // 64-row query tiles per workgroup
+  constexpr int BM = kWaveRows * ROW_TILES;     // query rows per workgroup
+  __shared__ __attribute__((aligned(1024))) char lds_k[2][kTileBytes];
+  __shared__ __attribute__((aligned(1024))) char lds_v[2][kTileBytes];
+
+  int seq_start, seq_len, row0;
+  // heaviest (latest) tiles are dispatched first
+  if (!locate_tile(a.cu_seqlens, a.num_seqs, (int)(gridDim.x - 1 - blockIdx.x), BM, seq_start, seq_len, row0)) return;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int group = a.num_heads / a.num_kv_heads;
+  const int chunks = group / HPW;                    // workgroups per kv head
+  const int g = blockIdx.y / chunks;                 // kv head
+  const int h = g * group + (blockIdx.y % chunks) * HPW + (wave % HPW);   // query head of this wave
+  const int r0 = row0 + kWaveRows * (wave / HPW);    // first query row of this wave (inside the sequence)
+  const bool active = r0 < seq_len;
+  const int jd = r0 / kBN;                           // diagonal K/V tile of this wave
+  const int wg_last = min(row0 + BM, seq_len) - 1;
+  const int ntiles = wg_last / kBN + 1;
+  const int l32 = lane & 31;
+  const int hi = lane >> 5;                          // 0/1: which half of the k-slots / rows
+
+  const T* q = reinterpret_cast<const T*>(a.q);
+  const char* kg = reinterpret_cast<const char*>(a.k);
+  const char* vg = reinterpret_cast<const char*>(a.v);
+  const int64_t kv_row_bytes = (int64_t)a.num_kv_heads * D * 2;
+  const int64_t last_token = a.total_tokens - 1;
+
+  // Q fragments (B operand): column = query row 32*tq + l32, k = 16*ks + 8*hi ..
+  uint4 qf[2][8];
+#pragma unroll
+  for (int tq = 0; tq < 2; ++tq) {
+    int64_t tok = (int64_t)seq_start + r0 + 32 * tq + l32;
+    if (tok > last_token) tok = last_token;
+    const T* src = q + (tok * a.num_heads + h) * D + 8 * hi;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[tq][ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
+  }
+
+  v16f o[4][2];
+#pragma unroll
+  for (int td = 0; td < 4; ++td)
+#pragma unroll
+    for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[td][tq][r] = 0.f;
+  float m[2] = {-INFINITY, -INFINITY};
+  float l[2] = {0.f, 0.f};
+
+  // ---- K/V tile DMA: wave w moves rows 16w..16w+15 (4 instructions x 4 rows) of K and of V
+  const int ld_row = lane >> 4;        // row inside the 4-row group
+  const int ld_chunk = lane & 15;      // destination chunk inside the row
+  auto issue_tile = [&](int j, int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 16 * wave + 4 * i + ld_row;          // row inside the tile
+      int64_t tok = (int64_t)seq_start + (int64_t)j * kBN + row;
+      if (tok > last_token) tok = last_token;
+      const int kc = ld_chunk ^ (row & 15);
+      const int vc = ld_chunk ^ ((row & 3) << 2);
+      const char* ksrc = kg + tok * kv_row_bytes + (int64_t)g * (D * 2) + kc * 16;
+      const char* vsrc = vg + tok * kv_row_bytes + (int64_t)g * (D * 2) + vc * 16;
+      char* kdst = &lds_k[buf][(16 * wave + 4 * i) * 256];
+      char* vdst = &lds_v[buf][(16 * wave + 4 * i) * 256];
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)ksrc, (lds_ptr_t)kdst, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)vsrc, (lds_ptr_t)vdst, 16, 0, 0);
+    }
+  };
+
+  issue_tile(0, 0);
+  for (int j = 0; j < ntiles; ++j) {
+    const int buf = j & 1;
+    __builtin_amdgcn_s_waitcnt(0);     // this wave's share of tile j has landed
+    __syncthreads();                   // ... and everybody else's; tile j-1 is no longer read
+    if (j + 1 < ntiles) issue_tile(j + 1, buf ^ 1);
+    if (!active || j > jd) continue;
+
+    // ---- S^T = K Q^T ----
+    v16f s[2][2];
+#pragma unroll
+    for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[tq][tk][r] = 0.f;
+    const char* kb = lds_k[buf];
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk) {
+      const int row = 32 * tk + l32;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const int c = 2 * ks + hi;
+        const uint4 kf = *reinterpret_cast<const uint4*>(kb + row * 256 + ((c ^ (row & 15)) << 4));
+        s[0][tk] = mfma32x32x16<T>(kf, qf[0][ks], s[0][tk]);
+        s[1][tk] = mfma32x32x16<T>(kf, qf[1][ks], s[1][tk]);
+      }
+    }
+
+    // ---- online softmax, one query row per lane ----
+    const bool diag = (j == jd);
+#pragma unroll
+    for (int tq = 0; tq < 2; ++tq) {
+      const int qrow = r0 + 32 * tq + l32;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float x = s[tq][tk][r] * a.scale_log2;
+          if (diag) {
+            const int kv = j * kBN + 32 * tk + 8 * (r >> 2) + 4 * hi + (r & 3);
+            if (kv > qrow) x = -INFINITY;
+          }
+          s[tq][tk][r] = x;
+          mx = fmaxf(mx, x);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const bool grow = mx > m[tq] + 8.f || m[tq] == -INFINITY;
+      if (__any(grow)) {
+        const float m_new = grow ? mx : m[tq];
+        const float alpha = (m_new == m[tq]) ? 1.f : fast_exp2(m[tq] - m_new);   // exp2(-inf) = 0 on the first tile
+        l[tq] *= alpha;
+#pragma unroll
+        for (int td = 0; td < 4; ++td)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[td][tq][r] *= alpha;
+        m[tq] = m_new;
+      }
+      float sum = 0.f;
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float pv = fast_exp2(s[tq][tk][r] - m[tq]);
+          s[tq][tk][r] = pv;
+          sum += pv;
+        }
+      l[tq] += sum;       // partial: this lane's kv rows only; lanes l and l^32 are added at the end
+    }
+
+    // ---- O^T += V^T P^T ----
+    const char* vb = lds_v[buf];
+    const int i16 = lane & 15;
+    const int half = (lane >> 4) & 1;
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        uint4 pf[2];
+#pragma unroll
+        for (int tq = 0; tq < 2; ++tq) {
+          pf[tq].x = pack2<T>(s[tq][tk][8 * st + 0], s[tq][tk][8 * st + 1]);
+          pf[tq].y = pack2<T>(s[tq][tk][8 * st + 2], s[tq][tk][8 * st + 3]);
+          pf[tq].z = pack2<T>(s[tq][tk][8 * st + 4], s[tq][tk][8 * st + 5]);
+          pf[tq].w = pack2<T>(s[tq][tk][8 * st + 6], s[tq][tk][8 * st + 7]);
+        }
+        const int kvrow = 32 * tk + 16 * st + 4 * hi + (i16 >> 2);
+        const int swz = (kvrow & 3) << 2;
+#pragma unroll
+        for (int td = 0; td < 4; ++td) {
+          const int c = (4 * td + 2 * half + ((i16 & 3) >> 1)) ^ swz;
+          const char* p0 = vb + kvrow * 256 + (c << 4) + ((i16 & 1) << 3);
+          const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
+          const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * 256));
+          uint4 af;
+          af.x = __builtin_bit_cast(uint2, a0).x; af.y = __builtin_bit_cast(uint2, a0).y;
+          af.z = __builtin_bit_cast(uint2, a1).x; af.w = __builtin_bit_cast(uint2, a1).y;
+          o[td][0] = mfma32x32x16<T>(af, pf[0], o[td][0]);
+          o[td][1] = mfma32x32x16<T>(af, pf[1], o[td][1]);
+        }
+      }
+    }
+  }
+
+  if (!active) return;
+  // ---- epilogue: normalise and store; lane holds row 32*tq + l32, dims 32*td + 8*(r/4) + 4*hi + r%4 ----
+  T* out = reinterpret_cast<T*>(a.out);
+#pragma unroll
+  for (int tq = 0; tq < 2; ++tq) {
+    const int qrow = r0 + 32 * tq + l32;
+    const float lt = l[tq] + __shfl_xor(l[tq], 32, 64);
+    const float inv = 1.f / lt;
+    if (qrow < seq_len) {
+      T* dst = out + ((int64_t)(seq_start + qrow) * a.num_heads + h) * D + 4 * hi;
+#pragma unroll
+      for (int td = 0; td < 4; ++td)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          uint2 w;
+          w.x = pack2<T>(o[td][tq][4 * r4 + 0] * inv, o[td][tq][4 * r4 + 1] * inv);
+          w.y = pack2<T>(o[td][tq][4 * r4 + 2] * inv, o[td][tq][4 * r4 + 3] * inv);
+          *reinterpret_cast<uint2*>(dst + 32 * td + 8 * r4) = w;
+        }
+    }
+  }
+}
+
+template <typename T>
+static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
+  const int group = a.num_heads / a.num_kv_heads;
+  const int hpw = group >= 4 ? 4 : group;              // 1, 2 or 4 (group is 1, 2 or a multiple of 4)
+  const int bm = kWaveRows * (4 / hpw);
+  const int64_t tiles = a.total_tokens / bm + a.num_seqs;
+  dim3 grid((unsigned)tiles, (unsigned)(a.num_kv_heads * (group / hpw)));
+  if (hpw == 4) prefill_mfma_kernel<T, 4><<<grid, dim3(256), 0, stream>>>(a);
+  else if (hpw == 2) prefill_mfma_kernel<T, 2><<<grid, dim3(256), 0, stream>>>(a);
+  else prefill_mfma_kernel<T, 1><<<grid, dim3(256), 0, stream>>>(a);
+  return launch_status();
+}
+
 template <typename T>
 static int launch_prefill_generic(const PrefillArgs& a, hipStream_t stream) {
   const int64_t tiles = a.total_tokens / kGenRows + a.num_seqs;
@@ -140,6 +398,11 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   a.total_tokens = total_tokens; a.num_seqs = num_seqs; a.num_heads = num_heads;
   a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
   hipStream_t s = (hipStream_t)stream;
+  const int group = num_heads / num_kv_heads;
+  const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 && (group == 1 || group == 2 || group % 4 == 0) &&
+                       aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
+                       num_kv_heads * group <= 65535;
+  if (mfma_ok) return dtype == MVLLM_BF16 ? launch_prefill_mfma<bf16_t>(a, s) : launch_prefill_mfma<f16_t>(a, s);
   switch (dtype) {
     case MVLLM_F32: return launch_prefill_generic<float>(a, s);
     case MVLLM_BF16: return launch_prefill_generic<bf16_t>(a, s);
