@@ -115,9 +115,9 @@ __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs 
 // ---------------------------------------------------------------------------
 // MFMA path: 16-bit inputs, head_dim 128.
 //
-// Workgroup = 4 waves = (one kv head, HPW of the query heads that share it,
-// 4/HPW consecutive 64-row query tiles); every wave owns 64 query rows of one
-// head.  All waves walk the same 64-row K/V tiles, which are DMA'd from global
+// Workgroup = 8 waves = (one kv head, HPW of the query heads that share it,
+// 8/HPW consecutive 32-row query tiles); every wave owns 32 query rows of one
+// head; two waves per SIMD so one wave's softmax overlaps the other's MFMAs.  All waves walk the same 64-row K/V tiles, which are DMA'd from global
 // into LDS once per workgroup (global_load_lds, 16 B per lane, double
 // buffered), so K/V traffic is shared by the GQA group inside the tile.
 //
@@ -140,7 +140,7 @@ typedef __attribute__((ext_vector_type(2))) __bf16 v2bf16;
 typedef __attribute__((ext_vector_type(2))) _Float16 v2f16;
 
 constexpr int kBN = 64;                 // K/V rows per LDS tile
-constexpr int kWaveRows = 64;           // query rows per wave
+constexpr int kWaveRows = 32;           // query rows per wave
 constexpr int kTileBytes = kBN * 256;   // one K (or V) tile, head_dim 128 x 2 B
 
 template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
@@ -153,13 +153,22 @@ template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, v2f16));
 }
 
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+// 16 bytes per lane from global straight into LDS at lds_base + 16 * lane (global_load_lds_dwordx4).
+// Written as inline asm on purpose: the compiler then neither tracks the transfer in vmcnt nor
+// inserts a full vmcnt(0) wait before the next LDS read, so the copy of tile j+1 really overlaps
+// the math on tile j; completion is awaited explicitly with dma_wait_all() before the barrier.
+__device__ __forceinline__ void dma16_to_lds(const void* gsrc, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gsrc) : "memory");
+}
+__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
 
 template <typename T, int HPW>
-__global__ __launch_bounds__(256, 1) void prefill_mfma_kernel(const PrefillArgs a) {
+__global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs a) {
   constexpr int D = 128;
-  constexpr int ROW_TILES = 4 / HPW;            // 64-row query tiles per workgroup
+  constexpr int ROW_TILES = 8 / HPW;            // 32-row query tiles per workgroup
   constexpr int BM = kWaveRows * ROW_TILES;     // query rows per workgroup
   __shared__ __attribute__((aligned(1024))) char lds_k[2][kTileBytes];
   __shared__ __attribute__((aligned(1024))) char lds_v[2][kTileBytes];
@@ -181,6 +190,7 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_kernel(const PrefillArgs 
   const int ntiles = wg_last / kBN + 1;
   const int l32 = lane & 31;
   const int hi = lane >> 5;                          // 0/1: which half of the k-slots / rows
+  const int qrow = r0 + l32;                         // query row of this lane
 
   const T* q = reinterpret_cast<const T*>(a.q);
   const char* kg = reinterpret_cast<const char*>(a.k);
@@ -188,172 +198,168 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_kernel(const PrefillArgs 
   const int64_t kv_row_bytes = (int64_t)a.num_kv_heads * D * 2;
   const int64_t last_token = a.total_tokens - 1;
 
-  // Q fragments (B operand): column = query row 32*tq + l32, k = 16*ks + 8*hi ..
-  uint4 qf[2][8];
-#pragma unroll
-  for (int tq = 0; tq < 2; ++tq) {
-    int64_t tok = (int64_t)seq_start + r0 + 32 * tq + l32;
-    if (tok > last_token) tok = last_token;
-    const T* src = q + (tok * a.num_heads + h) * D + 8 * hi;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[tq][ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
-  }
-
-  v16f o[4][2];
-#pragma unroll
-  for (int td = 0; td < 4; ++td)
-#pragma unroll
-    for (int tq = 0; tq < 2; ++tq)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[td][tq][r] = 0.f;
-  float m[2] = {-INFINITY, -INFINITY};
-  float l[2] = {0.f, 0.f};
-
-  // ---- K/V tile DMA: wave w moves rows 16w..16w+15 (4 instructions x 4 rows) of K and of V
+  // ---- K/V tile DMA: wave w moves rows 8w..8w+7 (2 instructions x 4 rows) of K and of V
   const int ld_row = lane >> 4;        // row inside the 4-row group
   const int ld_chunk = lane & 15;      // destination chunk inside the row
   auto issue_tile = [&](int j, int buf) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = 16 * wave + 4 * i + ld_row;          // row inside the tile
+    for (int i = 0; i < 2; ++i) {
+      const int row = 8 * wave + 4 * i + ld_row;           // row inside the tile
       int64_t tok = (int64_t)seq_start + (int64_t)j * kBN + row;
       if (tok > last_token) tok = last_token;
       const int kc = ld_chunk ^ (row & 15);
       const int vc = ld_chunk ^ ((row & 3) << 2);
       const char* ksrc = kg + tok * kv_row_bytes + (int64_t)g * (D * 2) + kc * 16;
       const char* vsrc = vg + tok * kv_row_bytes + (int64_t)g * (D * 2) + vc * 16;
-      char* kdst = &lds_k[buf][(16 * wave + 4 * i) * 256];
-      char* vdst = &lds_v[buf][(16 * wave + 4 * i) * 256];
-      __builtin_amdgcn_global_load_lds((gbl_ptr_t)ksrc, (lds_ptr_t)kdst, 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gbl_ptr_t)vsrc, (lds_ptr_t)vdst, 16, 0, 0);
+      const uint32_t kdst = __builtin_amdgcn_readfirstlane(lds_address(&lds_k[buf][(8 * wave + 4 * i) * 256]));
+      const uint32_t vdst = __builtin_amdgcn_readfirstlane(lds_address(&lds_v[buf][(8 * wave + 4 * i) * 256]));
+      dma16_to_lds(ksrc, kdst);
+      dma16_to_lds(vsrc, vdst);
     }
   };
-
   issue_tile(0, 0);
+
+  // Q fragments (B operand): column = query row l32, k = 16*ks + 8*hi ..
+  uint4 qf[8];
+  {
+    int64_t tok = (int64_t)seq_start + qrow;
+    if (tok > last_token) tok = last_token;
+    const T* src = q + (tok * a.num_heads + h) * D + 8 * hi;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
+  }
+  // Make the compiler retire the Q loads here: otherwise it carries "Q may still be in flight" into
+  // the loop and its vmcnt waits there would also wait for the tile prefetch.
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) asm volatile("" ::"v"(qf[ks].x), "v"(qf[ks].w));
+
+  v16f o[4];
+#pragma unroll
+  for (int td = 0; td < 4; ++td)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[td][r] = 0.f;
+  float m = -INFINITY;
+  float l = 0.f;
+
+  // per-lane constant parts of the LDS addresses
+  const int k_row_off = l32 * 256;                         // K: row l32 (+32*tk), chunk (2*ks+hi) ^ (row&15)
+  const int k_swz = l32 & 15;
+  const int i16 = lane & 15;
+  const int half = (lane >> 4) & 1;
+  const int v_row = 4 * hi + (i16 >> 2);                   // V: row 32*tk + 16*st + v_row (+8)
+  const int v_swz = (v_row & 3) << 2;
+  const int v_chunk = 2 * half + ((i16 & 3) >> 1);         // + 4*td
+  const int v_byte = (i16 & 1) << 3;
+
   for (int j = 0; j < ntiles; ++j) {
     const int buf = j & 1;
-    __builtin_amdgcn_s_waitcnt(0);     // this wave's share of tile j has landed
+    dma_wait_all();                    // this wave's share of tile j has landed
     __syncthreads();                   // ... and everybody else's; tile j-1 is no longer read
     if (j + 1 < ntiles) issue_tile(j + 1, buf ^ 1);
     if (!active || j > jd) continue;
+    const bool diag = (j == jd);
+    // on the diagonal tile a wave whose rows sit in the first half never sees kv rows 32..63
+    const int ntk = (diag && (r0 & 32) == 0) ? 1 : 2;
 
     // ---- S^T = K Q^T ----
-    v16f s[2][2];
-#pragma unroll
-    for (int tq = 0; tq < 2; ++tq)
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[tq][tk][r] = 0.f;
+    v16f s[2];
     const char* kb = lds_k[buf];
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk) {
-      const int row = 32 * tk + l32;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const int c = 2 * ks + hi;
-        const uint4 kf = *reinterpret_cast<const uint4*>(kb + row * 256 + ((c ^ (row & 15)) << 4));
-        s[0][tk] = mfma32x32x16<T>(kf, qf[0][ks], s[0][tk]);
-        s[1][tk] = mfma32x32x16<T>(kf, qf[1][ks], s[1][tk]);
+      for (int r = 0; r < 16; ++r) s[tk][r] = 0.f;
+      if (tk < ntk) {
+        uint4 kf[8];
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+          kf[ks] = *reinterpret_cast<const uint4*>(kb + tk * 32 * 256 + k_row_off + (((2 * ks + hi) ^ k_swz) << 4));
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) s[tk] = mfma32x32x16<T>(kf[ks], qf[ks], s[tk]);
       }
     }
 
     // ---- online softmax, one query row per lane ----
-    const bool diag = (j == jd);
+    float mx = -INFINITY;
 #pragma unroll
-    for (int tq = 0; tq < 2; ++tq) {
-      const int qrow = r0 + 32 * tq + l32;
-      float mx = -INFINITY;
+    for (int tk = 0; tk < 2; ++tk)
 #pragma unroll
-      for (int tk = 0; tk < 2; ++tk)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float x = s[tq][tk][r] * a.scale_log2;
-          if (diag) {
-            const int kv = j * kBN + 32 * tk + 8 * (r >> 2) + 4 * hi + (r & 3);
-            if (kv > qrow) x = -INFINITY;
-          }
-          s[tq][tk][r] = x;
-          mx = fmaxf(mx, x);
+      for (int r = 0; r < 16; ++r) {
+        float x = s[tk][r] * a.scale_log2;
+        if (diag) {
+          const int kv = j * kBN + 32 * tk + 8 * (r >> 2) + 4 * hi + (r & 3);
+          if (kv > qrow) x = -INFINITY;
         }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const bool grow = mx > m[tq] + 8.f || m[tq] == -INFINITY;
-      if (__any(grow)) {
-        const float m_new = grow ? mx : m[tq];
-        const float alpha = (m_new == m[tq]) ? 1.f : fast_exp2(m[tq] - m_new);   // exp2(-inf) = 0 on the first tile
-        l[tq] *= alpha;
-#pragma unroll
-        for (int td = 0; td < 4; ++td)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) o[td][tq][r] *= alpha;
-        m[tq] = m_new;
+        s[tk][r] = x;
+        mx = fmaxf(mx, x);
       }
-      float sum = 0.f;
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const bool grow = mx > m + 8.f || m == -INFINITY;
+    if (__any(grow)) {
+      const float m_new = grow ? mx : m;
+      const float alpha = (m_new == m) ? 1.f : fast_exp2(m - m_new);   // exp2(-inf) = 0 on the first tile
+      l *= alpha;
 #pragma unroll
-      for (int tk = 0; tk < 2; ++tk)
+      for (int td = 0; td < 4; ++td)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float pv = fast_exp2(s[tq][tk][r] - m[tq]);
-          s[tq][tk][r] = pv;
-          sum += pv;
-        }
-      l[tq] += sum;       // partial: this lane's kv rows only; lanes l and l^32 are added at the end
+        for (int r = 0; r < 16; ++r) o[td][r] *= alpha;
+      m = m_new;
     }
+    float sum = 0.f;
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pv = fast_exp2(s[tk][r] - m);
+        s[tk][r] = pv;
+        sum += pv;
+      }
+    l += sum;       // partial: this lane's kv rows only; lanes l and l^32 are added at the end
 
     // ---- O^T += V^T P^T ----
     const char* vb = lds_v[buf];
-    const int i16 = lane & 15;
-    const int half = (lane >> 4) & 1;
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk) {
+      if (tk < ntk) {
 #pragma unroll
-      for (int st = 0; st < 2; ++st) {
-        uint4 pf[2];
+        for (int st = 0; st < 2; ++st) {
+          uint4 pf;
+          pf.x = pack2<T>(s[tk][8 * st + 0], s[tk][8 * st + 1]);
+          pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
+          pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
+          pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
+          const char* vrow = vb + (32 * tk + 16 * st + v_row) * 256 + v_byte;
+          uint4 af[4];
 #pragma unroll
-        for (int tq = 0; tq < 2; ++tq) {
-          pf[tq].x = pack2<T>(s[tq][tk][8 * st + 0], s[tq][tk][8 * st + 1]);
-          pf[tq].y = pack2<T>(s[tq][tk][8 * st + 2], s[tq][tk][8 * st + 3]);
-          pf[tq].z = pack2<T>(s[tq][tk][8 * st + 4], s[tq][tk][8 * st + 5]);
-          pf[tq].w = pack2<T>(s[tq][tk][8 * st + 6], s[tq][tk][8 * st + 7]);
-        }
-        const int kvrow = 32 * tk + 16 * st + 4 * hi + (i16 >> 2);
-        const int swz = (kvrow & 3) << 2;
+          for (int td = 0; td < 4; ++td) {
+            const char* p0 = vrow + (((4 * td + v_chunk) ^ v_swz) << 4);
+            const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
+            const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * 256));
+            af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;
+            af[td].z = __builtin_bit_cast(uint2, a1).x; af[td].w = __builtin_bit_cast(uint2, a1).y;
+          }
 #pragma unroll
-        for (int td = 0; td < 4; ++td) {
-          const int c = (4 * td + 2 * half + ((i16 & 3) >> 1)) ^ swz;
-          const char* p0 = vb + kvrow * 256 + (c << 4) + ((i16 & 1) << 3);
-          const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
-          const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * 256));
-          uint4 af;
-          af.x = __builtin_bit_cast(uint2, a0).x; af.y = __builtin_bit_cast(uint2, a0).y;
-          af.z = __builtin_bit_cast(uint2, a1).x; af.w = __builtin_bit_cast(uint2, a1).y;
-          o[td][0] = mfma32x32x16<T>(af, pf[0], o[td][0]);
-          o[td][1] = mfma32x32x16<T>(af, pf[1], o[td][1]);
+          for (int td = 0; td < 4; ++td) o[td] = mfma32x32x16<T>(af[td], pf, o[td]);
         }
       }
     }
   }
 
   if (!active) return;
-  // ---- epilogue: normalise and store; lane holds row 32*tq + l32, dims 32*td + 8*(r/4) + 4*hi + r%4 ----
+  // ---- epilogue: normalise and store; lane holds row l32, dims 32*td + 8*(r/4) + 4*hi + r%4 ----
   T* out = reinterpret_cast<T*>(a.out);
+  const float lt = l + __shfl_xor(l, 32, 64);
+  const float inv = 1.f / lt;
+  if (qrow < seq_len) {
+    T* dst = out + ((int64_t)(seq_start + qrow) * a.num_heads + h) * D + 4 * hi;
 #pragma unroll
-  for (int tq = 0; tq < 2; ++tq) {
-    const int qrow = r0 + 32 * tq + l32;
-    const float lt = l[tq] + __shfl_xor(l[tq], 32, 64);
-    const float inv = 1.f / lt;
-    if (qrow < seq_len) {
-      T* dst = out + ((int64_t)(seq_start + qrow) * a.num_heads + h) * D + 4 * hi;
+    for (int td = 0; td < 4; ++td)
 #pragma unroll
-      for (int td = 0; td < 4; ++td)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          uint2 w;
-          w.x = pack2<T>(o[td][tq][4 * r4 + 0] * inv, o[td][tq][4 * r4 + 1] * inv);
-          w.y = pack2<T>(o[td][tq][4 * r4 + 2] * inv, o[td][tq][4 * r4 + 3] * inv);
-          *reinterpret_cast<uint2*>(dst + 32 * td + 8 * r4) = w;
-        }
-    }
+      for (int r4 = 0; r4 < 4; ++r4) {
+        uint2 w;
+        w.x = pack2<T>(o[td][4 * r4 + 0] * inv, o[td][4 * r4 + 1] * inv);
+        w.y = pack2<T>(o[td][4 * r4 + 2] * inv, o[td][4 * r4 + 3] * inv);
+        *reinterpret_cast<uint2*>(dst + 32 * td + 8 * r4) = w;
+      }
   }
 }
 
@@ -361,15 +367,14 @@ template <typename T>
 static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   const int group = a.num_heads / a.num_kv_heads;
   const int hpw = group >= 4 ? 4 : group;              // 1, 2 or 4 (group is 1, 2 or a multiple of 4)
-  const int bm = kWaveRows * (4 / hpw);
+  const int bm = kWaveRows * (8 / hpw);
   const int64_t tiles = a.total_tokens / bm + a.num_seqs;
   dim3 grid((unsigned)tiles, (unsigned)(a.num_kv_heads * (group / hpw)));
-  if (hpw == 4) prefill_mfma_kernel<T, 4><<<grid, dim3(256), 0, stream>>>(a);
-  else if (hpw == 2) prefill_mfma_kernel<T, 2><<<grid, dim3(256), 0, stream>>>(a);
-  else prefill_mfma_kernel<T, 1><<<grid, dim3(256), 0, stream>>>(a);
+  if (hpw == 4) prefill_mfma_kernel<T, 4><<<grid, dim3(512), 0, stream>>>(a);
+  else if (hpw == 2) prefill_mfma_kernel<T, 2><<<grid, dim3(512), 0, stream>>>(a);
+  else prefill_mfma_kernel<T, 1><<<grid, dim3(512), 0, stream>>>(a);
   return launch_status();
 }
-
 template <typename T>
 static int launch_prefill_generic(const PrefillArgs& a, hipStream_t stream) {
   const int64_t tiles = a.total_tokens / kGenRows + a.num_seqs;
