@@ -22,25 +22,43 @@ struct PrefillArgs {
   int num_kv_heads;
   int head_dim;
   float scale_log2;
+  int tiles_x;      // MFMA path: query-tile upper bound (total_tokens / BM + num_seqs)
+  int heads_y;      // MFMA path: head slices (kv heads x query-head chunks)
 };
 
-// Tile `tile` (global numbering) -> sequence and first row inside it.
+// Tile `tile` (global numbering) -> sequence and first row inside it.  Wave-parallel: 64 sequences
+// per step (tile counts, inclusive prefix sum by shuffles, ballot to pick the owner), so the cost is
+// a few hundred cycles per 64 sequences instead of one dependent load per sequence.  Every lane of
+// the calling wave must be active; all lanes return the same values.
 __device__ __forceinline__ bool locate_tile(const int32_t* __restrict__ cu, int num_seqs, int tile, int bm,
                                             int& seq_start, int& seq_len, int& row0) {
+  const int lane = threadIdx.x & 63;
   int first = 0;
-  int prev = cu[0];
-  for (int s = 0; s < num_seqs; ++s) {
-    const int next = cu[s + 1];
-    const int len = next - prev;
+  for (int base = 0; base < num_seqs; base += 64) {
+    const int s = base + lane;
+    int lo = 0, len = 0;
+    if (s < num_seqs) {
+      lo = cu[s];
+      len = cu[s + 1] - lo;
+    }
     const int n = (len + bm - 1) / bm;
-    if (tile < first + n) {
-      seq_start = prev;
-      seq_len = len;
-      row0 = (tile - first) * bm;
+    int incl = n;                                   // inclusive prefix sum of tile counts over the lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += t;
+    }
+    const int total = __shfl(incl, 63, 64);
+    if (tile < first + total) {
+      const unsigned long long owners = __ballot(tile < first + incl);   // first lane whose prefix passes the tile
+      const int owner = __ffsll((long long)owners) - 1;
+      const int start_tile = first + __shfl(incl - n, owner, 64);
+      seq_start = __shfl(lo, owner, 64);
+      seq_len = __shfl(len, owner, 64);
+      row0 = (tile - start_tile) * bm;
       return true;
     }
-    first += n;
-    prev = next;
+    first += total;
   }
   return false;
 }
@@ -139,6 +157,10 @@ typedef __attribute__((ext_vector_type(2))) float v2f;
 typedef __attribute__((ext_vector_type(2))) __bf16 v2bf16;
 typedef __attribute__((ext_vector_type(2))) _Float16 v2f16;
 
+#ifndef MVLLM_PF_XCD_CHUNK
+#define MVLLM_PF_XCD_CHUNK 32
+#endif
+constexpr unsigned kXcdChunk = MVLLM_PF_XCD_CHUNK;   // consecutive work items handed to one XCD
 constexpr int kBN = 64;                 // K/V rows per LDS tile
 constexpr int kWaveRows = 32;           // query rows per wave
 constexpr int kTileBytes = kBN * 256;   // one K (or V) tile, head_dim 128 x 2 B
@@ -173,21 +195,38 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
   __shared__ __attribute__((aligned(1024))) char lds_k[2][kTileBytes];
   __shared__ __attribute__((aligned(1024))) char lds_v[2][kTileBytes];
 
+  // Work item = (head slice y, query tile x), x fastest.  Workgroups are dealt to the 8 XCDs round-robin by
+  // linear id; items are handed out in chunks of kXcdChunk consecutive items per XCD so that workgroups
+  // sharing one sequence's K/V run on the same XCD (same L2) at about the same time.
+  const int tiles_x = a.tiles_x;
+  const unsigned id = blockIdx.x;
+  const unsigned slot = id >> 3, xcd = id & 7;
+  // round q of an XCD takes chunk 8q + (xcd + q) % 8: the rotation spreads the heavy (late-tile) chunks of
+  // a long sequence over all XCDs instead of always handing them to the same one
+  const unsigned round = slot / kXcdChunk;
+  const unsigned item = (round * 8 + ((xcd + round) & 7)) * kXcdChunk + slot % kXcdChunk;
+  if (item >= (unsigned)tiles_x * (unsigned)a.heads_y) return;
+  const int item_y = (int)(item / (unsigned)tiles_x);
+  const int item_x = (int)(item % (unsigned)tiles_x);
   int seq_start, seq_len, row0;
-  // heaviest (latest) tiles are dispatched first
-  if (!locate_tile(a.cu_seqlens, a.num_seqs, (int)(gridDim.x - 1 - blockIdx.x), BM, seq_start, seq_len, row0)) return;
+  // latest (heaviest) tiles of a sequence first
+  if (!locate_tile(a.cu_seqlens, a.num_seqs, tiles_x - 1 - item_x, BM, seq_start, seq_len, row0)) return;
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int group = a.num_heads / a.num_kv_heads;
   const int chunks = group / HPW;                    // workgroups per kv head
-  const int g = blockIdx.y / chunks;                 // kv head
-  const int h = g * group + (blockIdx.y % chunks) * HPW + (wave % HPW);   // query head of this wave
+  const int g = item_y / chunks;                     // kv head
+  const int h = g * group + (item_y % chunks) * HPW + (wave % HPW);   // query head of this wave
   const int r0 = row0 + kWaveRows * (wave / HPW);    // first query row of this wave (inside the sequence)
   const bool active = r0 < seq_len;
   const int jd = r0 / kBN;                           // diagonal K/V tile of this wave
   const int wg_last = min(row0 + BM, seq_len) - 1;
+#ifdef MVLLM_PF_ONETILE
+  const int ntiles = 1;      // experiment only: wrong results
+#else
   const int ntiles = wg_last / kBN + 1;
+#endif
   const int l32 = lane & 31;
   const int hi = lane >> 5;                          // 0/1: which half of the k-slots / rows
   const int qrow = r0 + l32;                         // query row of this lane
@@ -264,35 +303,45 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
     // ---- S^T = K Q^T ----
     v16f s[2];
     const char* kb = lds_k[buf];
+#ifdef MVLLM_PF_PRIO
+    __builtin_amdgcn_s_setprio(MVLLM_PF_PRIO);
+#endif
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[tk][r] = 0.f;
       if (tk < ntk) {
         uint4 kf[8];
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks)
           kf[ks] = *reinterpret_cast<const uint4*>(kb + tk * 32 * 256 + k_row_off + (((2 * ks + hi) ^ k_swz) << 4));
+        const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        s[tk] = mfma32x32x16<T>(kf[0], qf[0], zero);
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) s[tk] = mfma32x32x16<T>(kf[ks], qf[ks], s[tk]);
+        for (int ks = 1; ks < 8; ++ks) s[tk] = mfma32x32x16<T>(kf[ks], qf[ks], s[tk]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[tk][r] = -INFINITY;   // never visited: masked out
       }
     }
+#ifdef MVLLM_PF_PRIO
+    __builtin_amdgcn_s_setprio(0);
+#endif
 
-    // ---- online softmax, one query row per lane ----
+    // ---- online softmax, one query row per lane (scores stay unscaled; the scale is folded
+    //      into the exp2 argument) ----
+    if (diag) {
+      const int thr = qrow - j * kBN - 4 * hi;       // kv offset inside the tile must be <= thr
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (32 * tk + 8 * (r >> 2) + (r & 3) > thr) s[tk][r] = -INFINITY;
+    }
     float mx = -INFINITY;
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float x = s[tk][r] * a.scale_log2;
-        if (diag) {
-          const int kv = j * kBN + 32 * tk + 8 * (r >> 2) + 4 * hi + (r & 3);
-          if (kv > qrow) x = -INFINITY;
-        }
-        s[tk][r] = x;
-        mx = fmaxf(mx, x);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[tk][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * a.scale_log2;
     const bool grow = mx > m + 8.f || m == -INFINITY;
     if (__any(grow)) {
       const float m_new = grow ? mx : m;
@@ -305,11 +354,12 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
       m = m_new;
     }
     float sum = 0.f;
+    const float neg_m = -m;
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float pv = fast_exp2(s[tk][r] - m);
+        const float pv = fast_exp2(fmaf(s[tk][r], a.scale_log2, neg_m));
         s[tk][r] = pv;
         sum += pv;
       }
@@ -317,6 +367,9 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
 
     // ---- O^T += V^T P^T ----
     const char* vb = lds_v[buf];
+#ifdef MVLLM_PF_PRIO
+    __builtin_amdgcn_s_setprio(MVLLM_PF_PRIO);
+#endif
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk) {
       if (tk < ntk) {
@@ -342,15 +395,20 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
         }
       }
     }
+#ifdef MVLLM_PF_PRIO
+    __builtin_amdgcn_s_setprio(0);
+#endif
   }
 
+  // ---- epilogue: normalise, transpose through LDS (the K buffers are free now), store whole rows ----
+  // lane holds row l32, dims 32*td + 8*(r/4) + 4*hi + r%4  ->  wave-private [32 rows][256 B] tile with
+  // 16-byte chunks xor-swizzled by row, read back as 16 B per lane so every global store is a full row.
+  __syncthreads();                                   // every wave is done reading K/V tiles
   if (!active) return;
-  // ---- epilogue: normalise and store; lane holds row l32, dims 32*td + 8*(r/4) + 4*hi + r%4 ----
-  T* out = reinterpret_cast<T*>(a.out);
-  const float lt = l + __shfl_xor(l, 32, 64);
-  const float inv = 1.f / lt;
-  if (qrow < seq_len) {
-    T* dst = out + ((int64_t)(seq_start + qrow) * a.num_heads + h) * D + 4 * hi;
+  char* ot = &lds_k[0][0] + wave * (kWaveRows * 256);   // 8 waves x 8 KB = both K buffers
+  {
+    const float lt = l + __shfl_xor(l, 32, 64);
+    const float inv = 1.f / lt;
 #pragma unroll
     for (int td = 0; td < 4; ++td)
 #pragma unroll
@@ -358,8 +416,22 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
         uint2 w;
         w.x = pack2<T>(o[td][4 * r4 + 0] * inv, o[td][4 * r4 + 1] * inv);
         w.y = pack2<T>(o[td][4 * r4 + 2] * inv, o[td][4 * r4 + 3] * inv);
-        *reinterpret_cast<uint2*>(dst + 32 * td + 8 * r4) = w;
+        *reinterpret_cast<uint2*>(ot + l32 * 256 + (((4 * td + r4) ^ (l32 & 15)) << 4) + 8 * hi) = w;
       }
+  }
+  // wave-private tile: the writes above and the reads below are ordered by the LDS queue of this wave
+  T* out = reinterpret_cast<T*>(a.out);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = 4 * i + (lane >> 4);
+    const int c = lane & 15;
+    const uint4 w = *reinterpret_cast<const uint4*>(ot + row * 256 + ((c ^ (row & 15)) << 4));
+#ifdef MVLLM_PF_NOSTORE
+    if (w.x == 0x12345678u)
+#else
+    if (r0 + row < seq_len)
+#endif
+      *reinterpret_cast<uint4*>(out + ((int64_t)(seq_start + r0 + row) * a.num_heads + h) * D + 8 * c) = w;
   }
 }
 
@@ -368,11 +440,15 @@ static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   const int group = a.num_heads / a.num_kv_heads;
   const int hpw = group >= 4 ? 4 : group;              // 1, 2 or 4 (group is 1, 2 or a multiple of 4)
   const int bm = kWaveRows * (8 / hpw);
-  const int64_t tiles = a.total_tokens / bm + a.num_seqs;
-  dim3 grid((unsigned)tiles, (unsigned)(a.num_kv_heads * (group / hpw)));
-  if (hpw == 4) prefill_mfma_kernel<T, 4><<<grid, dim3(512), 0, stream>>>(a);
-  else if (hpw == 2) prefill_mfma_kernel<T, 2><<<grid, dim3(512), 0, stream>>>(a);
-  else prefill_mfma_kernel<T, 1><<<grid, dim3(512), 0, stream>>>(a);
+  PrefillArgs b = a;
+  b.tiles_x = (int)(a.total_tokens / bm + a.num_seqs);
+  b.heads_y = a.num_kv_heads * (group / hpw);
+  const int64_t items = (int64_t)b.tiles_x * b.heads_y;
+  const int64_t span = 8 * (int64_t)kXcdChunk;
+  dim3 grid((unsigned)((items + span - 1) / span * span));
+  if (hpw == 4) prefill_mfma_kernel<T, 4><<<grid, dim3(512), 0, stream>>>(b);
+  else if (hpw == 2) prefill_mfma_kernel<T, 2><<<grid, dim3(512), 0, stream>>>(b);
+  else prefill_mfma_kernel<T, 1><<<grid, dim3(512), 0, stream>>>(b);
   return launch_status();
 }
 template <typename T>
@@ -402,6 +478,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   a.out = out; a.q = q; a.k = k; a.v = v; a.cu_seqlens = cu_seqlens;
   a.total_tokens = total_tokens; a.num_seqs = num_seqs; a.num_heads = num_heads;
   a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
+  a.tiles_x = 0; a.heads_y = 0;
   hipStream_t s = (hipStream_t)stream;
   const int group = num_heads / num_kv_heads;
   const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 && (group == 1 || group == 2 || group % 4 == 0) &&
