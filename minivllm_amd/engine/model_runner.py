@@ -1,0 +1,100 @@
+"""Model runner: builds the model and the paged KV pool, turns scheduled sequences into the per-step
+``Context`` and runs one engine step (src/myvllm/engine/model_runner.py:14-308, single GPU, no process
+group, no SHM workers).
+
+Config keys (one set of names; the reference's runner and engine disagree on two of them): model keys
+``vocab_size hidden_size num_layers num_heads num_kv_heads head_dim intermediate_size base
+rms_norm_epsilon qkv_bias ffn_bias scale tie_word_embeddings max_position``; engine keys ``block_size
+max_cached_blocks max_num_sequences max_num_batched_tokens dtype kv_cache_dtype seed``.
+"""
+from __future__ import annotations
+
+import torch
+
+from minivllm_amd.engine.metadata import decode_metadata, prefill_metadata
+from minivllm_amd.layers.basic import Sampler
+from minivllm_amd.models.qwen3 import Qwen3ForCausalLM
+from minivllm_amd.utils.context import reset_context, set_context
+
+_DTYPES = {"bf16": torch.bfloat16, "bfloat16": torch.bfloat16, "fp16": torch.float16, "float16": torch.float16,
+           "fp32": torch.float32, "float32": torch.float32}
+
+
+class ModelRunner:
+    def __init__(self, config: dict, device: str = "cuda:0"):
+        self.config = config
+        self.device = torch.device(device)
+        self.block_size = config.get("block_size", 256)
+        self.num_blocks = config.get("max_cached_blocks", 1024)
+        self.dtype = _DTYPES[config.get("dtype", "bf16")]
+        self.kv_cache_dtype = config.get("kv_cache_dtype", "auto")
+        head_dim = config.get("head_dim") or config["hidden_size"] // config["num_heads"]
+        self.model = Qwen3ForCausalLM(
+            vocab_size=config["vocab_size"], hidden_size=config["hidden_size"], num_heads=config["num_heads"],
+            head_dim=head_dim, scale=config.get("scale", 1.0), num_kv_heads=config.get("num_kv_heads"),
+            rms_norm_epsilon=config.get("rms_norm_epsilon", 1e-6), qkv_bias=config.get("qkv_bias", False),
+            base=config.get("base", 1_000_000), max_position=config.get("max_position", 4096),
+            intermediate_size=config["intermediate_size"], ffn_bias=config.get("ffn_bias", True),
+            num_layers=config["num_layers"], tie_word_embeddings=config.get("tie_word_embeddings", True),
+            block_size=self.block_size, kv_cache_dtype=self.kv_cache_dtype)
+        self.model.reset_parameters(seed=config.get("seed", 0))
+        self.model.to(device=self.device, dtype=self.dtype).eval()
+        self.sampler = Sampler()
+        self.generator = torch.Generator(device=self.device).manual_seed(config.get("seed", 0))
+        self.allocate_kv_cache()
+
+    def allocate_kv_cache(self):
+        """One pool ``[2, L, num_blocks, block_size, Hkv, D]``; each ``Attention`` gets its layer's views
+        (model_runner.py:140-168).  With an INT8 cache a second pool holds the fp32 scales."""
+        cfg = self.config
+        hkv = cfg.get("num_kv_heads") or cfg["num_heads"]
+        d = cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_heads"]
+        layers = cfg["num_layers"]
+        int8 = self.kv_cache_dtype == "int8"
+        self.kv_cache = torch.zeros(2, layers, self.num_blocks, self.block_size, hkv, d,
+                                    dtype=torch.int8 if int8 else self.dtype, device=self.device)
+        self.kv_scale = (torch.zeros(2, layers, self.num_blocks, self.block_size, hkv, dtype=torch.float32,
+                                     device=self.device) if int8 else None)
+        layer_id = 0
+        for module in self.model.modules():
+            if hasattr(module, "k_cache") and hasattr(module, "v_cache"):
+                module.k_cache = self.kv_cache[0, layer_id]
+                module.v_cache = self.kv_cache[1, layer_id]
+                if int8:
+                    module.k_scale = self.kv_scale[0, layer_id]
+                    module.v_scale = self.kv_scale[1, layer_id]
+                layer_id += 1
+        assert layer_id == layers
+
+    def _to_device(self, values, dtype):
+        return torch.tensor(values, dtype=dtype, pin_memory=True).to(self.device, non_blocking=True)
+
+    def prepare_prefill(self, seqs):
+        md = prefill_metadata(seqs, self.block_size, reuse_cached_kv=False)
+        positions = [p for seq in seqs for p in range(len(seq))]
+        set_context(True,
+                    cu_seqlens_q=self._to_device(md["cu_seqlens_q"], torch.int32),
+                    cu_seqlens_k=self._to_device(md["cu_seqlens_k"], torch.int32),
+                    max_seqlen_q=md["max_seqlen_q"], max_seqlen_k=md["max_seqlen_k"],
+                    slot_mapping=self._to_device(md["slot_mapping"], torch.int64),
+                    context_lens=None, block_tables=None)
+        return self._to_device(md["input_ids"], torch.int64), self._to_device(positions, torch.int64)
+
+    def prepare_decode(self, seqs):
+        md = decode_metadata(seqs, self.block_size)
+        context_lens = self._to_device(md["context_lens"], torch.int64)
+        set_context(False,
+                    slot_mapping=self._to_device(md["slot_mapping"], torch.int64),
+                    context_lens=context_lens,
+                    block_tables=self._to_device(md["block_tables"], torch.int32))
+        return self._to_device(md["input_ids"], torch.int64), context_lens - 1
+
+    @torch.inference_mode()
+    def run(self, seqs, is_prefill: bool) -> list[int]:
+        input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
+        temperatures = self._to_device([seq.temperature for seq in seqs], torch.float32)
+        hidden = self.model(input_ids, positions)
+        logits = self.model.compute_logits(hidden)
+        token_ids = self.sampler(logits, temperatures, self.generator).tolist()
+        reset_context()
+        return token_ids

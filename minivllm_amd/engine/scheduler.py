@@ -1,0 +1,78 @@
+"""Prefill-first continuous batching (src/myvllm/engine/scheduler.py:6-82).
+
+Intended semantics where the reference is broken: limits are checked before a
+sequence is popped from ``running`` (the reference pops then breaks, losing
+it, scheduler.py:45,54-55), and ``postprocess`` advances the sequence with
+``append_token`` (the reference appends to ``token_ids`` only, so lengths never
+move, scheduler.py:78-79).
+"""
+from __future__ import annotations
+
+from collections import deque
+
+from minivllm_amd.engine.block_manager import BlockManager
+from minivllm_amd.engine.sequence import Sequence, SequenceStatus
+
+
+class Scheduler:
+    def __init__(self, max_num_sequences: int, max_num_batched_tokens: int, max_cached_blocks: int,
+                 block_size: int, eos: int):
+        self.block_manager = BlockManager(max_cached_blocks, block_size)
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.max_num_sequences = max_num_sequences
+        self.waiting: deque[Sequence] = deque()
+        self.running: deque[Sequence] = deque()
+        self.eos = eos
+
+    def is_finished(self):
+        return not self.waiting and not self.running
+
+    def add_sequence(self, sequence: Sequence):
+        self.waiting.append(sequence)
+
+    def schedule(self) -> tuple[list[Sequence], bool]:
+        scheduled: list[Sequence] = []
+        num_tokens = 0
+        # prefill: admit waiting sequences while blocks, token budget and batch slots last
+        while self.waiting and len(scheduled) < self.max_num_sequences:
+            seq = self.waiting[0]
+            if len(seq) + num_tokens > self.max_num_batched_tokens or not self.block_manager.can_allocate(seq):
+                break
+            self.waiting.popleft()
+            self.block_manager.allocate(seq)
+            seq.status = SequenceStatus.RUNNING
+            self.running.append(seq)
+            scheduled.append(seq)
+            num_tokens += len(seq)
+        if scheduled:
+            return scheduled, True
+
+        # decode: one token for each running sequence, preempting from the tail when blocks run out
+        while self.running and len(scheduled) < self.max_num_sequences and num_tokens < self.max_num_batched_tokens:
+            seq = self.running.popleft()
+            while not self.block_manager.can_append(seq):
+                if self.running:
+                    self.preempt(self.running.pop())
+                else:
+                    self.preempt(seq)
+                    break
+            else:
+                self.block_manager.append(seq)
+                scheduled.append(seq)
+                num_tokens += 1
+        if scheduled:
+            self.running.extendleft(reversed(scheduled))
+        return scheduled, False
+
+    def preempt(self, seq: Sequence) -> None:
+        self.block_manager.deallocate(seq)
+        seq.status = SequenceStatus.WAITING
+        self.waiting.appendleft(seq)
+
+    def postprocess(self, seqs: list[Sequence], token_ids: list[int]) -> None:
+        for seq, token_id in zip(seqs, token_ids):
+            seq.append_token(int(token_id))
+            if (not seq.ignore_eos and token_id == self.eos) or seq.num_completion_tokens >= seq.max_tokens:
+                seq.status = SequenceStatus.FINISHED
+                self.block_manager.deallocate(seq)
+                self.running.remove(seq)

@@ -1,0 +1,60 @@
+"""Plain PyTorch-ROCm counterparts of the reference's small layers (callers of the attention path,
+not kernel targets): RMSNorm with fused residual (layers/layernorm.py:9-28), NeoX half-split RoPE
+(layers/rotary_embedding.py:4-83), SiluAndMul (layers/activation.py:15-18) and the temperature /
+exponential-race sampler (layers/sampler.py:14-19)."""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, size: int, eps: float = 1e-6):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(size))
+        self.eps = eps
+
+    def _norm(self, x):
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + self.eps)
+        return (xf * self.weight.float()).to(x.dtype)
+
+    def forward(self, x, residual=None):
+        if residual is None:
+            return self._norm(x)
+        x = x + residual
+        return self._norm(x), x
+
+
+class RotaryEmbedding(nn.Module):
+    def __init__(self, base: float, rotary_dim: int, max_position: int):
+        super().__init__()
+        inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+        freqs = torch.outer(torch.arange(max_position, dtype=torch.float32), inv_freq)
+        self.register_buffer("cos_sin_cache", torch.cat([freqs.cos(), freqs.sin()], dim=-1), persistent=False)
+
+    @staticmethod
+    def _rotate(x, cos, sin):
+        x1, x2 = x.float().chunk(2, dim=-1)
+        return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).to(x.dtype)
+
+    def forward(self, positions, query, key):
+        cos, sin = self.cos_sin_cache[positions].chunk(2, dim=-1)      # (T, D/2) each, fp32
+        cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
+        return self._rotate(query, cos, sin), self._rotate(key, cos, sin)
+
+
+class SiluAndMul(nn.Module):
+    def forward(self, x):
+        a, b = x.chunk(2, dim=-1)
+        return F.silu(a) * b
+
+
+class Sampler(nn.Module):
+    """argmax(softmax(logits / T) / E), E ~ Exp(1): one draw from the tempered distribution."""
+
+    def forward(self, logits, temperatures, generator=None):
+        probs = torch.softmax(logits.float() / temperatures.unsqueeze(-1), dim=-1)
+        noise = torch.empty_like(probs).exponential_(1.0, generator=generator).clamp_min_(1e-10)
+        return probs.div_(noise).argmax(dim=-1)

@@ -1,0 +1,1 @@
+from .qwen3 import Qwen3ForCausalLM  # noqa: F401

@@ -1,0 +1,171 @@
+"""Engine-side producers on the CPU: sequence block arithmetic, block manager (prefix hashes, ref counts),
+scheduler (prefill-first, preemption, finish) and the per-step metadata vs the producers oracle."""
+import random
+
+import pytest
+import xxhash
+import numpy as np
+
+import oracle
+from minivllm_amd.engine.block_manager import BlockManager
+from minivllm_amd.engine.llm_engine import LLMEngine
+from minivllm_amd.engine.metadata import decode_metadata, prefill_metadata
+from minivllm_amd.engine.scheduler import Scheduler
+from minivllm_amd.engine.sequence import Sequence, SequenceStatus
+from minivllm_amd.sampling_parameters import SamplingParams
+
+
+def _seq(n, bs, start=0, **kw):
+    return Sequence(list(range(start, start + n)), SamplingParams(**kw), bs)
+
+
+def test_sequence_block_arithmetic_including_exact_multiples():
+    s = _seq(8, 4)
+    assert (s.num_blocks, s.last_block_num_tokens, s.block(1)) == (2, 4, [4, 5, 6, 7])
+    s.append_token(99)
+    assert (len(s), s.num_blocks, s.last_block_num_tokens, s.block(2), s.last_token) == (9, 3, 1, [99], 99)
+    assert s.num_completion_tokens == 1 and s.completion_token_ids == [99]
+    with pytest.raises(AssertionError):
+        SamplingParams(temperature=0.0)
+
+
+def test_compute_hash_is_chained_xxh64_of_int32_bytes():
+    """XXH64 known answers: empty input with seed 0 is ef46db3751d8e999."""
+    assert xxhash.xxh64(b"").intdigest() == 0xEF46DB3751D8E999
+    toks = [1, 2, 3, 4]
+    raw = np.array(toks, dtype=np.int32).tobytes()
+    assert BlockManager.compute_hash(toks) == xxhash.xxh64(raw).intdigest()
+    prefix = 0x0123456789ABCDEF
+    assert BlockManager.compute_hash(toks, prefix) == xxhash.xxh64(prefix.to_bytes(8, "little") + raw).intdigest()
+    assert BlockManager.compute_hash(toks, prefix) != BlockManager.compute_hash(toks)
+
+
+def test_block_manager_allocate_free_and_prefix_sharing():
+    bm = BlockManager(8, 4)
+    a = _seq(10, 4)
+    bm.allocate(a)
+    assert len(a.block_table) == 3 and len(bm.free_block_ids) == 5 and a.num_cached_tokens == 0
+    b = Sequence(list(range(8)) + [70, 71], SamplingParams(), 4)       # shares the first two full blocks
+    bm.allocate(b)
+    assert b.block_table[:2] == a.block_table[:2] and b.block_table[2] != a.block_table[2]
+    assert b.num_cached_tokens == 8 and len(bm.free_block_ids) == 4
+    assert bm.blocks[a.block_table[0]].ref_count == 2
+    bm.deallocate(a)
+    assert len(bm.free_block_ids) == 5 and bm.blocks[b.block_table[0]].ref_count == 1
+    bm.deallocate(b)
+    assert len(bm.free_block_ids) == 8 and not bm.used_block_ids
+    c = _seq(8, 4)                                                      # cached hashes survive a free
+    bm.allocate(c)
+    assert c.num_cached_tokens == 8
+    d = Sequence([5, 5, 5, 5, 4, 5, 6, 7], SamplingParams(), 4)         # same 2nd block tokens, other prefix: no hit
+    bm.allocate(d)
+    assert d.num_cached_tokens == 0
+
+
+def test_block_manager_append_allocates_on_block_start_and_hashes_on_fill():
+    bm = BlockManager(4, 4)
+    s = _seq(4, 4)
+    bm.allocate(s)
+    assert len(s.block_table) == 1
+    s.append_token(100)                       # 5 tokens: the new token starts block 1
+    assert bm.can_append(s)
+    bm.append(s)
+    assert len(s.block_table) == 2 and bm.blocks[s.block_table[1]].hash == -1
+    for t in (101, 102):
+        s.append_token(t)
+        bm.append(s)
+    assert len(s.block_table) == 2
+    s.append_token(103)                       # 8 tokens: this step fills block 1 -> it gets its chained hash
+    bm.append(s)
+    blk = bm.blocks[s.block_table[1]]
+    assert blk.hash == BlockManager.compute_hash([100, 101, 102, 103], bm.blocks[s.block_table[0]].hash)
+    bm2 = BlockManager(1, 4)
+    t = _seq(4, 4)
+    bm2.allocate(t)
+    t.append_token(1)
+    assert not bm2.can_append(t)
+
+
+def _metadata_inputs(seqs):
+    return [dict(num_tokens=len(s), num_cached_tokens=s.num_cached_tokens, block_table=list(s.block_table),
+                 last_token=s.last_token) for s in seqs]
+
+
+def test_metadata_matches_producers_oracle():
+    rng = random.Random(0)
+    for bs in (1, 4, 16):
+        bm = BlockManager(200, bs)
+        seqs = []
+        for _ in range(5):
+            s = _seq(rng.randint(1, 50), bs, start=rng.randint(0, 3))
+            bm.allocate(s)
+            seqs.append(s)
+        got = prefill_metadata(seqs, bs, reuse_cached_kv=True)
+        want = oracle.prefill_metadata_oracle(_metadata_inputs(seqs), bs)
+        for key in ("cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "slot_mapping", "block_tables"):
+            assert got[key] == want[key], (bs, key)
+        full = prefill_metadata(seqs, bs, reuse_cached_kv=False)
+        uncached = [dict(m, num_cached_tokens=0) for m in _metadata_inputs(seqs)]
+        want_full = oracle.prefill_metadata_oracle(uncached, bs)
+        assert full["slot_mapping"] == want_full["slot_mapping"] and full["cu_seqlens_q"] == want_full["cu_seqlens_k"]
+        assert full["input_ids"] == [t for s in seqs for t in s.token_ids]
+        for s in seqs:
+            s.append_token(7)
+            bm.append(s)
+        got = decode_metadata(seqs, bs)
+        want = oracle.decode_metadata_oracle(_metadata_inputs(seqs), bs)
+        assert got == want
+
+
+class FakeRunner:
+    """Stands in for the model: returns a counter as the next token and records what it was asked to run."""
+
+    def __init__(self):
+        self.calls = []
+        self.next = 1000
+
+    def run(self, seqs, is_prefill):
+        self.calls.append((is_prefill, [s.seq_id for s in seqs], [len(s) for s in seqs]))
+        out = list(range(self.next, self.next + len(seqs)))
+        self.next += len(seqs)
+        return out
+
+
+def test_engine_loop_prefill_first_then_decode_until_max_tokens():
+    cfg = dict(max_num_sequences=2, max_num_batched_tokens=64, max_cached_blocks=16, block_size=4, eos=-1)
+    runner = FakeRunner()
+    eng = LLMEngine(cfg, model_runner=runner)
+    prompts = [[1, 2, 3], [4, 5, 6, 7, 8], [9]]
+    out = eng.generate(prompts, SamplingParams(temperature=0.6, max_tokens=4, ignore_eos=True))
+    assert [len(t) for t in out["token_ids"]] == [4, 4, 4]
+    # first two prompts admitted together (batch limit 2), then the third is prefilled before any decode
+    assert runner.calls[0][0] is True and len(runner.calls[0][1]) == 2
+    assert runner.calls[1][0] is True and len(runner.calls[1][1]) == 1
+    assert all(c[0] is False for c in runner.calls[2:])
+    # lengths advance by one per decode step (the sequence is really extended)
+    first = runner.calls[0][1][0]
+    lens = [c[2][c[1].index(first)] for c in runner.calls if first in c[1]]
+    assert lens == [3, 4, 5, 6]
+    assert eng.scheduler.is_finished() and len(eng.scheduler.block_manager.free_block_ids) == 16
+    assert eng.stats["decode_tokens"] == 9 and eng.stats["prefill_tokens"] == 3 + 5 + 1
+
+
+def test_scheduler_eos_and_token_budget_and_preemption():
+    sch = Scheduler(max_num_sequences=8, max_num_batched_tokens=8, max_cached_blocks=3, block_size=4, eos=42)
+    a, b = _seq(6, 4, max_tokens=10), _seq(4, 4, start=50, max_tokens=10)
+    sch.add_sequence(a)
+    sch.add_sequence(b)
+    seqs, is_prefill = sch.schedule()
+    assert is_prefill and seqs == [a]                 # 6 + 4 tokens exceed the 8-token budget
+    sch.postprocess(seqs, [5])
+    seqs, is_prefill = sch.schedule()
+    assert is_prefill and seqs == [b]                 # waiting prompts go before decode
+    sch.postprocess(seqs, [6])
+    # 3 blocks in total: a holds 2, b holds 1; b's 5th token needs a block -> the tail sequence is preempted
+    seqs, is_prefill = sch.schedule()
+    assert not is_prefill and seqs == [a]
+    assert b.status == SequenceStatus.WAITING and b.block_table == [] and sch.waiting[0] is b
+    sch.postprocess(seqs, [42])                       # eos finishes a and frees its blocks
+    assert a.is_finished and len(sch.block_manager.free_block_ids) == 3
+    seqs, is_prefill = sch.schedule()
+    assert is_prefill and seqs == [b] and len(b) == 5  # re-prefilled with prompt + generated token
