@@ -7,7 +7,7 @@ paged-attention decode, batch 256, context lengths log-uniform in [128, 32768],
 as algorithmic HBM GB/s.  A "step" is one decode call over the whole batch with
 all inputs resident in HBM.  `extra` carries the other measured workloads
 (decode at block_size 256, varlen prefill TFLOP/s and store_kvcache GB/s on
-config 2).  `cpu_baseline` times the CPU oracle's naive decode on a bounded
+config 2, the INT8 cache path of config 4, the engine generate loop of config 5).  `cpu_baseline` times the CPU oracle's naive decode on a bounded
 subset of the same batch on the host cores.
 """
 from __future__ import annotations
@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode,decode256,prefill,store,cpu to restrict the run")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,engine,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -190,6 +190,93 @@ def bench_prefill_store(args, which):
     return out
 
 
+def bench_int8(args):
+    """BASELINE config 4: B 128, ctx U[256,16384], Hq32/Hkv8/D128; K/V ~ N(0,1) with 1 % outliers at 8 sigma are
+    quantised by store_kvcache_int8 into a block-16 int8 cache, then decoded with in-kernel dequantisation."""
+    import torch
+    from minivllm_amd.layers.attention import paged_attention_decode_int8, store_kvcache_int8
+
+    dev = "cuda:0"
+    hq, hkv, d, batch, bs = 32, 8, 128, 128, 16
+    g = torch.Generator().manual_seed(args.seed)
+    ctx = torch.randint(256, 16385, (batch,), generator=g)
+    need = ((ctx + bs - 1) // bs).tolist()
+    nb = sum(need)
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.full((batch, max(need)), -1, dtype=torch.int32)
+    at = 0
+    for b, n in enumerate(need):
+        tables[b, :n] = perm[at:at + n].to(torch.int32)
+        at += n
+    dg = torch.Generator(device=dev).manual_seed(args.seed + 1)
+    kc = torch.zeros(nb, bs, hkv, d, dtype=torch.int8, device=dev)
+    vc = torch.zeros_like(kc)
+    ks = torch.zeros(nb, bs, hkv, dtype=torch.float32, device=dev)
+    vs = torch.zeros_like(ks)
+    total = nb * bs
+    store_ms, chunk = [], 1 << 16
+    for lo in range(0, total, chunk):                       # fill the whole cache through the INT8 store kernel
+        n = min(chunk, total - lo)
+        k = torch.randn(n, hkv, d, generator=dg, device=dev)
+        v = torch.randn(n, hkv, d, generator=dg, device=dev)
+        k = torch.where(torch.rand(k.shape, generator=dg, device=dev) < 0.01, k * 8, k).to(torch.bfloat16)
+        v = torch.where(torch.rand(v.shape, generator=dg, device=dev) < 0.01, v * 8, v).to(torch.bfloat16)
+        slots = torch.arange(lo, lo + n, device=dev)
+        if lo == 0:
+            _, ms = time_steps(lambda: store_kvcache_int8(k, v, kc, vc, ks, vs, slots, bs), 10, 2)
+            store_ms.append(ms)
+            store_bytes = 2 * n * hkv * d * (2 + 1) + 8 * n + 2 * n * hkv * 4
+        store_kvcache_int8(k, v, kc, vc, ks, vs, slots, bs)
+    q = torch.randn(batch, hq, d, generator=dg, device=dev).to(torch.bfloat16)
+    td, cd = tables.to(dev), ctx.to(dev)
+    scale = 1.0 / math.sqrt(d)
+    wall_ms, event_ms = time_steps(
+        lambda: paged_attention_decode_int8(q, kc, vc, ks, vs, td, cd, scale, hq, hkv, d, bs),
+        max(3, args.steps // 3), max(1, args.warmup // 2))
+    nbytes = decode_bytes(ctx, bs, hq, hkv, d, 1, 2, 8, int8_scales=True)
+    return {
+        "workload": "INT8 KV cache: decode B128 ctx~U[256,16384] Hq32 Hkv8 D128 block_size 16, bf16 q",
+        "tokens": int(ctx.sum()), "algorithmic_bytes": nbytes, "ms_per_step": wall_ms,
+        "event_ms_per_step": event_ms, "gbs": nbytes / (event_ms * 1e-3) / 1e9,
+        "store_int8_gbs": store_bytes / (store_ms[0] * 1e-3) / 1e9, "store_int8_tokens": chunk,
+    }
+
+
+def bench_engine(args, max_num_sequences):
+    """BASELINE config 5: random-init Qwen3-style decoder (hidden 1024, 8 layers, Hq16/Hkv8/D128, FFN 3072,
+    vocab 151936, bf16), 60 prompts of random ids with lengths U[32,96], 256 new tokens each, T 0.6."""
+    import torch
+    from minivllm_amd.engine.llm_engine import LLMEngine
+    from minivllm_amd.sampling_parameters import SamplingParams
+
+    cfg = dict(vocab_size=151936, hidden_size=1024, num_layers=8, num_heads=16, num_kv_heads=8, head_dim=128,
+               intermediate_size=3072, base=1_000_000, rms_norm_epsilon=1e-6, qkv_bias=False, ffn_bias=True,
+               scale=1.0, tie_word_embeddings=True, block_size=256, max_num_batched_tokens=16384,
+               max_num_sequences=max_num_sequences, max_cached_blocks=256, max_position=512, dtype="bf16",
+               eos=-1, seed=args.seed)
+    g = torch.Generator().manual_seed(args.seed)
+    lengths = torch.randint(32, 97, (60,), generator=g).tolist()
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lengths]
+    engine = LLMEngine(cfg)
+    sp = SamplingParams(temperature=0.6, max_tokens=256, ignore_eos=True)
+    engine.generate(prompts[:4], SamplingParams(temperature=0.6, max_tokens=4, ignore_eos=True))   # warm-up
+    for key in engine.stats:
+        engine.stats[key] = 0
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = engine.generate(prompts, sp)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    new_tokens = sum(len(t) for t in out["token_ids"])
+    assert new_tokens == 60 * 256
+    return {
+        "workload": "engine generate: 60 prompts L~U[32,96], 256 new tokens each, Qwen3-style 8x1024 bf16, "
+                    f"block_size 256, max_num_sequences {max_num_sequences}, eager decode",
+        "output_tokens": new_tokens, "wall_s": wall, "tok_per_s": new_tokens / wall,
+        "steps": engine.stats["steps"], "decode_s": engine.stats["decode_s"], "prefill_s": engine.stats["prefill_s"],
+    }
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -219,6 +306,11 @@ def main():
     which = [n for n in ("prefill", "store") if want(n)]
     if which:
         extra.update(bench_prefill_store(args, which))
+    if want("int8"):
+        extra["int8"] = bench_int8(args)
+    if want("engine"):
+        extra["engine_16seq"] = bench_engine(args, 16)
+        extra["engine_64seq"] = bench_engine(args, 64)
 
     line = {
         "metric": "decode-attn HBM GB/s (% peak); prefill TFLOP/s (% MFMA); engine out tok/s",
