@@ -358,6 +358,313 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_ke
 }
 
 // ---------------------------------------------------------------------------
+// Fast path, INT8 cache (head_dim 128, block_size % 16 == 0).  Same decomposition as the 16-bit kernel.
+//   QK^T   runs on v_mfma_i32_16x16x64_i8 with the int8 codes as they lie in memory (lane = token,
+//          16 bytes = 16 dims): the query row is turned once per wave into 15-bit fixed point
+//          q ~ (128*hi + lo) * amax/16256 with int8 hi/lo planes, so scores are exact integer dot
+//          products times (amax/16256) * k_scale[token];
+//   PV     on the VALU with v_cvt_f32_ubyte on codes biased by +128 (one xor per 4 codes); the bias is
+//          taken out at the end as 128 * sum(p * v_scale);
+//   scales one k_scale and one v_scale load per lane and tile (lane l%4 of a quad holds token 4*(l/16)+l%4),
+//          handed round inside the quad by DPP.
+// V rows are 128 B, so one 16-byte load per lane covers 8 rows: lane l reads token 4*(l/16) + 2i + (l%16)/8,
+// dims 16*(l%8).. in instruction i = 0, 1.
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(4))) int v4i;
+
+struct KVTileI8 {
+  uint4 k[2];
+  uint4 v[2];
+  float ks;
+  float vs;
+  int t0;
+  bool ok;
+};
+
+template <int SEL> __device__ __forceinline__ float byte_to_float(uint32_t w) {
+  return (float)((w >> (8 * SEL)) & 0xffu);      // v_cvt_f32_ubyteN
+}
+
+template <typename T, int NCH>
+__global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
+  constexpr int D = 128;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int waves_per_block = blockDim.x >> 6;
+  const int b = blockIdx.y;
+  const int p = (int)((blockIdx.x + (unsigned)b) % (unsigned)a.num_parts);   // see decode_mfma_kernel
+  const int g = blockIdx.z * waves_per_block + wave;
+  const int group = a.num_heads / a.num_kv_heads;
+  const bool direct = (a.num_parts == 1);
+  const int q4 = lane >> 4;            // token class: tokens 4*q4 .. 4*q4+3 of a tile
+  const int hb = (lane >> 3) & 1;      // which of the two V rows of an instruction this lane reads
+
+  const int ctx = (int)load_ctx(a, b);
+  const int part_start = p * a.part_tokens;
+  if (part_start >= ctx && !(direct && p == 0)) return;
+  const int part_end = min(ctx, part_start + a.part_tokens);
+  const int ntiles = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
+
+  // ---- query -> int8 hi/lo planes (B operand: column lane%16 -> head lane%4, bytes 16*q4.. of each 64-dim step)
+  v4i qhi[NCH][2], qlo[NCH][2];
+  float qscale[NCH];                   // amax/16256 * scale*log2e of head (lane%4) of chunk c
+  {
+    const T* q = reinterpret_cast<const T*>(a.q);
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int hl = c * 4 + (lane & 3);
+      const bool live = hl < group;
+      const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? hl : 0)) * D;
+      float x[2][16];
+      float amax = 0.f;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          x[j][e] = live ? to_float(src[64 * j + 16 * q4 + e]) : 0.f;
+          amax = fmaxf(amax, fabsf(x[j][e]));
+        }
+      amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+      const float to_fix = amax > 0.f ? 16256.f / amax : 0.f;
+      qscale[c] = amax * (1.f / 16256.f) * a.scale_log2;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        int hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int q16 = (int)rintf(x[j][e] * to_fix);            // |q16| <= 16256
+          const int l8 = ((q16 + 64) & 127) - 64;                  // [-64, 63]
+          const int h8 = (q16 - l8) >> 7;                          // [-127, 127]
+          hi[e >> 2] |= (h8 & 0xff) << (8 * (e & 3));
+          lo[e >> 2] |= (l8 & 0xff) << (8 * (e & 3));
+        }
+        qhi[c][j] = (v4i){hi[0], hi[1], hi[2], hi[3]};
+        qlo[c][j] = (v4i){lo[0], lo[1], lo[2], lo[3]};
+      }
+    }
+  }
+
+  float m[NCH], l[NCH], wsum[NCH], acc[NCH][4][16];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    m[c] = -INFINITY; l[c] = 0.f; wsum[c] = 0.f;
+#pragma unroll
+    for (int h = 0; h < 4; ++h)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[c][h][e] = 0.f;
+  }
+
+  const int bs = a.block_size;
+  const int64_t row = (int64_t)a.num_kv_heads * D;          // bytes per token row
+  const char* kc = reinterpret_cast<const char*>(a.k_cache) + (int64_t)g * D;
+  const char* vc = reinterpret_cast<const char*>(a.v_cache) + (int64_t)g * D;
+  const int32_t* table = a.block_tables + (int64_t)b * a.max_num_blocks;
+  int bi = part_start / bs;
+  int off = part_start - bi * bs;
+  int win_base = bi;
+  int win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
+  const int k_lane_off = (lane & 15) * (int)row + q4 * 16;                      // token lane%16, bytes 16*q4 (+64 j)
+  const int v_lane_off = (4 * q4 + hb) * (int)row + (lane & 7) * 16;            // token 4*q4 + hb (+2 i), dims 16*(lane%8)
+  const int s_lane_tok = 4 * q4 + (lane & 3);                                   // token whose scales this lane loads
+
+  auto load_tile = [&](KVTileI8& t, int tile) {
+    t.t0 = part_start + tile * kTile;
+    if (bi - win_base >= 64) {
+      win_base = bi;
+      win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
+    }
+    const int phys = __builtin_amdgcn_readlane(win, bi - win_base);
+    t.ok = (bi < a.max_num_blocks) && phys >= 0 && (int64_t)phys < a.num_blocks;
+    if (t.ok) {
+      const int64_t tok0 = (int64_t)phys * bs + off;
+      const char* kp = kc + tok0 * row + k_lane_off;
+      const char* vp = vc + tok0 * row + v_lane_off;
+      t.k[0] = *reinterpret_cast<const uint4*>(kp);
+      t.k[1] = *reinterpret_cast<const uint4*>(kp + 64);
+      t.v[0] = *reinterpret_cast<const uint4*>(vp);
+      t.v[1] = *reinterpret_cast<const uint4*>(vp + 2 * row);
+      const int64_t sidx = (tok0 + s_lane_tok) * a.num_kv_heads + g;
+      t.ks = a.k_scale[sidx];
+      t.vs = a.v_scale[sidx];
+    } else {
+      t.k[0] = t.k[1] = t.v[0] = t.v[1] = make_uint4(0u, 0u, 0u, 0u);
+      t.ks = t.vs = 0.f;
+    }
+    off += kTile;
+    if (off >= bs) { off = 0; ++bi; }
+  };
+
+  auto consume = [&](const KVTileI8& t) {
+    const int tok_base = t.t0 + 4 * q4;
+    const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
+    const float ks4[4] = {quad_bcast<0>(t.ks), quad_bcast<1>(t.ks), quad_bcast<2>(t.ks), quad_bcast<3>(t.ks)};
+    float vs4[4] = {quad_bcast<0>(t.vs), quad_bcast<1>(t.vs), quad_bcast<2>(t.vs), quad_bcast<3>(t.vs)};
+    if (partial) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (!t.ok || tok_base + r >= part_end) vs4[r] = 0.f;     // stale scale memory must not meet p = 0
+    }
+    float pr[NCH][4];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      v4i shi = {0, 0, 0, 0}, slo = {0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const v4i kf = (v4i){(int)t.k[j].x, (int)t.k[j].y, (int)t.k[j].z, (int)t.k[j].w};
+        shi = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qhi[c][j], shi, 0, 0, 0);
+        slo = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qlo[c][j], slo, 0, 0, 0);
+      }
+      float s2[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s2[r] = (float)(shi[r] * 128 + slo[r]) * (qscale[c] * ks4[r]);
+        if (partial && (!t.ok || tok_base + r >= part_end)) s2[r] = -INFINITY;
+      }
+      const float tile_max = fmaxf(fmaxf(s2[0], s2[1]), fmaxf(s2[2], s2[3]));
+      const bool grow = tile_max > m[c] + kLazyRescale || (m[c] == -INFINITY && tile_max > -INFINITY);
+      if (__any(grow)) {
+        const float m_new = grow ? tile_max : m[c];
+        const float al = (m_new == m[c]) ? 1.f : safe_exp2_diff(m[c], m_new);
+        l[c] *= al;
+        wsum[c] *= al;
+        const float a4[4] = {quad_bcast<0>(al), quad_bcast<1>(al), quad_bcast<2>(al), quad_bcast<3>(al)};
+#pragma unroll
+        for (int h = 0; h < 4; ++h)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[c][h][e] *= a4[h];
+        m[c] = m_new;
+      }
+      const float m_eff = (m[c] == -INFINITY) ? 0.f : m[c];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pr[c][r] = fast_exp2(s2[r] - m_eff);
+        l[c] += pr[c][r];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint4 raw = t.v[i];
+      const uint32_t w4[4] = {raw.x ^ 0x80808080u, raw.y ^ 0x80808080u, raw.z ^ 0x80808080u, raw.w ^ 0x80808080u};
+      float vf[16];
+#pragma unroll
+      for (int d4 = 0; d4 < 4; ++d4) {
+        vf[4 * d4 + 0] = byte_to_float<0>(w4[d4]);
+        vf[4 * d4 + 1] = byte_to_float<1>(w4[d4]);
+        vf[4 * d4 + 2] = byte_to_float<2>(w4[d4]);
+        vf[4 * d4 + 3] = byte_to_float<3>(w4[d4]);
+      }
+      const float vsel = hb ? vs4[2 * i + 1] : vs4[2 * i];
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const float wgt = (hb ? pr[c][2 * i + 1] : pr[c][2 * i]) * vsel;    // own head; other heads via the quad
+        wsum[c] += wgt;
+        const float w0 = quad_bcast<0>(wgt), w1 = quad_bcast<1>(wgt), w2 = quad_bcast<2>(wgt), w3 = quad_bcast<3>(wgt);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          acc[c][0][e] = fmaf(w0, vf[e], acc[c][0][e]);
+          acc[c][1][e] = fmaf(w1, vf[e], acc[c][1][e]);
+          acc[c][2][e] = fmaf(w2, vf[e], acc[c][2][e]);
+          acc[c][3][e] = fmaf(w3, vf[e], acc[c][3][e]);
+        }
+      }
+    }
+  };
+
+  KVTileI8 ta, tb;
+  if (ntiles > 0) load_tile(ta, 0);
+  int tile = 0;
+  while (tile < ntiles) {
+    if (tile + 1 < ntiles) load_tile(tb, tile + 1);
+    consume(ta);
+    ++tile;
+    if (tile >= ntiles) break;
+    if (tile + 1 < ntiles) load_tile(ta, tile + 1);
+    consume(tb);
+    ++tile;
+  }
+
+  // take the +128 bias out, then fold the token classes: first the two V-row halves (same m, l), then lane/16
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const float b4[4] = {quad_bcast<0>(wsum[c]), quad_bcast<1>(wsum[c]), quad_bcast<2>(wsum[c]), quad_bcast<3>(wsum[c])};
+#pragma unroll
+    for (int h = 0; h < 4; ++h)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        float x = fmaf(-128.f, b4[h], acc[c][h][e]);
+        x += __shfl_xor(x, 8, 64);
+        acc[c][h][e] = x;
+      }
+  }
+#pragma unroll
+  for (int offs = 16; offs <= 32; offs <<= 1) {
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const float mo = __shfl_xor(m[c], offs, 64);
+      const float lo = __shfl_xor(l[c], offs, 64);
+      const float mn = fmaxf(m[c], mo);
+      const float al = safe_exp2_diff(m[c], mn);
+      const float ao = safe_exp2_diff(mo, mn);
+      l[c] = l[c] * al + lo * ao;
+      m[c] = mn;
+      const float a4[4] = {quad_bcast<0>(al), quad_bcast<1>(al), quad_bcast<2>(al), quad_bcast<3>(al)};
+      const float o4[4] = {quad_bcast<0>(ao), quad_bcast<1>(ao), quad_bcast<2>(ao), quad_bcast<3>(ao)};
+#pragma unroll
+      for (int h = 0; h < 4; ++h)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float other = __shfl_xor(acc[c][h][e], offs, 64);
+          acc[c][h][e] = acc[c][h][e] * a4[h] + other * o4[h];
+        }
+    }
+  }
+
+  // lanes 0..7 hold dims 16*lane.. of heads 0..3 of every chunk
+  if (lane < 8) {
+    const int head0 = g * group;
+    if (direct) {
+      T* out = reinterpret_cast<T*>(a.out);
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const float linv = l[c] > 0.f ? 1.f / l[c] : 0.f;
+        const float li[4] = {quad_bcast<0>(linv), quad_bcast<1>(linv), quad_bcast<2>(linv), quad_bcast<3>(linv)};
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          if (c * 4 + h < group) {
+            T* dst = out + ((int64_t)b * a.num_heads + head0 + c * 4 + h) * D + lane * 16;
+            T o[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[e] = from_float<T>(acc[c][h][e] * li[h]);
+            reinterpret_cast<uint4*>(dst)[0] = reinterpret_cast<const uint4*>(o)[0];
+            reinterpret_cast<uint4*>(dst)[1] = reinterpret_cast<const uint4*>(o)[1];
+          }
+        }
+      }
+    } else {
+      const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          if (c * 4 + h < group) {
+            float* dst = a.ws_acc + (slot + c * 4 + h) * D + lane * 16;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4)
+              reinterpret_cast<float4*>(dst)[e4] = make_float4(acc[c][h][4 * e4], acc[c][h][4 * e4 + 1],
+                                                               acc[c][h][4 * e4 + 2], acc[c][h][4 * e4 + 3]);
+          }
+        }
+        if (lane < 4 && c * 4 + lane < group) {
+          float* ml = a.ws_ml + (slot + c * 4 + lane) * 2;
+          *reinterpret_cast<float2*>(ml) = make_float2(m[c], l[c]);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Generic path: any element type (fp32 included), head_dim <= 512, any
 // block_size and group size.  One wave per (partition, sequence, q head);
 // lanes split head_dim, one token per step.  Correctness path for shapes the
@@ -545,6 +852,11 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stre
       dim3 block(64 * wpb);
       if (group <= 4) decode_mfma_kernel<T, 1><<<grid, block, 0, stream>>>(a);
       else decode_mfma_kernel<T, 2><<<grid, block, 0, stream>>>(a);
+      launched = true;
+    } else if (fast_ok && int8 && group <= 4) {
+      const int wpb = largest_divisor_le(a.num_kv_heads, 8);
+      dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, (unsigned)(a.num_kv_heads / wpb));
+      decode_mfma_int8_kernel<T, 1><<<grid, dim3(64 * wpb), 0, stream>>>(a);
       launched = true;
     }
   }

@@ -1,0 +1,89 @@
+"""INT8 KV cache: store_kvcache_int8 then paged_attention_decode_int8 vs the CPU oracle.
+
+The INT8 format is defined by this build (the reference has none): the oracle dequantises code*scale in
+fp32 and runs the naive decode.  Tolerance: mean-abs 2e-3 and |err| <= 2e-2 + |want| * 2^-8 elementwise; the
+second term is the rounding of the 16-bit output itself, which matters here because the 8-sigma outliers of
+config 4 make single outputs as large as 30 (one bf16 ulp at 16..32 is 0.125)."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import error_stats, make_paged_case
+from minivllm_amd.layers.attention import paged_attention_decode_int8, store_kvcache_int8
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _quantised_case(seed, batch, ctx_lo, ctx_hi, hq, hkv, d, bs, dtype=torch.bfloat16, ctx_list=None):
+    q, kc, vc, tables, ctx = make_paged_case(seed, batch, ctx_lo, ctx_hi, hq, hkv, d, bs, ctx_list=ctx_list)
+    g = torch.Generator().manual_seed(seed + 100)
+    kc[torch.rand(kc.shape, generator=g) < 0.01] *= 8.0          # 1 % outliers at 8 sigma
+    vc[torch.rand(vc.shape, generator=g) < 0.01] *= 8.0
+    nb = kc.shape[0]
+    codes_k = torch.zeros(nb, bs, hkv, d, dtype=torch.int8, device=DEV)
+    codes_v = torch.zeros_like(codes_k)
+    sk = torch.zeros(nb, bs, hkv, device=DEV)
+    sv = torch.zeros_like(sk)
+    slots = torch.arange(nb * bs, device=DEV)
+    store_kvcache_int8(kc.view(-1, hkv, d).to(dtype).to(DEV), vc.view(-1, hkv, d).to(dtype).to(DEV),
+                       codes_k, codes_v, sk, sv, slots, bs)
+    return q.to(dtype), codes_k, codes_v, sk, sv, tables, ctx
+
+
+def _check(case, hq, hkv, d, bs, scale, ctx_dtype=torch.int64):
+    q, ck, cv, sk, sv, tables, ctx = case
+    got = paged_attention_decode_int8(q.to(DEV), ck, cv, sk, sv, tables.to(DEV), ctx.to(ctx_dtype).to(DEV), scale,
+                                      hq, hkv, d, bs).cpu()
+    want = oracle.decode_int8_oracle(q.float(), ck.cpu(), cv.cpu(), sk.cpu(), sv.cpu(), tables, ctx, scale,
+                                     hq, hkv, d, bs)
+    mx, mean = error_stats(got, want)
+    assert got.dtype == q.dtype and torch.isfinite(got).all()
+    excess = ((got.float() - want).abs() - want.abs() * 2.0 ** -8).max().item()
+    assert excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
+    return got
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,bs,ctx_hi", [(32, 8, 16, 700), (16, 8, 256, 1500), (8, 8, 32, 255), (6, 2, 48, 400)])
+def test_int8_fast_path(dtype, hq, hkv, bs, ctx_hi):
+    d = 128
+    _check(_quantised_case(61, 7, 1, ctx_hi, hq, hkv, d, bs, dtype), hq, hkv, d, bs, 1 / math.sqrt(d))
+
+
+@pytest.mark.parametrize("ctx_list", [[1, 2, 7, 8, 9, 15, 16, 17], [255, 256, 257, 1023, 1024, 1025]])
+def test_int8_context_boundaries(ctx_list):
+    hq, hkv, d, bs = 8, 2, 128, 16
+    _check(_quantised_case(62, 0, 0, 0, hq, hkv, d, bs, ctx_list=ctx_list), hq, hkv, d, bs, 0.1, torch.int32)
+
+
+@pytest.mark.parametrize("hq,hkv,d,bs", [(16, 16, 64, 16), (32, 4, 128, 16), (4, 2, 128, 8)])
+def test_int8_generic_path(hq, hkv, d, bs):
+    """head_dim 64, GQA 8 and block_size 8 run on the generic kernel."""
+    _check(_quantised_case(63, 5, 1, 300, hq, hkv, d, bs), hq, hkv, d, bs, 1 / math.sqrt(d))
+
+
+def test_int8_zero_context_and_missing_blocks():
+    hq, hkv, d, bs = 8, 2, 128, 16
+    q, ck, cv, sk, sv, tables, ctx = _quantised_case(64, 0, 0, 0, hq, hkv, d, bs, ctx_list=[40, 0, 100])
+    sk[0].fill_(float("nan"))                                  # stale memory in a block nobody owns... 
+    sv[0].fill_(float("nan"))
+    owned = set(tables[tables >= 0].tolist())
+    if 0 in owned:                                             # keep the poison only if block 0 is unowned
+        sk[0].zero_()
+        sv[0].zero_()
+    got = paged_attention_decode_int8(q.to(DEV), ck, cv, sk, sv, tables.to(DEV), ctx.to(DEV), 0.09, hq, hkv, d, bs).cpu()
+    assert torch.isfinite(got).all() and torch.count_nonzero(got[1]) == 0
+    hole = tables.clone()
+    hole[0, :] = -1
+    got2 = paged_attention_decode_int8(q.to(DEV), ck, cv, sk, sv, hole.to(DEV), ctx.to(DEV), 0.09, hq, hkv, d, bs).cpu()
+    assert torch.count_nonzero(got2[0]) == 0 and torch.equal(got2[2], got[2])
+
+
+def test_config4_subset():
+    """BASELINE config 4 shape (B 128 is cut to 24 sequences here, ctx U[256,16384]) on the fast path."""
+    hq, hkv, d, bs = 32, 8, 128, 16
+    case = _quantised_case(65, 24, 256, 16384, hq, hkv, d, bs)
+    _check(case, hq, hkv, d, bs, 1 / math.sqrt(d))
