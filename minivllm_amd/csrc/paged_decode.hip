@@ -31,6 +31,9 @@ namespace mvllm {
 #ifndef MVLLM_DECODE_WAVES_PER_EU
 #define MVLLM_DECODE_WAVES_PER_EU 2
 #endif
+#ifndef MVLLM_DECODE_WPB
+#define MVLLM_DECODE_WPB 8          // waves (= kv heads) per workgroup, upper bound
+#endif
 
 constexpr int kTile = 16;                                 // tokens per MFMA tile
 constexpr int kMaxParts = MVLLM_DECODE_MAX_PARTS;         // split-K partitions per sequence (upper bound)
@@ -79,6 +82,15 @@ __device__ __forceinline__ int64_t load_ctx(const DecodeArgs& a, int b) {
 __device__ __forceinline__ float safe_exp2_diff(float m_old, float m_new) {
   // exp2(m_old - m_new) with -inf - -inf := 0 contribution
   return (m_old == -INFINITY) ? 0.f : fast_exp2(m_old - m_new);
+}
+
+// (sequence, partition) of this workgroup.  The partition index is rotated by the sequence index:
+// workgroups are dealt to the 8 XCDs round-robin by linear id, and without the rotation every short
+// sequence (only partition 0 live) would land on the same XCD.
+__device__ __forceinline__ bool decode_item(const DecodeArgs& a, int& b, int& p) {
+  b = blockIdx.y;
+  p = (int)((blockIdx.x + (unsigned)b) % (unsigned)a.num_parts);
+  return true;
 }
 
 // ---------------------------------------------------------------------------
@@ -220,15 +232,8 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_ke
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int waves_per_block = blockDim.x >> 6;
-  const int b = blockIdx.y;
-  // Rotate the partition index by the sequence index: workgroups are dealt to the 8 XCDs
-  // round-robin by linear id, and without the rotation every short sequence (only partition 0
-  // live) would land on the same XCD.
-#ifndef MVLLM_DECODE_NO_SWIZZLE
-  const int p = (int)((blockIdx.x + (unsigned)b) % (unsigned)a.num_parts);
-#else
-  const int p = blockIdx.x;
-#endif
+  int b, p;
+  if (!decode_item(a, b, p)) return;
   const int g = blockIdx.z * waves_per_block + wave;   // kv head
   const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head
   const bool direct = (a.num_parts == 1);
@@ -391,8 +396,8 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_in
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int waves_per_block = blockDim.x >> 6;
-  const int b = blockIdx.y;
-  const int p = (int)((blockIdx.x + (unsigned)b) % (unsigned)a.num_parts);   // see decode_mfma_kernel
+  int b, p;
+  if (!decode_item(a, b, p)) return;
   const int g = blockIdx.z * waves_per_block + wave;
   const int group = a.num_heads / a.num_kv_heads;
   const bool direct = (a.num_parts == 1);
@@ -766,57 +771,49 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(const DecodeArgs a) 
 // ---------------------------------------------------------------------------
 // Second pass: merge the per-partition partials of one (sequence, q head).
 // ---------------------------------------------------------------------------
+// One wave per (sequence, query head), four heads per block; a lane owns dims lane + 64 r.  Partitions
+// are folded with a running max in one pass; the loads of successive partitions do not depend on the
+// arithmetic, so the unrolled loop keeps several in flight and the kernel is one short latency chain.
 template <typename T>
 __global__ __launch_bounds__(256) void decode_reduce_kernel(const DecodeArgs a) {
-  __shared__ float s_max[4];
-  __shared__ float s_l[4];
-  __shared__ float s_acc[4][64 * kGenericMaxR];
-  const int h = blockIdx.x;
-  const int b = blockIdx.y;
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int h = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int b = blockIdx.y;
+  if (h >= a.num_heads) return;
   const int D = a.head_dim;
   const int ctx = (int)load_ctx(a, b);
   int np = (ctx + a.part_tokens - 1) / a.part_tokens;
   if (np > a.num_parts) np = a.num_parts;
   const int64_t slot0 = ((int64_t)b * a.num_parts) * a.num_heads + h;
   const int64_t stride = a.num_heads;
-
-  // global max over the partitions
-  float mloc = -INFINITY;
-  for (int p = threadIdx.x; p < np; p += 256) mloc = fmaxf(mloc, a.ws_ml[(slot0 + p * stride) * 2]);
-  mloc = wave_max(mloc);
-  if (lane == 0) s_max[wave] = mloc;
-  __syncthreads();
-  const float mx = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
-
-  // wave w folds partitions w, w+4, ...; lane owns dims lane + 64 r
   float acc[kGenericMaxR];
 #pragma unroll
   for (int r = 0; r < kGenericMaxR; ++r) acc[r] = 0.f;
-  float lsum = 0.f;
+  float mx = -INFINITY, lsum = 0.f;
 #pragma unroll 4
-  for (int p = wave; p < np; p += 4) {
+  for (int p = 0; p < np; ++p) {
     const int64_t s = slot0 + p * stride;
     const float2 ml = *reinterpret_cast<const float2*>(a.ws_ml + s * 2);
-    const float wgt = safe_exp2_diff(ml.x, mx);
-    lsum = fmaf(wgt, ml.y, lsum);
+    float part[kGenericMaxR];
 #pragma unroll
     for (int r = 0; r < kGenericMaxR; ++r) {
       const int d = lane + 64 * r;
-      if (d < D) acc[r] = fmaf(wgt, a.ws_acc[s * D + d], acc[r]);
+      part[r] = d < D ? a.ws_acc[s * D + d] : 0.f;
     }
-  }
+    const float mn = fmaxf(mx, ml.x);
+    const float keep = safe_exp2_diff(mx, mn);
+    const float wgt = safe_exp2_diff(ml.x, mn);
+    lsum = lsum * keep + ml.y * wgt;
 #pragma unroll
-  for (int r = 0; r < kGenericMaxR; ++r) s_acc[wave][lane + 64 * r] = acc[r];
-  if (lane == 0) s_l[wave] = lsum;
-  __syncthreads();
+    for (int r = 0; r < kGenericMaxR; ++r) acc[r] = acc[r] * keep + part[r] * wgt;
+    mx = mn;
+  }
   T* out = reinterpret_cast<T*>(a.out) + ((int64_t)b * a.num_heads + h) * D;
-  const float ltot = s_l[0] + s_l[1] + s_l[2] + s_l[3];
-  const float linv = ltot > 0.f ? 1.f / ltot : 0.f;
-  for (int d = threadIdx.x; d < D; d += 256) {
-    const float o = s_acc[0][d] + s_acc[1][d] + s_acc[2][d] + s_acc[3][d];
-    out[d] = from_float<T>(o * linv);
+  const float linv = lsum > 0.f ? 1.f / lsum : 0.f;
+#pragma unroll
+  for (int r = 0; r < kGenericMaxR; ++r) {
+    const int d = lane + 64 * r;
+    if (d < D) out[d] = from_float<T>(acc[r] * linv);
   }
 }
 
@@ -846,17 +843,13 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stre
   const int group = a.num_heads / a.num_kv_heads;
   bool launched = false;
   if constexpr (IsSixteenBit<T>::value) {
-    if (fast_ok && !int8) {
-      const int wpb = largest_divisor_le(a.num_kv_heads, 8);
+    if (fast_ok && (!int8 || group <= 4)) {
+      const int wpb = largest_divisor_le(a.num_kv_heads, MVLLM_DECODE_WPB);
       dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, (unsigned)(a.num_kv_heads / wpb));
       dim3 block(64 * wpb);
-      if (group <= 4) decode_mfma_kernel<T, 1><<<grid, block, 0, stream>>>(a);
+      if (int8) decode_mfma_int8_kernel<T, 1><<<grid, block, 0, stream>>>(a);
+      else if (group <= 4) decode_mfma_kernel<T, 1><<<grid, block, 0, stream>>>(a);
       else decode_mfma_kernel<T, 2><<<grid, block, 0, stream>>>(a);
-      launched = true;
-    } else if (fast_ok && int8 && group <= 4) {
-      const int wpb = largest_divisor_le(a.num_kv_heads, 8);
-      dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, (unsigned)(a.num_kv_heads / wpb));
-      decode_mfma_int8_kernel<T, 1><<<grid, dim3(64 * wpb), 0, stream>>>(a);
       launched = true;
     }
   }
@@ -868,7 +861,7 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stre
   int st = launch_status();
   if (st != 0) return st;
   if (a.num_parts > 1) {
-    decode_reduce_kernel<T><<<dim3((unsigned)a.num_heads, (unsigned)a.batch), dim3(256), 0, stream>>>(a);
+    decode_reduce_kernel<T><<<dim3((unsigned)((a.num_heads + 3) / 4), (unsigned)a.batch), dim3(256), 0, stream>>>(a);
     st = launch_status();
   }
   return st;

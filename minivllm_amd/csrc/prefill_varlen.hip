@@ -222,11 +222,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
   const bool active = r0 < seq_len;
   const int jd = r0 / kBN;                           // diagonal K/V tile of this wave
   const int wg_last = min(row0 + BM, seq_len) - 1;
-#ifdef MVLLM_PF_ONETILE
-  const int ntiles = 1;      // experiment only: wrong results
-#else
   const int ntiles = wg_last / kBN + 1;
-#endif
   const int l32 = lane & 31;
   const int hi = lane >> 5;                          // 0/1: which half of the k-slots / rows
   const int qrow = r0 + l32;                         // query row of this lane
@@ -303,9 +299,6 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
     // ---- S^T = K Q^T ----
     v16f s[2];
     const char* kb = lds_k[buf];
-#ifdef MVLLM_PF_PRIO
-    __builtin_amdgcn_s_setprio(MVLLM_PF_PRIO);
-#endif
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk) {
       if (tk < ntk) {
@@ -322,9 +315,6 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
         for (int r = 0; r < 16; ++r) s[tk][r] = -INFINITY;   // never visited: masked out
       }
     }
-#ifdef MVLLM_PF_PRIO
-    __builtin_amdgcn_s_setprio(0);
-#endif
 
     // ---- online softmax, one query row per lane (scores stay unscaled; the scale is folded
     //      into the exp2 argument) ----
@@ -367,9 +357,6 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
 
     // ---- O^T += V^T P^T ----
     const char* vb = lds_v[buf];
-#ifdef MVLLM_PF_PRIO
-    __builtin_amdgcn_s_setprio(MVLLM_PF_PRIO);
-#endif
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk) {
       if (tk < ntk) {
@@ -395,9 +382,6 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
         }
       }
     }
-#ifdef MVLLM_PF_PRIO
-    __builtin_amdgcn_s_setprio(0);
-#endif
   }
 
   // ---- epilogue: normalise, transpose through LDS (the K buffers are free now), store whole rows ----
@@ -426,11 +410,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
     const int row = 4 * i + (lane >> 4);
     const int c = lane & 15;
     const uint4 w = *reinterpret_cast<const uint4*>(ot + row * 256 + ((c ^ (row & 15)) << 4));
-#ifdef MVLLM_PF_NOSTORE
-    if (w.x == 0x12345678u)
-#else
     if (r0 + row < seq_len)
-#endif
       *reinterpret_cast<uint4*>(out + ((int64_t)(seq_start + r0 + row) * a.num_heads + h) * D + 8 * c) = w;
   }
 }
