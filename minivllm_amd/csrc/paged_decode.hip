@@ -236,9 +236,10 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_ke
   if (!decode_item(a, b, p)) return;
   const int g = blockIdx.z * waves_per_block + wave;   // kv head
   const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head
-  const bool direct = (a.num_parts == 1);
 
   const int ctx = (int)load_ctx(a, b);
+  // a sequence that fits one partition (or is empty) is finished here: partition 0 writes the output row
+  const bool direct = ctx <= a.part_tokens;
   const int part_start = p * a.part_tokens;
   if (part_start >= ctx && !(direct && p == 0)) return;
   const int part_end = min(ctx, part_start + a.part_tokens);
@@ -400,11 +401,12 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_in
   if (!decode_item(a, b, p)) return;
   const int g = blockIdx.z * waves_per_block + wave;
   const int group = a.num_heads / a.num_kv_heads;
-  const bool direct = (a.num_parts == 1);
   const int q4 = lane >> 4;            // token class: tokens 4*q4 .. 4*q4+3 of a tile
   const int hb = (lane >> 3) & 1;      // which of the two V rows of an instruction this lane reads
 
   const int ctx = (int)load_ctx(a, b);
+  // a sequence that fits one partition (or is empty) is finished here: partition 0 writes the output row
+  const bool direct = ctx <= a.part_tokens;
   const int part_start = p * a.part_tokens;
   if (part_start >= ctx && !(direct && p == 0)) return;
   const int part_end = min(ctx, part_start + a.part_tokens);
@@ -686,9 +688,10 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(const DecodeArgs a) 
   const int D = a.head_dim;
   const int group = a.num_heads / a.num_kv_heads;
   const int g = h / group;
-  const bool direct = (a.num_parts == 1);
 
   const int ctx = (int)load_ctx(a, b);
+  // a sequence that fits one partition (or is empty) is finished here: partition 0 writes the output row
+  const bool direct = ctx <= a.part_tokens;
   const int part_start = p * a.part_tokens;
   if (part_start >= ctx && !(direct && p == 0)) return;
   const int part_end = min(ctx, part_start + a.part_tokens);
@@ -784,6 +787,7 @@ __global__ __launch_bounds__(256) void decode_reduce_kernel(const DecodeArgs a) 
   const int ctx = (int)load_ctx(a, b);
   int np = (ctx + a.part_tokens - 1) / a.part_tokens;
   if (np > a.num_parts) np = a.num_parts;
+  if (np <= 1) return;                               // written directly by the partition-0 workgroup
   const int64_t slot0 = ((int64_t)b * a.num_parts) * a.num_heads + h;
   const int64_t stride = a.num_heads;
   float acc[kGenericMaxR];
