@@ -242,7 +242,7 @@ def bench_int8(args):
     }
 
 
-def bench_engine(args, max_num_sequences):
+def bench_engine(args, max_num_sequences, graph):
     """BASELINE config 5: random-init Qwen3-style decoder (hidden 1024, 8 layers, Hq16/Hkv8/D128, FFN 3072,
     vocab 151936, bf16), 60 prompts of random ids with lengths U[32,96], 256 new tokens each, T 0.6."""
     import torch
@@ -252,8 +252,8 @@ def bench_engine(args, max_num_sequences):
     cfg = dict(vocab_size=151936, hidden_size=1024, num_layers=8, num_heads=16, num_kv_heads=8, head_dim=128,
                intermediate_size=3072, base=1_000_000, rms_norm_epsilon=1e-6, qkv_bias=False, ffn_bias=True,
                scale=1.0, tie_word_embeddings=True, block_size=256, max_num_batched_tokens=16384,
-               max_num_sequences=max_num_sequences, max_cached_blocks=256, max_position=512, dtype="bf16",
-               eos=-1, seed=args.seed)
+               max_num_sequences=max_num_sequences, max_cached_blocks=256, max_position=512,
+               max_model_length=512, enforce_eager=not graph, dtype="bf16", eos=-1, seed=args.seed)
     g = torch.Generator().manual_seed(args.seed)
     lengths = torch.randint(32, 97, (60,), generator=g).tolist()
     prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lengths]
@@ -271,7 +271,8 @@ def bench_engine(args, max_num_sequences):
     assert new_tokens == 60 * 256
     return {
         "workload": "engine generate: 60 prompts L~U[32,96], 256 new tokens each, Qwen3-style 8x1024 bf16, "
-                    f"block_size 256, max_num_sequences {max_num_sequences}, eager decode",
+                    f"block_size 256, max_num_sequences {max_num_sequences}, "
+                    + ("hipGraph decode" if graph else "eager decode"),
         "output_tokens": new_tokens, "wall_s": wall, "tok_per_s": new_tokens / wall,
         "steps": engine.stats["steps"], "decode_s": engine.stats["decode_s"], "prefill_s": engine.stats["prefill_s"],
     }
@@ -309,8 +310,9 @@ def main():
     if want("int8"):
         extra["int8"] = bench_int8(args)
     if want("engine"):
-        extra["engine_16seq"] = bench_engine(args, 16)
-        extra["engine_64seq"] = bench_engine(args, 64)
+        extra["engine_16seq_eager"] = bench_engine(args, 16, False)
+        extra["engine_16seq_graph"] = bench_engine(args, 16, True)
+        extra["engine_64seq_graph"] = bench_engine(args, 64, True)
 
     line = {
         "metric": "decode-attn HBM GB/s (% peak); prefill TFLOP/s (% MFMA); engine out tok/s",

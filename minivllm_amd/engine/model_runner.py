@@ -42,6 +42,9 @@ class ModelRunner:
         self.sampler = Sampler()
         self.generator = torch.Generator(device=self.device).manual_seed(config.get("seed", 0))
         self.allocate_kv_cache()
+        self.graphs = {}
+        if not config.get("enforce_eager", True):
+            self.capture_decode_graphs()
 
     def allocate_kv_cache(self):
         """One pool ``[2, L, num_blocks, block_size, Hkv, D]``; each ``Attention`` gets its layer's views
@@ -90,10 +93,68 @@ class ModelRunner:
         return self._to_device(md["input_ids"], torch.int64), context_lens - 1
 
     @torch.inference_mode()
+    def capture_decode_graphs(self):
+        """Record one hipGraph of the decode forward pass per batch-size bucket (model_runner.py:316-369).
+
+        The step metadata lives in static device buffers that ``run`` refills before every replay; rows past
+        the real batch carry slot -1, context length 0 and whatever table entries were there, which the
+        kernels treat as "store nothing, output zeros".  Positions are derived from the context lengths inside
+        the graph.  The attention library allocates nothing and its grids depend only on the static shapes
+        (batch bucket, table width), so a replay is valid for any contents of the buffers."""
+        cfg = self.config
+        max_bs = cfg.get("max_num_sequences", 16)
+        max_len = cfg.get("max_model_length", cfg.get("max_position", 4096))
+        max_blocks = -(-max_len // self.block_size)
+        dev = self.device
+        self.graph_vars = dict(
+            input_ids=torch.zeros(max_bs, dtype=torch.int64, device=dev),
+            slot_mapping=torch.full((max_bs,), -1, dtype=torch.int64, device=dev),
+            context_lens=torch.zeros(max_bs, dtype=torch.int64, device=dev),
+            block_tables=torch.zeros(max_bs, max_blocks, dtype=torch.int32, device=dev),
+            outputs=torch.zeros(max_bs, cfg["hidden_size"], dtype=self.dtype, device=dev))
+        v = self.graph_vars
+        buckets = sorted({b for b in [1, 2, 4, 8] + list(range(16, max_bs + 1, 16)) + [max_bs] if b <= max_bs})
+        pool = None
+        for bs in reversed(buckets):
+            set_context(False, slot_mapping=v["slot_mapping"][:bs], context_lens=v["context_lens"][:bs],
+                        block_tables=v["block_tables"][:bs])
+
+            def forward():
+                positions = (v["context_lens"][:bs] - 1).clamp_min(0)
+                v["outputs"][:bs] = self.model(v["input_ids"][:bs], positions)
+
+            forward()                                    # warm-up: sizes the attention workspace before capture
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool):
+                forward()
+            pool = graph.pool() if pool is None else pool
+            self.graphs[bs] = graph
+            torch.cuda.synchronize()
+            reset_context()
+
+    def _replay_decode(self, input_ids, bs):
+        from minivllm_amd.utils.context import get_context
+        ctx = get_context()
+        gbs = next(b for b in sorted(self.graphs) if b >= bs)
+        v = self.graph_vars
+        v["input_ids"][:bs].copy_(input_ids)
+        v["slot_mapping"][:gbs].fill_(-1)
+        v["slot_mapping"][:bs].copy_(ctx.slot_mapping)
+        v["context_lens"][:gbs].zero_()
+        v["context_lens"][:bs].copy_(ctx.context_lens)
+        v["block_tables"][:bs, :ctx.block_tables.size(1)].copy_(ctx.block_tables)
+        self.graphs[gbs].replay()
+        return v["outputs"][:bs]
+
+    @torch.inference_mode()
     def run(self, seqs, is_prefill: bool) -> list[int]:
         input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
         temperatures = self._to_device([seq.temperature for seq in seqs], torch.float32)
-        hidden = self.model(input_ids, positions)
+        if not is_prefill and self.graphs and len(seqs) <= max(self.graphs):
+            hidden = self._replay_decode(input_ids, len(seqs))
+        else:
+            hidden = self.model(input_ids, positions)
         logits = self.model.compute_logits(hidden)
         token_ids = self.sampler(logits, temperatures, self.generator).tolist()
         reset_context()
