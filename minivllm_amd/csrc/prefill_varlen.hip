@@ -6,6 +6,7 @@
 // and a workgroup finds its (sequence, local tile) by walking cu_seqlens, so
 // the grid needs only total_tokens and num_seqs (upper bound
 // total_tokens/BM + num_seqs tiles) and no host-side maximum length.
+#include <type_traits>
 #include "common.h"
 
 namespace mvllm {
@@ -165,6 +166,14 @@ constexpr int kBN = 64;                 // K/V rows per LDS tile
 constexpr int kWaveRows = 32;           // query rows per wave
 constexpr int kTileBytes = kBN * 256;   // one K (or V) tile, head_dim 128 x 2 B
 
+// v_max3_f32 without the canonicalising self-max the compiler puts in front of every fmaxf operand that
+// comes out of an MFMA (scores are finite or -inf here, never NaN).
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
 template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
   v2f x = {a, b};
@@ -276,43 +285,42 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
   float m = -INFINITY;
   float l = 0.f;
 
-  // per-lane constant parts of the LDS addresses
-  const int k_row_off = l32 * 256;                         // K: row l32 (+32*tk), chunk (2*ks+hi) ^ (row&15)
-  const int k_swz = l32 & 15;
+  // Per-lane LDS byte offsets, computed once: the xor swizzle keeps the compiler from folding them into
+  // instruction offsets, so they live in registers and every LDS read below is base + immediate.
+  //   K: row l32 (+32 rows per tk = +8192 B), 16-byte chunk (2*ks + hi) ^ (l32 & 15)
+  //   V: row 4*hi + (lane&15)/4 (+8, +16*st, +32*tk rows), chunk (4*td + 2*half + ...) ^ 4*(row & 3)
   const int i16 = lane & 15;
   const int half = (lane >> 4) & 1;
-  const int v_row = 4 * hi + (i16 >> 2);                   // V: row 32*tk + 16*st + v_row (+8)
-  const int v_swz = (v_row & 3) << 2;
-  const int v_chunk = 2 * half + ((i16 & 3) >> 1);         // + 4*td
-  const int v_byte = (i16 & 1) << 3;
+  int k_off[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) k_off[ks] = l32 * 256 + (((2 * ks + hi) ^ (l32 & 15)) << 4);
+  const int v_row = 4 * hi + (i16 >> 2);
+  int v_off[4];
+#pragma unroll
+  for (int td = 0; td < 4; ++td)
+    v_off[td] = v_row * 256 + (((4 * td + 2 * half + ((i16 & 3) >> 1)) ^ ((v_row & 3) << 2)) << 4) + ((i16 & 1) << 3);
 
-  for (int j = 0; j < ntiles; ++j) {
-    const int buf = j & 1;
-    dma_wait_all();                    // this wave's share of tile j has landed
-    __syncthreads();                   // ... and everybody else's; tile j-1 is no longer read
-    if (j + 1 < ntiles) issue_tile(j + 1, buf ^ 1);
-    if (!active || j > jd) continue;
+  // One K/V tile: scores, softmax, P.V.  BUF is a compile-time buffer index so that all LDS addresses are
+  // register + constant.
+  auto tile_step = [&](int j, auto BUF) {
+    constexpr int buf = decltype(BUF)::value;
     const bool diag = (j == jd);
-    // on the diagonal tile a wave whose rows sit in the first half never sees kv rows 32..63
-    const int ntk = (diag && (r0 & 32) == 0) ? 1 : 2;
 
-    // ---- S^T = K Q^T ----
+    // ---- S^T = K Q^T (on the diagonal tile rows past the causal limit are computed and then masked) ----
+    // The two 32-row halves of the tile form two independent accumulator chains that are issued
+    // alternately, so no MFMA waits for the result of the one before it.
     v16f s[2];
-    const char* kb = lds_k[buf];
+    const char* kb = &lds_k[buf][0];
+    {
+      const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      s[0] = zero;
+      s[1] = zero;
 #pragma unroll
-    for (int tk = 0; tk < 2; ++tk) {
-      if (tk < ntk) {
-        uint4 kf[8];
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks)
-          kf[ks] = *reinterpret_cast<const uint4*>(kb + tk * 32 * 256 + k_row_off + (((2 * ks + hi) ^ k_swz) << 4));
-        const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        s[tk] = mfma32x32x16<T>(kf[0], qf[0], zero);
-#pragma unroll
-        for (int ks = 1; ks < 8; ++ks) s[tk] = mfma32x32x16<T>(kf[ks], qf[ks], s[tk]);
-      } else {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[tk][r] = -INFINITY;   // never visited: masked out
+      for (int ks = 0; ks < 8; ++ks) {
+        const uint4 k0 = *reinterpret_cast<const uint4*>(kb + k_off[ks]);
+        const uint4 k1 = *reinterpret_cast<const uint4*>(kb + k_off[ks] + 32 * 256);
+        s[0] = mfma32x32x16<T>(k0, qf[ks], s[0]);
+        s[1] = mfma32x32x16<T>(k1, qf[ks], s[1]);
       }
     }
 
@@ -326,11 +334,13 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
         for (int r = 0; r < 16; ++r)
           if (32 * tk + 8 * (r >> 2) + (r & 3) > thr) s[tk][r] = -INFINITY;
     }
-    float mx = -INFINITY;
+    float mx = max3(s[0][0], s[0][1], s[0][2]);
 #pragma unroll
-    for (int tk = 0; tk < 2; ++tk)
+    for (int r = 3; r < 15; r += 2) mx = max3(mx, s[0][r], s[0][r + 1]);
+    mx = max3(mx, s[0][15], s[1][0]);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[tk][r]);
+    for (int r = 1; r < 15; r += 2) mx = max3(mx, s[1][r], s[1][r + 1]);
+    mx = fmaxf(mx, s[1][15]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * a.scale_log2;
     const bool grow = mx > m + 8.f || m == -INFINITY;
     if (__any(grow)) {
@@ -343,7 +353,6 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
         for (int r = 0; r < 16; ++r) o[td][r] *= alpha;
       m = m_new;
     }
-    float sum = 0.f;
     const float neg_m = -m;
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk)
@@ -351,36 +360,47 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
       for (int r = 0; r < 16; ++r) {
         const float pv = fast_exp2(fmaf(s[tk][r], a.scale_log2, neg_m));
         s[tk][r] = pv;
-        sum += pv;
+        l += pv;      // partial: this lane's kv rows only; lanes l and l^32 are added at the end
       }
-    l += sum;       // partial: this lane's kv rows only; lanes l and l^32 are added at the end
 
     // ---- O^T += V^T P^T ----
-    const char* vb = lds_v[buf];
+    const char* vb = &lds_v[buf][0];
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk) {
-      if (tk < ntk) {
 #pragma unroll
-        for (int st = 0; st < 2; ++st) {
-          uint4 pf;
-          pf.x = pack2<T>(s[tk][8 * st + 0], s[tk][8 * st + 1]);
-          pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
-          pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
-          pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
-          const char* vrow = vb + (32 * tk + 16 * st + v_row) * 256 + v_byte;
-          uint4 af[4];
+      for (int st = 0; st < 2; ++st) {
+        uint4 pf;
+        pf.x = pack2<T>(s[tk][8 * st + 0], s[tk][8 * st + 1]);
+        pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
+        pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
+        pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
+        uint4 af[4];
 #pragma unroll
-          for (int td = 0; td < 4; ++td) {
-            const char* p0 = vrow + (((4 * td + v_chunk) ^ v_swz) << 4);
-            const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
-            const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * 256));
-            af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;
-            af[td].z = __builtin_bit_cast(uint2, a1).x; af[td].w = __builtin_bit_cast(uint2, a1).y;
-          }
-#pragma unroll
-          for (int td = 0; td < 4; ++td) o[td] = mfma32x32x16<T>(af[td], pf, o[td]);
+        for (int td = 0; td < 4; ++td) {
+          const char* p0 = vb + v_off[td] + (32 * tk + 16 * st) * 256;
+          const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
+          const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * 256));
+          af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;
+          af[td].z = __builtin_bit_cast(uint2, a1).x; af[td].w = __builtin_bit_cast(uint2, a1).y;
         }
+#pragma unroll
+        for (int td = 0; td < 4; ++td) o[td] = mfma32x32x16<T>(af[td], pf, o[td]);
       }
+    }
+  };
+
+  // Double-buffered main loop, unrolled by two so that the buffer index is a compile-time constant.
+  auto sync_and_prefetch = [&](int j, int next_buf) {
+    dma_wait_all();                    // this wave's share of tile j has landed
+    __syncthreads();                   // ... and everybody else's; tile j-1 is no longer read
+    if (j + 1 < ntiles) issue_tile(j + 1, next_buf);
+  };
+  for (int j = 0; j < ntiles; j += 2) {
+    sync_and_prefetch(j, 1);
+    if (active && j <= jd) tile_step(j, std::integral_constant<int, 0>{});
+    if (j + 1 < ntiles) {
+      sync_and_prefetch(j + 1, 0);
+      if (active && j + 1 <= jd) tile_step(j + 1, std::integral_constant<int, 1>{});
     }
   }
 
