@@ -162,6 +162,10 @@ typedef __attribute__((ext_vector_type(2))) _Float16 v2f16;
 #define MVLLM_PF_XCD_CHUNK 32
 #endif
 constexpr unsigned kXcdChunk = MVLLM_PF_XCD_CHUNK;   // consecutive work items handed to one XCD
+#ifndef MVLLM_PF_WAVES
+#define MVLLM_PF_WAVES 4
+#endif
+constexpr int kPfWaves = MVLLM_PF_WAVES;             // waves per workgroup: 4, so that two workgroups share a CU
 constexpr int kBN = 64;                 // K/V rows per LDS tile
 constexpr int kWaveRows = 32;           // query rows per wave
 constexpr int kTileBytes = kBN * 256;   // one K (or V) tile, head_dim 128 x 2 B
@@ -197,9 +201,10 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 }
 
 template <typename T, int HPW>
-__global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs a) {
+__global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const PrefillArgs a) {
   constexpr int D = 128;
-  constexpr int ROW_TILES = 8 / HPW;            // 32-row query tiles per workgroup
+  constexpr int ROW_TILES = kPfWaves / HPW;     // 32-row query tiles per workgroup
+  constexpr int ROWS_PER_WAVE = kBN / kPfWaves; // K/V tile rows one wave copies (4 per instruction)
   constexpr int BM = kWaveRows * ROW_TILES;     // query rows per workgroup
   __shared__ __attribute__((aligned(1024))) char lds_k[2][kTileBytes];
   __shared__ __attribute__((aligned(1024))) char lds_v[2][kTileBytes];
@@ -247,16 +252,16 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_kernel(const PrefillArgs 
   const int ld_chunk = lane & 15;      // destination chunk inside the row
   auto issue_tile = [&](int j, int buf) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int row = 8 * wave + 4 * i + ld_row;           // row inside the tile
+    for (int i = 0; i < ROWS_PER_WAVE / 4; ++i) {
+      const int row = ROWS_PER_WAVE * wave + 4 * i + ld_row;   // row inside the tile
       int64_t tok = (int64_t)seq_start + (int64_t)j * kBN + row;
       if (tok > last_token) tok = last_token;
       const int kc = ld_chunk ^ (row & 15);
       const int vc = ld_chunk ^ ((row & 3) << 2);
       const char* ksrc = kg + tok * kv_row_bytes + (int64_t)g * (D * 2) + kc * 16;
       const char* vsrc = vg + tok * kv_row_bytes + (int64_t)g * (D * 2) + vc * 16;
-      const uint32_t kdst = __builtin_amdgcn_readfirstlane(lds_address(&lds_k[buf][(8 * wave + 4 * i) * 256]));
-      const uint32_t vdst = __builtin_amdgcn_readfirstlane(lds_address(&lds_v[buf][(8 * wave + 4 * i) * 256]));
+      const uint32_t kdst = __builtin_amdgcn_readfirstlane(lds_address(&lds_k[buf][(ROWS_PER_WAVE * wave + 4 * i) * 256]));
+      const uint32_t vdst = __builtin_amdgcn_readfirstlane(lds_address(&lds_v[buf][(ROWS_PER_WAVE * wave + 4 * i) * 256]));
       dma16_to_lds(ksrc, kdst);
       dma16_to_lds(vsrc, vdst);
     }
@@ -439,16 +444,16 @@ template <typename T>
 static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   const int group = a.num_heads / a.num_kv_heads;
   const int hpw = group >= 4 ? 4 : group;              // 1, 2 or 4 (group is 1, 2 or a multiple of 4)
-  const int bm = kWaveRows * (8 / hpw);
+  const int bm = kWaveRows * (kPfWaves / hpw);
   PrefillArgs b = a;
   b.tiles_x = (int)(a.total_tokens / bm + a.num_seqs);
   b.heads_y = a.num_kv_heads * (group / hpw);
   const int64_t items = (int64_t)b.tiles_x * b.heads_y;
   const int64_t span = 8 * (int64_t)kXcdChunk;
   dim3 grid((unsigned)((items + span - 1) / span * span));
-  if (hpw == 4) prefill_mfma_kernel<T, 4><<<grid, dim3(512), 0, stream>>>(b);
-  else if (hpw == 2) prefill_mfma_kernel<T, 2><<<grid, dim3(512), 0, stream>>>(b);
-  else prefill_mfma_kernel<T, 1><<<grid, dim3(512), 0, stream>>>(b);
+  if (hpw == 4) prefill_mfma_kernel<T, 4><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
+  else if (hpw == 2) prefill_mfma_kernel<T, 2><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
+  else prefill_mfma_kernel<T, 1><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
   return launch_status();
 }
 template <typename T>
