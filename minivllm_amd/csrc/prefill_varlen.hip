@@ -188,12 +188,13 @@ template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, v2f16));
 }
 
-// 16 bytes per lane from global straight into LDS at lds_base + 16 * lane (global_load_lds_dwordx4).
-// Written as inline asm on purpose: the compiler then neither tracks the transfer in vmcnt nor
-// inserts a full vmcnt(0) wait before the next LDS read, so the copy of tile j+1 really overlaps
-// the math on tile j; completion is awaited explicitly with dma_wait_all() before the barrier.
-__device__ __forceinline__ void dma16_to_lds(const void* gsrc, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gsrc) : "memory");
+// 16 bytes per lane from global (wave-uniform base + per-lane 32-bit byte offset) straight into LDS at
+// lds_base + 16 * lane (global_load_lds_dwordx4).  Written as inline asm on purpose: the compiler then neither
+// tracks the transfer in vmcnt nor inserts a full vmcnt(0) wait before the next LDS read, so the copy of tile
+// j+1 really overlaps the math on tile j; completion is awaited explicitly with dma_wait_all() before the
+// barrier.
+__device__ __forceinline__ void dma16_to_lds(const void* gbase, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(lane_off), "s"(gbase) : "memory");
 }
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
@@ -225,9 +226,14 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   int seq_start, seq_len, row0;
   // latest (heaviest) tiles of a sequence first
   if (!locate_tile(a.cu_seqlens, a.num_seqs, tiles_x - 1 - item_x, BM, seq_start, seq_len, row0)) return;
+  // Wave-uniform by construction; say so, so that everything derived from them (tile counts, loop bounds,
+  // tile base addresses, branches) lives in scalar registers and runs on the scalar unit.
+  seq_start = __builtin_amdgcn_readfirstlane(seq_start);
+  seq_len = __builtin_amdgcn_readfirstlane(seq_len);
+  row0 = __builtin_amdgcn_readfirstlane(row0);
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int group = a.num_heads / a.num_kv_heads;
   const int chunks = group / HPW;                    // workgroups per kv head
   const int g = item_y / chunks;                     // kv head
@@ -247,23 +253,40 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   const int64_t kv_row_bytes = (int64_t)a.num_kv_heads * D * 2;
   const int64_t last_token = a.total_tokens - 1;
 
-  // ---- K/V tile DMA: wave w moves rows 8w..8w+7 (2 instructions x 4 rows) of K and of V
+  // ---- K/V tile DMA: wave w moves ROWS_PER_WAVE rows (4 per instruction) of K and of V.
+  // Addresses are a wave-uniform 64-bit base (tile start, SALU arithmetic) plus a per-lane 32-bit offset that
+  // never changes, so a tile costs no VALU address math.  Only a tile that runs past the last packed token
+  // (the tail of the last sequence) recomputes clamped offsets.
   const int ld_row = lane >> 4;        // row inside the 4-row group
   const int ld_chunk = lane & 15;      // destination chunk inside the row
-  auto issue_tile = [&](int j, int buf) {
+  constexpr int kCopies = ROWS_PER_WAVE / 4;
+  uint32_t k_src_off[kCopies], v_src_off[kCopies];
 #pragma unroll
-    for (int i = 0; i < ROWS_PER_WAVE / 4; ++i) {
-      const int row = ROWS_PER_WAVE * wave + 4 * i + ld_row;   // row inside the tile
-      int64_t tok = (int64_t)seq_start + (int64_t)j * kBN + row;
-      if (tok > last_token) tok = last_token;
-      const int kc = ld_chunk ^ (row & 15);
-      const int vc = ld_chunk ^ ((row & 3) << 2);
-      const char* ksrc = kg + tok * kv_row_bytes + (int64_t)g * (D * 2) + kc * 16;
-      const char* vsrc = vg + tok * kv_row_bytes + (int64_t)g * (D * 2) + vc * 16;
-      const uint32_t kdst = __builtin_amdgcn_readfirstlane(lds_address(&lds_k[buf][(ROWS_PER_WAVE * wave + 4 * i) * 256]));
-      const uint32_t vdst = __builtin_amdgcn_readfirstlane(lds_address(&lds_v[buf][(ROWS_PER_WAVE * wave + 4 * i) * 256]));
-      dma16_to_lds(ksrc, kdst);
-      dma16_to_lds(vsrc, vdst);
+  for (int i = 0; i < kCopies; ++i) {
+    const int row = ROWS_PER_WAVE * wave + 4 * i + ld_row;   // row inside the tile
+    k_src_off[i] = (uint32_t)(row * (int)kv_row_bytes + ((ld_chunk ^ (row & 15)) << 4));
+    v_src_off[i] = (uint32_t)(row * (int)kv_row_bytes + ((ld_chunk ^ ((row & 3) << 2)) << 4));
+  }
+  auto issue_tile = [&](int j, int buf) {
+    const int64_t tok0 = (int64_t)seq_start + (int64_t)j * kBN;          // first row of the tile
+    const char* kbase = kg + tok0 * kv_row_bytes + (int64_t)g * (D * 2);
+    const char* vbase = vg + tok0 * kv_row_bytes + (int64_t)g * (D * 2);
+    const bool inside = tok0 + kBN - 1 <= last_token;
+#pragma unroll
+    for (int i = 0; i < kCopies; ++i) {
+      uint32_t ko = k_src_off[i], vo = v_src_off[i];
+      if (!inside) {                                                      // clamp rows past the end onto the last token
+        const int row = ROWS_PER_WAVE * wave + 4 * i + ld_row;
+        const int over = (int)(tok0 + row - last_token);
+        if (over > 0) {
+          ko -= (uint32_t)(over * (int)kv_row_bytes);
+          vo -= (uint32_t)(over * (int)kv_row_bytes);
+        }
+      }
+      const uint32_t kdst = lds_address(&lds_k[buf][(ROWS_PER_WAVE * wave + 4 * i) * 256]);
+      const uint32_t vdst = lds_address(&lds_v[buf][(ROWS_PER_WAVE * wave + 4 * i) * 256]);
+      dma16_to_lds(kbase, ko, kdst);
+      dma16_to_lds(vbase, vo, vdst);
     }
   };
   issue_tile(0, 0);
