@@ -178,6 +178,16 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return r;
 }
 
+// Compile-time loop: f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{}).
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
 template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
   v2f x = {a, b};
@@ -188,13 +198,28 @@ template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, v2f16));
 }
 
-// 16 bytes per lane from global (wave-uniform base + per-lane 32-bit byte offset) straight into LDS at
-// lds_base + 16 * lane (global_load_lds_dwordx4).  Written as inline asm on purpose: the compiler then neither
-// tracks the transfer in vmcnt nor inserts a full vmcnt(0) wait before the next LDS read, so the copy of tile
-// j+1 really overlaps the math on tile j; completion is awaited explicitly with dma_wait_all() before the
-// barrier.
-__device__ __forceinline__ void dma16_to_lds(const void* gbase, uint32_t lane_off, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(lane_off), "s"(gbase) : "memory");
+// 16 bytes per lane from a buffer resource (wave-uniform descriptor + per-lane 32-bit byte offset) straight
+// into LDS at lds_base + 16 * lane (buffer_load_dwordx4 ... lds).  Lanes whose offset is at or past the
+// descriptor's size read nothing and get zeros written, so tiles that run past the end of the tensor need no
+// clamping.  Written as inline asm on purpose: the compiler then neither tracks the transfer in vmcnt nor
+// inserts a full vmcnt(0) wait before the next LDS read, so the copy of tile j+1 really overlaps the math on
+// tile j; completion is awaited explicitly with dma_wait_all() before the barrier.  No "memory" clobber: the
+// destination buffer is not touched by ordinary code until after that wait and barrier (which do clobber), and
+// a clobber here would pin every LDS read of the tile in flight to its side of the copy.
+typedef __attribute__((ext_vector_type(4))) int v4i;
+template <int LDS_IMM>   // LDS destination = lds_base + LDS_IMM: one scalar register serves all copies of a wave
+__device__ __forceinline__ void dma16_to_lds(v4i rsrc, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_add_u32 m0, %0, %3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(lane_off), "s"(rsrc), "n"(LDS_IMM) : "scc");
+}
+// Raw buffer descriptor: 48-bit base, stride 0, size in bytes, 32-bit untyped data.
+__device__ __forceinline__ v4i make_rsrc(const char* base, uint32_t bytes) {
+  const uint64_t b = (uint64_t)base;
+  v4i r;
+  r[0] = (int)(uint32_t)b;
+  r[1] = (int)((uint32_t)(b >> 32) & 0xffffu);
+  r[2] = (int)bytes;
+  r[3] = 0x00020000;
+  return r;
 }
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
@@ -207,8 +232,8 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   constexpr int ROW_TILES = kPfWaves / HPW;     // 32-row query tiles per workgroup
   constexpr int ROWS_PER_WAVE = kBN / kPfWaves; // K/V tile rows one wave copies (4 per instruction)
   constexpr int BM = kWaveRows * ROW_TILES;     // query rows per workgroup
-  __shared__ __attribute__((aligned(1024))) char lds_k[2][kTileBytes];
-  __shared__ __attribute__((aligned(1024))) char lds_v[2][kTileBytes];
+  struct Tiles { char k[2][kTileBytes]; char v[2][kTileBytes]; };     // double-buffered K and V tiles
+  __shared__ __attribute__((aligned(1024))) Tiles lds;
 
   // Work item = (head slice y, query tile x), x fastest.  Workgroups are dealt to the 8 XCDs round-robin by
   // linear id; items are handed out in chunks of kXcdChunk consecutive items per XCD so that workgroups
@@ -267,27 +292,46 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     k_src_off[i] = (uint32_t)(row * (int)kv_row_bytes + ((ld_chunk ^ (row & 15)) << 4));
     v_src_off[i] = (uint32_t)(row * (int)kv_row_bytes + ((ld_chunk ^ ((row & 3) << 2)) << 4));
   }
-  auto issue_tile = [&](int j, int buf) {
-    const int64_t tok0 = (int64_t)seq_start + (int64_t)j * kBN;          // first row of the tile
-    const char* kbase = kg + tok0 * kv_row_bytes + (int64_t)g * (D * 2);
-    const char* vbase = vg + tok0 * kv_row_bytes + (int64_t)g * (D * 2);
-    const bool inside = tok0 + kBN - 1 <= last_token;
-#pragma unroll
-    for (int i = 0; i < kCopies; ++i) {
-      uint32_t ko = k_src_off[i], vo = v_src_off[i];
-      if (!inside) {                                                      // clamp rows past the end onto the last token
-        const int row = ROWS_PER_WAVE * wave + 4 * i + ld_row;
-        const int over = (int)(tok0 + row - last_token);
-        if (over > 0) {
-          ko -= (uint32_t)(over * (int)kv_row_bytes);
-          vo -= (uint32_t)(over * (int)kv_row_bytes);
-        }
-      }
-      const uint32_t kdst = lds_address(&lds_k[buf][(ROWS_PER_WAVE * wave + 4 * i) * 256]);
-      const uint32_t vdst = lds_address(&lds_v[buf][(ROWS_PER_WAVE * wave + 4 * i) * 256]);
-      dma16_to_lds(kbase, ko, kdst);
-      dma16_to_lds(vbase, vo, vdst);
-    }
+  // One tile's copy is 2 * kCopies instructions per wave (K copies first, then V).  Inside tile_step they are
+  // issued one at a time, spread between the MFMAs of the tile before, because a wave that issues them back
+  // to back sits in the memory pipeline's queue instead of feeding the matrix unit.  The descriptor of a tile
+  // starts at the tile's first row and ends with the tensor, so rows past the last packed token arrive as
+  // zeros; a descriptor of size 0 (enable = false) turns the copy into a zero fill that touches no memory,
+  // which keeps the last tile's code free of branches.
+  struct TileSrc { v4i k, v; };
+  const int row_bytes = (int)kv_row_bytes;
+  const int total_rows = (int)a.total_tokens;
+  const int rows_4g = (int)(0xffffffffu / (uint32_t)row_bytes);   // rows whose bytes no longer fit 32 bits
+  auto tile_src = [&](int j, bool enable) {
+    const int row0 = seq_start + j * kBN;                          // first row of the tile
+    const int rows_left = total_rows - row0;
+    const uint32_t size = (!enable || rows_left <= 0) ? 0u
+                          : rows_left > rows_4g       ? 0xffffffffu
+                                                      : (uint32_t)(rows_left * row_bytes - g * (D * 2));
+    const int64_t start = (int64_t)row0 * kv_row_bytes + (int64_t)g * (D * 2);
+    TileSrc t;
+    t.k = make_rsrc(kg + start, size);
+    t.v = make_rsrc(vg + start, size);
+    return t;
+  };
+  // LDS byte address of this wave's first row in buffer 0 of K; V, buffer 1 and later copies are constants away
+  // (the two arrays are laid out back to back by the struct below).
+  const uint32_t lds_wave_base = lds_address(&lds.k[0][0]) + (uint32_t)(ROWS_PER_WAVE * wave * 256);
+  auto issue_copy = [&](const TileSrc& t, auto BUF, auto C) {               // C < kCopies: K copy C, else V copy C - kCopies
+    constexpr int c = decltype(C)::value;
+    constexpr bool is_k = c < kCopies;
+    constexpr int i = is_k ? c : c - kCopies;
+    constexpr int imm = (is_k ? 0 : 2 * kTileBytes) + decltype(BUF)::value * kTileBytes + 4 * i * 256;
+    dma16_to_lds<imm>(is_k ? t.k : t.v, is_k ? k_src_off[i] : v_src_off[i], lds_wave_base);
+  };
+  auto issue_tile = [&](int j, int buf) {                        // whole tile at once, buffer chosen at run time
+    const TileSrc t = tile_src(j, true);
+    const uint32_t base = lds_wave_base + (uint32_t)buf * kTileBytes;
+    static_for<kCopies>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      dma16_to_lds<4 * i * 256>(t.k, k_src_off[i], base);
+      dma16_to_lds<2 * kTileBytes + 4 * i * 256>(t.v, v_src_off[i], base);
+    });
   };
   issue_tile(0, 0);
 
@@ -330,26 +374,29 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
 
   // One K/V tile: scores, softmax, P.V.  BUF is a compile-time buffer index so that all LDS addresses are
   // register + constant.
-  auto tile_step = [&](int j, auto BUF) {
+  auto tile_step = [&](int j, auto BUF, bool prefetch) {
     constexpr int buf = decltype(BUF)::value;
+    using NEXT_BUF = std::integral_constant<int, buf ^ 1>;
     const bool diag = (j == jd);
+    const TileSrc next = tile_src(j + 1, prefetch);
 
     // ---- S^T = K Q^T (on the diagonal tile rows past the causal limit are computed and then masked) ----
     // The two 32-row halves of the tile form two independent accumulator chains that are issued
     // alternately, so no MFMA waits for the result of the one before it.
     v16f s[2];
-    const char* kb = &lds_k[buf][0];
+    const char* kb = &lds.k[buf][0];
     {
       const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       s[0] = zero;
       s[1] = zero;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
+      static_for<8>([&](auto KS) {
+        constexpr int ks = decltype(KS)::value;
         const uint4 k0 = *reinterpret_cast<const uint4*>(kb + k_off[ks]);
         const uint4 k1 = *reinterpret_cast<const uint4*>(kb + k_off[ks] + 32 * 256);
         s[0] = mfma32x32x16<T>(k0, qf[ks], s[0]);
         s[1] = mfma32x32x16<T>(k1, qf[ks], s[1]);
-      }
+        if constexpr (ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);           // copies of the next tile, K first
+      });
     }
 
     // ---- online softmax, one query row per lane (scores stay unscaled; the scale is folded
@@ -392,52 +439,61 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       }
 
     // ---- O^T += V^T P^T ----
-    const char* vb = &lds_v[buf][0];
+    const char* vb = &lds.v[buf][0];
+    static_for<4>([&](auto STEP) {                     // 16 kv rows per step
+      constexpr int tk = decltype(STEP)::value / 2, st = decltype(STEP)::value % 2;
+      uint4 pf;
+      pf.x = pack2<T>(s[tk][8 * st + 0], s[tk][8 * st + 1]);
+      pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
+      pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
+      pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
+      uint4 af[4];
 #pragma unroll
-    for (int tk = 0; tk < 2; ++tk) {
-#pragma unroll
-      for (int st = 0; st < 2; ++st) {
-        uint4 pf;
-        pf.x = pack2<T>(s[tk][8 * st + 0], s[tk][8 * st + 1]);
-        pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
-        pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
-        pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
-        uint4 af[4];
-#pragma unroll
-        for (int td = 0; td < 4; ++td) {
-          const char* p0 = vb + v_off[td] + (32 * tk + 16 * st) * 256;
-          const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
-          const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * 256));
-          af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;
-          af[td].z = __builtin_bit_cast(uint2, a1).x; af[td].w = __builtin_bit_cast(uint2, a1).y;
-        }
-#pragma unroll
-        for (int td = 0; td < 4; ++td) o[td] = mfma32x32x16<T>(af[td], pf, o[td]);
+      for (int td = 0; td < 4; ++td) {
+        const char* p0 = vb + v_off[td] + (32 * tk + 16 * st) * 256;
+        const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
+        const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * 256));
+        af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;
+        af[td].z = __builtin_bit_cast(uint2, a1).x; af[td].w = __builtin_bit_cast(uint2, a1).y;
       }
-    }
+#pragma unroll
+      for (int td = 0; td < 4; ++td) o[td] = mfma32x32x16<T>(af[td], pf, o[td]);
+    });
   };
 
-  // Double-buffered main loop, unrolled by two so that the buffer index is a compile-time constant.
-  auto sync_and_prefetch = [&](int j, int next_buf) {
+  // Tile j lives in buffer j % 2.  The main loop is unrolled by two so that the buffer index is a compile-time
+  // constant inside tile_step (all LDS addresses are register + immediate).
+  auto math_step = [&](int j, auto BUF) {
     dma_wait_all();                    // this wave's share of tile j has landed
     __syncthreads();                   // ... and everybody else's; tile j-1 is no longer read
-    if (j + 1 < ntiles) issue_tile(j + 1, next_buf);
+    tile_step(j, BUF, j + 1 < ntiles);
   };
-  for (int j = 0; j < ntiles; j += 2) {
-    sync_and_prefetch(j, 1);
-    if (active && j <= jd) tile_step(j, std::integral_constant<int, 0>{});
-    if (j + 1 < ntiles) {
-      sync_and_prefetch(j + 1, 0);
-      if (active && j + 1 <= jd) tile_step(j + 1, std::integral_constant<int, 1>{});
-    }
+  const int nmath = active ? jd + 1 : 0;               // tiles this wave computes on (<= ntiles)
+  int j = 0;
+  for (; j + 1 < nmath; j += 2) {
+    math_step(j, std::integral_constant<int, 0>{});
+    math_step(j + 1, std::integral_constant<int, 1>{});
+  }
+  if (j < nmath) {
+    math_step(j, std::integral_constant<int, 0>{});
+    ++j;
+  }
+  // Tiles that only other waves of the workgroup still compute on (their rows are further down): keep copying
+  // this wave's share and meeting the barriers.  Kept out of the loop above so that the accumulators have one
+  // straight-line life there.
+  for (; j < ntiles; ++j) {
+    dma_wait_all();
+    __syncthreads();
+    if (j + 1 < ntiles) issue_tile(j + 1, (j + 1) & 1);
   }
 
   // ---- epilogue: normalise, transpose through LDS (the K buffers are free now), store whole rows ----
   // lane holds row l32, dims 32*td + 8*(r/4) + 4*hi + r%4  ->  wave-private [32 rows][256 B] tile with
   // 16-byte chunks xor-swizzled by row, read back as 16 B per lane so every global store is a full row.
+  dma_wait_all();                                    // the zero fill issued during the last tile has landed
   __syncthreads();                                   // every wave is done reading K/V tiles
   if (!active) return;
-  char* ot = &lds_k[0][0] + wave * (kWaveRows * 256);   // 8 waves x 8 KB = both K buffers
+  char* ot = &lds.k[0][0] + wave * (kWaveRows * 256);   // 8 waves x 8 KB = both K buffers
   {
     const float lt = l + __shfl_xor(l, 32, 64);
     const float inv = 1.f / lt;
