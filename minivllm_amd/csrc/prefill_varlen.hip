@@ -372,39 +372,44 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   for (int td = 0; td < 4; ++td)
     v_off[td] = v_row * 256 + (((4 * td + 2 * half + ((i16 & 3) >> 1)) ^ ((v_row & 3) << 2)) << 4) + ((i16 & 1) << 3);
 
-  // One K/V tile: scores, softmax, P.V.  BUF is a compile-time buffer index so that all LDS addresses are
-  // register + constant.
-  auto tile_step = [&](int j, auto BUF, bool prefetch) {
+  // One K/V tile: scores, softmax, P.V.  Compile-time parameters: BUF, the buffer index (so that all LDS
+  // addresses are register + constant); DIAG, set for the wave's last tile, the one the causal diagonal runs
+  // through (the only one that is masked); NH, the number of 32-row halves of the tile that are computed at
+  // all: 1 when the wave's rows are the upper half of the 64-row block, so that the diagonal tile's second
+  // half is masked entirely.
+  auto tile_step = [&](int j, auto BUF, auto DIAG, auto NHALF, bool prefetch) {
     constexpr int buf = decltype(BUF)::value;
+    constexpr bool diag = decltype(DIAG)::value;
+    constexpr int NH = decltype(NHALF)::value;
     using NEXT_BUF = std::integral_constant<int, buf ^ 1>;
-    const bool diag = (j == jd);
     const TileSrc next = tile_src(j + 1, prefetch);
 
     // ---- S^T = K Q^T (on the diagonal tile rows past the causal limit are computed and then masked) ----
     // The two 32-row halves of the tile form two independent accumulator chains that are issued
     // alternately, so no MFMA waits for the result of the one before it.
-    v16f s[2];
+    v16f s[NH];
     const char* kb = &lds.k[buf][0];
     {
       const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      s[0] = zero;
-      s[1] = zero;
+#pragma unroll
+      for (int tk = 0; tk < NH; ++tk) s[tk] = zero;
       static_for<8>([&](auto KS) {
         constexpr int ks = decltype(KS)::value;
-        const uint4 k0 = *reinterpret_cast<const uint4*>(kb + k_off[ks]);
-        const uint4 k1 = *reinterpret_cast<const uint4*>(kb + k_off[ks] + 32 * 256);
-        s[0] = mfma32x32x16<T>(k0, qf[ks], s[0]);
-        s[1] = mfma32x32x16<T>(k1, qf[ks], s[1]);
+        uint4 kf[NH];
+#pragma unroll
+        for (int tk = 0; tk < NH; ++tk) kf[tk] = *reinterpret_cast<const uint4*>(kb + k_off[ks] + tk * 32 * 256);
+#pragma unroll
+        for (int tk = 0; tk < NH; ++tk) s[tk] = mfma32x32x16<T>(kf[tk], qf[ks], s[tk]);
         if constexpr (ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);           // copies of the next tile, K first
       });
     }
 
     // ---- online softmax, one query row per lane (scores stay unscaled; the scale is folded
     //      into the exp2 argument) ----
-    if (diag) {
+    if constexpr (diag) {
       const int thr = qrow - j * kBN - 4 * hi;       // kv offset inside the tile must be <= thr
 #pragma unroll
-      for (int tk = 0; tk < 2; ++tk)
+      for (int tk = 0; tk < NH; ++tk)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           if (32 * tk + 8 * (r >> 2) + (r & 3) > thr) s[tk][r] = -INFINITY;
@@ -412,10 +417,12 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     float mx = max3(s[0][0], s[0][1], s[0][2]);
 #pragma unroll
     for (int r = 3; r < 15; r += 2) mx = max3(mx, s[0][r], s[0][r + 1]);
-    mx = max3(mx, s[0][15], s[1][0]);
+    if constexpr (NH == 2) {
+      mx = max3(mx, s[0][15], s[NH - 1][0]);
 #pragma unroll
-    for (int r = 1; r < 15; r += 2) mx = max3(mx, s[1][r], s[1][r + 1]);
-    mx = fmaxf(mx, s[1][15]);
+      for (int r = 1; r < 15; r += 2) mx = max3(mx, s[NH - 1][r], s[NH - 1][r + 1]);
+    }
+    mx = fmaxf(mx, s[NH - 1][15]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * a.scale_log2;
     const bool grow = mx > m + 8.f || m == -INFINITY;
     if (__any(grow)) {
@@ -430,7 +437,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     }
     const float neg_m = -m;
 #pragma unroll
-    for (int tk = 0; tk < 2; ++tk)
+    for (int tk = 0; tk < NH; ++tk)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float pv = fast_exp2(fmaf(s[tk][r], a.scale_log2, neg_m));
@@ -440,7 +447,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
 
     // ---- O^T += V^T P^T ----
     const char* vb = &lds.v[buf][0];
-    static_for<4>([&](auto STEP) {                     // 16 kv rows per step
+    static_for<2 * NH>([&](auto STEP) {                // 16 kv rows per step
       constexpr int tk = decltype(STEP)::value / 2, st = decltype(STEP)::value % 2;
       uint4 pf;
       pf.x = pack2<T>(s[tk][8 * st + 0], s[tk][8 * st + 1]);
@@ -462,21 +469,36 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   };
 
   // Tile j lives in buffer j % 2.  The main loop is unrolled by two so that the buffer index is a compile-time
-  // constant inside tile_step (all LDS addresses are register + immediate).
-  auto math_step = [&](int j, auto BUF) {
+  // constant inside tile_step.  A wave's tiles are jd full ones and then the diagonal one.
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
+  using H1 = std::integral_constant<int, 1>;
+  using H2 = std::integral_constant<int, 2>;
+  auto full_step = [&](int j, auto BUF) {
     dma_wait_all();                    // this wave's share of tile j has landed
     __syncthreads();                   // ... and everybody else's; tile j-1 is no longer read
-    tile_step(j, BUF, j + 1 < ntiles);
+    tile_step(j, BUF, std::false_type{}, H2{}, j + 1 < ntiles);
   };
-  const int nmath = active ? jd + 1 : 0;               // tiles this wave computes on (<= ntiles)
+  auto diag_step = [&](int j, auto BUF) {
+    dma_wait_all();
+    __syncthreads();
+    if ((r0 & 32) == 0) tile_step(j, BUF, std::true_type{}, H1{}, j + 1 < ntiles);
+    else tile_step(j, BUF, std::true_type{}, H2{}, j + 1 < ntiles);
+  };
   int j = 0;
-  for (; j + 1 < nmath; j += 2) {
-    math_step(j, std::integral_constant<int, 0>{});
-    math_step(j + 1, std::integral_constant<int, 1>{});
-  }
-  if (j < nmath) {
-    math_step(j, std::integral_constant<int, 0>{});
-    ++j;
+  if (active) {
+    for (; j + 1 < jd; j += 2) {
+      full_step(j, B0{});
+      full_step(j + 1, B1{});
+    }
+    if (j < jd) {
+      full_step(j, B0{});
+      diag_step(j + 1, B1{});
+      j += 2;
+    } else {
+      diag_step(j, B0{});
+      j += 1;
+    }
   }
   // Tiles that only other waves of the workgroup still compute on (their rows are further down): keep copying
   // this wave's share and meeting the barriers.  Kept out of the loop above so that the accumulators have one
