@@ -134,11 +134,14 @@ __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs 
 // ---------------------------------------------------------------------------
 // MFMA path: 16-bit inputs, head_dim 128.
 //
-// Workgroup = 8 waves = (one kv head, HPW of the query heads that share it,
-// 8/HPW consecutive 32-row query tiles); every wave owns 32 query rows of one
-// head; two waves per SIMD so one wave's softmax overlaps the other's MFMAs.  All waves walk the same 64-row K/V tiles, which are DMA'd from global
-// into LDS once per workgroup (global_load_lds, 16 B per lane, double
-// buffered), so K/V traffic is shared by the GQA group inside the tile.
+// Workgroup = 4 waves = (one kv head, HPW of the query heads that share it,
+// 4/HPW consecutive 32-row query tiles); every wave owns 32 query rows of one
+// head.  Two workgroups share a CU (64 KB of LDS each), so every SIMD holds two
+// waves of different workgroups and one's softmax, prologue or epilogue fills
+// the gaps of the other.  All waves of a workgroup walk the same 64-row K/V
+// tiles, which are copied from global into LDS once per workgroup
+// (buffer_load ... lds, 16 B per lane, double buffered, bounds-checked by the
+// buffer descriptor), so K/V traffic is shared by the GQA group inside the tile.
 //
 // Per wave and K/V tile (all MFMA 32x32x16):
 //   S^T[kv][q]  = K (A operand, ds_read_b128 from LDS) x Q^T (B operand, registers)
