@@ -91,6 +91,15 @@ __device__ __forceinline__ float wave_max(float x) {
   return x;
 }
 
+// 16-byte global load with the non-temporal hint: for data that is read once and should stream through the
+// caches instead of displacing what is reused (K/V cache blocks in decode).  Measured on MI355X a pure read
+// stream reaches about 7.1 TB/s with the hint against 6.0-6.5 TB/s without.
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+__device__ __forceinline__ uint4 load16_stream(const void* p) {
+  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // ---- host helpers ----------------------------------------------------------

@@ -299,10 +299,14 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_ke
       const int64_t base = ((int64_t)phys * bs + off) * row;
       const T* kp = kc + base + k_lane_off;
       const T* vp = vc + base + v_lane_off;
+      // V is read once, in whole 256-byte rows per instruction: non-temporal loads stream it past the caches.
+      // K is read in the MFMA operand layout, 64 bytes of a row per instruction, so the second half of each
+      // 128-byte line has to survive in cache until the next instruction: ordinary loads (the hint costs 7 %
+      // there).
 #pragma unroll
       for (int j = 0; j < 4; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) t.v[i] = *reinterpret_cast<const uint4*>(vp + (int64_t)i * row);
+      for (int i = 0; i < 4; ++i) t.v[i] = load16_stream(vp + (int64_t)i * row);
     } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
@@ -495,8 +499,8 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_in
       const char* vp = vc + tok0 * row + v_lane_off;
       t.k[0] = *reinterpret_cast<const uint4*>(kp);
       t.k[1] = *reinterpret_cast<const uint4*>(kp + 64);
-      t.v[0] = *reinterpret_cast<const uint4*>(vp);
-      t.v[1] = *reinterpret_cast<const uint4*>(vp + 2 * row);
+      t.v[0] = load16_stream(vp);
+      t.v[1] = load16_stream(vp + 2 * row);
       const int64_t sidx = (tok0 + s_lane_tok) * a.num_kv_heads + g;
       t.ks = a.k_scale[sidx];
       t.vs = a.v_scale[sidx];
