@@ -140,6 +140,34 @@ int mvllm_prefill_varlen(void* out, const void* q, const void* k, const void* v,
                          int num_heads, int num_kv_heads, int head_dim,
                          float scale, int dtype, void* stream);
 
+/*
+ * The caller's per-layer chain between the QKV projection and the attention kernels, fused:
+ *   q = rms_norm(q); k = rms_norm(k)      src/myvllm/models/qwen3.py:104-106, layers/layernorm.py:9-17
+ *   q, k = rotary_emb(positions, q, k)    qwen3.py:108, layers/rotary_embedding.py:4-23, 77-83
+ *   store_kvcache(k, v, ...)              layers/attention.py:67-108 (called from Attention.forward :505-506)
+ * q, k, v are rows of num_heads*D / num_kv_heads*D / num_kv_heads*D elements with the given strides (in
+ * elements) between tokens, so the three slices of the packed QKV projection output can be passed as they
+ * lie.  gamma [D] fp32 is the shared RMSNorm weight (NULL: no norm, the reference's qkv_bias=True case);
+ * cos_sin_cache [max_position, D] fp32 holds cos (D/2) then sin (D/2) per position (rotary_embedding.py:61-70);
+ * positions int64 [T] are clamped to [0, max_position).  Rotation pairs element i with i + D/2.
+ * Rounding follows the unfused chain: norm result rounded to the element type, rotation in fp32 on the
+ * rounded values, rounded again.
+ * Outputs: q_out [T, Hq, D] always; k_out / v_out [T, Hkv, D] when not NULL (the prefill kernel reads them);
+ * when slot_mapping is not NULL the rotated k and v go to flat slot slot_mapping[t] of the caches
+ * (slots < 0 or >= num_slots skipped): element-type caches, or with cache_is_int8 != 0 int8 codes and
+ * fp32 scales exactly as mvllm_store_kvcache_int8 would write them from k_out / v.
+ * head_dim % 8 == 0, head_dim <= 512; 8-byte aligned pointers (16-byte for fp32), strides % 4 == 0.
+ */
+int mvllm_qk_norm_rope_store(void* q_out, void* k_out, void* v_out,
+                             const void* q, const void* k, const void* v,
+                             int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,
+                             const float* gamma, float eps,
+                             const float* cos_sin_cache, int64_t max_position,
+                             const int64_t* positions, const int64_t* slot_mapping,
+                             void* k_cache, void* v_cache, float* k_scale, float* v_scale, int cache_is_int8,
+                             int64_t num_tokens, int64_t num_slots,
+                             int num_heads, int num_kv_heads, int head_dim, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

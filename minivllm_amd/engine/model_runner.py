@@ -36,7 +36,8 @@ class ModelRunner:
             base=config.get("base", 1_000_000), max_position=config.get("max_position", 4096),
             intermediate_size=config["intermediate_size"], ffn_bias=config.get("ffn_bias", True),
             num_layers=config["num_layers"], tie_word_embeddings=config.get("tie_word_embeddings", True),
-            block_size=self.block_size, kv_cache_dtype=self.kv_cache_dtype)
+            block_size=self.block_size, kv_cache_dtype=self.kv_cache_dtype,
+            fused_qk=config.get("fused_qk", True))
         self.model.reset_parameters(seed=config.get("seed", 0))
         self.model.to(device=self.device, dtype=self.dtype).eval()
         self.sampler = Sampler()

@@ -17,6 +17,7 @@ import torch
 import torch.nn as nn
 
 from minivllm_amd import _C
+from minivllm_amd.layers.fused import qk_norm_rope_store
 from minivllm_amd.utils.context import get_context
 
 __all__ = [
@@ -262,6 +263,24 @@ class Attention(nn.Module):
         self.k_cache = self.v_cache = torch.tensor([])
         self.k_scale = self.v_scale = torch.tensor([])
 
+    def forward_fused(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor,
+                      cos_sin_cache: torch.Tensor, gamma: torch.Tensor | None, eps: float) -> torch.Tensor:
+        """``forward`` on q, k, v as they leave the QKV projection: the caller's RMSNorm of q and k (one
+        float32 ``gamma`` over head_dim, None = no norm), the rotary embedding at ``positions`` and the cache
+        store run in one launch in front of the prefill or decode kernel (qwen3.py:104-110)."""
+        context = get_context()
+        int8 = self.kv_cache_dtype == "int8"
+        store = self.k_cache.numel() > 0 and self.v_cache.numel() > 0 and context.slot_mapping is not None
+        if q.dim() == 4:          # (B, N, H, D) -> (B*N, H, D)
+            q, k, v = (t.reshape(-1, t.shape[-2], t.shape[-1]) for t in (q, k, v))
+        q, k, v = qk_norm_rope_store(
+            q, k, v, positions, cos_sin_cache, gamma, eps,
+            slot_mapping=context.slot_mapping if store else None,
+            k_cache=self.k_cache if store else None, v_cache=self.v_cache if store else None,
+            k_scale=self.k_scale if store and int8 else None, v_scale=self.v_scale if store and int8 else None,
+            need_kv=context.is_prefill)
+        return self._attend(context, q, k, v)
+
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
         context = get_context()
         k_cache, v_cache = self.k_cache, self.v_cache
@@ -279,6 +298,11 @@ class Attention(nn.Module):
             else:
                 store_kvcache(k_rows, v_rows, k_cache, v_cache, context.slot_mapping, self.block_size)
 
+        return self._attend(context, q, k, v)
+
+    def _attend(self, context, q, k, v):
+        k_cache, v_cache = self.k_cache, self.v_cache
+        int8 = self.kv_cache_dtype == "int8"
         scale = self.scale / (self.head_dim ** 0.5)
 
         if context.is_prefill:

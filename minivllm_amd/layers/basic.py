@@ -30,9 +30,20 @@ class RMSNorm(nn.Module):
 class RotaryEmbedding(nn.Module):
     def __init__(self, base: float, rotary_dim: int, max_position: int):
         super().__init__()
-        inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
-        freqs = torch.outer(torch.arange(max_position, dtype=torch.float32), inv_freq)
-        self.register_buffer("cos_sin_cache", torch.cat([freqs.cos(), freqs.sin()], dim=-1), persistent=False)
+        self.base, self.rotary_dim, self.max_position = base, rotary_dim, max_position
+        self.register_buffer("cos_sin_cache", self._table(), persistent=False)
+
+    def _table(self):
+        inv_freq = 1.0 / (self.base ** (torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / self.rotary_dim))
+        freqs = torch.outer(torch.arange(self.max_position, dtype=torch.float32), inv_freq)
+        return torch.cat([freqs.cos(), freqs.sin()], dim=-1)
+
+    def _apply(self, fn, recurse=True):
+        # the table stays float32 whatever dtype the model is cast to (rotary_embedding.py:61-70 builds it
+        # from float positions): rebuild it on the device the cast left it on
+        super()._apply(fn, recurse)
+        self.cos_sin_cache = self._table().to(self.cos_sin_cache.device)
+        return self
 
     @staticmethod
     def _rotate(x, cos, sin):

@@ -1,0 +1,111 @@
+"""Fused caller-side operator in front of the attention kernels.
+
+``qk_norm_rope_store`` does in one HIP launch what the reference's ``Qwen3Attention.forward`` does with
+three modules per layer and step (src/myvllm/models/qwen3.py:104-110): the shared-gamma RMSNorm of q and k
+(layers/layernorm.py:9-17), the half-split rotary embedding (layers/rotary_embedding.py:4-23, 77-83) and
+``store_kvcache`` of the rotated k and of v (layers/attention.py:67-108).  It reads q, k and v as the three
+column slices of the packed QKV projection output (no copies) and calls libminivllm_amd.so on the current
+torch stream; there is no PyTorch fallback.
+"""
+from __future__ import annotations
+
+import torch
+
+from minivllm_amd import _C
+
+__all__ = ["qk_norm_rope_store"]
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _rows(name, t, heads, head_dim):
+    """(T, heads, head_dim) view whose (head, dim) part is dense; returns the token stride in elements."""
+    if t.dim() != 3 or tuple(t.shape[1:]) != (heads, head_dim):
+        raise ValueError(f"{name} must be (num_tokens, {heads}, {head_dim}), got {tuple(t.shape)}")
+    if t.shape[0] > 1 and (t.stride(2) != 1 or t.stride(1) != head_dim):
+        raise ValueError(f"{name}: heads and head_dim must be contiguous inside a token row")
+    return t.stride(0) if t.shape[0] > 1 else heads * head_dim
+
+
+def qk_norm_rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor,
+                       cos_sin_cache: torch.Tensor, gamma: torch.Tensor | None = None, eps: float = 1e-6,
+                       slot_mapping: torch.Tensor | None = None, k_cache: torch.Tensor | None = None,
+                       v_cache: torch.Tensor | None = None, k_scale: torch.Tensor | None = None,
+                       v_scale: torch.Tensor | None = None, need_kv: bool = True):
+    """RMSNorm(q), RMSNorm(k) with one gamma over head_dim (skipped when ``gamma`` is None), rotary embedding
+    of both at ``positions``, and the cache store of the rotated k and of v at ``slot_mapping``.
+
+    q: (T, Hq, D); k, v: (T, Hkv, D), token rows may be strided (slices of the QKV projection);
+    positions int64 (T,); cos_sin_cache float32 (max_position, D) = cos | sin; gamma float32 (D,);
+    caches (num_blocks, block_size, Hkv, D) in q's dtype, or int8 with float32 k_scale / v_scale
+    (num_blocks, block_size, Hkv).  ``slot_mapping`` None stores nothing.
+    Returns (q_out, k_out, v_out) contiguous; k_out and v_out are None unless ``need_kv`` (prefill reads
+    them, decode reads the cache).
+    """
+    _C.require_cuda(q, k, v, positions, cos_sin_cache)
+    if q.dim() != 3 or k.dim() != 3:
+        raise ValueError("q, k and v must be (num_tokens, heads, head_dim)")
+    num_tokens, num_heads, head_dim = q.shape
+    num_kv_heads = k.shape[1]
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k and v must share one dtype")
+    if k.shape[0] != num_tokens or v.shape != k.shape:
+        raise ValueError("q, k and v must have the same number of tokens and k, v the same shape")
+    q_stride = _rows("q", q, num_heads, head_dim)
+    k_stride = _rows("k", k, num_kv_heads, head_dim)
+    v_stride = _rows("v", v, num_kv_heads, head_dim)
+    if positions.numel() != num_tokens:
+        raise ValueError("positions must have one entry per token")
+    if positions.dtype != torch.int64:
+        positions = positions.to(torch.int64)
+    positions = positions.contiguous()
+    if cos_sin_cache.dtype != torch.float32 or cos_sin_cache.dim() != 2 or cos_sin_cache.shape[1] != head_dim \
+            or not cos_sin_cache.is_contiguous():
+        raise ValueError(f"cos_sin_cache must be contiguous float32 (max_position, {head_dim})")
+    if gamma is not None:
+        _C.require_cuda(gamma)
+        if gamma.dtype != torch.float32 or gamma.numel() != head_dim or not gamma.is_contiguous():
+            raise ValueError(f"gamma must be contiguous float32 ({head_dim},)")
+    int8 = False
+    num_slots = 0
+    if slot_mapping is not None:
+        if k_cache is None or v_cache is None:
+            raise ValueError("slot_mapping given without caches")
+        _C.require_cuda(slot_mapping, k_cache, v_cache)
+        if slot_mapping.numel() != num_tokens:
+            raise ValueError("Slot mapping size must match number of tokens")
+        if slot_mapping.dtype != torch.int64:
+            slot_mapping = slot_mapping.to(torch.int64)
+        slot_mapping = slot_mapping.contiguous()
+        for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+            if c.dim() != 4 or tuple(c.shape[2:]) != (num_kv_heads, head_dim) or not c.is_contiguous():
+                raise ValueError(f"{name} must be contiguous [num_blocks, block_size, {num_kv_heads}, {head_dim}]")
+        if k_cache.shape != v_cache.shape:
+            raise ValueError("K and V cache shapes must match")
+        int8 = k_cache.dtype == torch.int8
+        if int8:
+            if v_cache.dtype != torch.int8:
+                raise ValueError("int8 caches expected")
+            for name, s in (("k_scale", k_scale), ("v_scale", v_scale)):
+                if s is None or s.dtype != torch.float32 or tuple(s.shape) != tuple(k_cache.shape[:3]) \
+                        or not s.is_contiguous():
+                    raise ValueError(f"{name} must be contiguous float32 {tuple(k_cache.shape[:3])}")
+        elif k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+            raise ValueError(f"cache dtype {k_cache.dtype} differs from q/k/v dtype {q.dtype}")
+        num_slots = k_cache.shape[0] * k_cache.shape[1]
+    q_out = torch.empty((num_tokens, num_heads, head_dim), dtype=q.dtype, device=q.device)
+    k_out = torch.empty((num_tokens, num_kv_heads, head_dim), dtype=q.dtype, device=q.device) if need_kv else None
+    v_out = torch.empty_like(k_out) if need_kv else None
+    if num_tokens == 0:
+        return q_out, k_out, v_out
+    lib = _C.load()
+    st = lib.mvllm_qk_norm_rope_store(
+        _ptr(q_out), _ptr(k_out), _ptr(v_out), _ptr(q), _ptr(k), _ptr(v), q_stride, k_stride, v_stride,
+        _ptr(gamma), float(eps), _ptr(cos_sin_cache), cos_sin_cache.shape[0], _ptr(positions),
+        _ptr(slot_mapping), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale if int8 else None),
+        _ptr(v_scale if int8 else None), int(int8), num_tokens, num_slots, num_heads, num_kv_heads, head_dim,
+        _C.dtype_code(q.dtype), _C.current_stream_ptr(q.device))
+    _C.check(st, "qk_norm_rope_store")
+    return q_out, k_out, v_out

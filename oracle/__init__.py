@@ -14,6 +14,10 @@ from .attention_oracle import (  # noqa: F401
     decode_int8_oracle,
     prefill_standard_oracle,
     gather_sequence_kv,
+    rms_norm_oracle,
+    rope_cos_sin_cache_oracle,
+    rope_oracle,
+    qk_norm_rope_store_oracle,
 )
 from .producers_oracle import (  # noqa: F401
     prefill_metadata_oracle,

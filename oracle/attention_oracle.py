@@ -16,6 +16,12 @@ pinned by ``tests/test_oracle_pins.py`` against what the mathematics fixes:
                                 |x-code*scale|<=scale/2, scale == amax/127 in fp32)
                                 -- "parity unpinned" by the reference: it has no
                                 INT8 code; the spec is defined by this build.
+* ``rms_norm_oracle`` / ``rope_cos_sin_cache_oracle`` / ``rope_oracle`` /
+  ``qk_norm_rope_store_oracle``   unit mean square, scale invariance, constant-vector
+                                closed form; table vs cos/sin of pos * base^(-2i/D) in
+                                fp64; position 0 identity, hand-worked quarter turn
+                                (sign and half-split pairing), pair norms kept,
+                                angles add, scores depend on position difference only
 """
 from __future__ import annotations
 
@@ -208,3 +214,49 @@ def prefill_standard_oracle(q, k, v, cu_seqlens, scale, num_heads, num_kv_heads,
         probs = torch.softmax(scores, dim=-1)
         out[lo:hi] = torch.matmul(probs, vs).transpose(0, 1)
     return out
+
+
+# --------------------------------------------------------------------------
+# caller-side chain in front of the attention kernels
+# reference: src/myvllm/models/qwen3.py:104-110, layers/layernorm.py:9-17,
+#            layers/rotary_embedding.py:4-23 and :48-83, layers/attention.py:505-506
+# --------------------------------------------------------------------------
+def rms_norm_oracle(x: torch.Tensor, gamma: torch.Tensor, eps: float) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * gamma over the last dim, fp32 math, result in x's dtype
+    (layernorm.py:13-15)."""
+    xf = x.float()
+    variance = xf.pow(2).mean(dim=-1, keepdim=True) + eps
+    return (xf / variance.sqrt() * gamma.float()).to(x.dtype)
+
+
+def rope_cos_sin_cache_oracle(base: float, rotary_dim: int, max_position: int) -> torch.Tensor:
+    """[max_position, rotary_dim] fp32: cos(pos * inv_freq) | sin(pos * inv_freq),
+    inv_freq[i] = base^(-2i/rotary_dim) (rotary_embedding.py:58-70)."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+    freqs = torch.einsum("i,j->ij", torch.arange(max_position, dtype=torch.float32), inv_freq)
+    return torch.cat([freqs.cos(), freqs.sin()], dim=-1)
+
+
+def rope_oracle(x: torch.Tensor, positions: torch.Tensor, cos_sin_cache: torch.Tensor) -> torch.Tensor:
+    """Half-split rotation of x (T, H, D): element i pairs with i + D/2
+    (rotary_embedding.py:4-23, 77-83).  fp32 math, result in x's dtype."""
+    cos, sin = cos_sin_cache[positions.long()].float().chunk(2, dim=-1)
+    cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
+    x1, x2 = x.float().chunk(2, dim=-1)
+    return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).to(x.dtype)
+
+
+def qk_norm_rope_store_oracle(q, k, v, positions, cos_sin_cache, gamma, eps, slot_mapping=None,
+                              k_cache=None, v_cache=None, k_scale=None, v_scale=None, block_size=0):
+    """The unfused chain: shared-gamma RMSNorm on q and k (skipped when gamma is None, the
+    reference's qkv_bias=True case), rotation, then the cache store of (rotated k, v).
+    Returns (q_out, k_out); caches are modified in place (int8 when k_scale is given)."""
+    if gamma is not None:
+        q, k = rms_norm_oracle(q, gamma, eps), rms_norm_oracle(k, gamma, eps)
+    q, k = rope_oracle(q, positions, cos_sin_cache), rope_oracle(k, positions, cos_sin_cache)
+    if slot_mapping is not None:
+        if k_scale is not None:
+            store_kvcache_int8_oracle(k, v, k_cache, v_cache, k_scale, v_scale, slot_mapping, block_size)
+        else:
+            store_kvcache_oracle(k, v, k_cache, v_cache, slot_mapping, block_size)
+    return q, k

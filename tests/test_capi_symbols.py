@@ -28,7 +28,7 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_prefill_varlen",
-              "mvllm_version", "mvllm_status_string"]:
+              "mvllm_qk_norm_rope_store", "mvllm_version", "mvllm_status_string"]:
         assert n in names
 
 
@@ -63,6 +63,13 @@ def test_argument_validation_without_gpu():
     assert lib.mvllm_paged_decode(0, 0, 0, 0, 0, 4, 0, 1, 2, 6, 4, 128, 16, 8, 1.0, 1, 0, 0, 0) == -3  # Hq % Hkv
     assert lib.mvllm_prefill_varlen(0, 0, 0, 0, 0, 0, 0, 4, 2, 128, 1.0, 1, 0) == 0      # empty batch
     assert lib.mvllm_prefill_varlen(0, 0, 0, 0, 0, 1, 5, 4, 2, 128, 1.0, 1, 0) == -1
+    fused = lib.mvllm_qk_norm_rope_store
+    #     q_out k_out v_out q k v | strides | gamma eps cos max_pos pos slots | caches scales int8 | T slots Hq Hkv D dt stream
+    assert fused(0, 0, 0, 0, 0, 0, 512, 256, 256, 0, 1e-6, 0, 64, 0, 0, 0, 0, 0, 0, 0, 0, 0, 4, 2, 128, 1, 0) == 0   # no tokens
+    assert fused(0, 0, 0, 0, 0, 0, 512, 256, 256, 0, 1e-6, 0, 64, 0, 0, 0, 0, 0, 0, 0, 3, 0, 4, 2, 128, 1, 0) == -1  # nulls
+    assert fused(0, 0, 0, 0, 0, 0, 512, 256, 256, 0, 1e-6, 0, 64, 0, 0, 0, 0, 0, 0, 0, 3, 0, 4, 2, 100, 1, 0) == -4  # D % 8
+    assert fused(0, 0, 0, 0, 0, 0, 100, 256, 256, 0, 1e-6, 0, 64, 0, 0, 0, 0, 0, 0, 0, 3, 0, 4, 2, 128, 1, 0) == -3  # stride < row
+    assert fused(0, 0, 0, 0, 0, 0, 512, 256, 256, 0, 1e-6, 0, 64, 0, 0, 0, 0, 0, 0, 0, 3, 0, 4, 2, 128, 9, 0) == -2  # dtype
     with pytest.raises(ValueError):
         _C.check(-3, "x")
     with pytest.raises(RuntimeError):

@@ -84,3 +84,24 @@ def test_graph_decode_matches_eager_decode():
     same = sum(a == b for a, b in zip(eager, graphed))
     # identical up to the rare tie that a 1-ulp GEMM difference between batch buckets can flip
     assert same >= 7, (same, eager, graphed)
+
+
+@pytest.mark.parametrize("kv_cache_dtype", ["auto", "int8"])
+def test_fused_qk_path_matches_unfused_modules(kv_cache_dtype):
+    """One prefill and one decode step through the model with the fused norm + rotary + store launch and
+    with the three separate modules: same hidden states (the fused kernel rounds where the modules round;
+    the sum of squares may differ in its last bit) and the same cache contents up to that."""
+    cfg = dict(SMALL, kv_cache_dtype=kv_cache_dtype, max_cached_blocks=32)
+    prompts = _prompts(4, 5, 50, seed=8)
+    sp = SamplingParams(temperature=0.5, max_tokens=6, ignore_eos=True)
+    outs, caches = [], []
+    for fused in (True, False):
+        eng = LLMEngine(dict(cfg, fused_qk=fused))
+        assert all(l.self_attn.fused_qk == fused for l in eng.model_runner.model.layer_stack)
+        outs.append(eng.generate(prompts, sp)["token_ids"])
+        caches.append(eng.model_runner.kv_cache.clone())
+    same = sum(a == b for a, b in zip(*outs))
+    assert same >= 3, outs                           # a 1-ulp difference may flip a sampling tie, rarely
+    a, b = caches[0].float(), caches[1].float()
+    if kv_cache_dtype == "auto" and same == 4:
+        assert (a - b).abs().max() <= 6e-2 and (a - b).abs().mean() <= 1e-3

@@ -309,3 +309,85 @@ def test_metadata_slots_unique_and_owned():
             assert slot == s["block_table"][(n - 1) // bs] * bs + (n - 1) % bs
 
     run()
+
+
+# ---------------------------------------------------------------------------
+# caller-side chain: RMSNorm, rotary table, rotation (layernorm.py:9-17, rotary_embedding.py:4-83)
+# ---------------------------------------------------------------------------
+def test_rms_norm_oracle_closed_forms():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(7, 3, 64, generator=g)
+    ones = torch.ones(64)
+    y = oracle.rms_norm_oracle(x, ones, 0.0)
+    assert torch.allclose(y.pow(2).mean(-1), torch.ones(7, 3), atol=1e-5)          # unit mean square
+    assert torch.allclose(oracle.rms_norm_oracle(3.5 * x, ones, 0.0), y, atol=1e-5)  # scale invariant at eps 0
+    c = torch.full((1, 1, 64), -2.0)
+    gamma = torch.linspace(0.5, 2.0, 64)
+    want = -2.0 / math.sqrt(4.0 + 0.25) * gamma                                    # constant vector, eps 0.25
+    assert torch.allclose(oracle.rms_norm_oracle(c, gamma, 0.25)[0, 0], want, atol=1e-6)
+    big_eps = oracle.rms_norm_oracle(x, ones, 1e6)                                 # eps sits inside the root
+    assert torch.allclose(big_eps, x / math.sqrt(1e6), rtol=1e-3, atol=1e-7)
+
+
+def test_rope_table_matches_fp64_formula():
+    base, d, n = 10000.0, 32, 50
+    table = oracle.rope_cos_sin_cache_oracle(base, d, n)
+    assert table.shape == (n, d) and table.dtype == torch.float32
+    pos = torch.arange(n, dtype=torch.float64).unsqueeze(1)
+    inv = torch.tensor([base ** (-2.0 * i / d) for i in range(d // 2)], dtype=torch.float64).unsqueeze(0)
+    assert torch.allclose(table[:, : d // 2].double(), torch.cos(pos * inv), atol=2e-5)
+    assert torch.allclose(table[:, d // 2:].double(), torch.sin(pos * inv), atol=2e-5)
+
+
+def test_rope_oracle_sign_pairing_and_group_law():
+    d = 8
+    table = oracle.rope_cos_sin_cache_oracle(10000.0, d, 64)
+    # position 0 is the identity
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(5, 2, d, generator=g)
+    assert torch.equal(oracle.rope_oracle(x, torch.zeros(5, dtype=torch.long), table), x)
+    # hand-worked: inv_freq[0] = 1, so at position 1 the unit vector e_0 turns by +1 rad in the (0, d/2) plane
+    e0 = torch.zeros(1, 1, d); e0[0, 0, 0] = 1.0
+    y = oracle.rope_oracle(e0, torch.tensor([1]), table)[0, 0]
+    want = torch.zeros(d); want[0] = math.cos(1.0); want[d // 2] = math.sin(1.0)
+    assert torch.allclose(y, want, atol=1e-6)
+    # e_{d/2} turns to (-sin, cos): the sign of the second row of the rotation
+    e4 = torch.zeros(1, 1, d); e4[0, 0, d // 2] = 1.0
+    y = oracle.rope_oracle(e4, torch.tensor([1]), table)[0, 0]
+    want = torch.zeros(d); want[0] = -math.sin(1.0); want[d // 2] = math.cos(1.0)
+    assert torch.allclose(y, want, atol=1e-6)
+    # every (i, i + d/2) pair keeps its norm, nothing leaks between pairs
+    pos = torch.tensor([3, 17, 40, 63, 1])
+    y = oracle.rope_oracle(x, pos, table)
+    n_in = x[..., : d // 2] ** 2 + x[..., d // 2:] ** 2
+    n_out = y[..., : d // 2] ** 2 + y[..., d // 2:] ** 2
+    assert torch.allclose(n_in, n_out, atol=1e-5)
+    # angles add: rotating to position a and then by b more equals rotating to a + b
+    a, b = torch.tensor([5] * 5), torch.tensor([9] * 5)
+    assert torch.allclose(oracle.rope_oracle(oracle.rope_oracle(x, a, table), b, table),
+                          oracle.rope_oracle(x, a + b, table), atol=1e-5)
+    # scores depend on the position difference only
+    q, k = torch.randn(1, 1, d, generator=g), torch.randn(1, 1, d, generator=g)
+    s1 = (oracle.rope_oracle(q, torch.tensor([20]), table) * oracle.rope_oracle(k, torch.tensor([13]), table)).sum()
+    s2 = (oracle.rope_oracle(q, torch.tensor([47]), table) * oracle.rope_oracle(k, torch.tensor([40]), table)).sum()
+    assert abs(float(s1 - s2)) < 1e-4
+
+
+def test_fused_chain_oracle_is_the_composition():
+    g = torch.Generator().manual_seed(11)
+    t, hq, hkv, d, bs = 9, 4, 2, 16, 4
+    q, k, v = (torch.randn(t, h, d, generator=g).to(torch.bfloat16) for h in (hq, hkv, hkv))
+    table = oracle.rope_cos_sin_cache_oracle(1e6, d, 32)
+    pos = torch.randint(0, 32, (t,), generator=g)
+    gamma = torch.rand(d, generator=g) + 0.5
+    slots = torch.tensor([0, 1, 2, -1, 8, 9, 10, 11, 5])
+    kc = torch.zeros(3, bs, hkv, d, dtype=torch.bfloat16); vc = torch.zeros_like(kc)
+    q_out, k_out = oracle.qk_norm_rope_store_oracle(q, k, v, pos, table, gamma, 1e-6, slots, kc, vc, block_size=bs)
+    assert torch.equal(q_out, oracle.rope_oracle(oracle.rms_norm_oracle(q, gamma, 1e-6), pos, table))
+    flat = kc.view(-1, hkv, d)
+    assert torch.equal(flat[8], k_out[4]) and torch.equal(flat[5], k_out[8])
+    assert torch.equal(vc.view(-1, hkv, d)[2], v[2])
+    assert float(flat[3].abs().sum()) == 0.0                                        # slot 3 never written (token 3 skipped)
+    # no gamma: rotation only
+    q2, _ = oracle.qk_norm_rope_store_oracle(q, k, v, pos, table, None, 1e-6)
+    assert torch.equal(q2, oracle.rope_oracle(q, pos, table))
