@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,engine,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,fused_qk,engine,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -242,6 +242,53 @@ def bench_int8(args):
     }
 
 
+def bench_fused_qk(args):
+    """The caller's chain in front of the attention kernels on the prefill batch of config 2 (same lengths):
+    q/k RMSNorm + rotary embedding + store into a block-256 bf16 cache, as one HIP launch reading the packed QKV
+    projection output, against the same chain as separate modules (torch ops + store_kvcache)."""
+    import torch
+    from helpers import make_slot_mapping
+    from minivllm_amd.layers.attention import store_kvcache
+    from minivllm_amd.layers.basic import RMSNorm, RotaryEmbedding
+    from minivllm_amd.layers.fused import qk_norm_rope_store
+
+    dev = "cuda:0"
+    hq, hkv, d, bs = 32, 8, 128, 256
+    g = torch.Generator().manual_seed(args.seed)
+    lengths = torch.randint(64, 2049, (16,), generator=g).tolist()
+    total = sum(lengths)
+    dg = torch.Generator(device=dev).manual_seed(args.seed + 1)
+    qkv = torch.randn(total, (hq + 2 * hkv) * d, generator=dg, device=dev).to(torch.bfloat16)
+    q, k, v = qkv.split([hq * d, hkv * d, hkv * d], dim=-1)
+    q, k, v = q.unflatten(-1, (hq, d)), k.unflatten(-1, (hkv, d)), v.unflatten(-1, (hkv, d))
+    pos = torch.cat([torch.arange(n) for n in lengths]).to(dev)
+    rotary = RotaryEmbedding(1_000_000, d, 4096).to(dev)
+    norm = RMSNorm(d, 1e-6).to(dev)
+    gamma = norm.weight.detach().float().contiguous()
+    slots, _, nb = make_slot_mapping(args.seed + 2, lengths, bs)
+    kc = torch.zeros(nb, bs, hkv, d, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    sl = slots.to(dev)
+
+    def unfused():
+        qq, kk = norm(q.reshape(-1, hq, d)), norm(k.reshape(-1, hkv, d))
+        qq, kk = rotary(pos, qq, kk)
+        store_kvcache(kk, v.reshape(-1, hkv, d), kc, vc, sl, bs)
+        return qq, kk
+
+    fused = lambda: qk_norm_rope_store(q, k, v, pos, rotary.cos_sin_cache, gamma, 1e-6, sl, kc, vc)
+    with torch.inference_mode():
+        _, fused_ms = time_steps(fused, args.steps, args.warmup)
+        _, unfused_ms = time_steps(unfused, max(3, args.steps // 3), max(1, args.warmup // 2))
+    # read q, k, v once; write q_out, k_out, v_out and the two cache rows; per token: position, slot, table row
+    nbytes = total * ((hq + 2 * hkv) * d * 2 * 2 + 2 * hkv * d * 2 + 8 + 8 + d * 4)
+    return {
+        "workload": "q/k RMSNorm + rotary + store_kvcache on the config-2 prefill batch, Hq32 Hkv8 D128 bf16, block 256",
+        "tokens": total, "algorithmic_bytes": nbytes, "event_ms_per_step": fused_ms,
+        "gbs": nbytes / (fused_ms * 1e-3) / 1e9, "unfused_modules_event_ms": unfused_ms,
+    }
+
+
 def bench_engine(args, max_num_sequences, graph):
     """BASELINE config 5: random-init Qwen3-style decoder (hidden 1024, 8 layers, Hq16/Hkv8/D128, FFN 3072,
     vocab 151936, bf16), 60 prompts of random ids with lengths U[32,96], 256 new tokens each, T 0.6."""
@@ -309,6 +356,8 @@ def main():
         extra.update(bench_prefill_store(args, which))
     if want("int8"):
         extra["int8"] = bench_int8(args)
+    if want("fused_qk"):
+        extra["fused_qk"] = bench_fused_qk(args)
     if want("engine"):
         extra["engine_16seq_eager"] = bench_engine(args, 16, False)
         extra["engine_16seq_graph"] = bench_engine(args, 16, True)

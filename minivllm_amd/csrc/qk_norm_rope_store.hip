@@ -8,8 +8,8 @@
 // from the rounded values and rounded again; products and sums are separate IEEE operations (no fused
 // multiply-add), division and square root are correctly rounded.  Only the order of the sum of squares is free.
 //
-// Work item = one (token, head) vector of q, k or v.  GROUP = head_dim / 8 lanes (next power of two) share a
-// vector; lane j holds elements [4j, 4j+4) of the first half and the same four of the second half, i.e.
+// Work item = one (token, head) vector of q, k or v.  GROUP lanes (a power of two) share a vector; lane j holds
+// EPL = 8 (4 when head_dim is not a multiple of 16) elements [EPL j, EPL j + EPL) of the first half and the same of the second half, i.e.
 // exactly the pairs the rotation mixes, so the rotation needs no cross-lane traffic; the sum of squares and the
 // INT8 amax are xor-shuffle reductions inside the group.
 #include "common.h"
@@ -42,27 +42,43 @@ struct FusedArgs {
   int num_heads, num_kv_heads, head_dim;
 };
 
-template <typename T> struct Vec4;
-template <> struct Vec4<float> {
-  static __device__ __forceinline__ void load(const float* p, float (&x)[4]) {
-    const float4 v = *reinterpret_cast<const float4*>(p);
-    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+// N = 4 or 8 consecutive elements of T <-> fp32 registers, as one 8- or 16-byte access (16 / 32 for fp32)
+template <typename T, int N> struct VecN;
+template <int N> struct VecN<float, N> {
+  static __device__ __forceinline__ void load(const float* p, float (&x)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; i += 4) {
+      const float4 v = *reinterpret_cast<const float4*>(p + i);
+      x[i] = v.x; x[i + 1] = v.y; x[i + 2] = v.z; x[i + 3] = v.w;
+    }
   }
-  static __device__ __forceinline__ void store(float* p, const float (&x)[4]) {
-    *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+  static __device__ __forceinline__ void store(float* p, const float (&x)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; i += 4) *reinterpret_cast<float4*>(p + i) = make_float4(x[i], x[i + 1], x[i + 2], x[i + 3]);
   }
 };
-template <typename T16> struct Vec4 {
-  static __device__ __forceinline__ void load(const T16* p, float (&x)[4]) {
-    const uint2 w = *reinterpret_cast<const uint2*>(p);
-    x[0] = lo_to_float<T16>(w.x); x[1] = hi_to_float<T16>(w.x);
-    x[2] = lo_to_float<T16>(w.y); x[3] = hi_to_float<T16>(w.y);
-  }
-  static __device__ __forceinline__ void store(T16* p, const float (&x)[4]) {
-    T16 o[4];
+template <typename T16, int N> struct VecN {
+  static __device__ __forceinline__ void load(const T16* p, float (&x)[N]) {
+    uint32_t w[N / 2];
+    if constexpr (N == 8) {
+      const uint4 v = *reinterpret_cast<const uint4*>(p);
+      w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    } else {
+      const uint2 v = *reinterpret_cast<const uint2*>(p);
+      w[0] = v.x; w[1] = v.y;
+    }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = from_float<T16>(x[e]);
-    *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(o);
+    for (int i = 0; i < N / 2; ++i) {
+      x[2 * i] = lo_to_float<T16>(w[i]);
+      x[2 * i + 1] = hi_to_float<T16>(w[i]);
+    }
+  }
+  static __device__ __forceinline__ void store(T16* p, const float (&x)[N]) {
+    T16 o[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) o[e] = from_float<T16>(x[e]);
+    if constexpr (N == 8) *reinterpret_cast<uint4*>(p) = *reinterpret_cast<const uint4*>(o);
+    else *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(o);
   }
 };
 
@@ -80,21 +96,27 @@ template <int GROUP> __device__ __forceinline__ float group_max(float x) {
   return x;
 }
 
-__device__ __forceinline__ uint32_t pack_codes(const float (&x)[4], float div, bool live) {
-  uint32_t w = 0u;
+// four codes per 32-bit word, element order = byte order
+template <int N>
+__device__ __forceinline__ void store_codes(int8_t* dst, const float (&x)[N], float div, bool live) {
+  uint32_t w[N / 4];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
+  for (int i = 0; i < N / 4; ++i) w[i] = 0u;
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
     float r = rintf(x[e] / div);
     r = fminf(fmaxf(r, -127.f), 127.f);
     const int c = live ? (int)r : 0;
-    w |= ((uint32_t)(c & 0xff)) << (8 * e);
+    w[e >> 2] |= ((uint32_t)(c & 0xff)) << (8 * (e & 3));
   }
-  return w;
+  if constexpr (N == 8) *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
+  else *reinterpret_cast<uint32_t*>(dst) = w[0];
 }
 
 constexpr int kFusedThreads = 256;
 
-template <typename T, int GROUP, bool INT8>
+// EPL = elements per lane and half: 8 when head_dim is a multiple of 16 (16-byte accesses), else 4.
+template <typename T, int GROUP, int EPL, bool INT8>
 __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(const FusedArgs a) {
   constexpr int kVecPerBlock = kFusedThreads / GROUP;
   const int j = threadIdx.x % GROUP;
@@ -104,8 +126,8 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(const
   const int64_t t = item / per_token;
   const int i = (int)(item - t * per_token);
   const int D = a.head_dim, half = D >> 1;
-  const bool lane_live = 8 * j < D;                      // GROUP may exceed head_dim / 8
-  const int e1 = 4 * j, e2 = half + 4 * j;
+  const bool lane_live = 2 * EPL * j < D;                // GROUP may exceed the lanes a vector needs
+  const int e1 = EPL * j, e2 = half + EPL * j;
 
   const int kind = i < a.num_heads ? 0 : (i < a.num_heads + a.num_kv_heads ? 1 : 2);   // q, k, v
   const int h = kind == 0 ? i : (kind == 1 ? i - a.num_heads : i - a.num_heads - a.num_kv_heads);
@@ -114,10 +136,12 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(const
                              : reinterpret_cast<const T*>(a.v) + t * a.v_stride;
   src += (int64_t)h * D;
 
-  float x1[4] = {0.f, 0.f, 0.f, 0.f}, x2[4] = {0.f, 0.f, 0.f, 0.f};
+  float x1[EPL], x2[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) x1[e] = x2[e] = 0.f;
   if (lane_live) {
-    Vec4<T>::load(src + e1, x1);
-    Vec4<T>::load(src + e2, x2);
+    VecN<T, EPL>::load(src + e1, x1);
+    VecN<T, EPL>::load(src + e2, x2);
   }
 
   if (kind != 2) {
@@ -125,17 +149,17 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(const
       // x / sqrt(mean(x^2) + eps) * gamma, rounded to T  (layernorm.py:13-15)
       float ss = 0.f;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) ss = ss + x1[e] * x1[e];
+      for (int e = 0; e < EPL; ++e) ss = ss + x1[e] * x1[e];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) ss = ss + x2[e] * x2[e];
+      for (int e = 0; e < EPL; ++e) ss = ss + x2[e] * x2[e];
       ss = group_sum<GROUP>(ss);
       const float denom = sqrtf(ss / (float)D + a.eps);
       if (lane_live) {
-        float g1[4], g2[4];
-        Vec4<float>::load(a.gamma + e1, g1);
-        Vec4<float>::load(a.gamma + e2, g2);
+        float g1[EPL], g2[EPL];
+        VecN<float, EPL>::load(a.gamma + e1, g1);
+        VecN<float, EPL>::load(a.gamma + e2, g2);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
+        for (int e = 0; e < EPL; ++e) {
           x1[e] = rounded<T>((x1[e] / denom) * g1[e]);
           x2[e] = rounded<T>((x2[e] / denom) * g2[e]);
         }
@@ -145,11 +169,11 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(const
     if (lane_live) {
       int64_t pos = a.positions[t];
       pos = pos < 0 ? 0 : (pos >= a.max_position ? a.max_position - 1 : pos);
-      float c[4], s[4];
-      Vec4<float>::load(a.cos_sin + pos * D + e1, c);
-      Vec4<float>::load(a.cos_sin + pos * D + e2, s);
+      float c[EPL], s[EPL];
+      VecN<float, EPL>::load(a.cos_sin + pos * D + e1, c);
+      VecN<float, EPL>::load(a.cos_sin + pos * D + e2, s);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
+      for (int e = 0; e < EPL; ++e) {
         const float o1 = x1[e] * c[e] - x2[e] * s[e];
         const float o2 = x1[e] * s[e] + x2[e] * c[e];
         x1[e] = rounded<T>(o1);
@@ -165,8 +189,8 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(const
   if (dense && lane_live) {
     const int heads = kind == 0 ? a.num_heads : a.num_kv_heads;
     T* dst = dense + (t * heads + h) * D;
-    Vec4<T>::store(dst + e1, x1);
-    Vec4<T>::store(dst + e2, x2);
+    VecN<T, EPL>::store(dst + e1, x1);
+    VecN<T, EPL>::store(dst + e2, x2);
   }
   if (kind == 0 || !a.slot_mapping) return;
 
@@ -177,41 +201,48 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(const
   if constexpr (INT8) {
     float amax = 0.f;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) amax = fmaxf(amax, fmaxf(fabsf(x1[e]), fabsf(x2[e])));
+    for (int e = 0; e < EPL; ++e) amax = fmaxf(amax, fmaxf(fabsf(x1[e]), fabsf(x2[e])));
     amax = group_max<GROUP>(amax);
     const float scale = amax / 127.0f;
     const bool live = scale > 0.f;
     const float div = live ? scale : 1.0f;
     int8_t* dst = reinterpret_cast<int8_t*>(kind == 1 ? a.k_cache : a.v_cache) + vec * D;
     if (lane_live) {
-      *reinterpret_cast<uint32_t*>(dst + e1) = pack_codes(x1, div, live);
-      *reinterpret_cast<uint32_t*>(dst + e2) = pack_codes(x2, div, live);
+      store_codes<EPL>(dst + e1, x1, div, live);
+      store_codes<EPL>(dst + e2, x2, div, live);
     }
     if (j == 0) (kind == 1 ? a.k_scale : a.v_scale)[vec] = scale;
   } else {
     if (lane_live) {
       T* dst = reinterpret_cast<T*>(kind == 1 ? a.k_cache : a.v_cache) + vec * D;
-      Vec4<T>::store(dst + e1, x1);
-      Vec4<T>::store(dst + e2, x2);
+      VecN<T, EPL>::store(dst + e1, x1);
+      VecN<T, EPL>::store(dst + e2, x2);
     }
   }
 }
 
 template <typename T>
-static int launch_fused(const FusedArgs& a, bool int8, hipStream_t stream) {
-  const int lanes = a.head_dim / 8;
+static int launch_fused(const FusedArgs& a, bool int8, bool wide, hipStream_t stream) {
+  const int lanes = a.head_dim / (wide ? 16 : 8);
   const int64_t vecs = a.num_tokens * (a.num_heads + 2 * a.num_kv_heads);
-#define MVLLM_LAUNCH_F(G)                                                                          \
+#define MVLLM_LAUNCH_F(G, E)                                                                       \
   do {                                                                                             \
     const int64_t blocks = (vecs + (kFusedThreads / G) - 1) / (kFusedThreads / G);                  \
-    if (int8) qk_norm_rope_store_kernel<T, G, true><<<dim3((unsigned)blocks), dim3(kFusedThreads), 0, stream>>>(a);  \
-    else qk_norm_rope_store_kernel<T, G, false><<<dim3((unsigned)blocks), dim3(kFusedThreads), 0, stream>>>(a);      \
+    if (int8) qk_norm_rope_store_kernel<T, G, E, true><<<dim3((unsigned)blocks), dim3(kFusedThreads), 0, stream>>>(a);  \
+    else qk_norm_rope_store_kernel<T, G, E, false><<<dim3((unsigned)blocks), dim3(kFusedThreads), 0, stream>>>(a);      \
   } while (0)
-  if (lanes <= 4) MVLLM_LAUNCH_F(4);
-  else if (lanes <= 8) MVLLM_LAUNCH_F(8);
-  else if (lanes <= 16) MVLLM_LAUNCH_F(16);
-  else if (lanes <= 32) MVLLM_LAUNCH_F(32);
-  else MVLLM_LAUNCH_F(64);
+  if (wide) {
+    if (lanes <= 4) MVLLM_LAUNCH_F(4, 8);
+    else if (lanes <= 8) MVLLM_LAUNCH_F(8, 8);
+    else if (lanes <= 16) MVLLM_LAUNCH_F(16, 8);
+    else MVLLM_LAUNCH_F(32, 8);
+  } else {
+    if (lanes <= 4) MVLLM_LAUNCH_F(4, 4);
+    else if (lanes <= 8) MVLLM_LAUNCH_F(8, 4);
+    else if (lanes <= 16) MVLLM_LAUNCH_F(16, 4);
+    else if (lanes <= 32) MVLLM_LAUNCH_F(32, 4);
+    else MVLLM_LAUNCH_F(64, 4);
+  }
 #undef MVLLM_LAUNCH_F
   return launch_status();
 }
@@ -239,7 +270,8 @@ extern "C" int mvllm_qk_norm_rope_store(void* q_out, void* k_out, void* v_out, c
   if (!q_out || !q || !k || !v || !cos_sin_cache || !positions) return MVLLM_ERR_NULL_POINTER;
   if (slot_mapping && (!k_cache || !v_cache)) return MVLLM_ERR_NULL_POINTER;
   if (slot_mapping && cache_is_int8 && (!k_scale || !v_scale)) return MVLLM_ERR_NULL_POINTER;
-  // every lane moves 4 elements at a time: 8-byte (16-bit types) or 16-byte (fp32) accesses
+  // every lane moves 4 elements at a time, 8 when head_dim is a multiple of 16 and everything is 16-byte
+  // aligned: 8- or 16-byte accesses for the 16-bit types, 16-byte ones for fp32
   const uintptr_t amask = esize == 4 ? 15u : 7u;
   const uintptr_t ptrs = reinterpret_cast<uintptr_t>(q_out) | reinterpret_cast<uintptr_t>(k_out) |
                          reinterpret_cast<uintptr_t>(v_out) | reinterpret_cast<uintptr_t>(q) |
@@ -247,6 +279,7 @@ extern "C" int mvllm_qk_norm_rope_store(void* q_out, void* k_out, void* v_out, c
                          (slot_mapping ? reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache) : 0);
   if ((ptrs & amask) != 0 || !aligned16(cos_sin_cache) || (gamma && !aligned16(gamma))) return MVLLM_ERR_MISALIGNED;
   if (((q_row_stride | k_row_stride | v_row_stride) & 3) != 0) return MVLLM_ERR_MISALIGNED;
+  const bool wide = head_dim % 16 == 0 && (ptrs & 15u) == 0 && ((q_row_stride | k_row_stride | v_row_stride) & 7) == 0;
 
   FusedArgs a;
   a.q_out = q_out; a.k_out = k_out; a.v_out = v_out;
@@ -261,8 +294,8 @@ extern "C" int mvllm_qk_norm_rope_store(void* q_out, void* k_out, void* v_out, c
   hipStream_t s = (hipStream_t)stream;
   const bool int8 = slot_mapping && cache_is_int8;
   switch (dtype) {
-    case MVLLM_F32: return launch_fused<float>(a, int8, s);
-    case MVLLM_BF16: return launch_fused<bf16_t>(a, int8, s);
-    default: return launch_fused<f16_t>(a, int8, s);
+    case MVLLM_F32: return launch_fused<float>(a, int8, wide, s);
+    case MVLLM_BF16: return launch_fused<bf16_t>(a, int8, wide, s);
+    default: return launch_fused<f16_t>(a, int8, wide, s);
   }
 }
