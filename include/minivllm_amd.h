@@ -141,6 +141,29 @@ int mvllm_prefill_varlen(void* out, const void* q, const void* k, const void* v,
                          float scale, int dtype, void* stream);
 
 /*
+ * Prefill over a paged cache: the same attention as mvllm_prefill_varlen for sequences whose first tokens are
+ * already in the cache (prefix-cache hits).  The reference prepares exactly this metadata in
+ * ModelRunner.prepare_prefill (src/myvllm/engine/model_runner.py:192-226: input_ids = tokens[num_cached:],
+ * cu_seqlens_q over the new tokens, cu_seqlens_k over all of them, block_tables when they differ) but its
+ * Attention.forward never consumes it (attention.py:518-523 passes cu_seqlens_q and the fresh k, v only).
+ *   q, out       [total_q_tokens, Hq, D]: rows of the new tokens only, packed by cu_seqlens_q
+ *   k/v_cache    [num_blocks, block_size, Hkv, D], already holding every key of every sequence
+ *                (prefix from earlier requests, new tokens from the store that precedes this call)
+ *   block_tables int32 [num_seqs, max_num_blocks]; cu_seqlens_q/k int32 [num_seqs+1]
+ * Query row r of sequence s (r counted over its new tokens) sits at position
+ * c_s + r, c_s = len_k(s) - len_q(s), and attends keys 0 .. c_s + r.  The first ceil(len_k/bs) table
+ * entries of a sequence are expected to be valid; an entry < 0 or >= num_blocks there is not followed (no
+ * out-of-range access): its keys and values read as zeros.  With c_s = 0 for every s the result equals
+ * mvllm_prefill_varlen bit for bit.
+ */
+int mvllm_prefill_paged(void* out, const void* q, const void* k_cache, const void* v_cache,
+                        const int32_t* block_tables, int max_num_blocks,
+                        const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                        int num_seqs, int64_t total_q_tokens,
+                        int num_heads, int num_kv_heads, int head_dim, int block_size,
+                        int64_t num_blocks, float scale, int dtype, void* stream);
+
+/*
  * The caller's per-layer chain between the QKV projection and the attention kernels, fused:
  *   q = rms_norm(q); k = rms_norm(k)      src/myvllm/models/qwen3.py:104-106, layers/layernorm.py:9-17
  *   q, k = rotary_emb(positions, q, k)    qwen3.py:108, layers/rotary_embedding.py:4-23, 77-83

@@ -32,6 +32,8 @@ SIGNATURES = {
                                                           c_void_p]),
     "mvllm_prefill_varlen": (c_int, [c_void_p] * 5 + [c_int, c_int64, c_int, c_int, c_int, c_float, c_int,
                                                        c_void_p]),
+    "mvllm_prefill_paged": (c_int, [c_void_p] * 5 + [c_int, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int,
+                                                      c_int, c_int64, c_float, c_int, c_void_p]),
     "mvllm_qk_norm_rope_store": (c_int, [c_void_p] * 6 + [c_int64] * 3 + [c_void_p, c_float, c_void_p, c_int64,
                                                            c_void_p, c_void_p] + [c_void_p] * 4 +
                                  [c_int, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p]),

@@ -25,6 +25,13 @@ struct PrefillArgs {
   float scale_log2;
   int tiles_x;      // MFMA path: query-tile upper bound (total_tokens / BM + num_seqs)
   int heads_y;      // MFMA path: head slices (kv heads x query-head chunks)
+  // Paged mode (k, v are caches [num_blocks, block_size, Hkv, D]; q holds only the tokens after each
+  // sequence's cached prefix): cu_seqlens counts the query rows, cu_seqlens_k the keys (prefix + new).
+  const int32_t* cu_seqlens_k;
+  const int32_t* block_tables;
+  int max_num_blocks;
+  int block_size;
+  int64_t num_blocks;
 };
 
 // Tile `tile` (global numbering) -> sequence and first row inside it.  Wave-parallel: 64 sequences
@@ -32,7 +39,7 @@ struct PrefillArgs {
 // a few hundred cycles per 64 sequences instead of one dependent load per sequence.  Every lane of
 // the calling wave must be active; all lanes return the same values.
 __device__ __forceinline__ bool locate_tile(const int32_t* __restrict__ cu, int num_seqs, int tile, int bm,
-                                            int& seq_start, int& seq_len, int& row0) {
+                                            int& seq_start, int& seq_len, int& row0, int& seq_index) {
   const int lane = threadIdx.x & 63;
   int first = 0;
   for (int base = 0; base < num_seqs; base += 64) {
@@ -57,6 +64,7 @@ __device__ __forceinline__ bool locate_tile(const int32_t* __restrict__ cu, int 
       seq_start = __shfl(lo, owner, 64);
       seq_len = __shfl(len, owner, 64);
       row0 = (tile - start_tile) * bm;
+      seq_index = base + owner;
       return true;
     }
     first += total;
@@ -72,10 +80,10 @@ __device__ __forceinline__ bool locate_tile(const int32_t* __restrict__ cu, int 
 constexpr int kGenRows = 16;   // query rows per workgroup (4 waves x 4 rows)
 constexpr int kGenMaxR = 8;
 
-template <typename T>
+template <typename T, bool PAGED>
 __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs a) {
-  int seq_start, seq_len, row0;
-  if (!locate_tile(a.cu_seqlens, a.num_seqs, blockIdx.x, kGenRows, seq_start, seq_len, row0)) return;
+  int seq_start, seq_len, row0, seq_index;
+  if (!locate_tile(a.cu_seqlens, a.num_seqs, blockIdx.x, kGenRows, seq_start, seq_len, row0, seq_index)) return;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int h = blockIdx.y;
@@ -87,6 +95,9 @@ __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs 
   T* out = reinterpret_cast<T*>(a.out);
   const int64_t qrow = (int64_t)a.num_heads * D;
   const int64_t kvrow = (int64_t)a.num_kv_heads * D;
+  // paged: keys 0 .. cached + r of the sequence, looked up through its block table row
+  const int cached = PAGED ? (a.cu_seqlens_k[seq_index + 1] - a.cu_seqlens_k[seq_index]) - seq_len : 0;
+  const int32_t* table = PAGED ? a.block_tables + (int64_t)seq_index * a.max_num_blocks : nullptr;
 
   for (int r = row0 + wave; r < min(row0 + kGenRows, seq_len); r += 4) {
     float qv[kGenMaxR], acc[kGenMaxR];
@@ -98,14 +109,23 @@ __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs 
       acc[i] = 0.f;
     }
     float m = -INFINITY, l = 0.f;
-    for (int j = 0; j <= r; ++j) {
-      const int64_t base = (int64_t)(seq_start + j) * kvrow + (int64_t)g * D;
+    for (int j = 0; j <= cached + r; ++j) {
+      int64_t base;
+      bool mapped = true;
+      if (PAGED) {
+        const int bi = j / a.block_size;
+        const int phys = bi < a.max_num_blocks ? table[bi] : -1;
+        mapped = phys >= 0 && phys < a.num_blocks;               // an unmapped block reads as zero keys and values
+        base = ((int64_t)(mapped ? phys : 0) * a.block_size + (j - bi * a.block_size)) * kvrow + (int64_t)g * D;
+      } else {
+        base = (int64_t)(seq_start + j) * kvrow + (int64_t)g * D;
+      }
       float vv[kGenMaxR];
       float dot = 0.f;
 #pragma unroll
       for (int i = 0; i < kGenMaxR; ++i) {
         const int d = lane + 64 * i;
-        if (d < D) {
+        if (d < D && mapped) {
           dot = fmaf(qv[i], to_float(k[base + d]), dot);
           vv[i] = to_float(v[base + d]);
         } else {
@@ -122,7 +142,7 @@ __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs 
       m = m_new;
     }
     T* op = out + (int64_t)(seq_start + r) * qrow + (int64_t)h * D;
-    const float linv = 1.f / l;
+    const float linv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
     for (int i = 0; i < kGenMaxR; ++i) {
       const int d = lane + 64 * i;
@@ -229,7 +249,7 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
 
-template <typename T, int HPW>
+template <typename T, int HPW, bool PAGED>
 __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const PrefillArgs a) {
   constexpr int D = 128;
   constexpr int ROW_TILES = kPfWaves / HPW;     // 32-row query tiles per workgroup
@@ -251,14 +271,19 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   if (item >= (unsigned)tiles_x * (unsigned)a.heads_y) return;
   const int item_y = (int)(item / (unsigned)tiles_x);
   const int item_x = (int)(item % (unsigned)tiles_x);
-  int seq_start, seq_len, row0;
+  int seq_start, seq_len, row0, seq_index;
   // latest (heaviest) tiles of a sequence first
-  if (!locate_tile(a.cu_seqlens, a.num_seqs, tiles_x - 1 - item_x, BM, seq_start, seq_len, row0)) return;
+  if (!locate_tile(a.cu_seqlens, a.num_seqs, tiles_x - 1 - item_x, BM, seq_start, seq_len, row0, seq_index)) return;
   // Wave-uniform by construction; say so, so that everything derived from them (tile counts, loop bounds,
   // tile base addresses, branches) lives in scalar registers and runs on the scalar unit.
   seq_start = __builtin_amdgcn_readfirstlane(seq_start);
   seq_len = __builtin_amdgcn_readfirstlane(seq_len);
   row0 = __builtin_amdgcn_readfirstlane(row0);
+  seq_index = __builtin_amdgcn_readfirstlane(seq_index);
+  // Keys of the sequence: its own rows, or in paged mode the cached prefix plus them (query row r sits at
+  // position cached + r and sees keys 0 .. cached + r).
+  const int kv_len = PAGED ? a.cu_seqlens_k[seq_index + 1] - a.cu_seqlens_k[seq_index] : seq_len;
+  const int cached = PAGED ? max(kv_len - seq_len, 0) : 0;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -268,9 +293,11 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   const int h = g * group + (item_y % chunks) * HPW + (wave % HPW);   // query head of this wave
   const int r0 = row0 + kWaveRows * (wave / HPW);    // first query row of this wave (inside the sequence)
   const bool active = r0 < seq_len;
-  const int jd = r0 / kBN;                           // diagonal K/V tile of this wave
+  const int pos0 = cached + r0;                      // position of that row among the keys
+  const int n_full = (pos0 + 1) / kBN;               // tiles every row of the wave sees completely
+  const int j_last = min(pos0 + kWaveRows - 1, kv_len - 1) / kBN;   // last tile any row of the wave sees
   const int wg_last = min(row0 + BM, seq_len) - 1;
-  const int ntiles = wg_last / kBN + 1;
+  const int ntiles = (cached + wg_last) / kBN + 1;
   const int l32 = lane & 31;
   const int hi = lane >> 5;                          // 0/1: which half of the k-slots / rows
   const int qrow = r0 + l32;                         // query row of this lane
@@ -288,12 +315,14 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   const int ld_row = lane >> 4;        // row inside the 4-row group
   const int ld_chunk = lane & 15;      // destination chunk inside the row
   constexpr int kCopies = ROWS_PER_WAVE / 4;
+  static_assert(!PAGED || ROWS_PER_WAVE == 16, "paged mode: one wave copies one 16-row piece of a cache block");
   uint32_t k_src_off[kCopies], v_src_off[kCopies];
 #pragma unroll
   for (int i = 0; i < kCopies; ++i) {
-    const int row = ROWS_PER_WAVE * wave + 4 * i + ld_row;   // row inside the tile
-    k_src_off[i] = (uint32_t)(row * (int)kv_row_bytes + ((ld_chunk ^ (row & 15)) << 4));
-    v_src_off[i] = (uint32_t)(row * (int)kv_row_bytes + ((ld_chunk ^ ((row & 3) << 2)) << 4));
+    const int row = ROWS_PER_WAVE * wave + 4 * i + ld_row;   // row inside the tile (decides the swizzle)
+    const int src_row = PAGED ? 4 * i + ld_row : row;        // paged: the descriptor starts at the wave's own rows
+    k_src_off[i] = (uint32_t)(src_row * (int)kv_row_bytes + ((ld_chunk ^ (row & 15)) << 4));
+    v_src_off[i] = (uint32_t)(src_row * (int)kv_row_bytes + ((ld_chunk ^ ((row & 3) << 2)) << 4));
   }
   // One tile's copy is 2 * kCopies instructions per wave (K copies first, then V).  Inside tile_step they are
   // issued one at a time, spread between the MFMAs of the tile before, because a wave that issues them back
@@ -301,20 +330,53 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   // starts at the tile's first row and ends with the tensor, so rows past the last packed token arrive as
   // zeros; a descriptor of size 0 (enable = false) turns the copy into a zero fill that touches no memory,
   // which keeps the last tile's code free of branches.
+  // Paged mode: the wave's 16 rows of a tile are one piece of one cache block (block_size % 16 == 0); the
+  // descriptor starts at that piece and ends with the sequence's last key, so rows of the block that were
+  // never written (and unmapped blocks) arrive as zeros.  Tiles are asked for in order, once each, so the
+  // piece's block index and offset advance by 64 keys per call; block-table entries come from a 64-entry
+  // window held one per lane, as in the decode kernel.
   struct TileSrc { v4i k, v; };
   const int row_bytes = (int)kv_row_bytes;
   const int total_rows = (int)a.total_tokens;
   const int rows_4g = (int)(0xffffffffu / (uint32_t)row_bytes);   // rows whose bytes no longer fit 32 bits
+  const int bs = PAGED ? a.block_size : 1;
+  const int32_t* table = PAGED ? a.block_tables + (int64_t)seq_index * a.max_num_blocks : nullptr;
+  int pg_pos = ROWS_PER_WAVE * wave;                 // key position of this wave's piece in the next tile asked for
+  int pg_bi = pg_pos / bs, pg_off = pg_pos - pg_bi * bs;
+  int win_base = 0;
+  int win = -1;
+  if (PAGED) win = lane < a.max_num_blocks ? table[lane] : -1;
   auto tile_src = [&](int j, bool enable) {
-    const int row0 = seq_start + j * kBN;                          // first row of the tile
-    const int rows_left = total_rows - row0;
-    const uint32_t size = (!enable || rows_left <= 0) ? 0u
-                          : rows_left > rows_4g       ? 0xffffffffu
-                                                      : (uint32_t)(rows_left * row_bytes - g * (D * 2));
-    const int64_t start = (int64_t)row0 * kv_row_bytes + (int64_t)g * (D * 2);
     TileSrc t;
-    t.k = make_rsrc(kg + start, size);
-    t.v = make_rsrc(vg + start, size);
+    if constexpr (PAGED) {
+      (void)j;
+      if (pg_bi - win_base >= 64) {
+        win_base = pg_bi;
+        win = win_base + lane < a.max_num_blocks ? table[win_base + lane] : -1;
+      }
+      const int phys = __builtin_amdgcn_readlane(win, pg_bi - win_base);
+      const int valid = min(ROWS_PER_WAVE, kv_len - pg_pos);
+      const bool ok = enable && valid > 0 && pg_bi < a.max_num_blocks && phys >= 0 && (int64_t)phys < a.num_blocks;
+      const uint32_t size = ok ? (uint32_t)((valid - 1) * row_bytes + D * 2) : 0u;
+      const int64_t start = ok ? ((int64_t)phys * bs + pg_off) * kv_row_bytes + (int64_t)g * (D * 2) : 0;
+      t.k = make_rsrc(kg + start, size);
+      t.v = make_rsrc(vg + start, size);
+      pg_pos += kBN;
+      pg_off += kBN;
+      while (pg_off >= bs) {
+        pg_off -= bs;
+        ++pg_bi;
+      }
+    } else {
+      const int row0 = seq_start + j * kBN;                          // first row of the tile
+      const int rows_left = total_rows - row0;
+      const uint32_t size = (!enable || rows_left <= 0) ? 0u
+                            : rows_left > rows_4g       ? 0xffffffffu
+                                                        : (uint32_t)(rows_left * row_bytes - g * (D * 2));
+      const int64_t start = (int64_t)row0 * kv_row_bytes + (int64_t)g * (D * 2);
+      t.k = make_rsrc(kg + start, size);
+      t.v = make_rsrc(vg + start, size);
+    }
     return t;
   };
   // LDS byte address of this wave's first row in buffer 0 of K; V, buffer 1 and later copies are constants away
@@ -410,7 +472,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     // ---- online softmax, one query row per lane (scores stay unscaled; the scale is folded
     //      into the exp2 argument) ----
     if constexpr (diag) {
-      const int thr = qrow - j * kBN - 4 * hi;       // kv offset inside the tile must be <= thr
+      const int thr = cached + qrow - j * kBN - 4 * hi;   // kv offset inside the tile must be <= thr
 #pragma unroll
       for (int tk = 0; tk < NH; ++tk)
 #pragma unroll
@@ -472,7 +534,8 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   };
 
   // Tile j lives in buffer j % 2.  The main loop is unrolled by two so that the buffer index is a compile-time
-  // constant inside tile_step.  A wave's tiles are jd full ones and then the diagonal one.
+  // constant inside tile_step.  A wave's tiles are n_full complete ones and then those the causal diagonal runs
+  // through: one when the rows start at a multiple of 32 keys (always, without a cached prefix), else up to two.
   using B0 = std::integral_constant<int, 0>;
   using B1 = std::integral_constant<int, 1>;
   using H1 = std::integral_constant<int, 1>;
@@ -485,22 +548,23 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   auto diag_step = [&](int j, auto BUF) {
     dma_wait_all();
     __syncthreads();
-    if ((r0 & 32) == 0) tile_step(j, BUF, std::true_type{}, H1{}, j + 1 < ntiles);
+    // no row of the wave reaches the second 32 keys of the tile: skip that half
+    if (pos0 + kWaveRows - 1 < j * kBN + 32) tile_step(j, BUF, std::true_type{}, H1{}, j + 1 < ntiles);
     else tile_step(j, BUF, std::true_type{}, H2{}, j + 1 < ntiles);
   };
   int j = 0;
   if (active) {
-    for (; j + 1 < jd; j += 2) {
+    for (; j + 1 < n_full; j += 2) {
       full_step(j, B0{});
       full_step(j + 1, B1{});
     }
-    if (j < jd) {
+    if (j < n_full) {
       full_step(j, B0{});
-      diag_step(j + 1, B1{});
-      j += 2;
-    } else {
-      diag_step(j, B0{});
-      j += 1;
+      ++j;
+    }
+    for (; j <= j_last; ++j) {
+      if (j & 1) diag_step(j, B1{});
+      else diag_step(j, B0{});
     }
   }
   // Tiles that only other waves of the workgroup still compute on (their rows are further down): keep copying
@@ -544,7 +608,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   }
 }
 
-template <typename T>
+template <typename T, bool PAGED>
 static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   const int group = a.num_heads / a.num_kv_heads;
   const int hpw = group >= 4 ? 4 : group;              // 1, 2 or 4 (group is 1, 2 or a multiple of 4)
@@ -555,16 +619,27 @@ static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   const int64_t items = (int64_t)b.tiles_x * b.heads_y;
   const int64_t span = 8 * (int64_t)kXcdChunk;
   dim3 grid((unsigned)((items + span - 1) / span * span));
-  if (hpw == 4) prefill_mfma_kernel<T, 4><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
-  else if (hpw == 2) prefill_mfma_kernel<T, 2><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
-  else prefill_mfma_kernel<T, 1><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
+  if (hpw == 4) prefill_mfma_kernel<T, 4, PAGED><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
+  else if (hpw == 2) prefill_mfma_kernel<T, 2, PAGED><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
+  else prefill_mfma_kernel<T, 1, PAGED><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
   return launch_status();
 }
-template <typename T>
+template <typename T, bool PAGED>
 static int launch_prefill_generic(const PrefillArgs& a, hipStream_t stream) {
   const int64_t tiles = a.total_tokens / kGenRows + a.num_seqs;
-  prefill_generic_kernel<T><<<dim3((unsigned)tiles, (unsigned)a.num_heads), dim3(256), 0, stream>>>(a);
+  prefill_generic_kernel<T, PAGED><<<dim3((unsigned)tiles, (unsigned)a.num_heads), dim3(256), 0, stream>>>(a);
   return launch_status();
+}
+
+template <bool PAGED>
+static int prefill_dispatch(const PrefillArgs& a, int dtype, bool mfma_ok, hipStream_t s) {
+  if (mfma_ok)
+    return dtype == MVLLM_BF16 ? launch_prefill_mfma<bf16_t, PAGED>(a, s) : launch_prefill_mfma<f16_t, PAGED>(a, s);
+  switch (dtype) {
+    case MVLLM_F32: return launch_prefill_generic<float, PAGED>(a, s);
+    case MVLLM_BF16: return launch_prefill_generic<bf16_t, PAGED>(a, s);
+    default: return launch_prefill_generic<f16_t, PAGED>(a, s);
+  }
 }
 
 }  // namespace mvllm
@@ -588,15 +663,40 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   a.total_tokens = total_tokens; a.num_seqs = num_seqs; a.num_heads = num_heads;
   a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
   a.tiles_x = 0; a.heads_y = 0;
-  hipStream_t s = (hipStream_t)stream;
+  a.cu_seqlens_k = nullptr; a.block_tables = nullptr; a.max_num_blocks = 0; a.block_size = 0; a.num_blocks = 0;
   const int group = num_heads / num_kv_heads;
   const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 && (group == 1 || group == 2 || group % 4 == 0) &&
                        aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
                        num_kv_heads * group <= 65535;
-  if (mfma_ok) return dtype == MVLLM_BF16 ? launch_prefill_mfma<bf16_t>(a, s) : launch_prefill_mfma<f16_t>(a, s);
-  switch (dtype) {
-    case MVLLM_F32: return launch_prefill_generic<float>(a, s);
-    case MVLLM_BF16: return launch_prefill_generic<bf16_t>(a, s);
-    default: return launch_prefill_generic<f16_t>(a, s);
-  }
+  return prefill_dispatch<false>(a, dtype, mfma_ok, (hipStream_t)stream);
+}
+
+extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                   const int32_t* block_tables, int max_num_blocks, const int32_t* cu_seqlens_q,
+                                   const int32_t* cu_seqlens_k, int num_seqs, int64_t total_q_tokens,
+                                   int num_heads, int num_kv_heads, int head_dim, int block_size,
+                                   int64_t num_blocks, float scale, int dtype, void* stream) {
+  if (dtype_size(dtype) == 0) return MVLLM_ERR_BAD_DTYPE;
+  if (num_seqs < 0 || total_q_tokens < 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 ||
+      block_size <= 0 || num_blocks < 0 || max_num_blocks < 0)
+    return MVLLM_ERR_BAD_SHAPE;
+  if (num_heads % num_kv_heads != 0) return MVLLM_ERR_BAD_SHAPE;
+  if (num_seqs == 0 || total_q_tokens == 0) return MVLLM_OK;
+  if (!out || !q || !k_cache || !v_cache || !block_tables || !cu_seqlens_q || !cu_seqlens_k)
+    return MVLLM_ERR_NULL_POINTER;
+  if (head_dim > 64 * kGenMaxR || num_heads > 65535) return MVLLM_ERR_UNSUPPORTED;
+  if (total_q_tokens > ((int64_t)1 << 30)) return MVLLM_ERR_UNSUPPORTED;
+  PrefillArgs a;
+  a.out = out; a.q = q; a.k = k_cache; a.v = v_cache; a.cu_seqlens = cu_seqlens_q;
+  a.total_tokens = total_q_tokens; a.num_seqs = num_seqs; a.num_heads = num_heads;
+  a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
+  a.tiles_x = 0; a.heads_y = 0;
+  a.cu_seqlens_k = cu_seqlens_k; a.block_tables = block_tables; a.max_num_blocks = max_num_blocks;
+  a.block_size = block_size; a.num_blocks = num_blocks;
+  const int group = num_heads / num_kv_heads;
+  const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 && (group == 1 || group == 2 || group % 4 == 0) &&
+                       block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) &&
+                       aligned16(out) && num_kv_heads * group <= 65535 &&
+                       (int64_t)block_size * num_kv_heads * head_dim * 2 < ((int64_t)1 << 31);
+  return prefill_dispatch<true>(a, dtype, mfma_ok, (hipStream_t)stream);
 }

@@ -89,6 +89,10 @@ class BlockManager:
                 block.update(h, token_ids)
                 self.hash_to_block_id[h] = block.block_id
             seq.block_table.append(block.block_id)
+        if seq.num_cached_tokens == len(seq):
+            # every block hit: the last one is recomputed anyway (identical values into the shared block), so
+            # that the step has at least one query token per sequence to take the next-token logits from
+            seq.num_cached_tokens -= self.block_size
 
     def deallocate(self, seq: Sequence) -> None:
         for block_id in reversed(seq.block_table):

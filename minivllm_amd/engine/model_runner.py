@@ -74,14 +74,20 @@ class ModelRunner:
         return torch.tensor(values, dtype=dtype, pin_memory=True).to(self.device, non_blocking=True)
 
     def prepare_prefill(self, seqs):
-        md = prefill_metadata(seqs, self.block_size, reuse_cached_kv=False)
-        positions = [p for seq in seqs for p in range(len(seq))]
+        """Packed prompt tokens and their metadata (model_runner.py:180-227).  Tokens covered by prefix-cache hits
+        are left out and read from the paged cache by the attention kernel; with an int8 cache (no paged prefill
+        for it) or ``prefix_caching=False`` they are recomputed into the shared blocks instead."""
+        reuse = self.kv_cache_dtype != "int8" and self.config.get("prefix_caching", True)
+        md = prefill_metadata(seqs, self.block_size, reuse_cached_kv=reuse)
+        positions = [p for seq in seqs for p in range(seq.num_cached_tokens if reuse else 0, len(seq))]
+        tables = md["block_tables"]
         set_context(True,
                     cu_seqlens_q=self._to_device(md["cu_seqlens_q"], torch.int32),
                     cu_seqlens_k=self._to_device(md["cu_seqlens_k"], torch.int32),
                     max_seqlen_q=md["max_seqlen_q"], max_seqlen_k=md["max_seqlen_k"],
                     slot_mapping=self._to_device(md["slot_mapping"], torch.int64),
-                    context_lens=None, block_tables=None)
+                    context_lens=None,
+                    block_tables=None if tables is None else self._to_device(tables, torch.int32))
         return self._to_device(md["input_ids"], torch.int64), self._to_device(positions, torch.int64)
 
     def prepare_decode(self, seqs):

@@ -21,7 +21,7 @@ from minivllm_amd.layers.fused import qk_norm_rope_store
 from minivllm_amd.utils.context import get_context
 
 __all__ = [
-    "store_kvcache", "store_kvcache_int8", "flash_attention_prefill",
+    "store_kvcache", "store_kvcache_int8", "flash_attention_prefill", "flash_attention_prefill_paged",
     "paged_attention_decode", "paged_attention_decode_int8", "Attention",
 ]
 
@@ -152,6 +152,48 @@ def flash_attention_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, c
     return output
 
 
+def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                                  block_tables: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                                  cu_seqlens_k: torch.Tensor, scale: float, num_heads: int, num_kv_heads: int,
+                                  head_dim: int, block_size: int) -> torch.Tensor:
+    """Causal prefill of the tokens that follow each sequence's cached prefix, with every key read from the
+    paged cache.  Consumes the metadata ``ModelRunner.prepare_prefill`` builds for prefix-cache hits
+    (model_runner.py:192-226), which the reference's ``Attention.forward`` ignores (attention.py:518-523).
+
+    q: (total_new_tokens, num_heads, head_dim) packed by ``cu_seqlens_q``; caches
+    (num_blocks, block_size, Hkv, D) already holding all ``cu_seqlens_k`` keys of every sequence;
+    block_tables int32 (num_seqs, max_num_blocks).  Returns a tensor like q.
+    """
+    _C.require_cuda(q, k_cache, v_cache, block_tables, cu_seqlens_q, cu_seqlens_k)
+    if q.dim() != 3 or tuple(q.shape[1:]) != (num_heads, head_dim):
+        raise ValueError(f"q must be (total_tokens, {num_heads}, {head_dim}), got {tuple(q.shape)}")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise ValueError(f"q {q.dtype} and cache {k_cache.dtype} dtypes differ (no int8 cache in paged prefill)")
+    _check_cache("k_cache", k_cache, num_kv_heads, head_dim)
+    _check_cache("v_cache", v_cache, num_kv_heads, head_dim)
+    if k_cache.shape != v_cache.shape:
+        raise ValueError("K and V cache shapes must match")
+    if k_cache.shape[1] != block_size:
+        raise ValueError(f"cache block dimension {k_cache.shape[1]} != block_size {block_size}")
+    num_seqs = cu_seqlens_q.shape[0] - 1
+    if cu_seqlens_k.shape[0] != num_seqs + 1:
+        raise ValueError("cu_seqlens_q and cu_seqlens_k must have the same length")
+    if block_tables.dim() != 2 or block_tables.shape[0] != num_seqs:
+        raise ValueError(f"block_tables must be ({num_seqs}, max_num_blocks), got {tuple(block_tables.shape)}")
+    q = q.contiguous()
+    block_tables = block_tables.to(torch.int32).contiguous()
+    cu_seqlens_q = cu_seqlens_q.to(torch.int32).contiguous()
+    cu_seqlens_k = cu_seqlens_k.to(torch.int32).contiguous()
+    output = torch.empty_like(q)
+    lib = _C.load()
+    st = lib.mvllm_prefill_paged(_ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                 block_tables.shape[1], _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), num_seqs,
+                                 q.shape[0], num_heads, num_kv_heads, head_dim, block_size, k_cache.shape[0],
+                                 float(scale), _C.dtype_code(q.dtype), _C.current_stream_ptr(q.device))
+    _C.check(st, "flash_attention_prefill_paged")
+    return output
+
+
 def _decode_common(query, k_cache, v_cache, block_tables, context_lens, num_heads, num_kv_heads, head_dim,
                    block_size):
     if query.dim() != 3 or tuple(query.shape[1:]) != (num_heads, head_dim):
@@ -278,7 +320,7 @@ class Attention(nn.Module):
             slot_mapping=context.slot_mapping if store else None,
             k_cache=self.k_cache if store else None, v_cache=self.v_cache if store else None,
             k_scale=self.k_scale if store and int8 else None, v_scale=self.v_scale if store and int8 else None,
-            need_kv=context.is_prefill)
+            need_kv=context.is_prefill and context.block_tables is None)
         return self._attend(context, q, k, v)
 
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
@@ -312,6 +354,17 @@ class Attention(nn.Module):
             cu_seqlens = context.cu_seqlens_q
             if cu_seqlens is None:
                 raise ValueError("cu_seqlens_q must be provided for varlen attention")
+            if context.block_tables is not None:
+                # some sequence starts after a cached prefix: every key comes from the paged cache, which the
+                # store above has just completed with the new tokens (model_runner.py:206-215)
+                if int8:
+                    raise ValueError("prefill over a cached prefix needs a cache in the model dtype, not int8")
+                if context.cu_seqlens_k is None or k_cache.numel() == 0:
+                    raise ValueError("cu_seqlens_k and the KV cache must be provided for prefill over a cached prefix")
+                o = flash_attention_prefill_paged(q, k_cache, v_cache, context.block_tables, cu_seqlens,
+                                                  context.cu_seqlens_k, scale, self.num_heads, self.num_kv_heads,
+                                                  self.head_dim, self.block_size)
+                return o.reshape(o.shape[0], self.num_heads * self.head_dim)
             o = flash_attention_prefill(q, k, v, cu_seqlens, scale, self.num_heads, self.num_kv_heads,
                                         self.head_dim)
             return o.reshape(o.shape[0], self.num_heads * self.head_dim)

@@ -13,6 +13,7 @@ from .attention_oracle import (  # noqa: F401
     decode_vectorised_oracle,
     decode_int8_oracle,
     prefill_standard_oracle,
+    prefill_paged_oracle,
     gather_sequence_kv,
     rms_norm_oracle,
     rope_cos_sin_cache_oracle,

@@ -16,6 +16,9 @@ pinned by ``tests/test_oracle_pins.py`` against what the mathematics fixes:
                                 |x-code*scale|<=scale/2, scale == amax/127 in fp32)
                                 -- "parity unpinned" by the reference: it has no
                                 INT8 code; the spec is defined by this build.
+* ``prefill_paged_oracle``       equals the last rows of ``prefill_standard_oracle`` on the
+                                full sequences; no cached prefix == plain prefill; one
+                                new token == the decode oracle
 * ``rms_norm_oracle`` / ``rope_cos_sin_cache_oracle`` / ``rope_oracle`` /
   ``qk_norm_rope_store_oracle``   unit mean square, scale invariance, constant-vector
                                 closed form; table vs cos/sin of pos * base^(-2i/D) in
@@ -213,6 +216,32 @@ def prefill_standard_oracle(q, k, v, cu_seqlens, scale, num_heads, num_kv_heads,
         scores = scores.masked_fill(future.unsqueeze(0), float("-inf"))
         probs = torch.softmax(scores, dim=-1)
         out[lo:hi] = torch.matmul(probs, vs).transpose(0, 1)
+    return out
+
+
+def prefill_paged_oracle(q, k_cache, v_cache, block_tables, cu_seqlens_q, cu_seqlens_k, scale,
+                         num_heads, num_kv_heads, head_dim, block_size):
+    """Prefill of the tokens after a cached prefix: what ``pytorch_standard_attention``
+    (benchmark_prefilling.py:9-52) gives for the LAST len_q rows of each sequence when its keys are gathered
+    from the paged cache in logical order (``gather_sequence_kv``, benchmark_decoding.py:228-233) --
+    the computation the metadata of model_runner.py:192-226 describes.  fp32 math, result in q's dtype."""
+    out = torch.empty_like(q)
+    group = num_heads // num_kv_heads
+    cq, ck = cu_seqlens_q.tolist(), cu_seqlens_k.tolist()
+    for s in range(len(cq) - 1):
+        lq, lk = cq[s + 1] - cq[s], ck[s + 1] - ck[s]
+        if lq == 0:
+            continue
+        cached = lk - lq
+        k = gather_sequence_kv(k_cache, block_tables[s], lk, block_size).float()
+        v = gather_sequence_kv(v_cache, block_tables[s], lk, block_size).float()
+        k = k.repeat_interleave(group, dim=1).transpose(0, 1)                 # (Hq, lk, D)
+        v = v.repeat_interleave(group, dim=1).transpose(0, 1)
+        qs = q[cq[s]:cq[s + 1]].float().transpose(0, 1)                       # (Hq, lq, D)
+        scores = torch.matmul(qs, k.transpose(1, 2)) * scale                  # (Hq, lq, lk)
+        pos = torch.arange(lq).unsqueeze(1) + cached                          # key j visible iff j <= cached + i
+        scores = scores.masked_fill(torch.arange(lk).unsqueeze(0) > pos, float("-inf"))
+        out[cq[s]:cq[s + 1]] = torch.matmul(torch.softmax(scores, dim=-1), v).transpose(0, 1).to(q.dtype)
     return out
 
 

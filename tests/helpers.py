@@ -105,3 +105,26 @@ def extract_sequence(k_cache, v_cache, tables, ctx, b, block_size):
     vc = v_cache[ids].cpu()
     table = torch.arange(need, dtype=torch.int32).unsqueeze(0)
     return kc, vc, table, ctx[b:b + 1]
+
+
+def make_paged_prefill_case(seed, kv_lengths, cached, num_heads, num_kv_heads, head_dim, block_size,
+                            dtype=torch.float32, poison=float("nan")):
+    """Sequences of ``kv_lengths`` tokens whose first ``cached`` tokens count as a cached prefix.
+
+    Returns the full packed (q, k, v, cu_k) of a plain prefill, the caches holding every key (rows of a block
+    past a sequence's end are filled with ``poison``: the kernel must not let them through), the padded block
+    tables, and the query rows / cu_seqlens_q of the new tokens only.
+    """
+    q, k, v, cu_k = make_varlen_case(seed, kv_lengths, num_heads, num_kv_heads, head_dim, dtype)
+    slots, tables, num_blocks = make_slot_mapping(seed + 1, kv_lengths, block_size)
+    k_cache = torch.full((num_blocks, block_size, num_kv_heads, head_dim), poison).to(dtype)
+    v_cache = torch.full((num_blocks, block_size, num_kv_heads, head_dim), poison).to(dtype)
+    k_cache.view(-1, num_kv_heads, head_dim)[slots] = k
+    v_cache.view(-1, num_kv_heads, head_dim)[slots] = v
+    width = max(len(t) for t in tables)
+    block_tables = torch.tensor([t + [-1] * (width - len(t)) for t in tables], dtype=torch.int32)
+    new_rows = torch.cat([torch.arange(int(cu_k[s]) + c, int(cu_k[s + 1])) for s, c in enumerate(cached)])
+    cu_q = torch.zeros(len(kv_lengths) + 1, dtype=torch.int32)
+    cu_q[1:] = torch.tensor([n - c for n, c in zip(kv_lengths, cached)], dtype=torch.int32).cumsum(0)
+    return dict(q=q, k=k, v=v, cu_k=cu_k, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables,
+                q_new=q[new_rows].contiguous(), new_rows=new_rows, cu_q=cu_q)

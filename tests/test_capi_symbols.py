@@ -28,7 +28,7 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_prefill_varlen",
-              "mvllm_qk_norm_rope_store", "mvllm_version", "mvllm_status_string"]:
+              "mvllm_prefill_paged", "mvllm_qk_norm_rope_store", "mvllm_version", "mvllm_status_string"]:
         assert n in names
 
 
@@ -63,6 +63,12 @@ def test_argument_validation_without_gpu():
     assert lib.mvllm_paged_decode(0, 0, 0, 0, 0, 4, 0, 1, 2, 6, 4, 128, 16, 8, 1.0, 1, 0, 0, 0) == -3  # Hq % Hkv
     assert lib.mvllm_prefill_varlen(0, 0, 0, 0, 0, 0, 0, 4, 2, 128, 1.0, 1, 0) == 0      # empty batch
     assert lib.mvllm_prefill_varlen(0, 0, 0, 0, 0, 1, 5, 4, 2, 128, 1.0, 1, 0) == -1
+    paged = lib.mvllm_prefill_paged
+    #            out q kc vc tables MB cu_q cu_k S  T  Hq Hkv D   bs  NB scale dt stream
+    assert paged(0, 0, 0, 0, 0, 4, 0, 0, 0, 0, 4, 2, 128, 16, 8, 1.0, 1, 0) == 0       # no sequences
+    assert paged(0, 0, 0, 0, 0, 4, 0, 0, 1, 5, 4, 2, 128, 16, 8, 1.0, 1, 0) == -1      # null pointers
+    assert paged(0, 0, 0, 0, 0, 4, 0, 0, 1, 5, 4, 3, 128, 16, 8, 1.0, 1, 0) == -3      # Hq % Hkv
+    assert paged(0, 0, 0, 0, 0, 4, 0, 0, 1, 5, 4, 2, 128, 0, 8, 1.0, 1, 0) == -3       # block_size
     fused = lib.mvllm_qk_norm_rope_store
     #     q_out k_out v_out q k v | strides | gamma eps cos max_pos pos slots | caches scales int8 | T slots Hq Hkv D dt stream
     assert fused(0, 0, 0, 0, 0, 0, 512, 256, 256, 0, 1e-6, 0, 64, 0, 0, 0, 0, 0, 0, 0, 0, 0, 4, 2, 128, 1, 0) == 0   # no tokens

@@ -56,7 +56,7 @@ def test_block_manager_allocate_free_and_prefix_sharing():
     assert len(bm.free_block_ids) == 8 and not bm.used_block_ids
     c = _seq(8, 4)                                                      # cached hashes survive a free
     bm.allocate(c)
-    assert c.num_cached_tokens == 8
+    assert c.num_cached_tokens == 4        # both blocks hit; the last one is handed back to be recomputed
     d = Sequence([5, 5, 5, 5, 4, 5, 6, 7], SamplingParams(), 4)         # same 2nd block tokens, other prefix: no hit
     bm.allocate(d)
     assert d.num_cached_tokens == 0
@@ -169,3 +169,24 @@ def test_scheduler_eos_and_token_budget_and_preemption():
     assert a.is_finished and len(sch.block_manager.free_block_ids) == 3
     seqs, is_prefill = sch.schedule()
     assert is_prefill and seqs == [b] and len(b) == 5  # re-prefilled with prompt + generated token
+
+
+def test_full_prefix_hit_still_leaves_one_block_to_compute():
+    """A prompt made only of cached full blocks would have no query token in its prefill step; the allocator
+    hands the last block back to be recomputed (it stays shared)."""
+    from minivllm_amd.engine.block_manager import BlockManager
+    from minivllm_amd.engine.metadata import prefill_metadata
+    from minivllm_amd.engine.sequence import Sequence
+    from minivllm_amd.sampling_parameters import SamplingParams
+    bm = BlockManager(8, 4)
+    sp = SamplingParams()
+    first = Sequence(list(range(12)), sp, 4)
+    bm.allocate(first)
+    again = Sequence(list(range(8)), sp, 4)                       # blocks 0 and 1 of `first`
+    bm.allocate(again)
+    assert again.block_table == first.block_table[:2]
+    assert again.num_cached_tokens == 4
+    md = prefill_metadata([again], 4, reuse_cached_kv=True)
+    assert md["input_ids"] == [4, 5, 6, 7] and md["cu_seqlens_q"] == [0, 4] and md["cu_seqlens_k"] == [0, 8]
+    assert md["slot_mapping"] == [again.block_table[1] * 4 + i for i in range(4)]
+    assert md["block_tables"] == [again.block_table]

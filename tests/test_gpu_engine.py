@@ -105,3 +105,31 @@ def test_fused_qk_path_matches_unfused_modules(kv_cache_dtype):
     a, b = caches[0].float(), caches[1].float()
     if kv_cache_dtype == "auto" and same == 4:
         assert (a - b).abs().max() <= 6e-2 and (a - b).abs().mean() <= 1e-3
+
+
+def test_prefix_cache_hits_are_read_from_the_paged_cache():
+    """Prompts that share whole blocks with an earlier request skip those tokens in prefill (the attention
+    kernel reads their keys from the paged cache).  The generated tokens must match a run that recomputes them."""
+    g = torch.Generator().manual_seed(12)
+    shared = torch.randint(0, 2048, (48,), generator=g).tolist()          # three full blocks of 16
+    prompts = [shared + torch.randint(0, 2048, (n,), generator=g).tolist() for n in (5, 21, 0, 16)]
+    prompts.append(shared[:32])                                            # exactly two cached blocks, nothing new
+    sp = SamplingParams(temperature=0.6, max_tokens=8, ignore_eos=True)
+    cfg = dict(SMALL, max_num_sequences=2, max_cached_blocks=64)           # two per step: later steps hit the cache
+    outs, skipped = [], []
+    for reuse in (True, False):
+        eng = LLMEngine(dict(cfg, prefix_caching=reuse))
+        fed = []
+        real = eng.model_runner.prepare_prefill
+
+        def spy(seqs, real=real, fed=fed):
+            ids, pos = real(seqs)
+            fed.append((ids.numel(), sum(len(s) for s in seqs)))
+            return ids, pos
+        eng.model_runner.prepare_prefill = spy
+        outs.append(eng.generate(prompts, sp)["token_ids"])
+        skipped.append(sum(total - n for n, total in fed))
+    assert skipped[1] == 0
+    assert skipped[0] >= 48 + 48 + 16, skipped            # the 2nd step reuses 3 blocks twice, the 3rd at least 1
+    same = sum(a == b for a, b in zip(*outs))
+    assert same >= 4, outs                                # a 1-ulp difference may flip a sampling tie, rarely

@@ -1,0 +1,129 @@
+"""flash_attention_prefill_paged (prefill after a cached prefix, keys from the paged cache) on the GPU vs the CPU
+oracle; tolerances as for the plain prefill: bf16/fp16 max-abs <= 2e-2 and mean-abs <= 2e-3, fp32 max-abs <= 2e-4,
+against the oracle evaluated in fp32 on the same inputs.  Cache rows past a sequence's end hold NaN in these
+cases: any leak shows up as NaN in the output."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import error_stats, make_paged_prefill_case
+from minivllm_amd.layers.attention import (Attention, flash_attention_prefill, flash_attention_prefill_paged,
+                                           paged_attention_decode)
+from minivllm_amd.utils import reset_context, set_context
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+MAX_ABS_16, MEAN_ABS_16, MAX_ABS_32 = 2e-2, 2e-3, 2e-4
+
+
+def _run(c, scale, hq, hkv, d, bs):
+    out = flash_attention_prefill_paged(c["q_new"].to(DEV), c["k_cache"].to(DEV), c["v_cache"].to(DEV),
+                                        c["block_tables"].to(DEV), c["cu_q"].to(DEV), c["cu_k"].to(DEV), scale,
+                                        hq, hkv, d, bs)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def _oracle32(c, scale, hq, hkv, d, bs):
+    return oracle.prefill_paged_oracle(c["q_new"].float(), c["k_cache"].float(), c["v_cache"].float(),
+                                       c["block_tables"], c["cu_q"], c["cu_k"], scale, hq, hkv, d, bs)
+
+
+def _check(got, want, dtype):
+    assert not torch.isnan(got.float()).any()
+    mx, mean = error_stats(got, want)
+    if dtype == torch.float32:
+        assert mx <= MAX_ABS_32, mx
+    else:
+        assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("hq,hkv,d,bs,lengths,cached", [
+    (32, 8, 128, 16, [300, 64, 129, 500], [256, 0, 16, 48]),       # prefixes at multiples of 16, 64-aligned or not
+    (32, 8, 128, 256, [700, 300, 257], [512, 256, 0]),             # the engine's block size
+    (16, 8, 128, 16, [200, 90], [160, 80]),                        # GQA 2
+    (8, 8, 128, 32, [150], [96]),                                  # no grouping
+    (32, 8, 128, 16, [131, 77, 260], [50, 1, 259]),                # prefixes at arbitrary token counts, 1 new token
+    (6, 2, 80, 8, [40, 23], [16, 8]),                              # generic kernel (head_dim 80)
+    (4, 4, 64, 16, [70], [32]),                                    # generic kernel (head_dim 64)
+])
+def test_paged_prefill_vs_oracle(dtype, hq, hkv, d, bs, lengths, cached):
+    c = make_paged_prefill_case(61, lengths, cached, hq, hkv, d, bs, dtype=dtype)
+    scale = 1 / math.sqrt(d)
+    got = _run(c, scale, hq, hkv, d, bs)
+    want = _oracle32(c, scale, hq, hkv, d, bs)
+    assert got.dtype == dtype and got.shape == want.shape
+    _check(got, want, dtype)
+
+
+def test_paged_prefill_without_prefix_matches_plain_prefill_bitwise():
+    """No cached prefix: same tiles, same arithmetic as the packed kernel, only the copies' source differs."""
+    hq, hkv, d, bs = 32, 8, 128, 16
+    lengths = [257, 64, 31, 400]
+    c = make_paged_prefill_case(62, lengths, [0] * 4, hq, hkv, d, bs, dtype=torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    got = _run(c, scale, hq, hkv, d, bs)
+    plain = flash_attention_prefill(c["q"].to(DEV), c["k"].to(DEV), c["v"].to(DEV), c["cu_k"].to(DEV), scale,
+                                    hq, hkv, d).cpu()
+    assert torch.equal(got, plain)
+
+
+def test_paged_prefill_single_new_token_matches_decode():
+    hq, hkv, d, bs = 32, 8, 128, 16
+    lengths = [300, 17, 1, 64]
+    c = make_paged_prefill_case(63, lengths, [n - 1 for n in lengths], hq, hkv, d, bs, dtype=torch.bfloat16,
+                                poison=0.0)
+    scale = 1 / math.sqrt(d)
+    got = _run(c, scale, hq, hkv, d, bs)
+    dec = paged_attention_decode(c["q_new"].to(DEV), c["k_cache"].to(DEV), c["v_cache"].to(DEV),
+                                 c["block_tables"].to(DEV), torch.tensor(lengths, device=DEV), scale, hq, hkv, d,
+                                 bs).cpu()
+    mx, mean = error_stats(got, dec.float())
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16
+
+
+def test_paged_prefill_unmapped_blocks_and_empty_sequences():
+    """A table entry outside the pool is not followed: its keys and values read as zeros, exactly as if the
+    entry pointed at a block of zeros.  A sequence without new tokens produces no rows."""
+    hq, hkv, d, bs = 8, 2, 128, 16
+    lengths, cached = [100, 40, 70], [32, 40, 0]                   # the second sequence has no new tokens
+    for dtype in (torch.bfloat16, torch.float32):
+        c = make_paged_prefill_case(64, lengths, cached, hq, hkv, d, bs, dtype=dtype)
+        zero_block = c["k_cache"].shape[0]
+        kc = torch.cat([c["k_cache"], torch.zeros(1, bs, hkv, d, dtype=dtype)])
+        vc = torch.cat([c["v_cache"], torch.zeros(1, bs, hkv, d, dtype=dtype)])
+        want_tables = c["block_tables"].clone()
+        want_tables[0, 1] = zero_block                             # oracle: the hole is a block of zeros
+        want = _oracle32(dict(c, k_cache=kc, v_cache=vc, block_tables=want_tables), 0.09, hq, hkv, d, bs)
+        for bad in (-1, 10 ** 6):
+            c["block_tables"][0, 1] = bad
+            got = _run(c, 0.09, hq, hkv, d, bs)
+            _check(got, want, dtype)
+        assert int(c["cu_q"][2] - c["cu_q"][1]) == 0 and got.shape[0] == 68 + 70
+
+
+def test_attention_module_uses_the_paged_prefill_when_block_tables_are_set():
+    """Store the new tokens, then prefill over (cached prefix + new tokens) through ``Attention.forward``, as the
+    engine does on a prefix-cache hit."""
+    hq, hkv, d, bs = 16, 8, 128, 16
+    lengths, cached = [120, 50], [64, 16]
+    c = make_paged_prefill_case(65, lengths, cached, hq, hkv, d, bs, dtype=torch.bfloat16, poison=0.0)
+    att = Attention(hq, d, 1.0, hkv, bs)
+    kc, vc = c["k_cache"].clone(), c["v_cache"].clone()
+    slots = torch.cat([torch.tensor([int(c["block_tables"][s, j // bs]) * bs + j % bs
+                                     for j in range(cached[s], lengths[s])]) for s in range(2)])
+    kc.view(-1, hkv, d)[slots] = 0                                  # the new tokens are not in the cache yet
+    vc.view(-1, hkv, d)[slots] = 0
+    att.k_cache, att.v_cache = kc.to(DEV), vc.to(DEV)
+    k_new, v_new = c["k"][c["new_rows"]], c["v"][c["new_rows"]]
+    set_context(True, c["cu_q"].to(DEV), c["cu_k"].to(DEV), 64, 128, slots.to(DEV), None, c["block_tables"].to(DEV))
+    try:
+        out = att(c["q_new"].to(DEV), k_new.to(DEV), v_new.to(DEV)).cpu()
+    finally:
+        reset_context()
+    want = _oracle32(c, 1 / math.sqrt(d), hq, hkv, d, bs).reshape(out.shape[0], -1)
+    mx, mean = error_stats(out, want)
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16

@@ -391,3 +391,33 @@ def test_fused_chain_oracle_is_the_composition():
     # no gamma: rotation only
     q2, _ = oracle.qk_norm_rope_store_oracle(q, k, v, pos, table, None, 1e-6)
     assert torch.equal(q2, oracle.rope_oracle(q, pos, table))
+
+
+# ---------------------------------------------------------------------------
+# prefill after a cached prefix (metadata of model_runner.py:192-226)
+# ---------------------------------------------------------------------------
+def test_prefill_paged_oracle_is_the_tail_of_a_full_prefill():
+    from helpers import make_paged_prefill_case
+    hq, hkv, d, bs = 4, 2, 16, 8
+    lengths, cached = [37, 8, 50, 19], [16, 0, 49, 8]
+    c = make_paged_prefill_case(31, lengths, cached, hq, hkv, d, bs)
+    scale = 1.0 / math.sqrt(d)
+    full = oracle.prefill_standard_oracle(c["q"], c["k"], c["v"], c["cu_k"], scale, hq, hkv, d)
+    got = oracle.prefill_paged_oracle(c["q_new"], c["k_cache"], c["v_cache"], c["block_tables"], c["cu_q"],
+                                      c["cu_k"], scale, hq, hkv, d, bs)
+    assert torch.allclose(got, full[c["new_rows"]], atol=1e-5)
+    # no cached prefix anywhere: it is the plain prefill
+    c0 = make_paged_prefill_case(32, lengths, [0] * 4, hq, hkv, d, bs)
+    got0 = oracle.prefill_paged_oracle(c0["q_new"], c0["k_cache"], c0["v_cache"], c0["block_tables"], c0["cu_q"],
+                                       c0["cu_k"], scale, hq, hkv, d, bs)
+    want0 = oracle.prefill_standard_oracle(c0["q"], c0["k"], c0["v"], c0["cu_k"], scale, hq, hkv, d)
+    assert torch.allclose(got0, want0, atol=1e-5)
+    # exactly one new token per sequence: it is a decode step over the same cache
+    c1 = make_paged_prefill_case(33, lengths, [n - 1 for n in lengths], hq, hkv, d, bs)
+    got1 = oracle.prefill_paged_oracle(c1["q_new"], c1["k_cache"], c1["v_cache"], c1["block_tables"], c1["cu_q"],
+                                       c1["cu_k"], scale, hq, hkv, d, bs)
+    kc = torch.nan_to_num(c1["k_cache"], nan=0.0)      # the decode oracle pads with whole blocks
+    vc = torch.nan_to_num(c1["v_cache"], nan=0.0)
+    dec = oracle.decode_naive_oracle(c1["q_new"], kc, vc, c1["block_tables"], torch.tensor(lengths), scale,
+                                     hq, hkv, d, bs)
+    assert torch.allclose(got1, dec, atol=1e-5)
