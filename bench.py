@@ -175,6 +175,34 @@ def bench_prefill_store(args, which):
             "tflops": flops / (event_ms * 1e-3) / 1e12,
             "frac_of_bf16_mfma_peak": flops / (event_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         }
+    if "prefill" in which:
+        # the same prompts with the first half (whole 16-token blocks) already cached: only the second half is
+        # computed, every key comes from a block-16 paged cache
+        from minivllm_amd.layers.attention import flash_attention_prefill_paged
+        pbs = 16
+        cached = [(n // 2) // pbs * pbs for n in lengths]
+        slots16, tables16, nb16 = make_slot_mapping(args.seed + 3, lengths, pbs)
+        kc16 = torch.zeros(nb16, pbs, hkv, d, dtype=torch.bfloat16, device=dev)
+        vc16 = torch.zeros_like(kc16)
+        store_kvcache(k, v, kc16, vc16, slots16.to(dev), pbs)
+        width = max(len(t) for t in tables16)
+        bt = torch.tensor([t + [-1] * (width - len(t)) for t in tables16], dtype=torch.int32, device=dev)
+        rows = torch.cat([torch.arange(int(cu[i]) + c, int(cu[i + 1])) for i, c in enumerate(cached)]).to(dev)
+        q_new = q[rows].contiguous()
+        cu_q = torch.zeros(17, dtype=torch.int32)
+        cu_q[1:] = torch.tensor([n - c for n, c in zip(lengths, cached)]).cumsum(0)
+        cu_q = cu_q.to(dev)
+        scale = 1.0 / math.sqrt(d)
+        _, event_ms = time_steps(lambda: flash_attention_prefill_paged(q_new, kc16, vc16, bt, cu_q, cu, scale, hq, hkv,
+                                                                       d, pbs),
+                                 max(3, args.steps // 3), max(1, args.warmup // 2))
+        flops = 4 * hq * d * sum((n - c) * c + (n - c) * (n - c + 1) // 2 for n, c in zip(lengths, cached))
+        out["prefill_cached_prefix"] = {
+            "workload": "same prompts, first half of each (whole blocks) cached: paged prefill of the rest, block_size 16",
+            "new_tokens": int(cu_q[-1]), "algorithmic_flops": flops, "event_ms_per_step": event_ms,
+            "tflops": flops / (event_ms * 1e-3) / 1e12,
+            "frac_of_bf16_mfma_peak": flops / (event_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        }
     if "store" in which:
         slots, _, nb = make_slot_mapping(args.seed + 2, lengths, bs)
         kc = torch.zeros(nb, bs, hkv, d, dtype=torch.bfloat16, device=dev)
