@@ -191,6 +191,23 @@ int mvllm_qk_norm_rope_store(void* q_out, void* k_out, void* v_out,
                              int64_t num_tokens, int64_t num_slots,
                              int num_heads, int num_kv_heads, int head_dim, int dtype, void* stream);
 
+/*
+ * SamplerLayer.forward -- src/myvllm/layers/sampler.py:14-19:
+ *   logits /= temperature; probs = softmax(logits); token = argmax(probs / exponential_(1).clamp_min_(1e-10))
+ * One launch, no (batch, vocab) probability tensor: out_ids[b] = argmax_i( logits[b,i] / temperatures[b]
+ * - log(max(E[b,i], 1e-10)) ), which is the same argmax (softmax only rescales a row by a positive factor).
+ * Ties go to the smallest index.
+ *   logits        [batch, vocab] in dtype, row_stride elements between rows (the LM-head GEMM output as it lies)
+ *   temperatures  fp32 [batch], > 0
+ *   noise         fp32 [batch, vocab] of Exp(1) draws, or NULL: then E comes from Philox4x32-10 with key = seed
+ *                 and counter = (i / 4, b, offset): lane (i % 4) of the output word gives u = ((x >> 8) + 0.5) * 2^-24
+ *                 and E = -log(u).  Advance `offset` by one per call for independent draws.
+ *   out_ids       int64 [batch]
+ */
+int mvllm_sample_tokens(int64_t* out_ids, const void* logits, int64_t row_stride,
+                        const float* temperatures, const float* noise,
+                        uint64_t seed, uint64_t offset, int batch, int vocab, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

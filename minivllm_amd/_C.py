@@ -17,6 +17,7 @@ DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 
 c_void_p, c_int, c_int64, c_size_t, c_float = (ctypes.c_void_p, ctypes.c_int, ctypes.c_int64,
                                                 ctypes.c_size_t, ctypes.c_float)
+c_uint64 = ctypes.c_uint64
 
 # name -> (restype, argtypes); mirrors include/minivllm_amd.h one to one
 SIGNATURES = {
@@ -34,6 +35,8 @@ SIGNATURES = {
                                                        c_void_p]),
     "mvllm_prefill_paged": (c_int, [c_void_p] * 5 + [c_int, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int,
                                                       c_int, c_int64, c_float, c_int, c_void_p]),
+    "mvllm_sample_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_uint64, c_uint64, c_int, c_int,
+                                    c_int, c_void_p]),
     "mvllm_qk_norm_rope_store": (c_int, [c_void_p] * 6 + [c_int64] * 3 + [c_void_p, c_float, c_void_p, c_int64,
                                                            c_void_p, c_void_p] + [c_void_p] * 4 +
                                  [c_int, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p]),

@@ -1,0 +1,144 @@
+// mvllm_sample_tokens: the reference's SamplerLayer.forward (src/myvllm/layers/sampler.py:14-19) in one launch
+// and without materialising a (batch, vocab) fp32 probability tensor:
+//   logits /= temperature;  probs = softmax(logits);  token = argmax(probs / max(Exp(1) noise, 1e-10))
+// softmax is a positive per-row rescaling of exp(logit / T), so the argmax is taken directly over
+//   logit / T - log(max(noise, 1e-10))
+// (the exponential race / Gumbel-max form of one draw from the tempered distribution).
+// The noise is either read from a caller tensor (what the reference's exponential_ call would have produced:
+// used by the parity tests) or generated in the kernel with Philox4x32-10, keyed by (seed) and counted by
+// (element group, row, call offset), so a (seed, offset) pair always yields the same tokens.
+#include "common.h"
+
+namespace mvllm {
+
+__device__ __forceinline__ uint4 philox4x32_10(uint4 c, uint2 k) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c.x), lo0 = 0xD2511F53u * c.x;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c.z), lo1 = 0xCD9E8D57u * c.z;
+    c = make_uint4(hi1 ^ c.y ^ k.x, lo1, hi0 ^ c.w ^ k.y, lo0);
+    k.x += 0x9E3779B9u;
+    k.y += 0xBB67AE85u;
+  }
+  return c;
+}
+
+// 32 random bits -> uniform in (0, 1): the 24 high bits plus one half, times 2^-24
+__device__ __forceinline__ float uniform_open(uint32_t x) { return ((float)(x >> 8) + 0.5f) * 5.9604644775390625e-08f; }
+
+// four consecutive logits as fp32 (one vector load when `vec`), -inf past the end of the row
+template <typename T16> __device__ __forceinline__ void load4(const T16* p, bool vec, int n, float (&x)[4]) {
+  if (vec) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    x[0] = lo_to_float<T16>(w.x); x[1] = hi_to_float<T16>(w.x);
+    x[2] = lo_to_float<T16>(w.y); x[3] = hi_to_float<T16>(w.y);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[e] = e < n ? to_float(p[e]) : -INFINITY;
+  }
+}
+template <> __device__ __forceinline__ void load4<float>(const float* p, bool vec, int n, float (&x)[4]) {
+  if (vec) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[e] = e < n ? p[e] : -INFINITY;
+  }
+}
+
+constexpr int kSampleThreads = 1024;
+
+// better = larger score, ties to the smaller index (first occurrence)
+__device__ __forceinline__ void keep_best(float& s, int& i, float s2, int i2) {
+  if (s2 > s || (s2 == s && i2 < i)) {
+    s = s2;
+    i = i2;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kSampleThreads) void sample_tokens_kernel(
+    int64_t* __restrict__ out, const T* __restrict__ logits, int64_t row_stride, const float* __restrict__ temperatures,
+    const float* __restrict__ noise, uint32_t seed_lo, uint32_t seed_hi, uint32_t off_lo, uint32_t off_hi, int vocab) {
+  __shared__ float best_s[kSampleThreads / 64];
+  __shared__ int best_i[kSampleThreads / 64];
+  const int b = blockIdx.x;
+  const T* row = logits + (int64_t)b * row_stride;
+  const float inv_t = 1.0f / temperatures[b];
+  // whole groups of four can be loaded as one vector when the row starts on a vector boundary
+  const bool row_vec = ((reinterpret_cast<uintptr_t>(row) & (4 * sizeof(T) - 1)) == 0);
+  float s = -INFINITY;
+  int idx = 0x7fffffff;
+  const int groups = (vocab + 3) >> 2;
+  for (int gi = threadIdx.x; gi < groups; gi += kSampleThreads) {
+    const int i0 = 4 * gi;
+    const int n = min(4, vocab - i0);
+    float x[4], e[4];
+    load4<T>(row + i0, row_vec && n == 4, n, x);
+    if (noise) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) e[k] = k < n ? noise[(int64_t)b * vocab + i0 + k] : 1.0f;
+    } else {
+      const uint4 r = philox4x32_10(make_uint4((uint32_t)gi, (uint32_t)b, off_lo, off_hi), make_uint2(seed_lo, seed_hi));
+      e[0] = -__logf(uniform_open(r.x));
+      e[1] = -__logf(uniform_open(r.y));
+      e[2] = -__logf(uniform_open(r.z));
+      e[3] = -__logf(uniform_open(r.w));
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float score = x[k] * inv_t - __logf(fmaxf(e[k], 1e-10f));
+      if (k < n) keep_best(s, idx, score, i0 + k);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float s2 = __shfl_xor(s, o, 64);
+    const int i2 = __shfl_xor(idx, o, 64);
+    keep_best(s, idx, s2, i2);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    best_s[wave] = s;
+    best_i[wave] = idx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kSampleThreads / 64; ++w) keep_best(s, idx, best_s[w], best_i[w]);
+    out[b] = idx == 0x7fffffff ? 0 : idx;        // a row of NaNs: token 0
+  }
+}
+
+}  // namespace mvllm
+
+using namespace mvllm;
+
+extern "C" int mvllm_sample_tokens(int64_t* out_ids, const void* logits, int64_t row_stride,
+                                   const float* temperatures, const float* noise, uint64_t seed, uint64_t offset,
+                                   int batch, int vocab, int dtype, void* stream) {
+  const int esize = dtype_size(dtype);
+  if (esize == 0) return MVLLM_ERR_BAD_DTYPE;
+  if (batch < 0 || vocab <= 0 || row_stride < vocab) return MVLLM_ERR_BAD_SHAPE;
+  if (batch == 0) return MVLLM_OK;
+  if (!out_ids || !logits || !temperatures) return MVLLM_ERR_NULL_POINTER;
+  if ((reinterpret_cast<uintptr_t>(logits) & (uintptr_t)(esize - 1)) != 0) return MVLLM_ERR_MISALIGNED;
+  hipStream_t s = (hipStream_t)stream;
+  const uint32_t sl = (uint32_t)seed, sh = (uint32_t)(seed >> 32), ol = (uint32_t)offset, oh = (uint32_t)(offset >> 32);
+  const dim3 grid((unsigned)batch), block(kSampleThreads);
+  switch (dtype) {
+    case MVLLM_F32:
+      sample_tokens_kernel<float><<<grid, block, 0, s>>>(out_ids, (const float*)logits, row_stride, temperatures, noise, sl,
+                                                        sh, ol, oh, vocab);
+      break;
+    case MVLLM_BF16:
+      sample_tokens_kernel<bf16_t><<<grid, block, 0, s>>>(out_ids, (const bf16_t*)logits, row_stride, temperatures, noise,
+                                                         sl, sh, ol, oh, vocab);
+      break;
+    default:
+      sample_tokens_kernel<f16_t><<<grid, block, 0, s>>>(out_ids, (const f16_t*)logits, row_stride, temperatures, noise, sl,
+                                                        sh, ol, oh, vocab);
+      break;
+  }
+  return launch_status();
+}

@@ -13,6 +13,7 @@ import torch
 
 from minivllm_amd.engine.metadata import decode_metadata, prefill_metadata
 from minivllm_amd.layers.basic import Sampler
+from minivllm_amd.layers.fused import sample_tokens
 from minivllm_amd.models.qwen3 import Qwen3ForCausalLM
 from minivllm_amd.utils.context import reset_context, set_context
 
@@ -41,6 +42,9 @@ class ModelRunner:
         self.model.reset_parameters(seed=config.get("seed", 0))
         self.model.to(device=self.device, dtype=self.dtype).eval()
         self.sampler = Sampler()
+        self.fused_sampler = config.get("fused_sampler", True)
+        self.seed = config.get("seed", 0)
+        self.sample_calls = 0
         self.generator = torch.Generator(device=self.device).manual_seed(config.get("seed", 0))
         self.allocate_kv_cache()
         self.graphs = {}
@@ -163,6 +167,11 @@ class ModelRunner:
         else:
             hidden = self.model(input_ids, positions)
         logits = self.model.compute_logits(hidden)
-        token_ids = self.sampler(logits, temperatures, self.generator).tolist()
+        if self.fused_sampler:
+            # one launch over the LM-head output; draws are a function of (seed, step), so a run is reproducible
+            token_ids = sample_tokens(logits, temperatures, self.seed, self.sample_calls).tolist()
+            self.sample_calls += 1
+        else:
+            token_ids = self.sampler(logits, temperatures, self.generator).tolist()
         reset_context()
         return token_ids

@@ -6,6 +6,9 @@ three modules per layer and step (src/myvllm/models/qwen3.py:104-110): the share
 ``store_kvcache`` of the rotated k and of v (layers/attention.py:67-108).  It reads q, k and v as the three
 column slices of the packed QKV projection output (no copies) and calls libminivllm_amd.so on the current
 torch stream; there is no PyTorch fallback.
+
+``sample_tokens`` is the reference's ``SamplerLayer.forward`` (layers/sampler.py:14-19) as one launch over the
+LM-head output, with the Exp(1) noise drawn inside the kernel (Philox4x32-10) or passed in.
 """
 from __future__ import annotations
 
@@ -13,7 +16,7 @@ import torch
 
 from minivllm_amd import _C
 
-__all__ = ["qk_norm_rope_store"]
+__all__ = ["qk_norm_rope_store", "sample_tokens"]
 
 
 def _ptr(t):
@@ -109,3 +112,38 @@ def qk_norm_rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positi
         _C.dtype_code(q.dtype), _C.current_stream_ptr(q.device))
     _C.check(st, "qk_norm_rope_store")
     return q_out, k_out, v_out
+
+
+def sample_tokens(logits: torch.Tensor, temperatures: torch.Tensor, seed: int = 0, offset: int = 0,
+                  noise: torch.Tensor | None = None) -> torch.Tensor:
+    """One token per row from softmax(logits / temperature): argmax of ``probs / Exp(1) noise`` as in
+    sampler.py:15-18, computed as argmax(logits / T - log(noise)) without a probability tensor.
+
+    logits: (batch, vocab) float32 / bfloat16 / float16, rows may be strided; temperatures float32 (batch,), > 0.
+    ``noise`` float32 (batch, vocab) supplies the draws (clamped below at 1e-10); without it they are generated
+    from (seed, offset): the same pair always gives the same tokens, advance ``offset`` per call.
+    Returns int64 (batch,).
+    """
+    _C.require_cuda(logits, temperatures, noise)
+    if logits.dim() != 2:
+        raise ValueError(f"logits must be (batch, vocab), got {tuple(logits.shape)}")
+    batch, vocab = logits.shape
+    if batch > 1 and logits.stride(1) != 1 or batch == 1 and vocab > 1 and logits.stride(1) != 1:
+        logits = logits.contiguous()
+    if temperatures.numel() != batch:
+        raise ValueError("temperatures must have one entry per row")
+    temperatures = temperatures.to(torch.float32).contiguous()
+    if noise is not None:
+        if tuple(noise.shape) != (batch, vocab) or noise.dtype != torch.float32:
+            raise ValueError(f"noise must be float32 ({batch}, {vocab})")
+        noise = noise.contiguous()
+    out = torch.empty(batch, dtype=torch.int64, device=logits.device)
+    if batch == 0:
+        return out
+    lib = _C.load()
+    st = lib.mvllm_sample_tokens(_ptr(out), _ptr(logits), logits.stride(0) if batch > 1 else vocab,
+                                 _ptr(temperatures), _ptr(noise), int(seed) & (2 ** 64 - 1),
+                                 int(offset) & (2 ** 64 - 1), batch, vocab, _C.dtype_code(logits.dtype),
+                                 _C.current_stream_ptr(logits.device))
+    _C.check(st, "sample_tokens")
+    return out

@@ -24,3 +24,8 @@ from .producers_oracle import (  # noqa: F401
     prefill_metadata_oracle,
     decode_metadata_oracle,
 )
+from .sampler_oracle import (  # noqa: F401
+    philox4x32_10_oracle,
+    exponential_noise_oracle,
+    sampler_oracle,
+)

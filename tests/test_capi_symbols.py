@@ -28,7 +28,7 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_prefill_varlen",
-              "mvllm_prefill_paged", "mvllm_qk_norm_rope_store", "mvllm_version", "mvllm_status_string"]:
+              "mvllm_prefill_paged", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_version", "mvllm_status_string"]:
         assert n in names
 
 
@@ -69,6 +69,11 @@ def test_argument_validation_without_gpu():
     assert paged(0, 0, 0, 0, 0, 4, 0, 0, 1, 5, 4, 2, 128, 16, 8, 1.0, 1, 0) == -1      # null pointers
     assert paged(0, 0, 0, 0, 0, 4, 0, 0, 1, 5, 4, 3, 128, 16, 8, 1.0, 1, 0) == -3      # Hq % Hkv
     assert paged(0, 0, 0, 0, 0, 4, 0, 0, 1, 5, 4, 2, 128, 0, 8, 1.0, 1, 0) == -3       # block_size
+    sample = lib.mvllm_sample_tokens
+    assert sample(0, 0, 100, 0, 0, 1, 2, 0, 100, 1, 0) == 0        # empty batch
+    assert sample(0, 0, 100, 0, 0, 1, 2, 4, 100, 1, 0) == -1       # null pointers
+    assert sample(0, 0, 50, 0, 0, 1, 2, 4, 100, 1, 0) == -3        # row stride < vocab
+    assert sample(0, 0, 100, 0, 0, 1, 2, 4, 100, 5, 0) == -2       # dtype
     fused = lib.mvllm_qk_norm_rope_store
     #     q_out k_out v_out q k v | strides | gamma eps cos max_pos pos slots | caches scales int8 | T slots Hq Hkv D dt stream
     assert fused(0, 0, 0, 0, 0, 0, 512, 256, 256, 0, 1e-6, 0, 64, 0, 0, 0, 0, 0, 0, 0, 0, 0, 4, 2, 128, 1, 0) == 0   # no tokens

@@ -421,3 +421,49 @@ def test_prefill_paged_oracle_is_the_tail_of_a_full_prefill():
     dec = oracle.decode_naive_oracle(c1["q_new"], kc, vc, c1["block_tables"], torch.tensor(lengths), scale,
                                      hq, hkv, d, bs)
     assert torch.allclose(got1, dec, atol=1e-5)
+
+
+# ---------------------------------------------------------------------------
+# sampler (sampler.py:14-19) and the counter-based noise of the HIP sampler
+# ---------------------------------------------------------------------------
+def test_philox_known_answer_vectors():
+    """Philox4x32-10 vectors published with the Random123 library (kat_vectors)."""
+    import numpy as np
+    kat = [
+        ([0, 0, 0, 0], (0, 0), "6627e8d5 e169c58d bc57ac4c 9b00dbd8"),
+        ([0xffffffff] * 4, (0xffffffff, 0xffffffff), "408f276d 41c83b0e a20bc7c6 6d5451fd"),
+        ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], (0xa4093822, 0x299f31d0),
+         "d16cfe09 94fdcceb 5001e420 24126ea1"),
+    ]
+    for ctr, key, want in kat:
+        got = oracle.philox4x32_10_oracle(np.array([ctr], dtype=np.uint32), key)[0]
+        assert " ".join("%08x" % int(x) for x in got) == want
+
+
+def test_exponential_noise_is_exponential_and_counter_addressed():
+    e = oracle.exponential_noise_oracle(seed=7, offset=3, batch=4, vocab=50001)
+    assert e.shape == (4, 50001) and e.dtype == torch.float32
+    assert float(e.min()) > 0 and float(e.max()) < 17.4               # u in (2^-25, 1 - 2^-25)
+    assert abs(float(e.mean()) - 1.0) < 0.01 and abs(float(e.var()) - 1.0) < 0.03
+    assert abs(float((e > 1.0).float().mean()) - math.exp(-1.0)) < 0.005
+    # rows, offsets and seeds address different streams; the same address repeats
+    assert not torch.equal(e[0], e[1])
+    assert torch.equal(e, oracle.exponential_noise_oracle(7, 3, 4, 50001))
+    assert not torch.equal(e, oracle.exponential_noise_oracle(7, 4, 4, 50001))
+    assert not torch.equal(e, oracle.exponential_noise_oracle(8, 3, 4, 50001))
+    # a shorter vocab is a prefix of the same stream
+    assert torch.equal(oracle.exponential_noise_oracle(7, 3, 4, 10)[:, :10], e[:, :10])
+
+
+def test_sampler_oracle_draws_from_the_tempered_softmax():
+    g = torch.Generator().manual_seed(4)
+    logits = torch.tensor([[2.0, 0.5, -1.0, 1.0, 0.0]]).repeat(40000, 1)
+    temps = torch.full((40000,), 0.7)
+    noise = torch.empty(40000, 5).exponential_(1.0, generator=g)
+    ids = oracle.sampler_oracle(logits, temps, noise)
+    freq = torch.bincount(ids, minlength=5).float() / 40000
+    want = torch.softmax(logits[0] / 0.7, dim=-1)
+    assert float((freq - want).abs().max()) < 0.01
+    # the clamp: a zero draw does not divide by zero, it wins
+    z = torch.ones(1, 5); z[0, 2] = 0.0
+    assert int(oracle.sampler_oracle(logits[:1], temps[:1], z)) == 2
