@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,fused_qk,engine,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,fused_qk,sampler,engine,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -317,6 +317,26 @@ def bench_fused_qk(args):
     }
 
 
+def bench_sampler(args):
+    """One sampling step of config 5's decode batch: 64 rows of bf16 logits over the 151 936-token vocabulary,
+    as one HIP launch against the module chain (fp32 softmax, exponential_, divide, argmax)."""
+    import torch
+    from minivllm_amd.layers.basic import Sampler
+    from minivllm_amd.layers.fused import sample_tokens
+
+    dev = "cuda:0"
+    batch, vocab = 64, 151936
+    dg = torch.Generator(device=dev).manual_seed(args.seed)
+    logits = (torch.randn(batch, vocab, generator=dg, device=dev) * 2).to(torch.bfloat16)
+    temps = torch.full((batch,), 0.6, device=dev)
+    sampler = Sampler()
+    _, fused_ms = time_steps(lambda: sample_tokens(logits, temps, 0, 0), args.steps, args.warmup)
+    _, modules_ms = time_steps(lambda: sampler(logits, temps, dg), max(3, args.steps // 3), max(1, args.warmup // 2))
+    nbytes = batch * vocab * 2 + batch * 12
+    return {"workload": "sampler: 64 x 151936 bf16 logits, T 0.6", "algorithmic_bytes": nbytes,
+            "event_ms_per_step": fused_ms, "gbs": nbytes / (fused_ms * 1e-3) / 1e9, "unfused_modules_event_ms": modules_ms}
+
+
 def bench_engine(args, max_num_sequences, graph):
     """BASELINE config 5: random-init Qwen3-style decoder (hidden 1024, 8 layers, Hq16/Hkv8/D128, FFN 3072,
     vocab 151936, bf16), 60 prompts of random ids with lengths U[32,96], 256 new tokens each, T 0.6."""
@@ -386,6 +406,8 @@ def main():
         extra["int8"] = bench_int8(args)
     if want("fused_qk"):
         extra["fused_qk"] = bench_fused_qk(args)
+    if want("sampler"):
+        extra["sampler"] = bench_sampler(args)
     if want("engine"):
         extra["engine_16seq_eager"] = bench_engine(args, 16, False)
         extra["engine_16seq_graph"] = bench_engine(args, 16, True)

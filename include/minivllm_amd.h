@@ -208,6 +208,26 @@ int mvllm_sample_tokens(int64_t* out_ids, const void* logits, int64_t row_stride
                         const float* temperatures, const float* noise,
                         uint64_t seed, uint64_t offset, int batch, int vocab, int dtype, void* stream);
 
+/*
+ * LayerNorm.forward with and without residual -- src/myvllm/layers/layernorm.py:9-28, called from
+ * Qwen3DecoderLayer.forward and the final norm (src/myvllm/models/qwen3.py:197-212, 306-312):
+ *   x = x + residual (rounded to the element type);  out = x / sqrt(mean(x^2) + eps) * gamma;  residual_out = x
+ * x [rows, hidden] with x_row_stride elements between rows; residual likewise or NULL (no add);
+ * residual_out [rows, hidden] dense or NULL; out [rows, hidden] dense; gamma fp32 [hidden].
+ * hidden % 8 == 0, hidden <= 8192, 16-byte aligned pointers, strides % 8 == 0.
+ */
+int mvllm_add_rms_norm(void* out, void* residual_out, const void* x, const void* residual,
+                       const float* gamma, float eps, int64_t rows, int hidden,
+                       int64_t x_row_stride, int64_t residual_row_stride, int dtype, void* stream);
+
+/*
+ * SiluAndMul.forward -- src/myvllm/layers/activation.py:15-18:  x, y = in.chunk(2, -1); out = silu(x) * y
+ * in [rows, 2*width] with in_row_stride elements between rows; out [rows, width] dense.  silu(x) is rounded to
+ * the element type before the product, as the two tensor operations would.  width a multiple of 16 bytes.
+ */
+int mvllm_silu_and_mul(void* out, const void* in, int64_t rows, int width, int64_t in_row_stride,
+                       int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

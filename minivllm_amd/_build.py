@@ -14,7 +14,8 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libminivllm_amd.so")
-SOURCES = ["capi.hip", "store_kvcache.hip", "paged_decode.hip", "prefill_varlen.hip", "qk_norm_rope_store.hip", "sampler.hip"]
+SOURCES = ["capi.hip", "store_kvcache.hip", "paged_decode.hip", "prefill_varlen.hip", "qk_norm_rope_store.hip", "sampler.hip",
+           "rms_norm.hip", "activation.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

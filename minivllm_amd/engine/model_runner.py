@@ -38,7 +38,7 @@ class ModelRunner:
             intermediate_size=config["intermediate_size"], ffn_bias=config.get("ffn_bias", True),
             num_layers=config["num_layers"], tie_word_embeddings=config.get("tie_word_embeddings", True),
             block_size=self.block_size, kv_cache_dtype=self.kv_cache_dtype,
-            fused_qk=config.get("fused_qk", True))
+            fused_qk=config.get("fused_qk", True), fused_elementwise=config.get("fused_elementwise", True))
         self.model.reset_parameters(seed=config.get("seed", 0))
         self.model.to(device=self.device, dtype=self.dtype).eval()
         self.sampler = Sampler()

@@ -1,5 +1,5 @@
-"""Plain PyTorch-ROCm counterparts of the reference's small layers (callers of the attention path,
-not kernel targets): RMSNorm with fused residual (layers/layernorm.py:9-28), NeoX half-split RoPE
+"""Counterparts of the reference's small layers around the attention path, as chains of PyTorch-ROCm tensor
+operations and, with ``fused=True``, as single HIP launches (minivllm_amd.layers.fused): RMSNorm with fused residual (layers/layernorm.py:9-28), NeoX half-split RoPE
 (layers/rotary_embedding.py:4-83), SiluAndMul (layers/activation.py:15-18) and the temperature /
 exponential-race sampler (layers/sampler.py:14-19)."""
 from __future__ import annotations
@@ -8,19 +8,35 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from minivllm_amd.layers.fused import add_rms_norm, silu_and_mul
+
 
 class RMSNorm(nn.Module):
-    def __init__(self, size: int, eps: float = 1e-6):
+    """x / sqrt(mean(x^2) + eps) * weight over the last dim, optionally after adding a residual
+    (layers/layernorm.py:9-28).  ``fused=True`` runs it as one HIP launch (``add_rms_norm``), otherwise as the
+    chain of tensor operations; both round where the chain rounds."""
+
+    def __init__(self, size: int, eps: float = 1e-6, fused: bool = False):
         super().__init__()
         self.weight = nn.Parameter(torch.ones(size))
         self.eps = eps
+        self.fused = fused
+        self._w32 = None
+
+    def weight_fp32(self):
+        """float32 copy of the weight for the HIP kernels (made once; weights do not change while serving)."""
+        if self._w32 is None or self._w32.device != self.weight.device:
+            self._w32 = self.weight.detach().float().contiguous()
+        return self._w32
 
     def _norm(self, x):
         xf = x.float()
-        xf = xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + self.eps)
+        xf = xf / torch.sqrt(xf.pow(2).mean(dim=-1, keepdim=True) + self.eps)
         return (xf * self.weight.float()).to(x.dtype)
 
     def forward(self, x, residual=None):
+        if self.fused and x.dim() == 2:
+            return add_rms_norm(x, self.weight_fp32(), self.eps, residual)
         if residual is None:
             return self._norm(x)
         x = x + residual
@@ -57,7 +73,13 @@ class RotaryEmbedding(nn.Module):
 
 
 class SiluAndMul(nn.Module):
+    def __init__(self, fused: bool = False):
+        super().__init__()
+        self.fused = fused
+
     def forward(self, x):
+        if self.fused and x.dim() == 2:
+            return silu_and_mul(x)
         a, b = x.chunk(2, dim=-1)
         return F.silu(a) * b
 

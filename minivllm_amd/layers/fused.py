@@ -16,7 +16,7 @@ import torch
 
 from minivllm_amd import _C
 
-__all__ = ["qk_norm_rope_store", "sample_tokens"]
+__all__ = ["qk_norm_rope_store", "sample_tokens", "add_rms_norm", "silu_and_mul"]
 
 
 def _ptr(t):
@@ -146,4 +146,56 @@ def sample_tokens(logits: torch.Tensor, temperatures: torch.Tensor, seed: int = 
                                  int(offset) & (2 ** 64 - 1), batch, vocab, _C.dtype_code(logits.dtype),
                                  _C.current_stream_ptr(logits.device))
     _C.check(st, "sample_tokens")
+    return out
+
+
+def _rows2d(name, t):
+    if t.dim() != 2:
+        raise ValueError(f"{name} must be (rows, features), got {tuple(t.shape)}")
+    if t.shape[0] > 1 and t.stride(1) != 1 or t.shape[0] == 1 and t.shape[1] > 1 and t.stride(1) != 1:
+        t = t.contiguous()
+    return t, (t.stride(0) if t.shape[0] > 1 else t.shape[1])
+
+
+def add_rms_norm(x: torch.Tensor, gamma: torch.Tensor, eps: float, residual: torch.Tensor | None = None):
+    """``LayerNorm.forward`` (layers/layernorm.py:9-28) in one launch.
+
+    Without ``residual``: returns ``x / sqrt(mean(x^2) + eps) * gamma``.  With it: returns
+    ``(norm(x + residual), x + residual)``, the sum rounded to x's dtype first.  x, residual: (rows, hidden),
+    rows may be strided; gamma float32 (hidden,).
+    """
+    _C.require_cuda(x, gamma, residual)
+    x, x_stride = _rows2d("x", x)
+    rows, hidden = x.shape
+    if gamma.dtype != torch.float32 or gamma.numel() != hidden or not gamma.is_contiguous():
+        raise ValueError(f"gamma must be contiguous float32 ({hidden},)")
+    r_stride = hidden
+    if residual is not None:
+        if residual.shape != x.shape or residual.dtype != x.dtype:
+            raise ValueError("residual must match x in shape and dtype")
+        residual, r_stride = _rows2d("residual", residual)
+    out = torch.empty((rows, hidden), dtype=x.dtype, device=x.device)
+    new_residual = torch.empty_like(out) if residual is not None else None
+    if rows:
+        lib = _C.load()
+        st = lib.mvllm_add_rms_norm(_ptr(out), _ptr(new_residual), _ptr(x), _ptr(residual), _ptr(gamma), float(eps),
+                                    rows, hidden, x_stride, r_stride, _C.dtype_code(x.dtype),
+                                    _C.current_stream_ptr(x.device))
+        _C.check(st, "add_rms_norm")
+    return out if residual is None else (out, new_residual)
+
+
+def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """``SiluAndMul.forward`` (layers/activation.py:15-18): silu(first half) * second half of the last dim."""
+    _C.require_cuda(x)
+    x, stride = _rows2d("x", x)
+    rows, two_w = x.shape
+    if two_w % 2:
+        raise ValueError("the last dimension must be even")
+    out = torch.empty((rows, two_w // 2), dtype=x.dtype, device=x.device)
+    if rows:
+        lib = _C.load()
+        st = lib.mvllm_silu_and_mul(_ptr(out), _ptr(x), rows, two_w // 2, stride, _C.dtype_code(x.dtype),
+                                    _C.current_stream_ptr(x.device))
+        _C.check(st, "silu_and_mul")
     return out

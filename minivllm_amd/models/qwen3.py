@@ -31,14 +31,6 @@ class Qwen3Attention(nn.Module):
         self.attention = Attention(num_heads, head_dim, scale, num_kv_heads, block_size, kv_cache_dtype)
         self.output_projection = nn.Linear(self.q_size, hidden_size, bias=False)
         self.fused_qk = fused_qk
-        self._gamma32 = None
-
-    def _gamma_fp32(self):
-        """float32 copy of the norm weight for the fused kernel (made once; weights do not change while serving)."""
-        w = self.rms_norm.weight
-        if self._gamma32 is None or self._gamma32.device != w.device:
-            self._gamma32 = w.detach().float().contiguous()
-        return self._gamma32
 
     def forward(self, x, positions):
         q, k, v = self.qkv_projection(x).split([self.q_size, self.kv_size, self.kv_size], dim=-1)
@@ -47,7 +39,7 @@ class Qwen3Attention(nn.Module):
             q = q.unflatten(-1, (self.num_heads, self.head_dim))
             k = k.unflatten(-1, (self.num_kv_heads, self.head_dim))
             v = v.unflatten(-1, (self.num_kv_heads, self.head_dim))
-            gamma = None if self.qkv_bias else self._gamma_fp32()
+            gamma = None if self.qkv_bias else self.rms_norm.weight_fp32()
             o = self.attention.forward_fused(q, k, v, positions, self.rotary_emb.cos_sin_cache, gamma,
                                              self.rms_norm.eps)
             return self.output_projection(o)
@@ -61,10 +53,10 @@ class Qwen3Attention(nn.Module):
 
 
 class Qwen3MLP(nn.Module):
-    def __init__(self, hidden_size, intermediate_size, bias):
+    def __init__(self, hidden_size, intermediate_size, bias, fused=True):
         super().__init__()
         self.gate_up = nn.Linear(hidden_size, 2 * intermediate_size, bias=bias)
-        self.activation = SiluAndMul()
+        self.activation = SiluAndMul(fused)
         self.gate_down = nn.Linear(intermediate_size, hidden_size, bias=bias)
 
     def forward(self, x):
@@ -72,12 +64,13 @@ class Qwen3MLP(nn.Module):
 
 
 class Qwen3DecoderLayer(nn.Module):
-    def __init__(self, hidden_size, intermediate_size, ffn_bias, rms_norm_epsilon, **attn_kwargs):
+    def __init__(self, hidden_size, intermediate_size, ffn_bias, rms_norm_epsilon, fused_elementwise=True,
+                 **attn_kwargs):
         super().__init__()
-        self.input_layernorm = RMSNorm(hidden_size, rms_norm_epsilon)
+        self.input_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
         self.self_attn = Qwen3Attention(hidden_size=hidden_size, rms_norm_epsilon=rms_norm_epsilon, **attn_kwargs)
-        self.post_attention_layernorm = RMSNorm(hidden_size, rms_norm_epsilon)
-        self.mlp = Qwen3MLP(hidden_size, intermediate_size, ffn_bias)
+        self.post_attention_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
+        self.mlp = Qwen3MLP(hidden_size, intermediate_size, ffn_bias, fused_elementwise)
 
     def forward(self, x, residual, positions):
         if residual is None:
@@ -94,7 +87,7 @@ class Qwen3ForCausalLM(nn.Module):
     def __init__(self, vocab_size, hidden_size, num_heads, head_dim=None, scale=1.0, num_kv_heads=None,
                  rms_norm_epsilon=1e-6, qkv_bias=False, base=1_000_000, max_position=4096,
                  intermediate_size=3072, ffn_bias=True, num_layers=8, tie_word_embeddings=True,
-                 block_size=256, kv_cache_dtype="auto", fused_qk=True):
+                 block_size=256, kv_cache_dtype="auto", fused_qk=True, fused_elementwise=True):
         super().__init__()
         head_dim = head_dim if head_dim is not None else hidden_size // num_heads
         num_kv_heads = num_kv_heads if num_kv_heads is not None else num_heads
@@ -104,9 +97,9 @@ class Qwen3ForCausalLM(nn.Module):
             Qwen3DecoderLayer(hidden_size, intermediate_size, ffn_bias, rms_norm_epsilon, num_heads=num_heads,
                               head_dim=head_dim, scale=scale, num_kv_heads=num_kv_heads, qkv_bias=qkv_bias,
                               rotary=rotary, block_size=block_size, kv_cache_dtype=kv_cache_dtype,
-                              fused_qk=fused_qk)
+                              fused_qk=fused_qk, fused_elementwise=fused_elementwise)
             for _ in range(num_layers)])
-        self.final_layernorm = RMSNorm(hidden_size, rms_norm_epsilon)
+        self.final_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
         self.lm_head_weight = self.embedding_layer.weight if tie_word_embeddings else nn.Parameter(
             torch.empty(vocab_size, hidden_size))
         self.max_position = max_position

@@ -19,6 +19,8 @@ from .attention_oracle import (  # noqa: F401
     rope_cos_sin_cache_oracle,
     rope_oracle,
     qk_norm_rope_store_oracle,
+    add_rms_norm_oracle,
+    silu_and_mul_oracle,
 )
 from .producers_oracle import (  # noqa: F401
     prefill_metadata_oracle,

@@ -289,3 +289,21 @@ def qk_norm_rope_store_oracle(q, k, v, positions, cos_sin_cache, gamma, eps, slo
         else:
             store_kvcache_oracle(k, v, k_cache, v_cache, slot_mapping, block_size)
     return q, k
+
+
+def add_rms_norm_oracle(x, gamma, eps, residual=None):
+    """LayerNorm.forward (layernorm.py:19-28): with a residual the sum is formed (and rounded) in x's dtype,
+    normalised, and returned next to the sum."""
+    if residual is None:
+        return rms_norm_oracle(x, gamma, eps)
+    s = x + residual
+    return rms_norm_oracle(s, gamma, eps), s
+
+
+def silu_and_mul_oracle(x):
+    """SiluAndMul.forward (activation.py:15-18) as two tensor operations: silu in fp32 rounded to x's dtype,
+    then the product rounded again."""
+    a, b = x.chunk(2, dim=-1)
+    af = a.float()
+    s = (af / (1.0 + torch.exp(-af))).to(x.dtype)
+    return (s.float() * b.float()).to(x.dtype)

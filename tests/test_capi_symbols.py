@@ -28,7 +28,8 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_prefill_varlen",
-              "mvllm_prefill_paged", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_version", "mvllm_status_string"]:
+              "mvllm_prefill_paged", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_add_rms_norm",
+              "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
         assert n in names
 
 
@@ -74,6 +75,16 @@ def test_argument_validation_without_gpu():
     assert sample(0, 0, 100, 0, 0, 1, 2, 4, 100, 1, 0) == -1       # null pointers
     assert sample(0, 0, 50, 0, 0, 1, 2, 4, 100, 1, 0) == -3        # row stride < vocab
     assert sample(0, 0, 100, 0, 0, 1, 2, 4, 100, 5, 0) == -2       # dtype
+    norm = lib.mvllm_add_rms_norm
+    assert norm(0, 0, 0, 0, 0, 1e-6, 0, 1024, 1024, 1024, 1, 0) == 0       # no rows
+    assert norm(0, 0, 0, 0, 0, 1e-6, 4, 1024, 1024, 1024, 1, 0) == -1      # null pointers
+    assert norm(0, 0, 0, 0, 0, 1e-6, 4, 1004, 1004, 1004, 1, 0) == -4      # hidden % 8
+    assert norm(0, 0, 0, 0, 0, 1e-6, 4, 1024, 512, 1024, 1, 0) == -3       # stride < hidden
+    act = lib.mvllm_silu_and_mul
+    assert act(0, 0, 0, 3072, 6144, 1, 0) == 0
+    assert act(0, 0, 2, 3072, 6144, 1, 0) == -1
+    assert act(0, 0, 2, 3072, 3072, 1, 0) == -3                            # stride < 2 * width
+    assert act(0, 0, 2, 3001, 6002, 1, 0) == -4                            # width not a multiple of 16 bytes
     fused = lib.mvllm_qk_norm_rope_store
     #     q_out k_out v_out q k v | strides | gamma eps cos max_pos pos slots | caches scales int8 | T slots Hq Hkv D dt stream
     assert fused(0, 0, 0, 0, 0, 0, 512, 256, 256, 0, 1e-6, 0, 64, 0, 0, 0, 0, 0, 0, 0, 0, 0, 4, 2, 128, 1, 0) == 0   # no tokens

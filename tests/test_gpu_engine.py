@@ -88,16 +88,17 @@ def test_graph_decode_matches_eager_decode():
 
 @pytest.mark.parametrize("kv_cache_dtype", ["auto", "int8"])
 def test_fused_qk_path_matches_unfused_modules(kv_cache_dtype):
-    """One prefill and one decode step through the model with the fused norm + rotary + store launch and
-    with the three separate modules: same hidden states (the fused kernel rounds where the modules round;
+    """Generation with the fused HIP launches (q/k norm + rotary + store, residual RMSNorm, SiLU-and-multiply)
+    and with the separate modules as chains of tensor operations: same hidden states (the fused kernel rounds where the modules round;
     the sum of squares may differ in its last bit) and the same cache contents up to that."""
     cfg = dict(SMALL, kv_cache_dtype=kv_cache_dtype, max_cached_blocks=32)
     prompts = _prompts(4, 5, 50, seed=8)
     sp = SamplingParams(temperature=0.5, max_tokens=6, ignore_eos=True)
     outs, caches = [], []
     for fused in (True, False):
-        eng = LLMEngine(dict(cfg, fused_qk=fused))
-        assert all(l.self_attn.fused_qk == fused for l in eng.model_runner.model.layer_stack)
+        eng = LLMEngine(dict(cfg, fused_qk=fused, fused_elementwise=fused))
+        assert all(l.self_attn.fused_qk == fused and l.input_layernorm.fused == fused and l.mlp.activation.fused == fused
+                   for l in eng.model_runner.model.layer_stack)
         outs.append(eng.generate(prompts, sp)["token_ids"])
         caches.append(eng.model_runner.kv_cache.clone())
     same = sum(a == b for a, b in zip(*outs))

@@ -467,3 +467,25 @@ def test_sampler_oracle_draws_from_the_tempered_softmax():
     # the clamp: a zero draw does not divide by zero, it wins
     z = torch.ones(1, 5); z[0, 2] = 0.0
     assert int(oracle.sampler_oracle(logits[:1], temps[:1], z)) == 2
+
+
+def test_silu_and_add_norm_oracles():
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(5, 32, generator=g) * 3
+    got = oracle.silu_and_mul_oracle(x)
+    assert torch.allclose(got, F.silu(x[:, :16]) * x[:, 16:], atol=1e-6)        # library routine
+    a = x[:, :16]
+    silu = lambda t: oracle.silu_and_mul_oracle(torch.cat([t, torch.ones_like(t)], dim=-1))
+    assert torch.allclose(silu(a) - silu(-a), a, atol=1e-6)                     # x s(x) - (-x) s(-x) = x
+    assert float(silu(torch.zeros(1, 4)).abs().max()) == 0.0
+    assert torch.allclose(silu(torch.full((1, 4), 30.0)), torch.full((1, 4), 30.0))
+    # bf16: the intermediate silu is rounded before the product
+    xb = x.to(torch.bfloat16)
+    two_step = (F.silu(xb[:, :16].float()).to(torch.bfloat16).float() * xb[:, 16:].float()).to(torch.bfloat16)
+    assert torch.equal(oracle.silu_and_mul_oracle(xb), two_step)
+    # residual form = norm of the rounded sum, returned with the sum
+    r = torch.randn(5, 32, generator=g).to(torch.bfloat16)
+    gamma = torch.rand(32, generator=g) + 0.5
+    y, s = oracle.add_rms_norm_oracle(xb, gamma, 1e-6, r)
+    assert torch.equal(s, xb + r) and torch.equal(y, oracle.rms_norm_oracle(xb + r, gamma, 1e-6))
+    assert torch.equal(oracle.add_rms_norm_oracle(xb, gamma, 1e-6), oracle.rms_norm_oracle(xb, gamma, 1e-6))
