@@ -67,12 +67,15 @@ struct DecodeArgs {
 // Partition length.  Lower bound: the smallest multiple of 256 tokens that covers the widest context with
 // kMaxParts partitions.  Longer partitions amortise the per-workgroup start-up better (1024 tokens measured
 // best on MI355X), so the length is doubled up to 1024 while the grid still offers at least four
-// workgroups per CU.
+// workgroups per CU.  A small batch of short contexts is the opposite case: too few (sequence, partition)
+// pairs to occupy 256 CUs, each walking its tokens tile after tile at memory latency; there the length is
+// halved, down to 64 tokens, until there are 256 pairs.
 __host__ __device__ inline int partition_tokens_for(int64_t max_ctx, int batch) {
   const int64_t per_part = (max_ctx + kMaxParts - 1) / kMaxParts;
   int64_t part = (per_part + kMinPartTokens - 1) / kMinPartTokens * kMinPartTokens;
   if (part < kMinPartTokens) part = kMinPartTokens;
   while (part < 1024 && (int64_t)batch * ((max_ctx + 2 * part - 1) / (2 * part)) >= 1024) part *= 2;
+  while (part > 64 && part / 2 >= per_part && (int64_t)batch * ((max_ctx + part - 1) / part) < 256) part /= 2;
   return (int)part;
 }
 
@@ -858,7 +861,11 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stre
   bool launched = false;
   if constexpr (IsSixteenBit<T>::value) {
     if (fast_ok && (!int8 || group <= 4)) {
-      const int wpb = largest_divisor_le(a.num_kv_heads, MVLLM_DECODE_WPB);
+      // kv heads (waves) per workgroup: as many as allowed, so that a workgroup streams whole token rows;
+      // fewer when the grid would otherwise leave most CUs without a workgroup
+      int wpb = largest_divisor_le(a.num_kv_heads, MVLLM_DECODE_WPB);
+      while (wpb > 1 && (int64_t)a.num_parts * a.batch * (a.num_kv_heads / wpb) < 512)
+        wpb = largest_divisor_le(a.num_kv_heads, wpb - 1);
       dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, (unsigned)(a.num_kv_heads / wpb));
       dim3 block(64 * wpb);
       if (int8) decode_mfma_int8_kernel<T, 1><<<grid, block, 0, stream>>>(a);
