@@ -203,10 +203,15 @@ int mvllm_qk_norm_rope_store(void* q_out, void* k_out, void* v_out,
  *                 and counter = (i / 4, b, offset): lane (i % 4) of the output word gives u = ((x >> 8) + 0.5) * 2^-24
  *                 and E = -log(u).  Advance `offset` by one per call for independent draws.
  *   out_ids       int64 [batch]
+ *   workspace     optional scratch of mvllm_sample_tokens_workspace_bytes(batch, vocab) bytes: with it a row is
+ *                 scanned by several workgroups (a small batch alone cannot occupy the GPU) and a second tiny
+ *                 launch picks the winner; NULL or too small: one workgroup per row, same result.
  */
+size_t mvllm_sample_tokens_workspace_bytes(int batch, int vocab);
 int mvllm_sample_tokens(int64_t* out_ids, const void* logits, int64_t row_stride,
                         const float* temperatures, const float* noise,
-                        uint64_t seed, uint64_t offset, int batch, int vocab, int dtype, void* stream);
+                        uint64_t seed, uint64_t offset, int batch, int vocab, int dtype,
+                        void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * LayerNorm.forward with and without residual -- src/myvllm/layers/layernorm.py:9-28, called from

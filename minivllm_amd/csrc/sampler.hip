@@ -14,8 +14,9 @@ namespace mvllm {
 __device__ __forceinline__ uint4 philox4x32_10(uint4 c, uint2 k) {
 #pragma unroll
   for (int r = 0; r < 10; ++r) {
-    const uint32_t hi0 = __umulhi(0xD2511F53u, c.x), lo0 = 0xD2511F53u * c.x;
-    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c.z), lo1 = 0xCD9E8D57u * c.z;
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c.x, p1 = (uint64_t)0xCD9E8D57u * c.z;   // one 32x32->64 multiply each
+    const uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0;
+    const uint32_t hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
     c = make_uint4(hi1 ^ c.y ^ k.x, lo1, hi0 ^ c.w ^ k.y, lo0);
     k.x += 0x9E3779B9u;
     k.y += 0xBB67AE85u;
@@ -57,10 +58,14 @@ __device__ __forceinline__ void keep_best(float& s, int& i, float s2, int i2) {
   }
 }
 
+// One workgroup scans one slice of one row: slices > 1 spreads a row over several workgroups (a small batch
+// would otherwise occupy only `batch` CUs with a kernel that is bound by Philox's integer multiplies); each then
+// leaves its (score, index) in `partial` and sample_combine_kernel picks the winner.
 template <typename T>
 __global__ __launch_bounds__(kSampleThreads) void sample_tokens_kernel(
-    int64_t* __restrict__ out, const T* __restrict__ logits, int64_t row_stride, const float* __restrict__ temperatures,
-    const float* __restrict__ noise, uint32_t seed_lo, uint32_t seed_hi, uint32_t off_lo, uint32_t off_hi, int vocab) {
+    int64_t* __restrict__ out, float2* __restrict__ partial, const T* __restrict__ logits, int64_t row_stride,
+    const float* __restrict__ temperatures, const float* __restrict__ noise, uint32_t seed_lo, uint32_t seed_hi,
+    uint32_t off_lo, uint32_t off_hi, int vocab, int slices) {
   __shared__ float best_s[kSampleThreads / 64];
   __shared__ int best_i[kSampleThreads / 64];
   const int b = blockIdx.x;
@@ -71,7 +76,9 @@ __global__ __launch_bounds__(kSampleThreads) void sample_tokens_kernel(
   float s = -INFINITY;
   int idx = 0x7fffffff;
   const int groups = (vocab + 3) >> 2;
-  for (int gi = threadIdx.x; gi < groups; gi += kSampleThreads) {
+  const int per_slice = (groups + slices - 1) / slices;
+  const int g_end = min(groups, (int)(blockIdx.y + 1) * per_slice);
+  for (int gi = blockIdx.y * per_slice + threadIdx.x; gi < g_end; gi += kSampleThreads) {
     const int i0 = 4 * gi;
     const int n = min(4, vocab - i0);
     float x[4], e[4];
@@ -106,39 +113,77 @@ __global__ __launch_bounds__(kSampleThreads) void sample_tokens_kernel(
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int w = 1; w < kSampleThreads / 64; ++w) keep_best(s, idx, best_s[w], best_i[w]);
-    out[b] = idx == 0x7fffffff ? 0 : idx;        // a row of NaNs: token 0
+    if (slices == 1) out[b] = idx == 0x7fffffff ? 0 : idx;        // a row of NaNs: token 0
+    else partial[(int64_t)b * slices + blockIdx.y] = make_float2(s, __int_as_float(idx));
   }
+}
+
+__global__ __launch_bounds__(64) void sample_combine_kernel(int64_t* __restrict__ out, const float2* __restrict__ partial,
+                                                            int slices) {
+  const int b = blockIdx.x;
+  float s = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = threadIdx.x; i < slices; i += 64) {
+    const float2 p = partial[(int64_t)b * slices + i];
+    keep_best(s, idx, p.x, __float_as_int(p.y));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float s2 = __shfl_xor(s, o, 64);
+    const int i2 = __shfl_xor(idx, o, 64);
+    keep_best(s, idx, s2, i2);
+  }
+  if (threadIdx.x == 0) out[b] = idx == 0x7fffffff ? 0 : idx;
 }
 
 }  // namespace mvllm
 
 using namespace mvllm;
 
+extern "C" size_t mvllm_sample_tokens_workspace_bytes(int batch, int vocab) {
+  if (batch <= 0 || vocab <= 0) return 0;
+  // enough slices for about two workgroups per CU, each with at least 4096 logits
+  int slices = (512 + batch - 1) / batch;
+  const int max_slices = (vocab + 4095) / 4096;
+  if (slices > max_slices) slices = max_slices;
+  return slices <= 1 ? 0 : (size_t)batch * (size_t)slices * sizeof(float2);
+}
+
 extern "C" int mvllm_sample_tokens(int64_t* out_ids, const void* logits, int64_t row_stride,
                                    const float* temperatures, const float* noise, uint64_t seed, uint64_t offset,
-                                   int batch, int vocab, int dtype, void* stream) {
+                                   int batch, int vocab, int dtype, void* workspace, size_t workspace_bytes,
+                                   void* stream) {
   const int esize = dtype_size(dtype);
   if (esize == 0) return MVLLM_ERR_BAD_DTYPE;
   if (batch < 0 || vocab <= 0 || row_stride < vocab) return MVLLM_ERR_BAD_SHAPE;
   if (batch == 0) return MVLLM_OK;
   if (!out_ids || !logits || !temperatures) return MVLLM_ERR_NULL_POINTER;
   if ((reinterpret_cast<uintptr_t>(logits) & (uintptr_t)(esize - 1)) != 0) return MVLLM_ERR_MISALIGNED;
+  // a row is split over as many workgroups as the workspace has room for (none: one workgroup per row)
+  const size_t want = mvllm_sample_tokens_workspace_bytes(batch, vocab);
+  int slices = 1;
+  if (workspace && want > 0 && workspace_bytes >= want) {
+    if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MVLLM_ERR_WORKSPACE;
+    slices = (int)(want / ((size_t)batch * sizeof(float2)));
+  }
   hipStream_t s = (hipStream_t)stream;
   const uint32_t sl = (uint32_t)seed, sh = (uint32_t)(seed >> 32), ol = (uint32_t)offset, oh = (uint32_t)(offset >> 32);
-  const dim3 grid((unsigned)batch), block(kSampleThreads);
+  const dim3 grid((unsigned)batch, (unsigned)slices), block(kSampleThreads);
+  float2* part = reinterpret_cast<float2*>(workspace);
   switch (dtype) {
     case MVLLM_F32:
-      sample_tokens_kernel<float><<<grid, block, 0, s>>>(out_ids, (const float*)logits, row_stride, temperatures, noise, sl,
-                                                        sh, ol, oh, vocab);
+      sample_tokens_kernel<float><<<grid, block, 0, s>>>(out_ids, part, (const float*)logits, row_stride, temperatures,
+                                                        noise, sl, sh, ol, oh, vocab, slices);
       break;
     case MVLLM_BF16:
-      sample_tokens_kernel<bf16_t><<<grid, block, 0, s>>>(out_ids, (const bf16_t*)logits, row_stride, temperatures, noise,
-                                                         sl, sh, ol, oh, vocab);
+      sample_tokens_kernel<bf16_t><<<grid, block, 0, s>>>(out_ids, part, (const bf16_t*)logits, row_stride, temperatures,
+                                                         noise, sl, sh, ol, oh, vocab, slices);
       break;
     default:
-      sample_tokens_kernel<f16_t><<<grid, block, 0, s>>>(out_ids, (const f16_t*)logits, row_stride, temperatures, noise, sl,
-                                                        sh, ol, oh, vocab);
+      sample_tokens_kernel<f16_t><<<grid, block, 0, s>>>(out_ids, part, (const f16_t*)logits, row_stride, temperatures,
+                                                        noise, sl, sh, ol, oh, vocab, slices);
       break;
   }
+  if (slices > 1) sample_combine_kernel<<<dim3((unsigned)batch), dim3(64), 0, s>>>(out_ids, part, slices);
   return launch_status();
 }

@@ -115,13 +115,14 @@ def qk_norm_rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positi
 
 
 def sample_tokens(logits: torch.Tensor, temperatures: torch.Tensor, seed: int = 0, offset: int = 0,
-                  noise: torch.Tensor | None = None) -> torch.Tensor:
+                  noise: torch.Tensor | None = None, use_workspace: bool = True) -> torch.Tensor:
     """One token per row from softmax(logits / temperature): argmax of ``probs / Exp(1) noise`` as in
     sampler.py:15-18, computed as argmax(logits / T - log(noise)) without a probability tensor.
 
     logits: (batch, vocab) float32 / bfloat16 / float16, rows may be strided; temperatures float32 (batch,), > 0.
     ``noise`` float32 (batch, vocab) supplies the draws (clamped below at 1e-10); without it they are generated
     from (seed, offset): the same pair always gives the same tokens, advance ``offset`` per call.
+    ``use_workspace=False`` keeps every row in one workgroup (same tokens, slower for small batches).
     Returns int64 (batch,).
     """
     _C.require_cuda(logits, temperatures, noise)
@@ -141,10 +142,12 @@ def sample_tokens(logits: torch.Tensor, temperatures: torch.Tensor, seed: int = 
     if batch == 0:
         return out
     lib = _C.load()
+    nbytes = lib.mvllm_sample_tokens_workspace_bytes(batch, vocab) if use_workspace else 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=logits.device) if nbytes else None
     st = lib.mvllm_sample_tokens(_ptr(out), _ptr(logits), logits.stride(0) if batch > 1 else vocab,
                                  _ptr(temperatures), _ptr(noise), int(seed) & (2 ** 64 - 1),
                                  int(offset) & (2 ** 64 - 1), batch, vocab, _C.dtype_code(logits.dtype),
-                                 _C.current_stream_ptr(logits.device))
+                                 _ptr(ws), nbytes, _C.current_stream_ptr(logits.device))
     _C.check(st, "sample_tokens")
     return out
 

@@ -28,7 +28,8 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_prefill_varlen",
-              "mvllm_prefill_paged", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_add_rms_norm",
+              "mvllm_prefill_paged", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_workspace_bytes",
+              "mvllm_add_rms_norm",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
         assert n in names
 
@@ -73,10 +74,12 @@ def test_argument_validation_without_gpu():
     assert paged(0, 0, 0, 0, 0, 4, 0, 0, 1, 5, 4, 3, 128, 16, 8, 1.0, 1, 0) == -3      # Hq % Hkv
     assert paged(0, 0, 0, 0, 0, 4, 0, 0, 1, 5, 4, 2, 128, 0, 8, 1.0, 1, 0) == -3       # block_size
     sample = lib.mvllm_sample_tokens
-    assert sample(0, 0, 100, 0, 0, 1, 2, 0, 100, 1, 0) == 0        # empty batch
-    assert sample(0, 0, 100, 0, 0, 1, 2, 4, 100, 1, 0) == -1       # null pointers
-    assert sample(0, 0, 50, 0, 0, 1, 2, 4, 100, 1, 0) == -3        # row stride < vocab
-    assert sample(0, 0, 100, 0, 0, 1, 2, 4, 100, 5, 0) == -2       # dtype
+    assert sample(0, 0, 100, 0, 0, 1, 2, 0, 100, 1, 0, 0, 0) == 0        # empty batch
+    assert sample(0, 0, 100, 0, 0, 1, 2, 4, 100, 1, 0, 0, 0) == -1       # null pointers
+    assert sample(0, 0, 50, 0, 0, 1, 2, 4, 100, 1, 0, 0, 0) == -3        # row stride < vocab
+    assert sample(0, 0, 100, 0, 0, 1, 2, 4, 100, 5, 0, 0, 0) == -2       # dtype
+    ws = lib.mvllm_sample_tokens_workspace_bytes
+    assert ws(64, 151936) == 64 * 8 * 8 and ws(1024, 151936) == 0 and ws(4, 1000) == 0 and ws(1, 151936) == 38 * 8
     norm = lib.mvllm_add_rms_norm
     assert norm(0, 0, 0, 0, 0, 1e-6, 0, 1024, 1024, 1024, 1, 0) == 0       # no rows
     assert norm(0, 0, 0, 0, 0, 1e-6, 4, 1024, 1024, 1024, 1, 0) == -1      # null pointers

@@ -24,6 +24,8 @@ def test_sampler_with_given_noise_matches_oracle(dtype, batch, vocab):
     want = oracle.sampler_oracle(logits, temps, noise)
     got = sample_tokens(logits.to(DEV), temps.to(DEV), noise=noise.to(DEV)).cpu()
     assert got.dtype == torch.int64 and torch.equal(got, want)
+    one = sample_tokens(logits.to(DEV), temps.to(DEV), noise=noise.to(DEV), use_workspace=False).cpu()
+    assert torch.equal(one, want)                                  # one workgroup per row: same tokens
 
 
 def test_sampler_generated_noise_matches_the_counter_stream():
