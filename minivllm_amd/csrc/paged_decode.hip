@@ -382,14 +382,19 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_ke
 //          16 bytes = 16 dims): the query row is turned once per wave into 15-bit fixed point
 //          q ~ (128*hi + lo) * amax/16256 with int8 hi/lo planes, so scores are exact integer dot
 //          products times (amax/16256) * k_scale[token];
-//   PV     on the VALU with v_cvt_f32_ubyte on codes biased by +128 (one xor per 4 codes); the bias is
-//          taken out at the end as 128 * sum(p * v_scale);
+//   PV     on the VALU, two tokens per instruction: the codes, biased by +128 (one xor per 4 codes), of a
+//          lane's two V rows are paired per dim as fp16 (1024 + u_a, 1024 + u_b) (v_perm + or of the exponent
+//          bits), the weights p * v_scale of the two tokens as an fp16 pair, and v_dot2_f32_f16 accumulates both
+//          in fp32; the bias is taken out at the end as 1152 * sum(weights).  The running maximum is kept over
+//          score + log2 v_scale, so weights lie in (0, 2^8] for any scales;
 //   scales one k_scale and one v_scale load per lane and tile (lane l%4 of a quad holds token 4*(l/16)+l%4),
 //          handed round inside the quad by DPP.
 // V rows are 128 B, so one 16-byte load per lane covers 8 rows: lane l reads token 4*(l/16) + 2i + (l%16)/8,
 // dims 16*(l%8).. in instruction i = 0, 1.
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(4))) int v4i;
+typedef __attribute__((ext_vector_type(2))) _Float16 v2f16;
+typedef __attribute__((ext_vector_type(2))) float v2f;
 
 struct KVTileI8 {
   uint4 k[2];
@@ -525,7 +530,13 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_in
       for (int r = 0; r < 4; ++r)
         if (!t.ok || tok_base + r >= part_end) vs4[r] = 0.f;     // stale scale memory must not meet p = 0
     }
-    float pr[NCH][4];
+    // log2 of the V scales: the weight of a token in the second product is p * v_scale = exp2(score + log2
+    // v_scale - m), and m tracks the maximum of score + log2 v_scale, so that weights stay in (0, 2^8] whatever
+    // the scales are and fit fp16 (a zero scale counts as 2^-40: such a token has only zero codes)
+    float lv4[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) lv4[r] = __log2f(fmaxf(vs4[r], 9.094947e-13f));
+    uint32_t wpk[NCH];                 // fp16 pair: weights of this lane's two V rows, for its own head
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       v4i shi = {0, 0, 0, 0}, slo = {0, 0, 0, 0};
@@ -535,13 +546,14 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_in
         shi = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qhi[c][j], shi, 0, 0, 0);
         slo = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qlo[c][j], slo, 0, 0, 0);
       }
-      float s2[4];
+      float s2[4], t2[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         s2[r] = (float)(shi[r] * 128 + slo[r]) * (qscale[c] * ks4[r]);
         if (partial && (!t.ok || tok_base + r >= part_end)) s2[r] = -INFINITY;
+        t2[r] = s2[r] + lv4[r];
       }
-      const float tile_max = fmaxf(fmaxf(s2[0], s2[1]), fmaxf(s2[2], s2[3]));
+      const float tile_max = fmaxf(fmaxf(t2[0], t2[1]), fmaxf(t2[2], t2[3]));
       const bool grow = tile_max > m[c] + kLazyRescale || (m[c] == -INFINITY && tile_max > -INFINITY);
       if (__any(grow)) {
         const float m_new = grow ? tile_max : m[c];
@@ -556,37 +568,43 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_in
         m[c] = m_new;
       }
       const float m_eff = (m[c] == -INFINITY) ? 0.f : m[c];
+      float wr[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        pr[c][r] = fast_exp2(s2[r] - m_eff);
-        l[c] += pr[c][r];
+        l[c] += fast_exp2(s2[r] - m_eff);          // softmax denominator, in the same units as the weights / v_scale
+        wr[r] = fast_exp2(t2[r] - m_eff);
       }
+      // this lane's V rows are tokens hb and 2 + hb of its token class
+      v2f wab = {hb ? wr[1] : wr[0], hb ? wr[3] : wr[2]};
+      const v2f16 wh = __builtin_convertvector(wab, v2f16);
+      wsum[c] += (float)wh[0] + (float)wh[1];      // of the weights as they are used
+      wpk[c] = __builtin_bit_cast(uint32_t, wh);
+    }
+    // V codes biased to 0..255, two tokens per register as the fp16 pair (1024 + u_a, 1024 + u_b): 0x6400 | u is
+    // exactly 1024 + u.  One v_dot2 then adds both tokens' contribution for one dim and head; the 1024 + 128 is
+    // taken out at the end as 1152 * sum(weights).
+    const uint32_t va[4] = {t.v[0].x ^ 0x80808080u, t.v[0].y ^ 0x80808080u, t.v[0].z ^ 0x80808080u, t.v[0].w ^ 0x80808080u};
+    const uint32_t vb[4] = {t.v[1].x ^ 0x80808080u, t.v[1].y ^ 0x80808080u, t.v[1].z ^ 0x80808080u, t.v[1].w ^ 0x80808080u};
+    v2f16 vp[16];
+#pragma unroll
+    for (int d4 = 0; d4 < 4; ++d4) {
+      vp[4 * d4 + 0] = __builtin_bit_cast(v2f16, __builtin_amdgcn_perm(vb[d4], va[d4], 0x0c040c00u) | 0x64006400u);
+      vp[4 * d4 + 1] = __builtin_bit_cast(v2f16, __builtin_amdgcn_perm(vb[d4], va[d4], 0x0c050c01u) | 0x64006400u);
+      vp[4 * d4 + 2] = __builtin_bit_cast(v2f16, __builtin_amdgcn_perm(vb[d4], va[d4], 0x0c060c02u) | 0x64006400u);
+      vp[4 * d4 + 3] = __builtin_bit_cast(v2f16, __builtin_amdgcn_perm(vb[d4], va[d4], 0x0c070c03u) | 0x64006400u);
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint4 raw = t.v[i];
-      const uint32_t w4[4] = {raw.x ^ 0x80808080u, raw.y ^ 0x80808080u, raw.z ^ 0x80808080u, raw.w ^ 0x80808080u};
-      float vf[16];
+    for (int c = 0; c < NCH; ++c) {
+      const v2f16 w0 = __builtin_bit_cast(v2f16, __builtin_amdgcn_update_dpp(0, (int)wpk[c], 0 * 0x55, 0xf, 0xf, false));
+      const v2f16 w1 = __builtin_bit_cast(v2f16, __builtin_amdgcn_update_dpp(0, (int)wpk[c], 1 * 0x55, 0xf, 0xf, false));
+      const v2f16 w2 = __builtin_bit_cast(v2f16, __builtin_amdgcn_update_dpp(0, (int)wpk[c], 2 * 0x55, 0xf, 0xf, false));
+      const v2f16 w3 = __builtin_bit_cast(v2f16, __builtin_amdgcn_update_dpp(0, (int)wpk[c], 3 * 0x55, 0xf, 0xf, false));
 #pragma unroll
-      for (int d4 = 0; d4 < 4; ++d4) {
-        vf[4 * d4 + 0] = byte_to_float<0>(w4[d4]);
-        vf[4 * d4 + 1] = byte_to_float<1>(w4[d4]);
-        vf[4 * d4 + 2] = byte_to_float<2>(w4[d4]);
-        vf[4 * d4 + 3] = byte_to_float<3>(w4[d4]);
-      }
-      const float vsel = hb ? vs4[2 * i + 1] : vs4[2 * i];
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        const float wgt = (hb ? pr[c][2 * i + 1] : pr[c][2 * i]) * vsel;    // own head; other heads via the quad
-        wsum[c] += wgt;
-        const float w0 = quad_bcast<0>(wgt), w1 = quad_bcast<1>(wgt), w2 = quad_bcast<2>(wgt), w3 = quad_bcast<3>(wgt);
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          acc[c][0][e] = fmaf(w0, vf[e], acc[c][0][e]);
-          acc[c][1][e] = fmaf(w1, vf[e], acc[c][1][e]);
-          acc[c][2][e] = fmaf(w2, vf[e], acc[c][2][e]);
-          acc[c][3][e] = fmaf(w3, vf[e], acc[c][3][e]);
-        }
+      for (int e = 0; e < 16; ++e) {
+        acc[c][0][e] = __builtin_amdgcn_fdot2(w0, vp[e], acc[c][0][e], false);
+        acc[c][1][e] = __builtin_amdgcn_fdot2(w1, vp[e], acc[c][1][e], false);
+        acc[c][2][e] = __builtin_amdgcn_fdot2(w2, vp[e], acc[c][2][e], false);
+        acc[c][3][e] = __builtin_amdgcn_fdot2(w3, vp[e], acc[c][3][e], false);
       }
     }
   };
@@ -604,7 +622,7 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_in
     ++tile;
   }
 
-  // take the +128 bias out, then fold the token classes: first the two V-row halves (same m, l), then lane/16
+  // take the 1024 + 128 bias out, then fold the token classes: first the two V-row halves (same m, l), then lane/16
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     const float b4[4] = {quad_bcast<0>(wsum[c]), quad_bcast<1>(wsum[c]), quad_bcast<2>(wsum[c]), quad_bcast<3>(wsum[c])};
@@ -612,7 +630,7 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_in
     for (int h = 0; h < 4; ++h)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        float x = fmaf(-128.f, b4[h], acc[c][h][e]);
+        float x = fmaf(-1152.f, b4[h], acc[c][h][e]);
         x += __shfl_xor(x, 8, 64);
         acc[c][h][e] = x;
       }
