@@ -31,6 +31,15 @@ namespace mvllm {
 #ifndef MVLLM_DECODE_WAVES_PER_EU
 #define MVLLM_DECODE_WAVES_PER_EU 2
 #endif
+#ifndef MVLLM_DECODE_I8_WPB
+#define MVLLM_DECODE_I8_WPB 4       // INT8 kernel: 4-wave workgroups, three of which fit a CU (more waves to hide latency)
+#endif
+#ifndef MVLLM_DECODE_I8_THREADS
+#define MVLLM_DECODE_I8_THREADS 256
+#endif
+#ifndef MVLLM_DECODE_I8_WAVES_PER_EU
+#define MVLLM_DECODE_I8_WAVES_PER_EU 3
+#endif
 #ifndef MVLLM_DECODE_WPB
 #define MVLLM_DECODE_WPB 8          // waves (= kv heads) per workgroup, upper bound
 #endif
@@ -410,7 +419,7 @@ template <int SEL> __device__ __forceinline__ float byte_to_float(uint32_t w) {
 }
 
 template <typename T, int NCH>
-__global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(MVLLM_DECODE_I8_THREADS, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
   constexpr int D = 128;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -881,7 +890,7 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stre
     if (fast_ok && (!int8 || group <= 4)) {
       // kv heads (waves) per workgroup: as many as allowed, so that a workgroup streams whole token rows;
       // fewer when the grid would otherwise leave most CUs without a workgroup
-      int wpb = largest_divisor_le(a.num_kv_heads, MVLLM_DECODE_WPB);
+      int wpb = largest_divisor_le(a.num_kv_heads, int8 ? MVLLM_DECODE_I8_WPB : MVLLM_DECODE_WPB);
       while (wpb > 1 && (int64_t)a.num_parts * a.batch * (a.num_kv_heads / wpb) < 512)
         wpb = largest_divisor_le(a.num_kv_heads, wpb - 1);
       dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, (unsigned)(a.num_kv_heads / wpb));
