@@ -41,7 +41,8 @@ namespace mvllm {
 #define MVLLM_DECODE_I8_WAVES_PER_EU 3
 #endif
 #ifndef MVLLM_DECODE_WPB
-#define MVLLM_DECODE_WPB 8          // waves (= kv heads) per workgroup, upper bound
+#define MVLLM_DECODE_WPB 4          // waves (= kv heads) per workgroup, upper bound: three 4-wave workgroups fit a CU
+                                    // (162 VGPRs), one more wave per SIMD than with 8-wave workgroups (+1.5 %)
 #endif
 
 constexpr int kTile = 16;                                 // tokens per MFMA tile
