@@ -102,6 +102,19 @@ __device__ __forceinline__ uint4 load16_stream(const void* p) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// x / d for many x and one d: r = 1 / d is computed once (correctly rounded), then each quotient costs a
+// multiply and two FMAs instead of a full division sequence: q = x r, q + (x - q d) r.  With a correctly rounded
+// reciprocal the corrected quotient is the correctly rounded x / d for normal operands (Markstein), up to rare
+// last-bit cases.
+struct SharedDivisor {
+  float d, r;
+  __device__ __forceinline__ explicit SharedDivisor(float divisor) : d(divisor), r(1.0f / divisor) {}
+  __device__ __forceinline__ float divide(float x) const {
+    const float q = x * r;
+    return fmaf(fmaf(-q, d, x), r, q);
+  }
+};
+
 // ---- host helpers ----------------------------------------------------------
 inline int dtype_size(int dtype) {
   switch (dtype) {

@@ -6,7 +6,8 @@
 //   store_kvcache(k, v, k_cache, v_cache, slot_mapping)   layers/attention.py:67-108
 // Rounding follows that chain: the norm result is rounded to the element type, the rotation is computed in fp32
 // from the rounded values and rounded again; products and sums are separate IEEE operations (no fused
-// multiply-add), division and square root are correctly rounded.  Only the order of the sum of squares is free.
+// multiply-add), the square root is correctly rounded and x / denominator is taken with one correction step from
+// the correctly rounded reciprocal (SharedDivisor).  Only the order of the sum of squares is free.
 //
 // Work item = one (token, head) vector of q, k or v.  GROUP lanes (a power of two) share a vector; lane j holds
 // EPL = 8 (4 when head_dim is not a multiple of 16) elements [EPL j, EPL j + EPL) of the first half and the same of the second half, i.e.
@@ -153,15 +154,15 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(const
 #pragma unroll
       for (int e = 0; e < EPL; ++e) ss = ss + x2[e] * x2[e];
       ss = group_sum<GROUP>(ss);
-      const float denom = sqrtf(ss / (float)D + a.eps);
+      const SharedDivisor denom(sqrtf(ss / (float)D + a.eps));
       if (lane_live) {
         float g1[EPL], g2[EPL];
         VecN<float, EPL>::load(a.gamma + e1, g1);
         VecN<float, EPL>::load(a.gamma + e2, g2);
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
-          x1[e] = rounded<T>((x1[e] / denom) * g1[e]);
-          x2[e] = rounded<T>((x2[e] / denom) * g2[e]);
+          x1[e] = rounded<T>(denom.divide(x1[e]) * g1[e]);
+          x2[e] = rounded<T>(denom.divide(x2[e]) * g2[e]);
         }
       }
     }

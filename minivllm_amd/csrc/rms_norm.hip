@@ -3,8 +3,9 @@
 //   x = x + residual                                   (in the element type: the sum is rounded to it)
 //   out = x / sqrt(mean(x^2) + eps) * gamma, residual_out = x
 // as called twice per layer and once after the last layer (src/myvllm/models/qwen3.py:197-212, 306-312).
-// The norm is computed in fp32 from the rounded sum with separate multiplies and adds (no contraction) and
-// correctly rounded division and square root; only the order of the sum of squares is free.
+// The norm is computed in fp32 from the rounded sum with separate multiplies and adds (no contraction), a
+// correctly rounded square root and the quotient x / denominator taken with one correction step from the
+// correctly rounded reciprocal (SharedDivisor); only the order of the sum of squares is free.
 //
 // One wave per row; lane l holds elements [8 (l + 64 c), +8) for chunks c = 0 .. CHUNKS-1 in registers, so the
 // row is read once and written once (16-byte accesses).
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) ss = ss + __shfl_xor(ss, o, 64);
-  const float denom = sqrtf(ss / (float)hidden + eps);
+  const SharedDivisor denom(sqrtf(ss / (float)hidden + eps));
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) {
     const int e0 = 8 * (lane + 64 * c);
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
       float g[8], y[8];
       Row8<float>::load(gamma + e0, g);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) y[e] = (v[c][e] / denom) * g[e];
+      for (int e = 0; e < 8; ++e) y[e] = denom.divide(v[c][e]) * g[e];
       Row8<T>::store(out + row * (int64_t)hidden + e0, y);
     }
   }
