@@ -31,6 +31,12 @@ namespace mvllm {
 #ifndef MVLLM_DECODE_WAVES_PER_EU
 #define MVLLM_DECODE_WAVES_PER_EU 2
 #endif
+#ifndef MVLLM_DECODE_SMALL_PAIRS
+#define MVLLM_DECODE_SMALL_PAIRS 1024  // partitions are shortened (to >= 64 tokens) while batch * partitions is below this
+#endif
+#ifndef MVLLM_DECODE_SMALL_GRID
+#define MVLLM_DECODE_SMALL_GRID 1024   // kv heads per workgroup are reduced while the grid has fewer workgroups than this
+#endif
 #ifndef MVLLM_DECODE_I8_WPB
 #define MVLLM_DECODE_I8_WPB 4       // INT8 kernel: 4-wave workgroups, three of which fit a CU (more waves to hide latency)
 #endif
@@ -79,13 +85,13 @@ struct DecodeArgs {
 // best on MI355X), so the length is doubled up to 1024 while the grid still offers at least four
 // workgroups per CU.  A small batch of short contexts is the opposite case: too few (sequence, partition)
 // pairs to occupy 256 CUs, each walking its tokens tile after tile at memory latency; there the length is
-// halved, down to 64 tokens, until there are 256 pairs.
+// halved, down to 64 tokens, until there are 1024 pairs.
 __host__ __device__ inline int partition_tokens_for(int64_t max_ctx, int batch) {
   const int64_t per_part = (max_ctx + kMaxParts - 1) / kMaxParts;
   int64_t part = (per_part + kMinPartTokens - 1) / kMinPartTokens * kMinPartTokens;
   if (part < kMinPartTokens) part = kMinPartTokens;
   while (part < 1024 && (int64_t)batch * ((max_ctx + 2 * part - 1) / (2 * part)) >= 1024) part *= 2;
-  while (part > 64 && part / 2 >= per_part && (int64_t)batch * ((max_ctx + part - 1) / part) < 256) part /= 2;
+  while (part > 64 && part / 2 >= per_part && (int64_t)batch * ((max_ctx + part - 1) / part) < MVLLM_DECODE_SMALL_PAIRS) part /= 2;
   return (int)part;
 }
 
@@ -892,7 +898,7 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stre
       // kv heads (waves) per workgroup: as many as allowed, so that a workgroup streams whole token rows;
       // fewer when the grid would otherwise leave most CUs without a workgroup
       int wpb = largest_divisor_le(a.num_kv_heads, int8 ? MVLLM_DECODE_I8_WPB : MVLLM_DECODE_WPB);
-      while (wpb > 1 && (int64_t)a.num_parts * a.batch * (a.num_kv_heads / wpb) < 512)
+      while (wpb > 1 && (int64_t)a.num_parts * a.batch * (a.num_kv_heads / wpb) < MVLLM_DECODE_SMALL_GRID)
         wpb = largest_divisor_le(a.num_kv_heads, wpb - 1);
       dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, (unsigned)(a.num_kv_heads / wpb));
       dim3 block(64 * wpb);

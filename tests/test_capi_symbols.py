@@ -48,8 +48,8 @@ def test_host_only_entry_points():
     assert lib.mvllm_version() >= 1000
     assert lib.mvllm_status_string(-5).decode().startswith("workspace")
     # pure host arithmetic: (D + 2) floats per (seq, partition, head); partitions of 256..1024 tokens, at most 32
-    # per sequence, shortened down to 64 tokens while batch * partitions < 256
-    assert lib.mvllm_paged_decode_workspace_bytes(256, 16, 128, 16, 16) == 0         # 256 tokens: 1 partition
+    # per sequence, shortened down to 64 tokens while batch * partitions < 1024
+    assert lib.mvllm_paged_decode_workspace_bytes(1024, 16, 128, 16, 16) == 0        # 256 tokens: 1 partition
     assert lib.mvllm_paged_decode_workspace_bytes(8, 16, 128, 16, 16) == 8 * 4 * 16 * 130 * 4     # 4 x 64 tokens
     assert lib.mvllm_paged_decode_workspace_bytes(2, 4, 128, 64, 16) == 2 * 16 * 4 * 130 * 4      # 16 x 64 tokens
     assert lib.mvllm_paged_decode_workspace_bytes(256, 32, 128, 2048, 16) == 256 * 32 * 32 * 130 * 4
