@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the paged-attention hot path on one MI355X.
 
-Prints ONE JSON line.  The headline (`metric`/`value`) is BASELINE config 3:
+Prints ONE JSON line.  The headline (`metric`/`value`) is BASELINE.json config 3:
 paged-attention decode, batch 256, context lengths log-uniform in [128, 32768],
 32 query heads / 8 KV heads / head_dim 128, bf16 cache, block_size 16, reported
 as algorithmic HBM GB/s.  A "step" is one decode call over the whole batch with
@@ -146,7 +146,7 @@ def bench_decode(args, block_size, want_cpu):
 
 
 def bench_prefill_store(args, which):
-    """BASELINE config 2: 16 prompts L~U[64,2048], Hq32/Hkv8/D128 bf16; store into a block-256 paged cache."""
+    """BASELINE.json config 2: 16 prompts L~U[64,2048], Hq32/Hkv8/D128 bf16; store into a block-256 paged cache."""
     import torch
     from helpers import make_slot_mapping
     from minivllm_amd.layers.attention import flash_attention_prefill, store_kvcache
@@ -219,7 +219,7 @@ def bench_prefill_store(args, which):
 
 
 def bench_int8(args):
-    """BASELINE config 4: B 128, ctx U[256,16384], Hq32/Hkv8/D128; K/V ~ N(0,1) with 1 % outliers at 8 sigma are
+    """BASELINE.json config 4: B 128, ctx U[256,16384], Hq32/Hkv8/D128; K/V ~ N(0,1) with 1 % outliers at 8 sigma are
     quantised by store_kvcache_int8 into a block-16 int8 cache, then decoded with in-kernel dequantisation."""
     import torch
     from minivllm_amd.layers.attention import paged_attention_decode_int8, store_kvcache_int8
@@ -338,7 +338,7 @@ def bench_sampler(args):
 
 
 def bench_engine(args, max_num_sequences, graph):
-    """BASELINE config 5: random-init Qwen3-style decoder (hidden 1024, 8 layers, Hq16/Hkv8/D128, FFN 3072,
+    """BASELINE.json config 5: random-init Qwen3-style decoder (hidden 1024, 8 layers, Hq16/Hkv8/D128, FFN 3072,
     vocab 151936, bf16), 60 prompts of random ids with lengths U[32,96], 256 new tokens each, T 0.6."""
     import torch
     from minivllm_amd.engine.llm_engine import LLMEngine

@@ -1,6 +1,6 @@
 """paged_attention_decode on the GPU vs the CPU oracle.
 
-Tolerances (BASELINE north_star): bf16/fp16 outputs max-abs <= 2e-2 and
+Tolerances (BASELINE.json north_star): bf16/fp16 outputs max-abs <= 2e-2 and
 mean-abs <= 2e-3 against the oracle evaluated in fp32 on the same (upcast)
 inputs; fp32 outputs max-abs <= 2e-4."""
 import math
@@ -30,7 +30,7 @@ def _oracle32(q, kc, vc, tables, ctx, scale, hq, hkv, d, bs):
 
 
 def test_config1_fp32_elementwise():
-    """BASELINE config 1: B 8, ctx U[16,512], Hq16/Hkv8, D128, bs16, fp32 cache, shuffled tables."""
+    """BASELINE.json config 1: B 8, ctx U[16,512], Hq16/Hkv8, D128, bs16, fp32 cache, shuffled tables."""
     hq, hkv, d, bs = 16, 8, 128, 16
     case = make_paged_case(31, 8, 16, 512, hq, hkv, d, bs)
     scale = 1 / math.sqrt(d)
@@ -148,7 +148,7 @@ def test_wider_table_same_result():
 
 @pytest.mark.parametrize("bs", [16, 256])
 def test_config3_full_size_subset_vs_oracle(bs):
-    """BASELINE config 3: B 256, ctx log-uniform [128, 32768], Hq32/Hkv8/D128 bf16.  The oracle is evaluated on
+    """BASELINE.json config 3: B 256, ctx log-uniform [128, 32768], Hq32/Hkv8/D128 bf16.  The oracle is evaluated on
     a seeded subset of sequences (the padded formulation does not fit in host memory for all 256)."""
     hq, hkv, d = 32, 8, 128
     q, kd, vd, tables, ctx = make_paged_case_on_device(40, DEV, 256, 128, 32768, hq, hkv, d, bs)

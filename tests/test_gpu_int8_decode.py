@@ -83,7 +83,7 @@ def test_int8_zero_context_and_missing_blocks():
 
 
 def test_config4_subset():
-    """BASELINE config 4 shape (B 128 is cut to 24 sequences here, ctx U[256,16384]) on the fast path."""
+    """BASELINE.json config 4 shape (B 128 is cut to 24 sequences here, ctx U[256,16384]) on the fast path."""
     hq, hkv, d, bs = 32, 8, 128, 16
     case = _quantised_case(65, 24, 256, 16384, hq, hkv, d, bs)
     _check(case, hq, hkv, d, bs, 1 / math.sqrt(d))

@@ -65,7 +65,7 @@ def test_prefill_zero_length_sequences_and_independence():
 
 
 def test_config2_full_size():
-    """BASELINE config 2: 16 prompts L U[64,2048], Hq32/Hkv8/D128 bf16; store into block-256 cache; the last
+    """BASELINE.json config 2: 16 prompts L U[64,2048], Hq32/Hkv8/D128 bf16; store into block-256 cache; the last
     row of each prompt must agree with a paged decode of that token over the stored cache."""
     hq, hkv, d, bs = 32, 8, 128, 256
     g = torch.Generator().manual_seed(53)

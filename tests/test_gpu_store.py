@@ -65,7 +65,7 @@ def test_store_non_contiguous_inputs_and_int32_slots_and_empty():
 
 
 def test_store_full_size_round_trip():
-    """BASELINE config 2 shape: 16 prompts, L in [64, 2048], Hkv 8, D 128, bf16, block 256."""
+    """BASELINE.json config 2 shape: 16 prompts, L in [64, 2048], Hkv 8, D 128, bf16, block 256."""
     g = torch.Generator().manual_seed(25)
     lengths = torch.randint(64, 2049, (16,), generator=g).tolist()
     bs, hkv, d = 256, 8, 128
@@ -106,7 +106,7 @@ def test_store_int8_bit_exact(dtype, hkv, d, bs):
 
 
 def test_store_int8_full_size_invariants():
-    """BASELINE config 4 style rows (1 % outliers at 8 sigma) at 64k tokens: spec invariants on the GPU result
+    """BASELINE.json config 4 style rows (1 % outliers at 8 sigma) at 64k tokens: spec invariants on the GPU result
     and bit-exact agreement with the oracle on the whole batch."""
     bs, hkv, d, t = 256, 8, 128, 65536
     k, v = _rows(29, t, hkv, d, torch.bfloat16, outliers=True)
