@@ -45,6 +45,8 @@ class ModelRunner:
         self.fused_sampler = config.get("fused_sampler", True)
         self.seed = config.get("seed", 0)
         self.sample_calls = 0
+        self._steady = None          # description of the batch in the static decode buffers (graph decode)
+        self._last_sampled = None    # device tensor of the ids sampled by the last graph decode step
         self.generator = torch.Generator(device=self.device).manual_seed(config.get("seed", 0))
         self.allocate_kv_cache()
         self.graphs = {}
@@ -144,34 +146,75 @@ class ModelRunner:
             torch.cuda.synchronize()
             reset_context()
 
-    def _replay_decode(self, input_ids, bs):
-        from minivllm_amd.utils.context import get_context
-        ctx = get_context()
-        gbs = next(b for b in sorted(self.graphs) if b >= bs)
+    def _fill_decode_buffers(self, seqs, gbs):
+        """Full refill of the static decode buffers from the host-side metadata (model_runner.py:231-256)."""
+        bs = len(seqs)
+        md = decode_metadata(seqs, self.block_size)
         v = self.graph_vars
-        v["input_ids"][:bs].copy_(input_ids)
+        v["input_ids"][:bs].copy_(self._to_device(md["input_ids"], torch.int64))
         v["slot_mapping"][:gbs].fill_(-1)
-        v["slot_mapping"][:bs].copy_(ctx.slot_mapping)
+        v["slot_mapping"][:bs].copy_(self._to_device(md["slot_mapping"], torch.int64))
         v["context_lens"][:gbs].zero_()
-        v["context_lens"][:bs].copy_(ctx.context_lens)
-        v["block_tables"][:bs, :ctx.block_tables.size(1)].copy_(ctx.block_tables)
+        v["context_lens"][:bs].copy_(self._to_device(md["context_lens"], torch.int64))
+        tables = self._to_device(md["block_tables"], torch.int32)
+        v["block_tables"][:bs, :tables.size(1)].copy_(tables)
+        self._steady = dict(key=tuple(seq.seq_id for seq in seqs), lens=[len(seq) for seq in seqs],
+                            temperatures=self._to_device([seq.temperature for seq in seqs], torch.float32))
+
+    def _advance_decode_buffers(self, seqs) -> bool:
+        """The same sequences as in the last graph decode step, each one token longer: the buffers move on the
+        device (input = the ids sampled last step, context length and slot + 1) and only sequences that started a
+        new block are patched from the host.  Returns False when the batch is not such a continuation."""
+        st = self._steady
+        if st is None or self._last_sampled is None or st["key"] != tuple(seq.seq_id for seq in seqs):
+            return False
+        lens = [len(seq) for seq in seqs]
+        if any(n != m + 1 for n, m in zip(lens, st["lens"])):
+            return False
+        bs = len(seqs)
+        v = self.graph_vars
+        v["input_ids"][:bs].copy_(self._last_sampled)
+        v["context_lens"][:bs] += 1
+        v["slot_mapping"][:bs] += 1
+        fresh = [i for i, n in enumerate(lens) if (n - 1) % self.block_size == 0]     # token n-1 opens a block
+        if fresh:
+            rows = self._to_device(fresh, torch.int64)
+            cols = self._to_device([len(seqs[i].block_table) - 1 for i in fresh], torch.int64)
+            blocks = [seqs[i].block_table[-1] for i in fresh]
+            v["block_tables"][rows, cols] = self._to_device(blocks, torch.int32)
+            v["slot_mapping"][rows] = self._to_device([b * self.block_size for b in blocks], torch.int64)
+        st["lens"] = lens
+        return True
+
+    def _replay_decode(self, seqs):
+        bs = len(seqs)
+        gbs = next(b for b in sorted(self.graphs) if b >= bs)
+        if not self._advance_decode_buffers(seqs):
+            self._fill_decode_buffers(seqs, gbs)
         self.graphs[gbs].replay()
-        return v["outputs"][:bs]
+        return self.graph_vars["outputs"][:bs], self._steady["temperatures"]
 
     @torch.inference_mode()
     def run(self, seqs, is_prefill: bool) -> list[int]:
-        input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
-        temperatures = self._to_device([seq.temperature for seq in seqs], torch.float32)
         if not is_prefill and self.graphs and len(seqs) <= max(self.graphs):
-            hidden = self._replay_decode(input_ids, len(seqs))
+            hidden, temperatures = self._replay_decode(seqs)
+            graphed = True
         else:
+            input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
+            temperatures = self._to_device([seq.temperature for seq in seqs], torch.float32)
             hidden = self.model(input_ids, positions)
-        logits = self.model.compute_logits(hidden)
+            graphed = False
+        logits = self.model.compute_logits(hidden) if not graphed else torch.nn.functional.linear(
+            hidden, self.model.lm_head_weight)
         if self.fused_sampler:
             # one launch over the LM-head output; draws are a function of (seed, step), so a run is reproducible
-            token_ids = sample_tokens(logits, temperatures, self.seed, self.sample_calls).tolist()
+            sampled = sample_tokens(logits, temperatures, self.seed, self.sample_calls)
             self.sample_calls += 1
         else:
-            token_ids = self.sampler(logits, temperatures, self.generator).tolist()
+            sampled = self.sampler(logits, temperatures, self.generator)
+        self._last_sampled = sampled if graphed else None      # next step's input ids, if it continues this batch
+        if not graphed:
+            self._steady = None
+        token_ids = sampled.tolist()
         reset_context()
         return token_ids
