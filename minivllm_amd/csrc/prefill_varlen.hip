@@ -194,7 +194,9 @@ constexpr int kWaveRows = 32;           // query rows per wave
 constexpr int kTileBytes = kBN * 256;   // one K (or V) tile, head_dim 128 x 2 B
 
 // v_max3_f32 without the canonicalising self-max the compiler puts in front of every fmaxf operand that
-// comes out of an MFMA (scores are finite or -inf here, never NaN).
+// comes out of an MFMA (scores are finite or -inf here, never NaN).  The compiler does not know what the asm
+// reads, so it does not space it from an MFMA that writes an operand: the caller has to order it after an
+// ordinary instruction that reads the newest MFMA result.
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
@@ -479,15 +481,20 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
         for (int r = 0; r < 16; ++r)
           if (32 * tk + 8 * (r >> 2) + (r & 3) > thr) s[tk][r] = -INFINITY;
     }
-    float mx = max3(s[0][0], s[0][1], s[0][2]);
+    // The chain starts from ordinary reads of one accumulator of each MFMA chain: the compiler keeps the
+    // distance an MFMA result needs before a vector instruction may read it only for instructions it knows,
+    // not for the v_max3 asm, and every max3 below depends on this first value (MFMAs finish in issue order,
+    // so once the last instruction of a chain has delivered, the chain's other registers are final too).
+    float mx = fmaxf(s[0][15], s[NH - 1][15]);
 #pragma unroll
-    for (int r = 3; r < 15; r += 2) mx = max3(mx, s[0][r], s[0][r + 1]);
+    for (int r = 0; r < 14; r += 2) mx = max3(mx, s[0][r], s[0][r + 1]);
     if constexpr (NH == 2) {
-      mx = max3(mx, s[0][15], s[NH - 1][0]);
+      mx = max3(mx, s[0][14], s[1][14]);
 #pragma unroll
-      for (int r = 1; r < 15; r += 2) mx = max3(mx, s[NH - 1][r], s[NH - 1][r + 1]);
+      for (int r = 0; r < 14; r += 2) mx = max3(mx, s[1][r], s[1][r + 1]);
+    } else {
+      mx = max3(mx, s[0][14], s[0][14]);
     }
-    mx = fmaxf(mx, s[NH - 1][15]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * a.scale_log2;
     const bool grow = mx > m + 8.f || m == -INFINITY;
     if (__any(grow)) {
