@@ -2,21 +2,21 @@
 // GQA-shared K/V reads, log-sum-exp merge in a second pass.
 // Replaces the Triton kernel of src/myvllm/layers/attention.py:283-415.
 //
-// Work decomposition (fast path, 16-bit cache, head_dim 128, block_size % 16 == 0)
-//   workgroup = (partition p, sequence b, group of <= 8 kv heads); wave w of the
+// Work decomposition (fast path, 16-bit cache, head_dim 128, block_size % 16 == 0, up to 16 query heads per kv head)
+//   workgroup = (partition p, sequence b, group of <= 4 kv heads); wave w of the
 //   workgroup owns kv head g and all Hq/Hkv query heads that share it, so the
-//   waves of one workgroup stream whole contiguous [token, Hkv, D] rows.
-//   A wave walks its partition in tiles of 16 tokens:
-//     S[16 tok x 16 col]   = K_tile (A operand, straight from global in MFMA
-//                            layout) x Q^T (B operand, column n = head n%4)
-//                            -> lane l holds tokens 4*(l/16)+i, head l%4
-//     online softmax       per lane over its token class, base-2, lazy rescale
-//     O[head][8 dims]     += p * V  on the VALU; V rows are loaded fully
-//                            coalesced (lane l: token 4*(l/16)+i, dims 8*(l%16)..)
-//                            and p of head h comes from quad lane h via DPP.
-//   The four token classes are merged once per partition with xor-shuffles.
-// Everything is HBM-bound by construction: QK^T costs no VALU, PV costs
-// ~5 lane-ops per cache element.
+//   waves of one workgroup stream contiguous pieces of the [token, Hkv, D] rows.
+//   A wave walks its partition in tiles of 16 tokens, both products on the matrix unit:
+//     S[16 tok x 16 head]  = K_tile (A operand, straight from global in MFMA
+//                            layout) x Q^T (B operand, column n = head n)
+//     online softmax       per lane over its four tokens, base-2, lazy rescale with one
+//                            maximum per head shared by the lanes that hold it
+//     O[16 head x 128]    += P (the scores' own layout, packed to 16 bit) x V; V rows are
+//                            loaded fully coalesced (lane l: tokens 4*(l/16)+i, dims 8*(l%16)..)
+//                            and two byte permutes per product turn them into the B operand.
+//   See decode_mfma_item for the operand layouts.
+// The kernel is HBM-bound: a kernel that only issues the same loads (no arithmetic) reaches
+// 6.25 TB/s on this access pattern, this one about 6.05.
 #include "common.h"
 
 namespace mvllm {
@@ -24,6 +24,12 @@ namespace mvllm {
 // Tuning constants (overridable at compile time for experiments).
 #ifndef MVLLM_DECODE_MAX_PARTS
 #define MVLLM_DECODE_MAX_PARTS 32
+#endif
+#ifndef MVLLM_DECODE_DEPTH
+#define MVLLM_DECODE_DEPTH 2          // K/V tiles per wave of the 16-bit kernel: one consumed, the others in flight
+#endif
+#ifndef MVLLM_DECODE_PART_CAP
+#define MVLLM_DECODE_PART_CAP 1024  // partitions grow to this many tokens while the grid stays large
 #endif
 #ifndef MVLLM_DECODE_MIN_PART
 #define MVLLM_DECODE_MIN_PART 256
@@ -47,8 +53,7 @@ namespace mvllm {
 #define MVLLM_DECODE_I8_WAVES_PER_EU 3
 #endif
 #ifndef MVLLM_DECODE_WPB
-#define MVLLM_DECODE_WPB 4          // waves (= kv heads) per workgroup, upper bound: three 4-wave workgroups fit a CU
-                                    // (162 VGPRs), one more wave per SIMD than with 8-wave workgroups (+1.5 %)
+#define MVLLM_DECODE_WPB 4          // waves (= kv heads) per workgroup, upper bound (8-wave workgroups: -1.5 %)
 #endif
 
 constexpr int kTile = 16;                                 // tokens per MFMA tile
@@ -90,7 +95,7 @@ __host__ __device__ inline int partition_tokens_for(int64_t max_ctx, int batch) 
   const int64_t per_part = (max_ctx + kMaxParts - 1) / kMaxParts;
   int64_t part = (per_part + kMinPartTokens - 1) / kMinPartTokens * kMinPartTokens;
   if (part < kMinPartTokens) part = kMinPartTokens;
-  while (part < 1024 && (int64_t)batch * ((max_ctx + 2 * part - 1) / (2 * part)) >= 1024) part *= 2;
+  while (part < MVLLM_DECODE_PART_CAP && (int64_t)batch * ((max_ctx + 2 * part - 1) / (2 * part)) >= 1024) part *= 2;
   while (part > 64 && part / 2 >= per_part && (int64_t)batch * ((max_ctx + part - 1) / part) < MVLLM_DECODE_SMALL_PAIRS) part /= 2;
   return (int)part;
 }
@@ -129,138 +134,43 @@ struct KVTile {
   bool ok;
 };
 
-template <typename T, int NCH>
-struct DecodeWave {
-  // per-lane online-softmax state for head (lane%4) of chunk c, token class lane/16
-  float m[NCH];
-  float l[NCH];
-  float acc[NCH][4][8];
-  uint4 qf[NCH][4];
+// 16-bit pair (a, b) in the element type
+template <typename T> __device__ __forceinline__ uint32_t pack_pair(float x, float y) {
+  T v[2] = {from_float<T>(x), from_float<T>(y)};
+  return __builtin_bit_cast(uint32_t, v);
+}
+typedef __attribute__((ext_vector_type(4))) short v4i16;
+typedef __attribute__((ext_vector_type(4))) _Float16 v4f16;
+// D[16x16] += A[16x16] B[16x16], four 16-bit k-values per lane
+template <typename T> __device__ __forceinline__ v4f mfma16x16x16(uint2 x, uint2 y, v4f c);
+template <> __device__ __forceinline__ v4f mfma16x16x16<bf16_t>(uint2 x, uint2 y, v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(v4i16, x), __builtin_bit_cast(v4i16, y), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ v4f mfma16x16x16<f16_t>(uint2 x, uint2 y, v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(v4f16, x), __builtin_bit_cast(v4f16, y), c, 0, 0, 0);
+}
 
-  __device__ __forceinline__ void init() {
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      m[c] = -INFINITY;
-      l[c] = 0.f;
-#pragma unroll
-      for (int h = 0; h < 4; ++h)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[c][h][e] = 0.f;
-    }
-  }
-
-  template <int H>
-  __device__ __forceinline__ void scale_head(int c, float a) {
-    const float ah = quad_bcast<H>(a);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[c][H][e] *= ah;
-  }
-  template <int H>
-  __device__ __forceinline__ void fma_head(int c, float p, const float (&vf)[8]) {
-    const float ph = quad_bcast<H>(p);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[c][H][e] = fmaf(ph, vf[e], acc[c][H][e]);
-  }
-
-  __device__ __forceinline__ void consume(const KVTile<T>& t, int part_end, float scale_log2, int lane) {
-    const int tok_base = t.t0 + 4 * (lane >> 4);
-    const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
-    float p[NCH][4];
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      v4f s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) s = mfma16x16x32<T>(t.k[j], qf[c][j], s);
-      float s2[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) s2[i] = s[i] * scale_log2;
-      if (partial) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (!t.ok || tok_base + i >= part_end) s2[i] = -INFINITY;
-      }
-      const float tile_max = fmaxf(fmaxf(s2[0], s2[1]), fmaxf(s2[2], s2[3]));
-      const bool grow = tile_max > m[c] + kLazyRescale || (m[c] == -INFINITY && tile_max > -INFINITY);
-      if (__any(grow)) {
-        const float m_new = grow ? tile_max : m[c];
-        const float a = (m_new == m[c]) ? 1.f : safe_exp2_diff(m[c], m_new);
-        l[c] *= a;
-        scale_head<0>(c, a);
-        scale_head<1>(c, a);
-        scale_head<2>(c, a);
-        scale_head<3>(c, a);
-        m[c] = m_new;
-      }
-      const float m_eff = (m[c] == -INFINITY) ? 0.f : m[c];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        p[c][i] = fast_exp2(s2[i] - m_eff);
-        l[c] += p[c][i];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      uint4 w = t.v[i];
-      if (partial && (!t.ok || tok_base + i >= part_end)) w = make_uint4(0u, 0u, 0u, 0u);
-      float vf[8];
-      vf[0] = lo_to_float<T>(w.x); vf[1] = hi_to_float<T>(w.x);
-      vf[2] = lo_to_float<T>(w.y); vf[3] = hi_to_float<T>(w.y);
-      vf[4] = lo_to_float<T>(w.z); vf[5] = hi_to_float<T>(w.z);
-      vf[6] = lo_to_float<T>(w.w); vf[7] = hi_to_float<T>(w.w);
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        fma_head<0>(c, p[c][i], vf);
-        fma_head<1>(c, p[c][i], vf);
-        fma_head<2>(c, p[c][i], vf);
-        fma_head<3>(c, p[c][i], vf);
-      }
-    }
-  }
-
-  template <int H>
-  __device__ __forceinline__ void merge_head(int c, float a, float ao, int off) {
-    const float ah = quad_bcast<H>(a);
-    const float aoh = quad_bcast<H>(ao);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float other = __shfl_xor(acc[c][H][e], off, 64);
-      acc[c][H][e] = acc[c][H][e] * ah + other * aoh;
-    }
-  }
-
-  // Fold the four token classes (lane/16) together; afterwards every lane holds
-  // the statistics of the whole partition for its head / dims.
-  __device__ __forceinline__ void merge_token_classes() {
-#pragma unroll
-    for (int off = 16; off <= 32; off <<= 1) {
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        const float mo = __shfl_xor(m[c], off, 64);
-        const float lo = __shfl_xor(l[c], off, 64);
-        const float mn = fmaxf(m[c], mo);
-        const float a = safe_exp2_diff(m[c], mn);
-        const float ao = safe_exp2_diff(mo, mn);
-        l[c] = l[c] * a + lo * ao;
-        m[c] = mn;
-        merge_head<0>(c, a, ao, off);
-        merge_head<1>(c, a, ao, off);
-        merge_head<2>(c, a, ao, off);
-        merge_head<3>(c, a, ao, off);
-      }
-    }
-  }
-};
-
-template <typename T, int NCH>
-__global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_kernel(const DecodeArgs a) {
+// One wave = one kv head of one (sequence, partition); both products run on the matrix unit.
+//   S[token][head] = K Q^T   v_mfma 16x16x32: A = 16 tokens x 32 dims (lane l: token l%16, dims 8*(l/16).. of each
+//                    32-dim step, 16 B straight from the cache row), B = the query heads of the group as columns
+//                    (column n = head n, zero past the group), four steps for 128 dims.  Lane l then holds
+//                    S[token 4*(l/16)+i][head l%16], i < 4.
+//   softmax          per lane over its four tokens; the running maximum m of a head is kept identical in the four
+//                    lanes (token classes) that hold the head, so it is only exchanged when a tile raises it by
+//                    more than 2^8 (lazy rescale), which is rare.
+//   O[head][dim] += P V   v_mfma 16x16x16: A = P with exactly the layout S came out in (row = head l%16,
+//                    k = tokens 4*(l/16)+i), packed to 16 bit; B = V with k = the same four tokens and column
+//                    n = one dim per lane.  A lane loads 16 B = 8 dims of each of its four tokens (whole 256-B
+//                    rows per instruction), so its dim e of step e is column l%16 of the e-th product:
+//                    column n of product e is dim 8 n + e, and two byte permutes per product gather the four
+//                    tokens' values of that dim.  Lane l ends with O[head 4*(l/16)+j][dims 8*(l%16) + e].
+template <typename T>
+__device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int p, int g) {   // g: kv head
   constexpr int D = 128;
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int waves_per_block = blockDim.x >> 6;
-  int b, p;
-  if (!decode_item(a, b, p)) return;
-  const int g = blockIdx.z * waves_per_block + wave;   // kv head
-  const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head
+  const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head (<= 16)
+  const int col = lane & 15;                           // head (first product), dim group (second product)
+  const int cls = lane >> 4;                           // token class: tokens 4*cls .. 4*cls+3 of a tile
 
   const int ctx = (int)load_ctx(a, b);
   // a sequence that fits one partition (or is empty) is finished here: partition 0 writes the output row
@@ -270,26 +180,23 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_ke
   const int part_end = min(ctx, part_start + a.part_tokens);
   const int ntiles = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
 
-  DecodeWave<T, NCH> w;
-  w.init();
-
-  // Q fragments: B operand, column n = lane%16 -> head (n%4) of chunk c, k = 8*(lane/16)+32j
+  // Q fragments: B operand, column n = head n, k = 8*cls + 32 j
+  uint4 qf[4];
   {
     const T* q = reinterpret_cast<const T*>(a.q);
-    const int hq = lane & 3;
-    const int kq = lane >> 4;
+    const bool live = col < group;
+    const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D + cls * 8;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int hl = c * 4 + hq;
-      const bool live = hl < group;
-      const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? hl : 0)) * D + kq * 8;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint4 x = *reinterpret_cast<const uint4*>(src + 32 * j);
-        w.qf[c][j] = live ? x : make_uint4(0u, 0u, 0u, 0u);
-      }
+    for (int j = 0; j < 4; ++j) {
+      const uint4 x = *reinterpret_cast<const uint4*>(src + 32 * j);
+      qf[j] = live ? x : make_uint4(0u, 0u, 0u, 0u);
     }
   }
+  float m = -INFINITY;        // running maximum of head `col` (log2 units), the same in its four lanes
+  float l = 0.f;              // this lane's share of the head's denominator
+  v4f o[8];                   // o[e][j] = O[head 4*cls + j][dim 8*col + e]
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
 
   const int bs = a.block_size;
   const int64_t row = (int64_t)a.num_kv_heads * D;       // elements per token row
@@ -303,8 +210,8 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_ke
   int win_base = bi;
   int win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
 
-  const int k_lane_off = (lane & 15) * (int)row + (lane >> 4) * 8;   // token lane%16, dims 8*(lane/16)
-  const int v_lane_off = 4 * (lane >> 4) * (int)row + (lane & 15) * 8;  // token 4*(lane/16), dims 8*(lane%16)
+  const int k_lane_off = col * (int)row + cls * 8;        // token lane%16, dims 8*(lane/16)
+  const int v_lane_off = 4 * cls * (int)row + col * 8;    // token 4*(lane/16), dims 8*(lane%16)
 
   auto load_tile = [&](KVTile<T>& t, int tile) {
     t.t0 = part_start + tile * kTile;
@@ -336,59 +243,112 @@ __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_ke
     if (off >= bs) { off = 0; ++bi; }
   };
 
-  KVTile<T> ta, tb;
-  if (ntiles > 0) load_tile(ta, 0);
-  int tile = 0;
-  while (tile < ntiles) {
-    if (tile + 1 < ntiles) load_tile(tb, tile + 1);
-    w.consume(ta, part_end, a.scale_log2, lane);
-    ++tile;
-    if (tile >= ntiles) break;
-    if (tile + 1 < ntiles) load_tile(ta, tile + 1);
-    w.consume(tb, part_end, a.scale_log2, lane);
-    ++tile;
-  }
-
-  w.merge_token_classes();
-
-  // Lanes 0..15 (token class 0) now hold dims 8*lane.. for heads 0..3 of every chunk.
-  if (lane < 16) {
-    const int head0 = g * group;
-    if (direct) {
-      T* out = reinterpret_cast<T*>(a.out);
+  auto consume = [&](const KVTile<T>& t) {
+    const int tok_base = t.t0 + 4 * cls;
+    const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
+    v4f s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        const float linv = w.l[c] > 0.f ? 1.f / w.l[c] : 0.f;
-        const float li[4] = {quad_bcast<0>(linv), quad_bcast<1>(linv), quad_bcast<2>(linv), quad_bcast<3>(linv)};
+    for (int j = 0; j < 4; ++j) s = mfma16x16x32<T>(t.k[j], qf[j], s);
+    float s2[4];
 #pragma unroll
-        for (int h = 0; h < 4; ++h) {
-          if (c * 4 + h < group) {
-            T* dst = out + ((int64_t)b * a.num_heads + head0 + c * 4 + h) * D + lane * 8;
-            T o[8];
+    for (int i = 0; i < 4; ++i) s2[i] = s[i] * a.scale_log2;
+    uint4 v[4] = {t.v[0], t.v[1], t.v[2], t.v[3]};
+    if (partial) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = from_float<T>(w.acc[c][h][e] * li[h]);
-            *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(o);
-          }
+      for (int i = 0; i < 4; ++i)
+        if (!t.ok || tok_base + i >= part_end) {
+          s2[i] = -INFINITY;
+          v[i] = make_uint4(0u, 0u, 0u, 0u);       // whatever lies there must not meet p = 0 as NaN or Inf
         }
-      }
-    } else {
-      const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
+    }
+    const float tile_max = fmaxf(fmaxf(s2[0], s2[1]), fmaxf(s2[2], s2[3]));
+    const bool grow = tile_max > m + kLazyRescale || (m == -INFINITY && tile_max > -INFINITY);
+    if (__any(grow)) {
+      // the head's maximum over its four token classes, then one decision for all four lanes
+      float mh = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+      mh = fmaxf(mh, __shfl_xor(mh, 32, 64));
+      const bool grow_h = mh > m + kLazyRescale || (m == -INFINITY && mh > -INFINITY);
+      const float m_new = grow_h ? mh : m;
+      const float al = (m_new == m) ? 1.f : safe_exp2_diff(m, m_new);
+      l *= al;
+      m = m_new;
+      // accumulator row j is head 4*cls + j, whose factor sits in lane 4*cls + j (any class would do)
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) {
+      for (int j = 0; j < 4; ++j) {
+        const float aj = __shfl(al, 4 * cls + j, 64);
 #pragma unroll
-        for (int h = 0; h < 4; ++h) {
-          if (c * 4 + h < group) {
-            float* dst = a.ws_acc + (slot + c * 4 + h) * D + lane * 8;
-            *reinterpret_cast<float4*>(dst) = make_float4(w.acc[c][h][0], w.acc[c][h][1], w.acc[c][h][2], w.acc[c][h][3]);
-            *reinterpret_cast<float4*>(dst + 4) = make_float4(w.acc[c][h][4], w.acc[c][h][5], w.acc[c][h][6], w.acc[c][h][7]);
-          }
-        }
-        if (lane < 4 && c * 4 + lane < group) {
-          float* ml = a.ws_ml + (slot + c * 4 + lane) * 2;
-          *reinterpret_cast<float2*>(ml) = make_float2(w.m[c], w.l[c]);
-        }
+        for (int e = 0; e < 8; ++e) o[e][j] *= aj;
       }
     }
+    const float m_eff = (m == -INFINITY) ? 0.f : m;
+    float pr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pr[i] = fast_exp2(s2[i] - m_eff);
+      l += pr[i];
+    }
+    const uint2 pa = make_uint2(pack_pair<T>(pr[0], pr[1]), pack_pair<T>(pr[2], pr[3]));
+    // dim e of the lane's 8: the low or high half of component e/2 of each token's 16 bytes
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+      const uint32_t c0 = e < 2 ? v[0].x : e < 4 ? v[0].y : e < 6 ? v[0].z : v[0].w;
+      const uint32_t c1 = e < 2 ? v[1].x : e < 4 ? v[1].y : e < 6 ? v[1].z : v[1].w;
+      const uint32_t c2 = e < 2 ? v[2].x : e < 4 ? v[2].y : e < 6 ? v[2].z : v[2].w;
+      const uint32_t c3 = e < 2 ? v[3].x : e < 4 ? v[3].y : e < 6 ? v[3].z : v[3].w;
+      const uint2 vb = make_uint2(__builtin_amdgcn_perm(c1, c0, sel), __builtin_amdgcn_perm(c3, c2, sel));
+      o[e] = mfma16x16x16<T>(pa, vb, o[e]);
+    }
+  };
+
+  // kDepth tiles per wave: kDepth - 1 in flight while one is consumed
+  constexpr int kDepth = MVLLM_DECODE_DEPTH;
+  KVTile<T> ring[kDepth];
+#pragma unroll
+  for (int i = 0; i < kDepth - 1; ++i)
+    if (i < ntiles) load_tile(ring[i], i);
+  int tile = 0;
+  while (tile < ntiles) {
+#pragma unroll
+    for (int u = 0; u < kDepth; ++u) {
+      if (tile + kDepth - 1 < ntiles) load_tile(ring[(u + kDepth - 1) % kDepth], tile + kDepth - 1);
+      consume(ring[u]);
+      ++tile;
+      if (tile >= ntiles) break;
+    }
+  }
+
+  // denominators: add the four token classes (every lane of a head then holds the head's total)
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  const int head0 = g * group;
+  if (direct) {
+    T* out = reinterpret_cast<T*>(a.out);
+    const float linv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int h = 4 * cls + j;
+      const float lj = __shfl(linv, h, 64);               // lane h (class 0) holds head h
+      if (h < group) {
+        T r[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r[e] = from_float<T>(o[e][j] * lj);
+        *reinterpret_cast<uint4*>(out + ((int64_t)b * a.num_heads + head0 + h) * D + col * 8) =
+            *reinterpret_cast<const uint4*>(r);
+      }
+    }
+  } else {
+    const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int h = 4 * cls + j;
+      if (h < group) {
+        float* dst = a.ws_acc + (slot + h) * D + col * 8;
+        *reinterpret_cast<float4*>(dst) = make_float4(o[0][j], o[1][j], o[2][j], o[3][j]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(o[4][j], o[5][j], o[6][j], o[7][j]);
+      }
+    }
+    if (lane < group && lane < 16) *reinterpret_cast<float2*>(a.ws_ml + (slot + lane) * 2) = make_float2(m, l);
   }
 }
 
@@ -426,14 +386,9 @@ template <int SEL> __device__ __forceinline__ float byte_to_float(uint32_t w) {
 }
 
 template <typename T, int NCH>
-__global__ __launch_bounds__(MVLLM_DECODE_I8_THREADS, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
+__device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b, int p, int g) {   // g: kv head
   constexpr int D = 128;
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int waves_per_block = blockDim.x >> 6;
-  int b, p;
-  if (!decode_item(a, b, p)) return;
-  const int g = blockIdx.z * waves_per_block + wave;
   const int group = a.num_heads / a.num_kv_heads;
   const int q4 = lane >> 4;            // token class: tokens 4*q4 .. 4*q4+3 of a tile
   const int hb = (lane >> 3) & 1;      // which of the two V rows of an instruction this lane reads
@@ -719,6 +674,23 @@ __global__ __launch_bounds__(MVLLM_DECODE_I8_THREADS, MVLLM_DECODE_I8_WAVES_PER_
 }
 
 // ---------------------------------------------------------------------------
+// Kernels of the fast path: one workgroup per (partition, sequence, group of kv heads); the partition index is
+// an upper bound, and a workgroup whose partition lies past its sequence's context returns at once.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_kernel(const DecodeArgs a) {
+  int b, p;
+  if (!decode_item(a, b, p)) return;
+  decode_mfma_item<T>(a, b, p, blockIdx.z * (blockDim.x >> 6) + (threadIdx.x >> 6));
+}
+template <typename T, int NCH>
+__global__ __launch_bounds__(MVLLM_DECODE_I8_THREADS, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
+  int b, p;
+  if (!decode_item(a, b, p)) return;
+  decode_mfma_int8_item<T, NCH>(a, b, p, blockIdx.z * (blockDim.x >> 6) + (threadIdx.x >> 6));
+}
+
+// ---------------------------------------------------------------------------
 // Generic path: any element type (fp32 included), head_dim <= 512, any
 // block_size and group size.  One wave per (partition, sequence, q head);
 // lanes split head_dim, one token per step.  Correctness path for shapes the
@@ -903,8 +875,7 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stre
       dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, (unsigned)(a.num_kv_heads / wpb));
       dim3 block(64 * wpb);
       if (int8) decode_mfma_int8_kernel<T, 1><<<grid, block, 0, stream>>>(a);
-      else if (group <= 4) decode_mfma_kernel<T, 1><<<grid, block, 0, stream>>>(a);
-      else decode_mfma_kernel<T, 2><<<grid, block, 0, stream>>>(a);
+      else decode_mfma_kernel<T><<<grid, block, 0, stream>>>(a);
       launched = true;
     }
   }
@@ -959,7 +930,7 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
     a.ws_ml = a.ws_acc + (size_t)batch * a.num_parts * num_heads * head_dim;
   }
   const int group = num_heads / num_kv_heads;
-  const bool fast_ok = dtype != MVLLM_F32 && head_dim == 128 && block_size % kTile == 0 && group <= 8 &&
+  const bool fast_ok = dtype != MVLLM_F32 && head_dim == 128 && block_size % kTile == 0 && group <= 16 &&
                        aligned16(q) && aligned16(out) && aligned16(k_cache) && aligned16(v_cache) &&
                        (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
   hipStream_t s = (hipStream_t)stream;

@@ -47,8 +47,11 @@ def test_config1_fp32_elementwise():
     (32, 8, 256, 1500),    # big blocks
     (16, 8, 16, 255),      # GQA 2, single partition (direct output)
     (8, 8, 32, 300),       # MHA
-    (32, 4, 16, 600),      # GQA 8 (two head chunks)
+    (32, 4, 16, 600),      # GQA 8
     (6, 2, 48, 500),       # GQA 3, block size not a power of two
+    (16, 1, 16, 900),      # MQA with 16 heads: every column of the score product is a live head
+    (24, 2, 32, 400),      # GQA 12: live heads in three of the four accumulator row groups
+    (5, 1, 16, 300),       # GQA 5: live heads end inside a row group
 ])
 def test_fast_path_vs_oracle(dtype, hq, hkv, bs, ctx_hi):
     d = 128
