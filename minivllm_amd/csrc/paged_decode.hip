@@ -14,7 +14,7 @@
 //     O[16 head x 128]    += P (the scores' own layout, packed to 16 bit) x V; V rows are
 //                            loaded fully coalesced (lane l: tokens 4*(l/16)+i, dims 8*(l%16)..)
 //                            and two byte permutes per product turn them into the B operand.
-//   See decode_mfma_item for the operand layouts.
+//   See DecodeHead for the operand layouts.
 // The kernel is HBM-bound: a kernel that only issues the same loads (no arithmetic) reaches
 // 6.25 TB/s on this access pattern, this one about 6.05.
 #include "common.h"
@@ -162,24 +162,15 @@ template <> __device__ __forceinline__ v4f mfma16x16x16<f16_t>(uint2 x, uint2 y,
 //                    column n of product e is dim 8 n + e, and two byte permutes per product gather the four
 //                    tokens' values of that dim.  Lane l ends with O[head 4*(l/16)+j][dims 8*(l%16) + e].
 template <typename T>
-__device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int p, int g) {   // g: kv head
-  constexpr int D = 128;
-  const int lane = threadIdx.x & 63;
-  const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head (<= 16)
-  const int col = lane & 15;                           // head (first product), dim group (second product)
-  const int cls = lane >> 4;                           // token class: tokens 4*cls .. 4*cls+3 of a tile
+struct DecodeHead {
+  uint4 qf[4];                // Q fragments: B operand, column n = head n, k = 8*cls + 32 j
+  float m;                    // running maximum of head `col` (log2 units), the same in its four lanes
+  float l;                    // this lane's share of the head's denominator
+  v4f o[8];                   // o[e][j] = O[head 4*cls + j][dim 8*col + e]
 
-  const int ctx = (int)load_ctx(a, b);
-  // a sequence that fits one partition (or is empty) is finished here: partition 0 writes the output row
-  const bool direct = ctx <= a.part_tokens;
-  const int part_start = p * a.part_tokens;
-  if (part_start >= ctx && !(direct && p == 0)) return;
-  const int part_end = min(ctx, part_start + a.part_tokens);
-  const int ntiles = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
-
-  // Q fragments: B operand, column n = head n, k = 8*cls + 32 j
-  uint4 qf[4];
-  {
+  __device__ __forceinline__ void start(const DecodeArgs& a, int b, int g, int group, int lane) {
+    constexpr int D = 128;
+    const int col = lane & 15, cls = lane >> 4;
     const T* q = reinterpret_cast<const T*>(a.q);
     const bool live = col < group;
     const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D + cls * 8;
@@ -188,59 +179,15 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
       const uint4 x = *reinterpret_cast<const uint4*>(src + 32 * j);
       qf[j] = live ? x : make_uint4(0u, 0u, 0u, 0u);
     }
+    m = -INFINITY;
+    l = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
   }
-  float m = -INFINITY;        // running maximum of head `col` (log2 units), the same in its four lanes
-  float l = 0.f;              // this lane's share of the head's denominator
-  v4f o[8];                   // o[e][j] = O[head 4*cls + j][dim 8*col + e]
-#pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  const int bs = a.block_size;
-  const int64_t row = (int64_t)a.num_kv_heads * D;       // elements per token row
-  const T* kc = reinterpret_cast<const T*>(a.k_cache) + (int64_t)g * D;
-  const T* vc = reinterpret_cast<const T*>(a.v_cache) + (int64_t)g * D;
-  const int32_t* table = a.block_tables + (int64_t)b * a.max_num_blocks;
-
-  // Block-table window: lane i holds entry (win_base + i) of this sequence.
-  int bi = part_start / bs;          // logical block of the next tile to load
-  int off = part_start - bi * bs;    // token offset inside that block
-  int win_base = bi;
-  int win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
-
-  const int k_lane_off = col * (int)row + cls * 8;        // token lane%16, dims 8*(lane/16)
-  const int v_lane_off = 4 * cls * (int)row + col * 8;    // token 4*(lane/16), dims 8*(lane%16)
-
-  auto load_tile = [&](KVTile<T>& t, int tile) {
-    t.t0 = part_start + tile * kTile;
-    if (bi - win_base >= 64) {
-      win_base = bi;
-      win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
-    }
-    const int phys = __builtin_amdgcn_readlane(win, bi - win_base);
-    t.ok = (bi < a.max_num_blocks) && phys >= 0 && (int64_t)phys < a.num_blocks;
-    if (t.ok) {
-      const int64_t base = ((int64_t)phys * bs + off) * row;
-      const T* kp = kc + base + k_lane_off;
-      const T* vp = vc + base + v_lane_off;
-      // V is read once, in whole 256-byte rows per instruction: non-temporal loads stream it past the caches.
-      // K is read in the MFMA operand layout, 64 bytes of a row per instruction, so the second half of each
-      // 128-byte line has to survive in cache until the next instruction: ordinary loads (the hint costs 7 %
-      // there).
-#pragma unroll
-      for (int j = 0; j < 4; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) t.v[i] = load16_stream(vp + (int64_t)i * row);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
-    }
-    off += kTile;
-    if (off >= bs) { off = 0; ++bi; }
-  };
-
-  auto consume = [&](const KVTile<T>& t) {
+  // one tile of 16 tokens starting at token t0 of the sequence; tokens at or past part_end do not count
+  __device__ __forceinline__ void consume(const KVTile<T>& t, int part_end, float scale_log2, int lane) {
+    const int cls = lane >> 4;
     const int tok_base = t.t0 + 4 * cls;
     const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
     v4f s = {0.f, 0.f, 0.f, 0.f};
@@ -248,7 +195,7 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
     for (int j = 0; j < 4; ++j) s = mfma16x16x32<T>(t.k[j], qf[j], s);
     float s2[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) s2[i] = s[i] * a.scale_log2;
+    for (int i = 0; i < 4; ++i) s2[i] = s[i] * scale_log2;
     uint4 v[4] = {t.v[0], t.v[1], t.v[2], t.v[3]};
     if (partial) {
 #pragma unroll
@@ -296,6 +243,109 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
       const uint2 vb = make_uint2(__builtin_amdgcn_perm(c1, c0, sel), __builtin_amdgcn_perm(c3, c2, sel));
       o[e] = mfma16x16x16<T>(pa, vb, o[e]);
     }
+  }
+
+  // write the output row (direct) or this partition's partial result
+  __device__ __forceinline__ void finish(const DecodeArgs& a, int b, int p, int g, int group, bool direct, int lane) {
+    constexpr int D = 128;
+    const int col = lane & 15, cls = lane >> 4;
+    // denominators: add the four token classes (every lane of a head then holds the head's total)
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int head0 = g * group;
+    if (direct) {
+      T* out = reinterpret_cast<T*>(a.out);
+      const float linv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int h = 4 * cls + j;
+        const float lj = __shfl(linv, h, 64);               // lane h (class 0) holds head h
+        if (h < group) {
+          T r[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) r[e] = from_float<T>(o[e][j] * lj);
+          *reinterpret_cast<uint4*>(out + ((int64_t)b * a.num_heads + head0 + h) * D + col * 8) =
+              *reinterpret_cast<const uint4*>(r);
+        }
+      }
+    } else {
+      const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int h = 4 * cls + j;
+        if (h < group) {
+          float* dst = a.ws_acc + (slot + h) * D + col * 8;
+          *reinterpret_cast<float4*>(dst) = make_float4(o[0][j], o[1][j], o[2][j], o[3][j]);
+          *reinterpret_cast<float4*>(dst + 4) = make_float4(o[4][j], o[5][j], o[6][j], o[7][j]);
+        }
+      }
+      if (lane < group && lane < 16) *reinterpret_cast<float2*>(a.ws_ml + (slot + lane) * 2) = make_float2(m, l);
+    }
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int p, int g) {   // g: kv head
+  constexpr int D = 128;
+  const int lane = threadIdx.x & 63;
+  const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head (<= 16)
+  const int col = lane & 15;                           // head (first product), dim group (second product)
+  const int cls = lane >> 4;                           // token class: tokens 4*cls .. 4*cls+3 of a tile
+
+  const int ctx = (int)load_ctx(a, b);
+  // a sequence that fits one partition (or is empty) is finished here: partition 0 writes the output row
+  const bool direct = ctx <= a.part_tokens;
+  const int part_start = p * a.part_tokens;
+  if (part_start >= ctx && !(direct && p == 0)) return;
+  const int part_end = min(ctx, part_start + a.part_tokens);
+  const int ntiles = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
+
+  DecodeHead<T> head;
+  head.start(a, b, g, group, lane);
+
+  const int bs = a.block_size;
+  const int64_t row = (int64_t)a.num_kv_heads * D;       // elements per token row
+  const T* kc = reinterpret_cast<const T*>(a.k_cache) + (int64_t)g * D;
+  const T* vc = reinterpret_cast<const T*>(a.v_cache) + (int64_t)g * D;
+  const int32_t* table = a.block_tables + (int64_t)b * a.max_num_blocks;
+
+  // Block-table window: lane i holds entry (win_base + i) of this sequence.
+  int bi = part_start / bs;          // logical block of the next tile to load
+  int off = part_start - bi * bs;    // token offset inside that block
+  int win_base = bi;
+  int win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
+
+  const int k_lane_off = col * (int)row + cls * 8;        // token lane%16, dims 8*(lane/16)
+  const int v_lane_off = 4 * cls * (int)row + col * 8;    // token 4*(lane/16), dims 8*(lane%16)
+
+  auto load_tile = [&](KVTile<T>& t, int tile) {
+    t.t0 = part_start + tile * kTile;
+    if (bi - win_base >= 64) {
+      win_base = bi;
+      win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
+    }
+    const int phys = __builtin_amdgcn_readlane(win, bi - win_base);
+    t.ok = (bi < a.max_num_blocks) && phys >= 0 && (int64_t)phys < a.num_blocks;
+    if (t.ok) {
+      const int64_t base = ((int64_t)phys * bs + off) * row;
+      const T* kp = kc + base + k_lane_off;
+      const T* vp = vc + base + v_lane_off;
+      // V is read once, in whole 256-byte rows per instruction: non-temporal loads stream it past the caches.
+      // K is read in the MFMA operand layout, 64 bytes of a row per instruction, so the second half of each
+      // 128-byte line has to survive in cache until the next instruction: ordinary loads (the hint costs 7 %
+      // there).
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.v[i] = load16_stream(vp + (int64_t)i * row);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    off += kTile;
+    if (off >= bs) { off = 0; ++bi; }
   };
 
   // Tiles in pairs (ta, tb: one consumed while the other is in flight), the odd one after the loop.  A single
@@ -306,44 +356,12 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
   int tile = 0;
   for (; tile + 1 < ntiles; tile += 2) {
     load_tile(tb, tile + 1);
-    consume(ta);
+    head.consume(ta, part_end, a.scale_log2, lane);
     if (tile + 2 < ntiles) load_tile(ta, tile + 2);
-    consume(tb);
+    head.consume(tb, part_end, a.scale_log2, lane);
   }
-  if (tile < ntiles) consume(ta);
-
-  // denominators: add the four token classes (every lane of a head then holds the head's total)
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  const int head0 = g * group;
-  if (direct) {
-    T* out = reinterpret_cast<T*>(a.out);
-    const float linv = l > 0.f ? 1.f / l : 0.f;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int h = 4 * cls + j;
-      const float lj = __shfl(linv, h, 64);               // lane h (class 0) holds head h
-      if (h < group) {
-        T r[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) r[e] = from_float<T>(o[e][j] * lj);
-        *reinterpret_cast<uint4*>(out + ((int64_t)b * a.num_heads + head0 + h) * D + col * 8) =
-            *reinterpret_cast<const uint4*>(r);
-      }
-    }
-  } else {
-    const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int h = 4 * cls + j;
-      if (h < group) {
-        float* dst = a.ws_acc + (slot + h) * D + col * 8;
-        *reinterpret_cast<float4*>(dst) = make_float4(o[0][j], o[1][j], o[2][j], o[3][j]);
-        *reinterpret_cast<float4*>(dst + 4) = make_float4(o[4][j], o[5][j], o[6][j], o[7][j]);
-      }
-    }
-    if (lane < group && lane < 16) *reinterpret_cast<float2*>(a.ws_ml + (slot + lane) * 2) = make_float2(m, l);
-  }
+  if (tile < ntiles) head.consume(ta, part_end, a.scale_log2, lane);
+  head.finish(a, b, p, g, group, direct, lane);
 }
 
 // ---------------------------------------------------------------------------
