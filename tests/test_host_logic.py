@@ -54,3 +54,19 @@ def test_prefill_without_cu_seqlens_raises_value_error():
     with pytest.raises(ValueError):
         a(torch.zeros(1, 3, 4, 8), torch.zeros(1, 3, 2, 8), torch.zeros(1, 3, 2, 8))
     reset_context()
+
+
+def test_bench_refuses_more_than_one_gpu_and_a_machine_without_one():
+    """bench.py measures one GPU: --gpus above 1 exits with a message; without a GPU it says so instead of
+    timing anything else (there is no CPU path to fall back to)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in (r.stdout + r.stderr)
+    import torch
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "1", "--warmup", "0"],
+                           capture_output=True, text=True)
+        assert r.returncode != 0 and "no GPU" in (r.stdout + r.stderr)
