@@ -365,45 +365,50 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
 }
 
 // ---------------------------------------------------------------------------
-// Fast path, INT8 cache (head_dim 128, block_size % 16 == 0).  Same decomposition as the 16-bit kernel.
-//   QK^T   runs on v_mfma_i32_16x16x64_i8 with the int8 codes as they lie in memory (lane = token,
-//          16 bytes = 16 dims): the query row is turned once per wave into 15-bit fixed point
-//          q ~ (128*hi + lo) * amax/16256 with int8 hi/lo planes, so scores are exact integer dot
-//          products times (amax/16256) * k_scale[token];
-//   PV     on the VALU, two tokens per instruction: the codes, biased by +128 (one xor per 4 codes), of a
-//          lane's two V rows are paired per dim as fp16 (1024 + u_a, 1024 + u_b) (v_perm + or of the exponent
-//          bits), the weights p * v_scale of the two tokens as an fp16 pair, and v_dot2_f32_f16 accumulates both
-//          in fp32; the bias is taken out at the end as 1152 * sum(weights).  The running maximum is kept over
-//          score + log2 v_scale, so weights lie in (0, 2^8] for any scales;
+// Fast path, INT8 cache (head_dim 128, block_size % 16 == 0, up to 16 query heads per kv head).  Same
+// decomposition as the 16-bit kernel, both products on the matrix unit.
+//   QK^T   v_mfma_i32_16x16x64_i8 with the int8 codes as they lie in memory (lane = token, 16 bytes = 16 dims):
+//          the query row is turned once per wave into 15-bit fixed point q ~ (128*hi + lo) * amax/16256 with
+//          int8 hi/lo planes (column n = head n), so scores are exact integer dot products times
+//          (amax/16256) * k_scale[token]; lane l holds S[token 4*(l/16)+r][head l%16].
+//   PV     v_mfma_f32_16x16x16_f16, as in the 16-bit kernel: A = the weights p * v_scale of the lane's four
+//          tokens as fp16, B = V with k = the same four tokens and column n = one dim per lane.  V rows are 128 B;
+//          a lane loads 8 bytes = 8 dims of each of its four tokens (lane l: tokens 4*(l/16)+i, dims 8*(l%16)..,
+//          whole rows per instruction).  The codes are biased by +128 (one xor per 4 codes) and the byte of dim e
+//          of two tokens becomes the fp16 pair (1024 + u_a, 1024 + u_b) with v_perm + an or of the exponent bits
+//          (0x6400 | u is exactly 1024 + u): four vector instructions per product, column n of product e is dim
+//          8 n + e.  The 1024 + 128 leaves at the end as 1152 * sum(weights).  The running maximum is kept over
+//          score + log2 v_scale, so weights lie in (0, 2^8] for any scales and fit fp16.
 //   scales one k_scale and one v_scale load per lane and tile (lane l%4 of a quad holds token 4*(l/16)+l%4),
 //          handed round inside the quad by DPP.
-// V rows are 128 B, so one 16-byte load per lane covers 8 rows: lane l reads token 4*(l/16) + 2i + (l%16)/8,
-// dims 16*(l%8).. in instruction i = 0, 1.
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(4))) int v4i;
 typedef __attribute__((ext_vector_type(2))) _Float16 v2f16;
 typedef __attribute__((ext_vector_type(2))) float v2f;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
 struct KVTileI8 {
   uint4 k[2];
-  uint4 v[2];
+  uint2 v[4];
   float ks;
   float vs;
   int t0;
   bool ok;
 };
 
-template <int SEL> __device__ __forceinline__ float byte_to_float(uint32_t w) {
-  return (float)((w >> (8 * SEL)) & 0xffu);      // v_cvt_f32_ubyteN
+__device__ __forceinline__ uint2 load8_stream(const void* p) {
+  const u32x2 x = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+  return make_uint2(x.x, x.y);
 }
 
 template <typename T, int NCH>
 __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b, int p, int g) {   // g: kv head
+  static_assert(NCH == 1, "one chunk of up to 16 heads");
   constexpr int D = 128;
   const int lane = threadIdx.x & 63;
   const int group = a.num_heads / a.num_kv_heads;
   const int q4 = lane >> 4;            // token class: tokens 4*q4 .. 4*q4+3 of a tile
-  const int hb = (lane >> 3) & 1;      // which of the two V rows of an instruction this lane reads
+  const int col = lane & 15;           // head (first product), dim group (second product)
 
   const int ctx = (int)load_ctx(a, b);
   // a sequence that fits one partition (or is empty) is finished here: partition 0 writes the output row
@@ -413,55 +418,48 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
   const int part_end = min(ctx, part_start + a.part_tokens);
   const int ntiles = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
 
-  // ---- query -> int8 hi/lo planes (B operand: column lane%16 -> head lane%4, bytes 16*q4.. of each 64-dim step)
-  v4i qhi[NCH][2], qlo[NCH][2];
-  float qscale[NCH];                   // amax/16256 * scale*log2e of head (lane%4) of chunk c
+  // ---- query -> int8 hi/lo planes (B operand: column lane%16 -> head, bytes 16*q4.. of each 64-dim step)
+  v4i qhi[2], qlo[2];
+  float qscale;                        // amax/16256 * scale*log2e of this lane's head
   {
     const T* q = reinterpret_cast<const T*>(a.q);
+    const bool live = col < group;
+    const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D;
+    float x[2][16];
+    float amax = 0.f;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int hl = c * 4 + (lane & 3);
-      const bool live = hl < group;
-      const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? hl : 0)) * D;
-      float x[2][16];
-      float amax = 0.f;
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          x[j][e] = live ? to_float(src[64 * j + 16 * q4 + e]) : 0.f;
-          amax = fmaxf(amax, fabsf(x[j][e]));
-        }
-      amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-      const float to_fix = amax > 0.f ? 16256.f / amax : 0.f;
-      qscale[c] = amax * (1.f / 16256.f) * a.scale_log2;
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        int hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int q16 = (int)rintf(x[j][e] * to_fix);            // |q16| <= 16256
-          const int l8 = ((q16 + 64) & 127) - 64;                  // [-64, 63]
-          const int h8 = (q16 - l8) >> 7;                          // [-127, 127]
-          hi[e >> 2] |= (h8 & 0xff) << (8 * (e & 3));
-          lo[e >> 2] |= (l8 & 0xff) << (8 * (e & 3));
-        }
-        qhi[c][j] = (v4i){hi[0], hi[1], hi[2], hi[3]};
-        qlo[c][j] = (v4i){lo[0], lo[1], lo[2], lo[3]};
+      for (int e = 0; e < 16; ++e) {
+        x[j][e] = live ? to_float(src[64 * j + 16 * q4 + e]) : 0.f;
+        amax = fmaxf(amax, fabsf(x[j][e]));
       }
+    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+    const float to_fix = amax > 0.f ? 16256.f / amax : 0.f;
+    qscale = amax * (1.f / 16256.f) * a.scale_log2;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      int hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int q16 = (int)rintf(x[j][e] * to_fix);            // |q16| <= 16256
+        const int l8 = ((q16 + 64) & 127) - 64;                  // [-64, 63]
+        const int h8 = (q16 - l8) >> 7;                          // [-127, 127]
+        hi[e >> 2] |= (h8 & 0xff) << (8 * (e & 3));
+        lo[e >> 2] |= (l8 & 0xff) << (8 * (e & 3));
+      }
+      qhi[j] = (v4i){hi[0], hi[1], hi[2], hi[3]};
+      qlo[j] = (v4i){lo[0], lo[1], lo[2], lo[3]};
     }
   }
 
-  float m[NCH], l[NCH], wsum[NCH], acc[NCH][4][16];
+  float m = -INFINITY;      // running maximum of score + log2 v_scale of head `col`, the same in its four lanes
+  float l = 0.f;            // this lane's share of the denominator (its four tokens)
+  float wsum = 0.f;         // this lane's share of the sum of weights as the second product uses them
+  v4f o[8];                 // o[e][j] = O[head 4*q4 + j][dim 8*col + e] (+ the bias)
 #pragma unroll
-  for (int c = 0; c < NCH; ++c) {
-    m[c] = -INFINITY; l[c] = 0.f; wsum[c] = 0.f;
-#pragma unroll
-    for (int h = 0; h < 4; ++h)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[c][h][e] = 0.f;
-  }
+  for (int e = 0; e < 8; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
 
   const int bs = a.block_size;
   const int64_t row = (int64_t)a.num_kv_heads * D;          // bytes per token row
@@ -472,9 +470,9 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
   int off = part_start - bi * bs;
   int win_base = bi;
   int win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
-  const int k_lane_off = (lane & 15) * (int)row + q4 * 16;                      // token lane%16, bytes 16*q4 (+64 j)
-  const int v_lane_off = (4 * q4 + hb) * (int)row + (lane & 7) * 16;            // token 4*q4 + hb (+2 i), dims 16*(lane%8)
-  const int s_lane_tok = 4 * q4 + (lane & 3);                                   // token whose scales this lane loads
+  const int k_lane_off = col * (int)row + q4 * 16;          // token lane%16, bytes 16*q4 (+64 j)
+  const int v_lane_off = 4 * q4 * (int)row + col * 8;       // tokens 4*q4 + i, dims 8*(lane%16)
+  const int s_lane_tok = 4 * q4 + (lane & 3);               // token whose scales this lane loads
 
   auto load_tile = [&](KVTileI8& t, int tile) {
     t.t0 = part_start + tile * kTile;
@@ -490,13 +488,15 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
       const char* vp = vc + tok0 * row + v_lane_off;
       t.k[0] = *reinterpret_cast<const uint4*>(kp);
       t.k[1] = *reinterpret_cast<const uint4*>(kp + 64);
-      t.v[0] = load16_stream(vp);
-      t.v[1] = load16_stream(vp + 2 * row);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.v[i] = load8_stream(vp + i * row);
       const int64_t sidx = (tok0 + s_lane_tok) * a.num_kv_heads + g;
       t.ks = a.k_scale[sidx];
       t.vs = a.v_scale[sidx];
     } else {
-      t.k[0] = t.k[1] = t.v[0] = t.v[1] = make_uint4(0u, 0u, 0u, 0u);
+      t.k[0] = t.k[1] = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.v[i] = make_uint2(0u, 0u);
       t.ks = t.vs = 0.f;
     }
     off += kTile;
@@ -519,170 +519,106 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
     float lv4[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) lv4[r] = __log2f(fmaxf(vs4[r], 9.094947e-13f));
-    uint32_t wpk[NCH];                 // fp16 pair: weights of this lane's two V rows, for its own head
+    v4i shi = {0, 0, 0, 0}, slo = {0, 0, 0, 0};
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      v4i shi = {0, 0, 0, 0}, slo = {0, 0, 0, 0};
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const v4i kf = (v4i){(int)t.k[j].x, (int)t.k[j].y, (int)t.k[j].z, (int)t.k[j].w};
-        shi = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qhi[c][j], shi, 0, 0, 0);
-        slo = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qlo[c][j], slo, 0, 0, 0);
-      }
-      float s2[4], t2[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        s2[r] = (float)(shi[r] * 128 + slo[r]) * (qscale[c] * ks4[r]);
-        if (partial && (!t.ok || tok_base + r >= part_end)) s2[r] = -INFINITY;
-        t2[r] = s2[r] + lv4[r];
-      }
-      const float tile_max = fmaxf(fmaxf(t2[0], t2[1]), fmaxf(t2[2], t2[3]));
-      const bool grow = tile_max > m[c] + kLazyRescale || (m[c] == -INFINITY && tile_max > -INFINITY);
-      if (__any(grow)) {
-        const float m_new = grow ? tile_max : m[c];
-        const float al = (m_new == m[c]) ? 1.f : safe_exp2_diff(m[c], m_new);
-        l[c] *= al;
-        wsum[c] *= al;
-        const float a4[4] = {quad_bcast<0>(al), quad_bcast<1>(al), quad_bcast<2>(al), quad_bcast<3>(al)};
-#pragma unroll
-        for (int h = 0; h < 4; ++h)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) acc[c][h][e] *= a4[h];
-        m[c] = m_new;
-      }
-      const float m_eff = (m[c] == -INFINITY) ? 0.f : m[c];
-      float wr[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        l[c] += fast_exp2(s2[r] - m_eff);          // softmax denominator, in the same units as the weights / v_scale
-        wr[r] = fast_exp2(t2[r] - m_eff);
-      }
-      // this lane's V rows are tokens hb and 2 + hb of its token class
-      v2f wab = {hb ? wr[1] : wr[0], hb ? wr[3] : wr[2]};
-      const v2f16 wh = __builtin_convertvector(wab, v2f16);
-      wsum[c] += (float)wh[0] + (float)wh[1];      // of the weights as they are used
-      wpk[c] = __builtin_bit_cast(uint32_t, wh);
+    for (int j = 0; j < 2; ++j) {
+      const v4i kf = (v4i){(int)t.k[j].x, (int)t.k[j].y, (int)t.k[j].z, (int)t.k[j].w};
+      shi = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qhi[j], shi, 0, 0, 0);
+      slo = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qlo[j], slo, 0, 0, 0);
     }
-    // V codes biased to 0..255, two tokens per register as the fp16 pair (1024 + u_a, 1024 + u_b): 0x6400 | u is
-    // exactly 1024 + u.  One v_dot2 then adds both tokens' contribution for one dim and head; the 1024 + 128 is
-    // taken out at the end as 1152 * sum(weights).
-    const uint32_t va[4] = {t.v[0].x ^ 0x80808080u, t.v[0].y ^ 0x80808080u, t.v[0].z ^ 0x80808080u, t.v[0].w ^ 0x80808080u};
-    const uint32_t vb[4] = {t.v[1].x ^ 0x80808080u, t.v[1].y ^ 0x80808080u, t.v[1].z ^ 0x80808080u, t.v[1].w ^ 0x80808080u};
-    v2f16 vp[16];
+    float s2[4], t2[4];
 #pragma unroll
-    for (int d4 = 0; d4 < 4; ++d4) {
-      vp[4 * d4 + 0] = __builtin_bit_cast(v2f16, __builtin_amdgcn_perm(vb[d4], va[d4], 0x0c040c00u) | 0x64006400u);
-      vp[4 * d4 + 1] = __builtin_bit_cast(v2f16, __builtin_amdgcn_perm(vb[d4], va[d4], 0x0c050c01u) | 0x64006400u);
-      vp[4 * d4 + 2] = __builtin_bit_cast(v2f16, __builtin_amdgcn_perm(vb[d4], va[d4], 0x0c060c02u) | 0x64006400u);
-      vp[4 * d4 + 3] = __builtin_bit_cast(v2f16, __builtin_amdgcn_perm(vb[d4], va[d4], 0x0c070c03u) | 0x64006400u);
+    for (int r = 0; r < 4; ++r) {
+      s2[r] = (float)(shi[r] * 128 + slo[r]) * (qscale * ks4[r]);
+      if (partial && (!t.ok || tok_base + r >= part_end)) s2[r] = -INFINITY;
+      t2[r] = s2[r] + lv4[r];
     }
+    const float tile_max = fmaxf(fmaxf(t2[0], t2[1]), fmaxf(t2[2], t2[3]));
+    const bool grow = tile_max > m + kLazyRescale || (m == -INFINITY && tile_max > -INFINITY);
+    if (__any(grow)) {
+      // the head's maximum over its four token classes, then one decision for all four lanes
+      float mh = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+      mh = fmaxf(mh, __shfl_xor(mh, 32, 64));
+      const bool grow_h = mh > m + kLazyRescale || (m == -INFINITY && mh > -INFINITY);
+      const float m_new = grow_h ? mh : m;
+      const float al = (m_new == m) ? 1.f : safe_exp2_diff(m, m_new);
+      l *= al;
+      wsum *= al;
+      m = m_new;
+      // accumulator row j is head 4*q4 + j, whose factor sits in lane 4*q4 + j (any class would do)
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const v2f16 w0 = __builtin_bit_cast(v2f16, __builtin_amdgcn_update_dpp(0, (int)wpk[c], 0 * 0x55, 0xf, 0xf, false));
-      const v2f16 w1 = __builtin_bit_cast(v2f16, __builtin_amdgcn_update_dpp(0, (int)wpk[c], 1 * 0x55, 0xf, 0xf, false));
-      const v2f16 w2 = __builtin_bit_cast(v2f16, __builtin_amdgcn_update_dpp(0, (int)wpk[c], 2 * 0x55, 0xf, 0xf, false));
-      const v2f16 w3 = __builtin_bit_cast(v2f16, __builtin_amdgcn_update_dpp(0, (int)wpk[c], 3 * 0x55, 0xf, 0xf, false));
+      for (int j = 0; j < 4; ++j) {
+        const float aj = __shfl(al, 4 * q4 + j, 64);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        acc[c][0][e] = __builtin_amdgcn_fdot2(w0, vp[e], acc[c][0][e], false);
-        acc[c][1][e] = __builtin_amdgcn_fdot2(w1, vp[e], acc[c][1][e], false);
-        acc[c][2][e] = __builtin_amdgcn_fdot2(w2, vp[e], acc[c][2][e], false);
-        acc[c][3][e] = __builtin_amdgcn_fdot2(w3, vp[e], acc[c][3][e], false);
+        for (int e = 0; e < 8; ++e) o[e][j] *= aj;
       }
+    }
+    const float m_eff = (m == -INFINITY) ? 0.f : m;
+    float wr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      l += fast_exp2(s2[r] - m_eff);          // softmax denominator, in the same units as the weights / v_scale
+      wr[r] = fast_exp2(t2[r] - m_eff);
+    }
+    const v2f16 w01 = __builtin_convertvector((v2f){wr[0], wr[1]}, v2f16);
+    const v2f16 w23 = __builtin_convertvector((v2f){wr[2], wr[3]}, v2f16);
+    wsum += ((float)w01[0] + (float)w01[1]) + ((float)w23[0] + (float)w23[1]);      // of the weights as they are used
+    const uint2 pa = make_uint2(__builtin_bit_cast(uint32_t, w01), __builtin_bit_cast(uint32_t, w23));
+    // V codes biased to 0..255; the byte of dim e of tokens (0, 1) and of tokens (2, 3) as fp16 pairs 1024 + u.
+    // Rows past the end hold arbitrary bytes, which are finite numbers here and meet a weight of zero.
+    const uint32_t v0[2] = {t.v[0].x ^ 0x80808080u, t.v[0].y ^ 0x80808080u};
+    const uint32_t v1[2] = {t.v[1].x ^ 0x80808080u, t.v[1].y ^ 0x80808080u};
+    const uint32_t v2[2] = {t.v[2].x ^ 0x80808080u, t.v[2].y ^ 0x80808080u};
+    const uint32_t v3[2] = {t.v[3].x ^ 0x80808080u, t.v[3].y ^ 0x80808080u};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t sel = 0x0c040c00u + 0x00010001u * (uint32_t)(e & 3);
+      const uint2 vb = make_uint2(__builtin_amdgcn_perm(v1[e >> 2], v0[e >> 2], sel) | 0x64006400u,
+                                  __builtin_amdgcn_perm(v3[e >> 2], v2[e >> 2], sel) | 0x64006400u);
+      o[e] = mfma16x16x16<f16_t>(pa, vb, o[e]);
     }
   };
 
+  // tiles in pairs, the odd one after the loop (see the 16-bit kernel)
   KVTileI8 ta, tb;
   if (ntiles > 0) load_tile(ta, 0);
   int tile = 0;
-  while (tile < ntiles) {
-    if (tile + 1 < ntiles) load_tile(tb, tile + 1);
+  for (; tile + 1 < ntiles; tile += 2) {
+    load_tile(tb, tile + 1);
     consume(ta);
-    ++tile;
-    if (tile >= ntiles) break;
-    if (tile + 1 < ntiles) load_tile(ta, tile + 1);
+    if (tile + 2 < ntiles) load_tile(ta, tile + 2);
     consume(tb);
-    ++tile;
   }
+  if (tile < ntiles) consume(ta);
 
-  // take the 1024 + 128 bias out, then fold the token classes: first the two V-row halves (same m, l), then lane/16
+  // denominators and weight sums over the four token classes (every lane of a head then holds the head's totals)
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  wsum += __shfl_xor(wsum, 16, 64);
+  wsum += __shfl_xor(wsum, 32, 64);
+  const int head0 = g * group;
+  const float linv = l > 0.f ? 1.f / l : 0.f;
+  const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
 #pragma unroll
-  for (int c = 0; c < NCH; ++c) {
-    const float b4[4] = {quad_bcast<0>(wsum[c]), quad_bcast<1>(wsum[c]), quad_bcast<2>(wsum[c]), quad_bcast<3>(wsum[c])};
+  for (int j = 0; j < 4; ++j) {
+    const int h = 4 * q4 + j;
+    const float bias = 1152.f * __shfl(wsum, h, 64);          // lane h (class 0) holds head h
+    const float lj = __shfl(linv, h, 64);
+    if (h < group) {
+      if (direct) {
+        T r[8];
 #pragma unroll
-    for (int h = 0; h < 4; ++h)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        float x = fmaf(-1152.f, b4[h], acc[c][h][e]);
-        x += __shfl_xor(x, 8, 64);
-        acc[c][h][e] = x;
-      }
-  }
-#pragma unroll
-  for (int offs = 16; offs <= 32; offs <<= 1) {
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const float mo = __shfl_xor(m[c], offs, 64);
-      const float lo = __shfl_xor(l[c], offs, 64);
-      const float mn = fmaxf(m[c], mo);
-      const float al = safe_exp2_diff(m[c], mn);
-      const float ao = safe_exp2_diff(mo, mn);
-      l[c] = l[c] * al + lo * ao;
-      m[c] = mn;
-      const float a4[4] = {quad_bcast<0>(al), quad_bcast<1>(al), quad_bcast<2>(al), quad_bcast<3>(al)};
-      const float o4[4] = {quad_bcast<0>(ao), quad_bcast<1>(ao), quad_bcast<2>(ao), quad_bcast<3>(ao)};
-#pragma unroll
-      for (int h = 0; h < 4; ++h)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const float other = __shfl_xor(acc[c][h][e], offs, 64);
-          acc[c][h][e] = acc[c][h][e] * a4[h] + other * o4[h];
-        }
-    }
-  }
-
-  // lanes 0..7 hold dims 16*lane.. of heads 0..3 of every chunk
-  if (lane < 8) {
-    const int head0 = g * group;
-    if (direct) {
-      T* out = reinterpret_cast<T*>(a.out);
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        const float linv = l[c] > 0.f ? 1.f / l[c] : 0.f;
-        const float li[4] = {quad_bcast<0>(linv), quad_bcast<1>(linv), quad_bcast<2>(linv), quad_bcast<3>(linv)};
-#pragma unroll
-        for (int h = 0; h < 4; ++h) {
-          if (c * 4 + h < group) {
-            T* dst = out + ((int64_t)b * a.num_heads + head0 + c * 4 + h) * D + lane * 16;
-            T o[16];
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o[e] = from_float<T>(acc[c][h][e] * li[h]);
-            reinterpret_cast<uint4*>(dst)[0] = reinterpret_cast<const uint4*>(o)[0];
-            reinterpret_cast<uint4*>(dst)[1] = reinterpret_cast<const uint4*>(o)[1];
-          }
-        }
-      }
-    } else {
-      const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-#pragma unroll
-        for (int h = 0; h < 4; ++h) {
-          if (c * 4 + h < group) {
-            float* dst = a.ws_acc + (slot + c * 4 + h) * D + lane * 16;
-#pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4)
-              reinterpret_cast<float4*>(dst)[e4] = make_float4(acc[c][h][4 * e4], acc[c][h][4 * e4 + 1],
-                                                               acc[c][h][4 * e4 + 2], acc[c][h][4 * e4 + 3]);
-          }
-        }
-        if (lane < 4 && c * 4 + lane < group) {
-          float* ml = a.ws_ml + (slot + c * 4 + lane) * 2;
-          *reinterpret_cast<float2*>(ml) = make_float2(m[c], l[c]);
-        }
+        for (int e = 0; e < 8; ++e) r[e] = from_float<T>((o[e][j] - bias) * lj);
+        *reinterpret_cast<uint4*>(reinterpret_cast<T*>(a.out) + ((int64_t)b * a.num_heads + head0 + h) * D + col * 8) =
+            *reinterpret_cast<const uint4*>(r);
+      } else {
+        float* dst = a.ws_acc + (slot + h) * D + col * 8;
+        *reinterpret_cast<float4*>(dst) = make_float4(o[0][j] - bias, o[1][j] - bias, o[2][j] - bias, o[3][j] - bias);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(o[4][j] - bias, o[5][j] - bias, o[6][j] - bias, o[7][j] - bias);
       }
     }
   }
+  if (!direct && lane < group && lane < 16) *reinterpret_cast<float2*>(a.ws_ml + (slot + lane) * 2) = make_float2(m, l);
 }
 
 // ---------------------------------------------------------------------------
@@ -878,7 +814,7 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stre
   const int group = a.num_heads / a.num_kv_heads;
   bool launched = false;
   if constexpr (IsSixteenBit<T>::value) {
-    if (fast_ok && (!int8 || group <= 4)) {
+    if (fast_ok) {
       // kv heads (waves) per workgroup: as many as allowed, so that a workgroup streams whole token rows;
       // fewer when the grid would otherwise leave most CUs without a workgroup
       int wpb = largest_divisor_le(a.num_kv_heads, int8 ? MVLLM_DECODE_I8_WPB : MVLLM_DECODE_WPB);

@@ -47,7 +47,8 @@ def _check(case, hq, hkv, d, bs, scale, ctx_dtype=torch.int64):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("hq,hkv,bs,ctx_hi", [(32, 8, 16, 700), (16, 8, 256, 1500), (8, 8, 32, 255), (6, 2, 48, 400)])
+@pytest.mark.parametrize("hq,hkv,bs,ctx_hi", [(32, 8, 16, 700), (16, 8, 256, 1500), (8, 8, 32, 255), (6, 2, 48, 400),
+                                              (32, 4, 16, 600), (16, 1, 32, 900), (24, 2, 16, 300), (5, 1, 64, 200)])
 def test_int8_fast_path(dtype, hq, hkv, bs, ctx_hi):
     d = 128
     _check(_quantised_case(61, 7, 1, ctx_hi, hq, hkv, d, bs, dtype), hq, hkv, d, bs, 1 / math.sqrt(d))
@@ -59,9 +60,9 @@ def test_int8_context_boundaries(ctx_list):
     _check(_quantised_case(62, 0, 0, 0, hq, hkv, d, bs, ctx_list=ctx_list), hq, hkv, d, bs, 0.1, torch.int32)
 
 
-@pytest.mark.parametrize("hq,hkv,d,bs", [(16, 16, 64, 16), (32, 4, 128, 16), (4, 2, 128, 8)])
+@pytest.mark.parametrize("hq,hkv,d,bs", [(16, 16, 64, 16), (34, 2, 128, 16), (4, 2, 128, 8)])
 def test_int8_generic_path(hq, hkv, d, bs):
-    """head_dim 64, GQA 8 and block_size 8 run on the generic kernel."""
+    """head_dim 64, GQA 17 and block_size 8 run on the generic kernel."""
     _check(_quantised_case(63, 5, 1, 300, hq, hkv, d, bs), hq, hkv, d, bs, 1 / math.sqrt(d))
 
 
