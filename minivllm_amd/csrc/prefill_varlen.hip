@@ -234,7 +234,7 @@ template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
 typedef __attribute__((ext_vector_type(4))) int v4i;
 template <int LDS_IMM>   // LDS destination = lds_base + LDS_IMM: one scalar register serves all copies of a wave
 __device__ __forceinline__ void dma16_to_lds(v4i rsrc, uint32_t lane_off, uint32_t lds_base) {
-  asm volatile("s_add_u32 m0, %0, %3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(lane_off), "s"(rsrc), "n"(LDS_IMM) : "scc");
+  asm volatile("s_add_u32 m0, %0, %3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(lane_off), "s"(rsrc), "n"(LDS_IMM) : "scc", "m0");
 }
 // Raw buffer descriptor: 48-bit base, stride 0, size in bytes, 32-bit untyped data.
 __device__ __forceinline__ v4i make_rsrc(const char* base, uint32_t bytes) {
