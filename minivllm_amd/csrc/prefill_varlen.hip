@@ -374,7 +374,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       const int rows_left = total_rows - row0;
       const uint32_t size = (!enable || rows_left <= 0) ? 0u
                             : rows_left > rows_4g       ? 0xffffffffu
-                                                        : (uint32_t)(rows_left * row_bytes - g * (D * 2));
+                                                        : (uint32_t)rows_left * (uint32_t)row_bytes - (uint32_t)(g * (D * 2));
       const int64_t start = (int64_t)row0 * kv_row_bytes + (int64_t)g * (D * 2);
       t.k = make_rsrc(kg + start, size);
       t.v = make_rsrc(vg + start, size);
