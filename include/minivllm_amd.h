@@ -91,6 +91,21 @@ size_t mvllm_paged_decode_workspace_bytes(int batch, int num_heads, int head_dim
                                           int max_num_blocks, int block_size);
 
 /*
+ * How mvllm_paged_decode{,_int8} split these static sizes (no counterpart in the reference, whose Triton kernel
+ * walks a whole context in one program, attention.py:283-415).  Pure host arithmetic:
+ *   *part_tokens      tokens of a partition; partition p of a sequence covers tokens [p, p+1) * part_tokens
+ *   *num_parts        partitions per sequence (1: no workspace is touched and no merge kernel is launched)
+ *   *waves_per_head   1: a workgroup holds up to 4 kv heads, one wave each, and every wave walks its partition;
+ *                     >1: small-batch form, a workgroup is that many waves on one kv head that share the
+ *                     partition's 16-token tiles and merge in LDS; 0: the generic kernel (fp32, head_dim != 128,
+ *                     block_size % 16 != 0 or more than 16 query heads per kv head)
+ * Returns MVLLM_OK or MVLLM_ERR_BAD_SHAPE / MVLLM_ERR_BAD_DTYPE.
+ */
+int mvllm_paged_decode_plan(int batch, int num_heads, int num_kv_heads, int head_dim,
+                            int max_num_blocks, int block_size, int dtype, int int8_cache,
+                            int* part_tokens, int* num_parts, int* waves_per_head);
+
+/*
  * paged_attention_decode -- src/myvllm/layers/attention.py:418-473 (kernel :283-415).
  * out[b,h,:] = softmax_t( scale * q[b,h,:] . K[b,t,g(h),:] ) V[b,t,g(h),:],
  * t in [0, context_lens[b]), g(h) = h / (Hq/Hkv); token t of sequence b lives at

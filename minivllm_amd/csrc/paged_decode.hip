@@ -97,6 +97,52 @@ __host__ __device__ inline int partition_tokens_for(int64_t max_ctx, int batch) 
   return (int)part;
 }
 
+inline int largest_divisor_le(int n, int cap) {
+  for (int d = cap; d >= 1; --d)
+    if (n % d == 0) return d;
+  return 1;
+}
+
+// Small batches (16-bit fast path).  The grid above needs many live (sequence, partition) pairs: when the batch
+// is small it shortens the partitions, every sequence then needs the second launch that merges them, and when the
+// contexts are much shorter than the block table is wide most of its workgroups are empty.  There a workgroup of
+// kSplitWaves waves takes one (sequence, partition, kv head) instead and its waves split the tiles
+// (decode_mfma_split_kernel); partitions are as long as still gives kSplitMinGroups workgroups, up to
+// kSplitMaxPart tokens, so that at common serving shapes (64 sequences x 8 kv heads, tables 4096 tokens wide) a
+// sequence is one workgroup and one launch.  It is chosen when partition_tokens_for could not reach its
+// 1024-token partitions, when the one-wave-per-head grid would have fewer workgroups than the GPU has CUs, and
+// for any batch when the table is at most kSplitMaxPart tokens wide (one partition, so never a second launch:
+// 256 sequences of 96-352 tokens in a 4096-token table 99 -> 45 us, all of 4096 tokens 661 -> 674 us).  With wider
+// tables and a large batch the first form is kept: it reads whole token rows and is up to 12 % faster when the
+// contexts are long, although up to 2x slower when they are much shorter than the table is wide, which the
+// host cannot know.
+// The partition is never shorter than partition_tokens_for's, so a workspace sized from it is always enough.
+#ifndef MVLLM_DECODE_SPLIT
+#define MVLLM_DECODE_SPLIT 1              // 0: never use the split kernel
+#endif
+#ifndef MVLLM_DECODE_SPLIT_WAVES
+#define MVLLM_DECODE_SPLIT_WAVES 4        // 8 waves: 1-3 us slower per call except at 16 sequences (merge cost, one workgroup per CU)
+#endif
+constexpr int kSplitWaves = MVLLM_DECODE_SPLIT_WAVES;
+constexpr int kSplitMinGroups = 512;
+constexpr int kSplitMaxPart = 4096;
+inline bool split_wanted(int64_t max_ctx, int batch, int num_kv_heads) {
+  if (!MVLLM_DECODE_SPLIT) return false;
+  if (MVLLM_DECODE_SPLIT == 2) return true;          // timing builds
+  const int part = partition_tokens_for(max_ctx, batch);
+  const int64_t parts = (max_ctx + part - 1) / part;
+  const int wpb = largest_divisor_le(num_kv_heads, MVLLM_DECODE_WPB);
+  return part < MVLLM_DECODE_PART_CAP || (int64_t)batch * parts * (num_kv_heads / wpb) < 256 || max_ctx <= kSplitMaxPart;
+}
+inline int split_partition_tokens(int64_t max_ctx, int batch, int num_kv_heads) {
+  const int64_t pairs = (int64_t)batch * num_kv_heads;
+  const int64_t want_parts = (kSplitMinGroups + pairs - 1) / pairs;
+  int64_t part = ((max_ctx + want_parts - 1) / want_parts + 63) / 64 * 64;
+  if (part > kSplitMaxPart) part = kSplitMaxPart;
+  const int64_t floor_part = partition_tokens_for(max_ctx, batch);
+  return (int)(part < floor_part ? floor_part : part);
+}
+
 __device__ __forceinline__ int64_t load_ctx(const DecodeArgs& a, int b) {
   int64_t c = a.ctx_is_i64 ? reinterpret_cast<const int64_t*>(a.context_lens)[b]
                            : (int64_t) reinterpret_cast<const int32_t*>(a.context_lens)[b];
@@ -253,6 +299,48 @@ struct DecodeHead {
     }
   }
 
+  // W waves hold partial results of the same heads over different tokens: waves 1 .. W-1 leave theirs in LDS
+  // (9 x 16 bytes per lane: m, l and the 8 x 4 accumulators), wave 0 folds them into its own with the usual
+  // log-sum-exp weights and is the only one to return true.  Every wave of the workgroup must call this.
+  template <int W>
+  __device__ __forceinline__ bool merge(int w, int lane) {
+    __shared__ float4 part[(W - 1) * 9 * 64];
+    const int cls = lane >> 4;
+    if (w > 0) {
+      float4* dst = part + (w - 1) * 9 * 64 + lane;
+      dst[0] = make_float4(m, l, 0.f, 0.f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dst[(1 + e) * 64] = make_float4(o[e][0], o[e][1], o[e][2], o[e][3]);
+    }
+    __syncthreads();
+    if (w > 0) return false;
+#pragma unroll 1
+    for (int x = 0; x < W - 1; ++x) {
+      const float4* src = part + x * 9 * 64 + lane;
+      const float4 ml = src[0];
+      const float m_new = fmaxf(m, ml.x);
+      const float f0 = safe_exp2_diff(m, m_new);          // both are 0 while neither wave has seen a token
+      const float f1 = safe_exp2_diff(ml.x, m_new);
+      m = m_new;
+      l = l * f0 + ml.y * f1;
+      float a0[4], a1[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {                        // accumulator row j is head 4*cls + j
+        a0[j] = __shfl(f0, 4 * cls + j, 64);
+        a1[j] = __shfl(f1, 4 * cls + j, 64);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float4 ow = src[(1 + e) * 64];
+        o[e][0] = o[e][0] * a0[0] + ow.x * a1[0];
+        o[e][1] = o[e][1] * a0[1] + ow.y * a1[1];
+        o[e][2] = o[e][2] * a0[2] + ow.z * a1[2];
+        o[e][3] = o[e][3] * a0[3] + ow.w * a1[3];
+      }
+    }
+    return true;
+  }
+
   // write the output row (direct) or this partition's partial result
   __device__ __forceinline__ void finish(const DecodeArgs& a, int b, int p, int g, int group, bool direct, int lane) {
     constexpr int D = 128;
@@ -292,42 +380,53 @@ struct DecodeHead {
   }
 };
 
-template <typename T>
-__device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int p, int g) {   // g: kv head
+// W = 1: the wave walks all tiles of its partition.  W > 1 (the workgroup is W waves on one kv head): wave w takes
+// tiles w, w + W, ... and the partial results meet in LDS (DecodeHead::merge), so a short context costs a few tiles
+// of latency per wave and no second launch.
+template <typename T, int W>
+__device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int p, int g, int w) {   // g: kv head
   constexpr int D = 128;
   const int lane = threadIdx.x & 63;
   const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head (<= 16)
   const int col = lane & 15;                           // head (first product), dim group (second product)
   const int cls = lane >> 4;                           // token class: tokens 4*cls .. 4*cls+3 of a tile
+  const int bs = a.block_size;
+  const int part_start = p * a.part_tokens;
+  const int first = part_start + (W == 1 ? 0 : w * kTile);      // first token of this wave's first tile
+  const int32_t* table = a.block_tables + (int64_t)b * a.max_num_blocks;
+
+  // The query rows and the block-table window (lane i holds entry win_base + i of this sequence) do not depend
+  // on the context length.  The split kernel, which is all latency, asks for them together with it; the
+  // one-wave form first drops the workgroups whose partition lies past the context (most of a ragged batch).
+  DecodeHead<T> head;
+  int bi = first / bs;               // logical block of the next tile to load
+  int off = first - bi * bs;         // token offset inside that block
+  int win_base = bi;
+  int win;
+  auto prologue = [&]() __attribute__((always_inline)) {
+    head.start(a, b, g, group, lane);
+    win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
+  };
+  if constexpr (W > 1) prologue();
 
   const int ctx = (int)load_ctx(a, b);
   // a sequence that fits one partition (or is empty) is finished here: partition 0 writes the output row
   const bool direct = ctx <= a.part_tokens;
-  const int part_start = p * a.part_tokens;
   if (part_start >= ctx && !(direct && p == 0)) return;
   const int part_end = min(ctx, part_start + a.part_tokens);
-  const int ntiles = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
+  const int tiles_all = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
+  const int ntiles = W == 1 ? tiles_all : (tiles_all > w ? (tiles_all - w + W - 1) / W : 0);   // this wave's
+  if constexpr (W == 1) prologue();
 
-  DecodeHead<T> head;
-  head.start(a, b, g, group, lane);
-
-  const int bs = a.block_size;
   const int64_t row = (int64_t)a.num_kv_heads * D;       // elements per token row
   const T* kc = reinterpret_cast<const T*>(a.k_cache) + (int64_t)g * D;
   const T* vc = reinterpret_cast<const T*>(a.v_cache) + (int64_t)g * D;
-  const int32_t* table = a.block_tables + (int64_t)b * a.max_num_blocks;
-
-  // Block-table window: lane i holds entry (win_base + i) of this sequence.
-  int bi = part_start / bs;          // logical block of the next tile to load
-  int off = part_start - bi * bs;    // token offset inside that block
-  int win_base = bi;
-  int win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
 
   const int k_lane_off = col * (int)row + cls * 8;        // token lane%16, dims 8*(lane/16)
   const int v_lane_off = 4 * cls * (int)row + col * 8;    // token 4*(lane/16), dims 8*(lane%16)
 
   auto load_tile = [&](KVTile<T>& t, int tile) {
-    t.t0 = part_start + tile * kTile;
+    t.t0 = first + tile * (W * kTile);
     if (bi - win_base >= 64) {
       win_base = bi;
       win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
@@ -352,8 +451,13 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
 #pragma unroll
       for (int i = 0; i < 4; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
     }
-    off += kTile;
-    if (off >= bs) { off = 0; ++bi; }
+    if constexpr (W == 1) {
+      off += kTile;
+      if (off >= bs) { off = 0; ++bi; }
+    } else {
+      off += W * kTile;
+      while (off >= bs) { off -= bs; ++bi; }
+    }
   };
 
   // Tiles in pairs (ta, tb: one consumed while the other is in flight), the odd one after the loop.  A single
@@ -369,6 +473,9 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
     head.consume(tb, part_end, a.scale_log2, lane);
   }
   if (tile < ntiles) head.consume(ta, part_end, a.scale_log2, lane);
+  if constexpr (W > 1) {
+    if (!head.template merge<W>(w, lane)) return;
+  }
   head.finish(a, b, p, g, group, direct, lane);
 }
 
@@ -637,7 +744,15 @@ template <typename T>
 __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_kernel(const DecodeArgs a) {
   int b, p, hg;
   if (!decode_item<false>(a, b, p, hg)) return;
-  decode_mfma_item<T>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6));
+  decode_mfma_item<T, 1>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
+}
+// Small batches: one workgroup of W waves per (partition, sequence, kv head), the waves splitting the tiles.
+template <typename T, int W>
+__global__ __launch_bounds__(64 * W, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_split_kernel(const DecodeArgs a) {
+  // kv head fastest: the workgroups of one (sequence, partition) start together and read the same token rows
+  const int g = blockIdx.x, b = blockIdx.z;
+  const int p = (int)((blockIdx.y + (unsigned)b) % (unsigned)a.num_parts);
+  decode_mfma_item<T, W>(a, b, p, g, threadIdx.x >> 6);
 }
 template <typename T, int NCH>
 __global__ __launch_bounds__(MVLLM_DECODE_I8_THREADS, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
@@ -799,12 +914,6 @@ __global__ __launch_bounds__(256) void decode_reduce_kernel(const DecodeArgs a) 
 // ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
-static int largest_divisor_le(int n, int cap) {
-  for (int d = cap; d >= 1; --d)
-    if (n % d == 0) return d;
-  return 1;
-}
-
 static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int max_num_blocks, int block_size) {
   if (batch <= 0 || num_heads <= 0 || head_dim <= 0 || max_num_blocks <= 0 || block_size <= 0) return 0;
   const int64_t max_ctx = (int64_t)max_num_blocks * block_size;
@@ -814,15 +923,38 @@ static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int ma
   return (size_t)batch * (size_t)np * (size_t)num_heads * (size_t)(head_dim + 2) * sizeof(float);
 }
 
+// shapes the MFMA kernels are built for (pointer alignment is checked by the caller)
+static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype) {
+  return dtype != MVLLM_F32 && head_dim == 128 && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
+         (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
+}
+
+struct DecodePlan {
+  int part_tokens, num_parts, waves_per_head;
+};
+static DecodePlan plan_decode(int batch, int num_kv_heads, int max_num_blocks, int block_size, bool fast_ok, bool int8) {
+  const int64_t max_ctx = (int64_t)max_num_blocks * block_size;
+  const bool split = fast_ok && !int8 && split_wanted(max_ctx, batch, num_kv_heads);
+  DecodePlan plan;
+  plan.part_tokens = split ? split_partition_tokens(max_ctx, batch, num_kv_heads) : partition_tokens_for(max_ctx, batch);
+  plan.num_parts = (int)((max_ctx + plan.part_tokens - 1) / plan.part_tokens);
+  plan.waves_per_head = !fast_ok ? 0 : split ? kSplitWaves : 1;
+  return plan;
+}
+
 template <typename T> struct IsSixteenBit { static constexpr bool value = true; };
 template <> struct IsSixteenBit<float> { static constexpr bool value = false; };
 
 template <typename T>
-static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, hipStream_t stream) {
+static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipStream_t stream) {
   const int group = a.num_heads / a.num_kv_heads;
   bool launched = false;
   if constexpr (IsSixteenBit<T>::value) {
-    if (fast_ok) {
+    if (fast_ok && split) {
+      decode_mfma_split_kernel<T, kSplitWaves><<<dim3((unsigned)a.num_kv_heads, (unsigned)a.num_parts, (unsigned)a.batch),
+                                                 dim3(64 * kSplitWaves), 0, stream>>>(a);
+      launched = true;
+    } else if (fast_ok) {
       // kv heads (waves) per workgroup: as many as allowed, so that a workgroup streams whole token rows;
       // fewer when the grid would otherwise leave most CUs without a workgroup
       int wpb = largest_divisor_le(a.num_kv_heads, int8 ? MVLLM_DECODE_I8_WPB : MVLLM_DECODE_WPB);
@@ -874,9 +1006,12 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
   a.num_blocks = num_blocks; a.ctx_is_i64 = ctx_is_i64; a.max_num_blocks = max_num_blocks;
   a.batch = batch; a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.head_dim = head_dim;
   a.block_size = block_size;
-  const int64_t max_ctx = (int64_t)max_num_blocks * block_size;
-  a.part_tokens = partition_tokens_for(max_ctx, batch);
-  a.num_parts = (int)((max_ctx + a.part_tokens - 1) / a.part_tokens);
+  const bool fast_ok = fast_shape(num_heads, num_kv_heads, head_dim, block_size, dtype) &&
+                       aligned16(q) && aligned16(out) && aligned16(k_cache) && aligned16(v_cache);
+  const DecodePlan plan = plan_decode(batch, num_kv_heads, max_num_blocks, block_size, fast_ok, int8);
+  const bool split = plan.waves_per_head > 1;
+  a.part_tokens = plan.part_tokens;
+  a.num_parts = plan.num_parts;
   a.scale_log2 = scale * kLog2e;
   a.ws_acc = nullptr; a.ws_ml = nullptr;
   if (a.num_parts > 1) {
@@ -885,15 +1020,11 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
     a.ws_acc = reinterpret_cast<float*>(workspace);
     a.ws_ml = a.ws_acc + (size_t)batch * a.num_parts * num_heads * head_dim;
   }
-  const int group = num_heads / num_kv_heads;
-  const bool fast_ok = dtype != MVLLM_F32 && head_dim == 128 && block_size % kTile == 0 && group <= 16 &&
-                       aligned16(q) && aligned16(out) && aligned16(k_cache) && aligned16(v_cache) &&
-                       (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case MVLLM_F32: return launch_decode<float>(a, int8, false, s);
-    case MVLLM_BF16: return launch_decode<bf16_t>(a, int8, fast_ok, s);
-    default: return launch_decode<f16_t>(a, int8, fast_ok, s);
+    case MVLLM_F32: return launch_decode<float>(a, int8, false, false, s);
+    case MVLLM_BF16: return launch_decode<bf16_t>(a, int8, fast_ok, split, s);
+    default: return launch_decode<f16_t>(a, int8, fast_ok, split, s);
   }
 }
 
@@ -904,6 +1035,21 @@ using namespace mvllm;
 extern "C" size_t mvllm_paged_decode_workspace_bytes(int batch, int num_heads, int head_dim,
                                                      int max_num_blocks, int block_size) {
   return workspace_bytes_for(batch, num_heads, head_dim, max_num_blocks, block_size);
+}
+
+extern "C" int mvllm_paged_decode_plan(int batch, int num_heads, int num_kv_heads, int head_dim, int max_num_blocks,
+                                       int block_size, int dtype, int int8_cache, int* part_tokens, int* num_parts,
+                                       int* waves_per_head) {
+  if (dtype_size(dtype) == 0) return MVLLM_ERR_BAD_DTYPE;
+  if (batch <= 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 || max_num_blocks <= 0 ||
+      num_heads % num_kv_heads != 0)
+    return MVLLM_ERR_BAD_SHAPE;
+  const DecodePlan plan = plan_decode(batch, num_kv_heads, max_num_blocks, block_size,
+                                      fast_shape(num_heads, num_kv_heads, head_dim, block_size, dtype), int8_cache != 0);
+  if (part_tokens) *part_tokens = plan.part_tokens;
+  if (num_parts) *num_parts = plan.num_parts;
+  if (waves_per_head) *waves_per_head = plan.waves_per_head;
+  return MVLLM_OK;
 }
 
 extern "C" int mvllm_paged_decode(void* out, const void* q, const void* k_cache, const void* v_cache,

@@ -220,6 +220,19 @@ def _decode_common(query, k_cache, v_cache, block_tables, context_lens, num_head
     return query.contiguous(), block_tables, context_lens
 
 
+def paged_decode_plan(batch: int, num_heads: int, num_kv_heads: int, head_dim: int, max_num_blocks: int,
+                      block_size: int, dtype: torch.dtype = torch.bfloat16, int8_cache: bool = False):
+    """(part_tokens, num_parts, waves_per_head) a decode call of these static sizes runs with (host arithmetic only).
+    waves_per_head: 1 = one wave per kv head walks a partition, >1 = the small-batch form (that many waves share
+    one kv head's partition), 0 = the generic kernel."""
+    import ctypes
+    out = [ctypes.c_int(0) for _ in range(3)]
+    st = _C.load().mvllm_paged_decode_plan(batch, num_heads, num_kv_heads, head_dim, max_num_blocks, block_size,
+                                           _C.dtype_code(dtype), int(int8_cache), *[ctypes.byref(x) for x in out])
+    _C.check(st, "paged_decode_plan")
+    return tuple(x.value for x in out)
+
+
 def paged_attention_decode(query: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                            block_tables: torch.Tensor, context_lens: torch.Tensor, scale: float,
                            num_heads: int, num_kv_heads: int, head_dim: int, block_size: int) -> torch.Tensor:

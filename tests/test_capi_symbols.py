@@ -27,7 +27,7 @@ def _lib():
 def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
-              "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_prefill_varlen",
+              "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_varlen",
               "mvllm_prefill_paged", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_workspace_bytes",
               "mvllm_add_rms_norm",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
@@ -53,6 +53,34 @@ def test_host_only_entry_points():
     assert lib.mvllm_paged_decode_workspace_bytes(8, 16, 128, 16, 16) == 8 * 4 * 16 * 130 * 4     # 4 x 64 tokens
     assert lib.mvllm_paged_decode_workspace_bytes(2, 4, 128, 64, 16) == 2 * 16 * 4 * 130 * 4      # 16 x 64 tokens
     assert lib.mvllm_paged_decode_workspace_bytes(256, 32, 128, 2048, 16) == 256 * 32 * 32 * 130 * 4
+
+
+def test_decode_plan_is_host_arithmetic():
+    """Which form a decode call takes, and that the split form never needs more workspace than is advertised."""
+    from minivllm_amd.layers.attention import paged_decode_plan
+    lib = _lib().load()
+    # one-wave-per-head form: large batch over a wide table (1024-token partitions)
+    assert paged_decode_plan(256, 32, 8, 128, 2048, 16) == (1024, 32, 1)
+    assert paged_decode_plan(64, 32, 8, 128, 2048, 16) == (1024, 32, 1)
+    # small-batch form: 64 sequences x 8 kv heads in a 4096-token table are one partition each, four waves per head
+    assert paged_decode_plan(64, 32, 8, 128, 256, 16) == (4096, 1, 4)
+    assert paged_decode_plan(256, 32, 8, 128, 16, 256) == (4096, 1, 4)        # any batch while the table is <= 4096
+    assert paged_decode_plan(1, 32, 8, 128, 2048, 16) == (1024, 32, 4)        # one long sequence: 256 workgroups
+    assert paged_decode_plan(16, 32, 8, 128, 512, 16) == (2048, 4, 4)
+    # INT8 caches and shapes outside the MFMA kernels
+    assert paged_decode_plan(64, 32, 8, 128, 256, 16, int8_cache=True)[2] == 1
+    assert paged_decode_plan(64, 16, 16, 64, 256, 16)[2] == 0                 # head_dim 64
+    import torch
+    assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32)[2] == 0
+    assert paged_decode_plan(8, 34, 2, 128, 64, 16)[2] == 0                   # 17 query heads per kv head
+    # the advertised workspace covers whatever form is chosen
+    for batch in (1, 3, 16, 64, 200, 1000):
+        for blocks, bs in ((16, 16), (64, 16), (300, 16), (2048, 16), (40, 256), (70000, 16)):
+            for hkv in (1, 2, 8):
+                part, parts, waves = paged_decode_plan(batch, 8 * hkv, hkv, 128, blocks, bs)
+                assert part % 16 == 0 and parts == -(-blocks * bs // part) and 1 <= parts <= 32
+                need = 0 if parts == 1 else batch * parts * 8 * hkv * 130 * 4
+                assert need <= lib.mvllm_paged_decode_workspace_bytes(batch, 8 * hkv, 128, blocks, bs)
 
 
 def test_argument_validation_without_gpu():

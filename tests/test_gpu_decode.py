@@ -10,7 +10,7 @@ import torch
 
 import oracle
 from helpers import error_stats, extract_sequence, make_paged_case, make_paged_case_on_device
-from minivllm_amd.layers.attention import Attention, paged_attention_decode
+from minivllm_amd.layers.attention import Attention, paged_attention_decode, paged_decode_plan
 from minivllm_amd.utils import reset_context, set_context
 
 pytestmark = pytest.mark.gpu
@@ -190,3 +190,45 @@ def test_attention_module_decode_dispatch():
     assert out.shape == (5, hq * d)
     mx, mean = error_stats(out.cpu(), want)
     assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16
+
+
+def _pad_tables(tables, width_tokens, bs):
+    width = max(tables.shape[1], width_tokens // bs)
+    out = torch.full((tables.shape[0], width), -1, dtype=torch.int32)
+    out[:, :tables.shape[1]] = tables
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,bs", [(32, 8, 16), (16, 8, 256), (16, 1, 32), (24, 2, 16), (5, 1, 64), (8, 8, 48)])
+@pytest.mark.parametrize("form", ["one wave per head", "waves share a head", "waves share a head, one partition"])
+def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, form):
+    """A ragged batch (contexts 1..1300, one empty) through both forms of the MFMA kernel: the batch size and the
+    width of the block table, not the contexts, decide the form.  64 sequences in a table of 32 K tokens take the
+    one-wave-per-head grid; 7 sequences in a table of 8 K tokens are spread over four waves per head in several
+    partitions; 64 sequences x 8 kv heads in a table of 4 K tokens are one partition each, written without the
+    merge kernel."""
+    d = 128
+    batch = 7 if form == "waves share a head" else 64
+    width = {"one wave per head": 32768, "waves share a head": 8192}.get(form, 4096) // bs * bs
+    g = torch.Generator().manual_seed(77)
+    ctx_list = torch.randint(1, 1301, (batch,), generator=g).tolist()
+    ctx_list[3] = 0
+    ctx_list[5] = 1300
+    q, kc, vc, tables, ctx = make_paged_case(78, 0, 0, 0, hq, hkv, d, bs, dtype=dtype, ctx_list=ctx_list)
+    tables = _pad_tables(tables, width, bs)
+    assert tables.shape[1] == width // bs
+    part, parts, waves = paged_decode_plan(batch, hq, hkv, d, tables.shape[1], bs, dtype)
+    if form == "one wave per head":
+        assert waves == 1 and part >= 1024
+    elif form == "waves share a head":
+        assert waves > 1 and parts > 1 and part < 1300
+    else:
+        assert waves > 1 and (parts == 1 or hkv < 8)
+    scale = 1 / math.sqrt(d)
+    got = _run(q, kc, vc, tables, ctx, scale, hq, hkv, d, bs)
+    live = ctx > 0                                    # the oracle, like the reference, has no answer for an empty context
+    want = _oracle32(q[live], kc, vc, tables[live][:, :-(-1300 // bs)], ctx[live], scale, hq, hkv, d, bs)
+    mx, mean = error_stats(got[live], want)
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+    assert torch.count_nonzero(got[3]) == 0
