@@ -103,7 +103,7 @@ inline int largest_divisor_le(int n, int cap) {
   return 1;
 }
 
-// Small batches (16-bit fast path).  The grid above needs many live (sequence, partition) pairs: when the batch
+// Small batches (fast path, both cache types).  The grid above needs many live (sequence, partition) pairs: when the batch
 // is small it shortens the partitions, every sequence then needs the second launch that merges them, and when the
 // contexts are much shorter than the block table is wide most of its workgroups are empty.  There a workgroup of
 // kSplitWaves waves takes one (sequence, partition, kv head) instead and its waves split the tiles
@@ -126,13 +126,19 @@ inline int largest_divisor_le(int n, int cap) {
 constexpr int kSplitWaves = MVLLM_DECODE_SPLIT_WAVES;
 constexpr int kSplitMinGroups = 512;
 constexpr int kSplitMaxPart = 4096;
-inline bool split_wanted(int64_t max_ctx, int batch, int num_kv_heads) {
+inline bool split_wanted(int64_t max_ctx, int batch, int num_kv_heads, bool int8) {
   if (!MVLLM_DECODE_SPLIT) return false;
   if (MVLLM_DECODE_SPLIT == 2) return true;          // timing builds
   const int part = partition_tokens_for(max_ctx, batch);
   const int64_t parts = (max_ctx + part - 1) / part;
   const int wpb = largest_divisor_le(num_kv_heads, MVLLM_DECODE_WPB);
-  return part < MVLLM_DECODE_PART_CAP || (int64_t)batch * parts * (num_kv_heads / wpb) < 256 || max_ctx <= kSplitMaxPart;
+  const bool few_groups = (int64_t)batch * parts * (num_kv_heads / wpb) < 256;
+  const bool short_parts = part < MVLLM_DECODE_PART_CAP, narrow_table = max_ctx <= kSplitMaxPart;
+  // INT8: a workgroup of the split form uses 4 of the 32 bytes of scales that a token's kv heads share, so with
+  // many long sequences every head's workgroup fetches the scale lines again (128 sequences x 4096 tokens:
+  // 218 -> 268 us, 256: 401 -> 467 us; 64: 123 -> 117 us): only up to 512 (sequence, kv head) pairs
+  if (int8) return few_groups || ((short_parts || narrow_table) && (int64_t)batch * num_kv_heads <= 512);
+  return few_groups || short_parts || narrow_table;
 }
 inline int split_partition_tokens(int64_t max_ctx, int batch, int num_kv_heads) {
   const int64_t pairs = (int64_t)batch * num_kv_heads;
@@ -516,22 +522,33 @@ __device__ __forceinline__ uint2 load8_stream(const void* p) {
   return make_uint2(x.x, x.y);
 }
 
-template <typename T, int NCH>
-__device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b, int p, int g) {   // g: kv head
+// W as in decode_mfma_item: 1 = the wave walks its partition, > 1 = W waves of the workgroup share it.
+template <typename T, int NCH, int W>
+__device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b, int p, int g, int w) {   // g: kv head
   static_assert(NCH == 1, "one chunk of up to 16 heads");
   constexpr int D = 128;
   const int lane = threadIdx.x & 63;
   const int group = a.num_heads / a.num_kv_heads;
   const int q4 = lane >> 4;            // token class: tokens 4*q4 .. 4*q4+3 of a tile
   const int col = lane & 15;           // head (first product), dim group (second product)
+  const int bs = a.block_size;
+  const int part_start = p * a.part_tokens;
+  const int first = part_start + (W == 1 ? 0 : w * kTile);      // first token of this wave's first tile
+  const int32_t* table = a.block_tables + (int64_t)b * a.max_num_blocks;
+  int bi = first / bs;
+  int off = first - bi * bs;
+  int win_base = bi;
+  int win;
+  if constexpr (W > 1) win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;   // before the context length
 
   const int ctx = (int)load_ctx(a, b);
   // a sequence that fits one partition (or is empty) is finished here: partition 0 writes the output row
   const bool direct = ctx <= a.part_tokens;
-  const int part_start = p * a.part_tokens;
   if (part_start >= ctx && !(direct && p == 0)) return;
   const int part_end = min(ctx, part_start + a.part_tokens);
-  const int ntiles = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
+  const int tiles_all = part_end > part_start ? (part_end - part_start + kTile - 1) / kTile : 0;
+  const int ntiles = W == 1 ? tiles_all : (tiles_all > w ? (tiles_all - w + W - 1) / W : 0);   // this wave's
+  if constexpr (W == 1) win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
 
   // ---- query -> int8 hi/lo planes (B operand: column lane%16 -> head, bytes 16*q4.. of each 64-dim step)
   v4i qhi[2], qlo[2];
@@ -576,21 +593,15 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
 #pragma unroll
   for (int e = 0; e < 8; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  const int bs = a.block_size;
   const int64_t row = (int64_t)a.num_kv_heads * D;          // bytes per token row
   const char* kc = reinterpret_cast<const char*>(a.k_cache) + (int64_t)g * D;
   const char* vc = reinterpret_cast<const char*>(a.v_cache) + (int64_t)g * D;
-  const int32_t* table = a.block_tables + (int64_t)b * a.max_num_blocks;
-  int bi = part_start / bs;
-  int off = part_start - bi * bs;
-  int win_base = bi;
-  int win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
   const int k_lane_off = col * (int)row + q4 * 16;          // token lane%16, bytes 16*q4 (+64 j)
   const int v_lane_off = 4 * q4 * (int)row + col * 8;       // tokens 4*q4 + i, dims 8*(lane%16)
   const int s_lane_tok = 4 * q4 + (lane & 3);               // token whose scales this lane loads
 
   auto load_tile = [&](KVTileI8& t, int tile) {
-    t.t0 = part_start + tile * kTile;
+    t.t0 = first + tile * (W * kTile);
     if (bi - win_base >= 64) {
       win_base = bi;
       win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
@@ -614,8 +625,13 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
       for (int i = 0; i < 4; ++i) t.v[i] = make_uint2(0u, 0u);
       t.ks = t.vs = 0.f;
     }
-    off += kTile;
-    if (off >= bs) { off = 0; ++bi; }
+    if constexpr (W == 1) {
+      off += kTile;
+      if (off >= bs) { off = 0; ++bi; }
+    } else {
+      off += W * kTile;
+      while (off >= bs) { off -= bs; ++bi; }
+    }
   };
 
   auto consume = [&](const KVTileI8& t) {
@@ -706,6 +722,45 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
   }
   if (tile < ntiles) consume(ta);
 
+  if constexpr (W > 1) {
+    // waves 1 .. W-1 leave m, l, the weight sum and their accumulators in LDS, wave 0 folds them in (as in
+    // DecodeHead::merge) and goes on alone
+    __shared__ float4 part[(W - 1) * 9 * 64];
+    if (w > 0) {
+      float4* dst = part + (w - 1) * 9 * 64 + lane;
+      dst[0] = make_float4(m, l, wsum, 0.f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dst[(1 + e) * 64] = make_float4(o[e][0], o[e][1], o[e][2], o[e][3]);
+    }
+    __syncthreads();
+    if (w > 0) return;
+#pragma unroll 1
+    for (int x = 0; x < W - 1; ++x) {
+      const float4* src = part + x * 9 * 64 + lane;
+      const float4 mlw = src[0];
+      const float m_new = fmaxf(m, mlw.x);
+      const float f0 = safe_exp2_diff(m, m_new);
+      const float f1 = safe_exp2_diff(mlw.x, m_new);
+      m = m_new;
+      l = l * f0 + mlw.y * f1;
+      wsum = wsum * f0 + mlw.z * f1;
+      float a0[4], a1[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        a0[j] = __shfl(f0, 4 * q4 + j, 64);
+        a1[j] = __shfl(f1, 4 * q4 + j, 64);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float4 ow = src[(1 + e) * 64];
+        o[e][0] = o[e][0] * a0[0] + ow.x * a1[0];
+        o[e][1] = o[e][1] * a0[1] + ow.y * a1[1];
+        o[e][2] = o[e][2] * a0[2] + ow.z * a1[2];
+        o[e][3] = o[e][3] * a0[3] + ow.w * a1[3];
+      }
+    }
+  }
+
   // denominators and weight sums over the four token classes (every lane of a head then holds the head's totals)
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -758,7 +813,13 @@ template <typename T, int NCH>
 __global__ __launch_bounds__(MVLLM_DECODE_I8_THREADS, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
   int b, p, hg;
   if (!decode_item<true>(a, b, p, hg)) return;
-  decode_mfma_int8_item<T, NCH>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6));
+  decode_mfma_int8_item<T, NCH, 1>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
+}
+template <typename T, int W>
+__global__ __launch_bounds__(64 * W, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_split_kernel(const DecodeArgs a) {
+  const int g = blockIdx.x, b = blockIdx.z;
+  const int p = (int)((blockIdx.y + (unsigned)b) % (unsigned)a.num_parts);
+  decode_mfma_int8_item<T, 1, W>(a, b, p, g, threadIdx.x >> 6);
 }
 
 // ---------------------------------------------------------------------------
@@ -934,7 +995,7 @@ struct DecodePlan {
 };
 static DecodePlan plan_decode(int batch, int num_kv_heads, int max_num_blocks, int block_size, bool fast_ok, bool int8) {
   const int64_t max_ctx = (int64_t)max_num_blocks * block_size;
-  const bool split = fast_ok && !int8 && split_wanted(max_ctx, batch, num_kv_heads);
+  const bool split = fast_ok && split_wanted(max_ctx, batch, num_kv_heads, int8);
   DecodePlan plan;
   plan.part_tokens = split ? split_partition_tokens(max_ctx, batch, num_kv_heads) : partition_tokens_for(max_ctx, batch);
   plan.num_parts = (int)((max_ctx + plan.part_tokens - 1) / plan.part_tokens);
@@ -951,8 +1012,9 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
   bool launched = false;
   if constexpr (IsSixteenBit<T>::value) {
     if (fast_ok && split) {
-      decode_mfma_split_kernel<T, kSplitWaves><<<dim3((unsigned)a.num_kv_heads, (unsigned)a.num_parts, (unsigned)a.batch),
-                                                 dim3(64 * kSplitWaves), 0, stream>>>(a);
+      const dim3 grid((unsigned)a.num_kv_heads, (unsigned)a.num_parts, (unsigned)a.batch), block(64 * kSplitWaves);
+      if (int8) decode_mfma_int8_split_kernel<T, kSplitWaves><<<grid, block, 0, stream>>>(a);
+      else decode_mfma_split_kernel<T, kSplitWaves><<<grid, block, 0, stream>>>(a);
       launched = true;
     } else if (fast_ok) {
       // kv heads (waves) per workgroup: as many as allowed, so that a workgroup streams whole token rows;

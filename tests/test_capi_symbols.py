@@ -67,8 +67,9 @@ def test_decode_plan_is_host_arithmetic():
     assert paged_decode_plan(256, 32, 8, 128, 16, 256) == (4096, 1, 4)        # any batch while the table is <= 4096
     assert paged_decode_plan(1, 32, 8, 128, 2048, 16) == (1024, 32, 4)        # one long sequence: 256 workgroups
     assert paged_decode_plan(16, 32, 8, 128, 512, 16) == (2048, 4, 4)
-    # INT8 caches and shapes outside the MFMA kernels
-    assert paged_decode_plan(64, 32, 8, 128, 256, 16, int8_cache=True)[2] == 1
+    # INT8 caches, and shapes outside the MFMA kernels
+    assert paged_decode_plan(64, 32, 8, 128, 256, 16, int8_cache=True) == (4096, 1, 4)
+    assert paged_decode_plan(256, 32, 8, 128, 256, 16, int8_cache=True) == (1024, 4, 1)     # large INT8 batch: first form
     assert paged_decode_plan(64, 16, 16, 64, 256, 16)[2] == 0                 # head_dim 64
     import torch
     assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32)[2] == 0

@@ -11,7 +11,7 @@ import torch
 
 import oracle
 from helpers import error_stats, make_paged_case
-from minivllm_amd.layers.attention import paged_attention_decode_int8, store_kvcache_int8
+from minivllm_amd.layers.attention import paged_attention_decode_int8, paged_decode_plan, store_kvcache_int8
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -88,3 +88,31 @@ def test_config4_subset():
     hq, hkv, d, bs = 32, 8, 128, 16
     case = _quantised_case(65, 24, 256, 16384, hq, hkv, d, bs)
     _check(case, hq, hkv, d, bs, 1 / math.sqrt(d))
+
+
+@pytest.mark.parametrize("hq,hkv,bs", [(32, 8, 16), (16, 8, 256), (16, 1, 32), (24, 2, 16), (5, 1, 64)])
+@pytest.mark.parametrize("form", ["one wave per head", "waves share a head", "waves share a head, one partition"])
+def test_int8_both_grid_forms(hq, hkv, bs, form):
+    """As test_both_grid_forms_vs_oracle of the 16-bit cache: the table width and the batch size pick the form."""
+    d = 128
+    batch = 7 if form == "waves share a head" else 64
+    width = {"one wave per head": 32768, "waves share a head": 8192}.get(form, 4096) // bs * bs
+    g = torch.Generator().manual_seed(66)
+    ctx_list = torch.randint(1, 1301, (batch,), generator=g).tolist()
+    ctx_list[2] = 1300
+    q, ck, cv, sk, sv, tables, ctx = _quantised_case(67, 0, 0, 0, hq, hkv, d, bs, ctx_list=ctx_list)
+    wide = torch.full((batch, width // bs), -1, dtype=torch.int32)
+    wide[:, :tables.shape[1]] = tables
+    part, parts, waves = paged_decode_plan(batch, hq, hkv, d, wide.shape[1], bs, q.dtype, int8_cache=True)
+    if form == "one wave per head":
+        assert waves == 1
+    elif form == "waves share a head":
+        assert waves > 1 and parts > 1 and part < 1300
+    else:
+        assert waves > 1 and (parts == 1 or hkv < 8)
+    scale = 1 / math.sqrt(d)
+    got = paged_attention_decode_int8(q.to(DEV), ck, cv, sk, sv, wide.to(DEV), ctx.to(DEV), scale, hq, hkv, d, bs).cpu()
+    want = oracle.decode_int8_oracle(q.float(), ck.cpu(), cv.cpu(), sk.cpu(), sv.cpu(), tables, ctx, scale, hq, hkv, d, bs)
+    mx, mean = error_stats(got, want)
+    excess = ((got.float() - want).abs() - want.abs() * 2.0 ** -8).max().item()
+    assert torch.isfinite(got).all() and excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
