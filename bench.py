@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,fused_qk,sampler,engine,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,decode_small,fused_qk,sampler,engine,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -337,6 +337,49 @@ def bench_sampler(args):
             "event_ms_per_step": fused_ms, "gbs": nbytes / (fused_ms * 1e-3) / 1e9, "unfused_modules_event_ms": modules_ms}
 
 
+def bench_decode_small(args):
+    """A serving-size decode call: 64 sequences of 96-352 tokens whose block table is 4096 tokens wide (the model
+    length, not the contexts), 16-bit and INT8 caches, timed as 20 calls inside one hipGraph (a call is latency,
+    not bandwidth, so back-to-back launches from the host would measure the host)."""
+    import torch
+    from helpers import make_paged_case_on_device
+    from minivllm_amd.layers.attention import (paged_attention_decode, paged_attention_decode_int8, paged_decode_plan,
+                                               store_kvcache_int8)
+
+    dev = "cuda:0"
+    hq, hkv, d, bs, batch, width = 32, 8, 128, 16, 64, 4096
+    q, kc, vc, tables, ctx = make_paged_case_on_device(args.seed, dev, batch, 96, 352, hq, hkv, d, bs, log_uniform=False)
+    wide = torch.full((batch, width // bs), -1, dtype=torch.int32)
+    wide[:, :tables.shape[1]] = tables
+    td, cd = wide.to(dev), ctx.to(dev)
+    nb = kc.shape[0]
+    ck, cv = (torch.zeros(nb, bs, hkv, d, dtype=torch.int8, device=dev) for _ in range(2))
+    sk, sv = (torch.zeros(nb, bs, hkv, device=dev) for _ in range(2))
+    store_kvcache_int8(kc.view(-1, hkv, d), vc.view(-1, hkv, d), ck, cv, sk, sv, torch.arange(nb * bs, device=dev), bs)
+    scale = 1 / math.sqrt(d)
+    calls = 20
+
+    def graph_us(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(calls):
+                fn()
+        _, ms = time_steps(g.replay, max(5, args.steps // 3), 2)
+        return ms * 1e3 / calls
+
+    us16 = graph_us(lambda: paged_attention_decode(q, kc, vc, td, cd, scale, hq, hkv, d, bs))
+    us8 = graph_us(lambda: paged_attention_decode_int8(q, ck, cv, sk, sv, td, cd, scale, hq, hkv, d, bs))
+    tokens = int(ctx.sum())
+    return {"workload": "decode B64 ctx~U[96,352] in a 4096-token block table, Hq32 Hkv8 D128 bf16, block_size 16, "
+                        "20 calls per hipGraph replay",
+            "tokens": tokens, "plan_part_tokens_parts_waves": list(paged_decode_plan(batch, hq, hkv, d, width // bs, bs)),
+            "us_per_call": us16, "gbs": tokens * hkv * d * 4 / (us16 * 1e-6) / 1e9,
+            "int8_us_per_call": us8, "int8_gbs": tokens * hkv * (2 * d + 8) / (us8 * 1e-6) / 1e9}
+
+
 def bench_engine(args, max_num_sequences, graph):
     """BASELINE.json config 5: random-init Qwen3-style decoder (hidden 1024, 8 layers, Hq16/Hkv8/D128, FFN 3072,
     vocab 151936, bf16), 60 prompts of random ids with lengths U[32,96], 256 new tokens each, T 0.6."""
@@ -404,6 +447,8 @@ def main():
         extra.update(bench_prefill_store(args, which))
     if want("int8"):
         extra["int8"] = bench_int8(args)
+    if want("decode_small"):
+        extra["decode_small_batch"] = bench_decode_small(args)
     if want("fused_qk"):
         extra["fused_qk"] = bench_fused_qk(args)
     if want("sampler"):
