@@ -55,7 +55,9 @@ template <int N> struct VecN<float, N> {
   }
   static __device__ __forceinline__ void store(float* p, const float (&x)[N]) {
 #pragma unroll
-    for (int i = 0; i < N; i += 4) *reinterpret_cast<float4*>(p + i) = make_float4(x[i], x[i + 1], x[i + 2], x[i + 3]);
+    for (int i = 0; i < N; i += 4)
+      store16_stream(p + i, make_uint4(__float_as_uint(x[i]), __float_as_uint(x[i + 1]), __float_as_uint(x[i + 2]),
+                                       __float_as_uint(x[i + 3])));
   }
 };
 template <typename T16, int N> struct VecN {
@@ -78,8 +80,8 @@ template <typename T16, int N> struct VecN {
     T16 o[N];
 #pragma unroll
     for (int e = 0; e < N; ++e) o[e] = from_float<T16>(x[e]);
-    if constexpr (N == 8) *reinterpret_cast<uint4*>(p) = *reinterpret_cast<const uint4*>(o);
-    else *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(o);
+    if constexpr (N == 8) store16_stream(p, *reinterpret_cast<const uint4*>(o));
+    else store8_stream(p, *reinterpret_cast<const uint2*>(o));
   }
 };
 
@@ -110,8 +112,8 @@ __device__ __forceinline__ void store_codes(int8_t* dst, const float (&x)[N], fl
     const int c = live ? (int)r : 0;
     w[e >> 2] |= ((uint32_t)(c & 0xff)) << (8 * (e & 3));
   }
-  if constexpr (N == 8) *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
-  else *reinterpret_cast<uint32_t*>(dst) = w[0];
+  if constexpr (N == 8) store8_stream(dst, make_uint2(w[0], w[1]));
+  else store4_stream(dst, w[0]);
 }
 
 constexpr int kFusedThreads = 256;
