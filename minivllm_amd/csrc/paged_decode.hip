@@ -2,7 +2,7 @@
 // GQA-shared K/V reads, log-sum-exp merge in a second pass.
 // Replaces the Triton kernel of src/myvllm/layers/attention.py:283-415.
 //
-// Work decomposition (fast path, 16-bit cache, head_dim 128, block_size % 16 == 0, up to 16 query heads per kv head)
+// Work decomposition (fast path, 16-bit cache, head_dim 128 or 64, block_size % 16 == 0, up to 16 query heads per kv head)
 //   workgroup = (partition p, sequence b, group of <= 4 kv heads); wave w of the
 //   workgroup owns kv head g and all Hq/Hkv query heads that share it, so the
 //   waves of one workgroup stream contiguous pieces of the [token, Hkv, D] rows.
@@ -221,21 +221,25 @@ template <> __device__ __forceinline__ v4f mfma16x16x16<f16_t>(uint2 x, uint2 y,
 //                    rows per instruction), so its dim e of step e is column l%16 of the e-th product:
 //                    column n of product e is dim 8 n + e, and two byte permutes per product gather the four
 //                    tokens' values of that dim.  Lane l ends with O[head 4*(l/16)+j][dims 8*(l%16) + e].
-template <typename T>
+// D = 128 or 64.  With 64 the first product has two steps instead of four, and of the second product's sixteen
+// columns (8 dims each) only the first eight exist: lanes l%16 >= 8 load no V, hold zero accumulators and write
+// nothing.
+template <typename T, int D>
 struct DecodeHead {
-  uint4 qf[4];                // Q fragments: B operand, column n = head n, k = 8*cls + 32 j
+  static constexpr int kSteps = D / 32;     // 32-dim steps of the first product
+  static constexpr int kCols = D / 8;       // lanes (l%16) that own 8 dims of the output
+  uint4 qf[kSteps];           // Q fragments: B operand, column n = head n, k = 8*cls + 32 j
   float m;                    // running maximum of head `col` (log2 units), the same in its four lanes
   float l;                    // this lane's share of the head's denominator
   v4f o[8];                   // o[e][j] = O[head 4*cls + j][dim 8*col + e]
 
   __device__ __forceinline__ void start(const DecodeArgs& a, int b, int g, int group, int lane) {
-    constexpr int D = 128;
     const int col = lane & 15, cls = lane >> 4;
     const T* q = reinterpret_cast<const T*>(a.q);
     const bool live = col < group;
     const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D + cls * 8;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kSteps; ++j) {
       const uint4 x = *reinterpret_cast<const uint4*>(src + 32 * j);
       qf[j] = live ? x : make_uint4(0u, 0u, 0u, 0u);
     }
@@ -252,7 +256,7 @@ struct DecodeHead {
     const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
     v4f s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) s = mfma16x16x32<T>(t.k[j], qf[j], s);
+    for (int j = 0; j < kSteps; ++j) s = mfma16x16x32<T>(t.k[j], qf[j], s);
     float s2[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) s2[i] = s[i] * scale_log2;
@@ -349,8 +353,8 @@ struct DecodeHead {
 
   // write the output row (direct) or this partition's partial result
   __device__ __forceinline__ void finish(const DecodeArgs& a, int b, int p, int g, int group, bool direct, int lane) {
-    constexpr int D = 128;
     const int col = lane & 15, cls = lane >> 4;
+    const bool owns = D == 128 || col < kCols;          // this lane's 8 dims exist
     // denominators: add the four token classes (every lane of a head then holds the head's total)
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -362,7 +366,7 @@ struct DecodeHead {
       for (int j = 0; j < 4; ++j) {
         const int h = 4 * cls + j;
         const float lj = __shfl(linv, h, 64);               // lane h (class 0) holds head h
-        if (h < group) {
+        if (h < group && owns) {
           T r[8];
 #pragma unroll
           for (int e = 0; e < 8; ++e) r[e] = from_float<T>(o[e][j] * lj);
@@ -375,7 +379,7 @@ struct DecodeHead {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int h = 4 * cls + j;
-        if (h < group) {
+        if (h < group && owns) {
           float* dst = a.ws_acc + (slot + h) * D + col * 8;
           *reinterpret_cast<float4*>(dst) = make_float4(o[0][j], o[1][j], o[2][j], o[3][j]);
           *reinterpret_cast<float4*>(dst + 4) = make_float4(o[4][j], o[5][j], o[6][j], o[7][j]);
@@ -389,9 +393,8 @@ struct DecodeHead {
 // W = 1: the wave walks all tiles of its partition.  W > 1 (the workgroup is W waves on one kv head): wave w takes
 // tiles w, w + W, ... and the partial results meet in LDS (DecodeHead::merge), so a short context costs a few tiles
 // of latency per wave and no second launch.
-template <typename T, int W>
+template <typename T, int W, int D>
 __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int p, int g, int w) {   // g: kv head
-  constexpr int D = 128;
   const int lane = threadIdx.x & 63;
   const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head (<= 16)
   const int col = lane & 15;                           // head (first product), dim group (second product)
@@ -404,7 +407,7 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
   // The query rows and the block-table window (lane i holds entry win_base + i of this sequence) do not depend
   // on the context length.  The split kernel, which is all latency, asks for them together with it; the
   // one-wave form first drops the workgroups whose partition lies past the context (most of a ragged batch).
-  DecodeHead<T> head;
+  DecodeHead<T, D> head;
   int bi = first / bs;               // logical block of the next tile to load
   int off = first - bi * bs;         // token offset inside that block
   int win_base = bi;
@@ -448,9 +451,10 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
       // 128-byte line has to survive in cache until the next instruction: ordinary loads (the hint costs 7 %
       // there).
 #pragma unroll
-      for (int j = 0; j < 4; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
+      for (int j = 0; j < D / 32; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) t.v[i] = load16_stream(vp + (int64_t)i * row);
+      for (int i = 0; i < 4; ++i)
+        t.v[i] = (D == 128 || col < D / 8) ? load16_stream(vp + (int64_t)i * row) : make_uint4(0u, 0u, 0u, 0u);
     } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
@@ -795,19 +799,19 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
 // Kernels of the fast path: one workgroup per (partition, sequence, group of kv heads); the partition index is
 // an upper bound, and a workgroup whose partition lies past its sequence's context returns at once.
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, int D>
 __global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_kernel(const DecodeArgs a) {
   int b, p, hg;
   if (!decode_item<false>(a, b, p, hg)) return;
-  decode_mfma_item<T, 1>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
+  decode_mfma_item<T, 1, D>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
 }
 // Small batches: one workgroup of W waves per (partition, sequence, kv head), the waves splitting the tiles.
-template <typename T, int W>
+template <typename T, int W, int D>
 __global__ __launch_bounds__(64 * W, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_split_kernel(const DecodeArgs a) {
   // kv head fastest: the workgroups of one (sequence, partition) start together and read the same token rows
   const int g = blockIdx.x, b = blockIdx.z;
   const int p = (int)((blockIdx.y + (unsigned)b) % (unsigned)a.num_parts);
-  decode_mfma_item<T, W>(a, b, p, g, threadIdx.x >> 6);
+  decode_mfma_item<T, W, D>(a, b, p, g, threadIdx.x >> 6);
 }
 template <typename T, int NCH>
 __global__ __launch_bounds__(MVLLM_DECODE_I8_THREADS, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
@@ -985,8 +989,9 @@ static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int ma
 }
 
 // shapes the MFMA kernels are built for (pointer alignment is checked by the caller)
-static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype) {
-  return dtype != MVLLM_F32 && head_dim == 128 && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
+static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool int8) {
+  const bool dim_ok = head_dim == 128 || (head_dim == 64 && !int8);     // the INT8 kernel is built for 128 only
+  return dtype != MVLLM_F32 && dim_ok && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
          (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
 }
 
@@ -1014,7 +1019,8 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
     if (fast_ok && split) {
       const dim3 grid((unsigned)a.num_kv_heads, (unsigned)a.num_parts, (unsigned)a.batch), block(64 * kSplitWaves);
       if (int8) decode_mfma_int8_split_kernel<T, kSplitWaves><<<grid, block, 0, stream>>>(a);
-      else decode_mfma_split_kernel<T, kSplitWaves><<<grid, block, 0, stream>>>(a);
+      else if (a.head_dim == 64) decode_mfma_split_kernel<T, kSplitWaves, 64><<<grid, block, 0, stream>>>(a);
+      else decode_mfma_split_kernel<T, kSplitWaves, 128><<<grid, block, 0, stream>>>(a);
       launched = true;
     } else if (fast_ok) {
       // kv heads (waves) per workgroup: as many as allowed, so that a workgroup streams whole token rows;
@@ -1025,7 +1031,8 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
       const unsigned groups = (unsigned)(a.num_kv_heads / wpb);
       dim3 block(64 * wpb);
       if (int8) decode_mfma_int8_kernel<T, 1><<<dim3((unsigned)a.num_parts, groups, (unsigned)a.batch), block, 0, stream>>>(a);
-      else decode_mfma_kernel<T><<<dim3((unsigned)a.num_parts, (unsigned)a.batch, groups), block, 0, stream>>>(a);
+      else if (a.head_dim == 64) decode_mfma_kernel<T, 64><<<dim3((unsigned)a.num_parts, (unsigned)a.batch, groups), block, 0, stream>>>(a);
+      else decode_mfma_kernel<T, 128><<<dim3((unsigned)a.num_parts, (unsigned)a.batch, groups), block, 0, stream>>>(a);
       launched = true;
     }
   }
@@ -1068,7 +1075,7 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
   a.num_blocks = num_blocks; a.ctx_is_i64 = ctx_is_i64; a.max_num_blocks = max_num_blocks;
   a.batch = batch; a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.head_dim = head_dim;
   a.block_size = block_size;
-  const bool fast_ok = fast_shape(num_heads, num_kv_heads, head_dim, block_size, dtype) &&
+  const bool fast_ok = fast_shape(num_heads, num_kv_heads, head_dim, block_size, dtype, int8) &&
                        aligned16(q) && aligned16(out) && aligned16(k_cache) && aligned16(v_cache);
   const DecodePlan plan = plan_decode(batch, num_kv_heads, max_num_blocks, block_size, fast_ok, int8);
   const bool split = plan.waves_per_head > 1;
@@ -1107,7 +1114,7 @@ extern "C" int mvllm_paged_decode_plan(int batch, int num_heads, int num_kv_head
       num_heads % num_kv_heads != 0)
     return MVLLM_ERR_BAD_SHAPE;
   const DecodePlan plan = plan_decode(batch, num_kv_heads, max_num_blocks, block_size,
-                                      fast_shape(num_heads, num_kv_heads, head_dim, block_size, dtype), int8_cache != 0);
+                                      fast_shape(num_heads, num_kv_heads, head_dim, block_size, dtype, int8_cache != 0), int8_cache != 0);
   if (part_tokens) *part_tokens = plan.part_tokens;
   if (num_parts) *num_parts = plan.num_parts;
   if (waves_per_head) *waves_per_head = plan.waves_per_head;

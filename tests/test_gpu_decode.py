@@ -75,7 +75,8 @@ def test_context_length_boundaries(ctx_list):
 
 @pytest.mark.parametrize("dtype,hq,hkv,d,bs", [
     (torch.float32, 4, 2, 64, 4),       # generic kernel: fp32
-    (torch.bfloat16, 16, 16, 64, 256),  # head_dim 64 (the reference demo's shape)
+    (torch.bfloat16, 16, 16, 64, 8),    # head_dim 64 with a block size the MFMA kernel is not built for
+    (torch.float32, 16, 8, 64, 16),     # the reference demo's shape and dtype (main.py)
     (torch.float16, 6, 3, 80, 3),       # odd head_dim and block size
     (torch.bfloat16, 4, 1, 256, 16),
 ])
@@ -200,15 +201,17 @@ def _pad_tables(tables, width_tokens, bs):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("hq,hkv,bs", [(32, 8, 16), (16, 8, 256), (16, 1, 32), (24, 2, 16), (5, 1, 64), (8, 8, 48)])
+@pytest.mark.parametrize("hq,hkv,bs,d", [(32, 8, 16, 128), (16, 8, 256, 128), (16, 1, 32, 128), (24, 2, 16, 128),
+                                         (5, 1, 64, 128), (8, 8, 48, 128),
+                                         (16, 8, 16, 64), (16, 16, 256, 64), (12, 1, 32, 64), (5, 5, 48, 64)])
 @pytest.mark.parametrize("form", ["one wave per head", "waves share a head", "waves share a head, one partition"])
-def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, form):
+def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, d, form):
     """A ragged batch (contexts 1..1300, one empty) through both forms of the MFMA kernel: the batch size and the
     width of the block table, not the contexts, decide the form.  64 sequences in a table of 32 K tokens take the
     one-wave-per-head grid; 7 sequences in a table of 8 K tokens are spread over four waves per head in several
     partitions; 64 sequences x 8 kv heads in a table of 4 K tokens are one partition each, written without the
-    merge kernel."""
-    d = 128
+    merge kernel.  head_dim 64 (the reference demo's model, qwen3.py:338) runs on the same kernels with half of
+    the second product's columns switched off."""
     batch = 7 if form == "waves share a head" else 64
     width = {"one wave per head": 32768, "waves share a head": 8192}.get(form, 4096) // bs * bs
     g = torch.Generator().manual_seed(77)
@@ -222,7 +225,7 @@ def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, form):
     if form == "one wave per head":
         assert waves == 1 and part >= 1024
     elif form == "waves share a head":
-        assert waves > 1 and parts > 1 and part < 1300
+        assert waves > 1 and parts > 1
     else:
         assert waves > 1 and (parts == 1 or hkv < 8)
     scale = 1 / math.sqrt(d)
