@@ -145,4 +145,59 @@ inline int launch_status() {
   return e == hipSuccess ? 0 : (int)e;
 }
 
+// Tile `tile` (global numbering) -> sequence and first row inside it.  Wave-parallel: 64 sequences
+// per step (tile counts, inclusive prefix sum by shuffles, ballot to pick the owner), so the cost is
+// a few hundred cycles per 64 sequences instead of one dependent load per sequence.  Every lane of
+// the calling wave must be active; all lanes return the same values.
+__device__ __forceinline__ bool locate_tile(const int32_t* __restrict__ cu, int num_seqs, int tile, int bm,
+                                            int& seq_start, int& seq_len, int& row0, int& seq_index) {
+  const int lane = threadIdx.x & 63;
+  int first = 0;
+  for (int base = 0; base < num_seqs; base += 64) {
+    const int s = base + lane;
+    int lo = 0, len = 0;
+    if (s < num_seqs) {
+      lo = cu[s];
+      len = cu[s + 1] - lo;
+    }
+    const int n = (len + bm - 1) / bm;
+    int incl = n;                                   // inclusive prefix sum of tile counts over the lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += t;
+    }
+    const int total = __shfl(incl, 63, 64);
+    if (tile < first + total) {
+      const unsigned long long owners = __ballot(tile < first + incl);   // first lane whose prefix passes the tile
+      const int owner = __ffsll((long long)owners) - 1;
+      const int start_tile = first + __shfl(incl - n, owner, 64);
+      seq_start = __shfl(lo, owner, 64);
+      seq_len = __shfl(len, owner, 64);
+      row0 = (tile - start_tile) * bm;
+      seq_index = base + owner;
+      return true;
+    }
+    first += total;
+  }
+  return false;
+}
+
+// Varlen causal prefill on the decode kernel's tile arithmetic, for 16-bit head dims the LDS-tiled prefill kernel is
+// not built for (head_dim 64).  Defined in paged_decode.hip, where that arithmetic lives; launched from the prefill
+// entry point.
+struct PrefillRowsArgs {
+  void* out;
+  const void* q;
+  const void* k;
+  const void* v;
+  const int32_t* cu_seqlens;
+  int64_t total_tokens;
+  int num_seqs;
+  int num_heads;
+  int num_kv_heads;
+  float scale_log2;
+};
+int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream);
+
 }  // namespace mvllm

@@ -250,7 +250,9 @@ struct DecodeHead {
   }
 
   // one tile of 16 tokens starting at token t0 of the sequence; tokens at or past part_end do not count
-  __device__ __forceinline__ void consume(const KVTile<T>& t, int part_end, float scale_log2, int lane) {
+  // (col_end: prefill only, where column n is a query row: tokens at or past it do not count for this lane's column)
+  __device__ __forceinline__ void consume(const KVTile<T>& t, int part_end, float scale_log2, int lane,
+                                          int col_end = 0x7fffffff) {
     const int cls = lane >> 4;
     const int tok_base = t.t0 + 4 * cls;
     const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
@@ -268,6 +270,11 @@ struct DecodeHead {
           s2[i] = -INFINITY;
           v[i] = make_uint4(0u, 0u, 0u, 0u);       // whatever lies there must not meet p = 0 as NaN or Inf
         }
+    }
+    if (col_end != 0x7fffffff) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (tok_base + i >= col_end) s2[i] = -INFINITY;
     }
     const float tile_max = fmaxf(fmaxf(s2[0], s2[1]), fmaxf(s2[2], s2[3]));
     const bool grow = tile_max > m + kLazyRescale || (m == -INFINITY && tile_max > -INFINITY);
@@ -487,6 +494,93 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
     if (!head.template merge<W>(w, lane)) return;
   }
   head.finish(a, b, p, g, group, direct, lane);
+}
+
+// ---------------------------------------------------------------------------
+// Varlen causal prefill on the same tile arithmetic (flash_attention_prefill, attention.py:212-280, for 16-bit
+// head dims the LDS-tiled kernel of prefill_varlen.hip is not built for: head_dim 64, the reference demo's model).
+// One wave = 16 consecutive query rows of one query head: the rows take the place of the heads of a group
+// (column n of the first product = row n), the keys 0 .. row are walked in 16-token tiles straight from the
+// packed k / v tensors, and the causal limit is applied per column.  The four waves of a workgroup are four query
+// heads on the same rows, so with grouped heads they read the same K/V tiles at the same time.  No LDS and no
+// reuse of K/V across row tiles beyond the caches: tens of TFLOP/s, not hundreds.
+// ---------------------------------------------------------------------------
+template <typename T, int D>
+__global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsArgs a, int tiles_x) {
+  int seq_start, seq_len, row0, seq_index;
+  // latest (heaviest) tiles first
+  if (!locate_tile(a.cu_seqlens, a.num_seqs, tiles_x - 1 - (int)blockIdx.x, kTile, seq_start, seq_len, row0, seq_index)) return;
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 15, cls = lane >> 4;
+  const int h = blockIdx.y * 4 + (threadIdx.x >> 6);   // query head of this wave
+  if (h >= a.num_heads) return;
+  const int g = h / (a.num_heads / a.num_kv_heads);
+  const int rows = min(kTile, seq_len - row0);          // live query rows of the tile
+
+  DecodeHead<T, D> head;
+  {
+    const bool live = col < rows;
+    const T* src = reinterpret_cast<const T*>(a.q) +
+                   ((int64_t)(seq_start + row0 + (live ? col : 0)) * a.num_heads + h) * D + cls * 8;
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+      const uint4 x = *reinterpret_cast<const uint4*>(src + 32 * j);
+      head.qf[j] = live ? x : make_uint4(0u, 0u, 0u, 0u);
+    }
+    head.m = -INFINITY;
+    head.l = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) head.o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
+  }
+  const int kv_end = row0 + rows;        // keys 0 .. kv_end - 1 are seen by at least one row of the tile
+  const int col_end = row0 + col + 1;    // keys seen by this lane's row
+  const int ntiles = (kv_end + kTile - 1) / kTile;
+  const int64_t row = (int64_t)a.num_kv_heads * D;
+  const T* kc = reinterpret_cast<const T*>(a.k) + (int64_t)seq_start * row + (int64_t)g * D + cls * 8;
+  const T* vc = reinterpret_cast<const T*>(a.v) + (int64_t)seq_start * row + (int64_t)g * D + col * 8;
+
+  // Tokens past kv_end are masked by consume(); their loads are redirected to the last visible row so that
+  // nothing past the end of the packed tensors is touched.
+  auto load_tile = [&](KVTile<T>& t, int tile) __attribute__((always_inline)) {
+    t.t0 = tile * kTile;
+    t.ok = true;
+    const T* kp = kc + (int64_t)min(t.t0 + col, kv_end - 1) * row;
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      t.v[i] = (D == 128 || col < D / 8) ? *reinterpret_cast<const uint4*>(vc + (int64_t)min(t.t0 + 4 * cls + i, kv_end - 1) * row)
+                                         : make_uint4(0u, 0u, 0u, 0u);
+  };
+  KVTile<T> ta, tb;
+  if (ntiles > 0) load_tile(ta, 0);
+  int tile = 0;
+  for (; tile + 1 < ntiles; tile += 2) {
+    load_tile(tb, tile + 1);
+    head.consume(ta, kv_end, a.scale_log2, lane, col_end);
+    if (tile + 2 < ntiles) load_tile(ta, tile + 2);
+    head.consume(tb, kv_end, a.scale_log2, lane, col_end);
+  }
+  if (tile < ntiles) head.consume(ta, kv_end, a.scale_log2, lane, col_end);
+
+  // denominators over the four token classes, then row 4*cls + j of the tile, dims 8*col .. of the head
+  float l = head.l;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  const float linv = l > 0.f ? 1.f / l : 0.f;
+  T* out = reinterpret_cast<T*>(a.out);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = 4 * cls + j;
+    const float lj = __shfl(linv, r, 64);                 // lane r (class 0) holds column r
+    if (r < rows && (D == 128 || col < D / 8)) {
+      T o8[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o8[e] = from_float<T>(head.o[e][j] * lj);
+      *reinterpret_cast<uint4*>(out + ((int64_t)(seq_start + row0 + r) * a.num_heads + h) * D + col * 8) =
+          *reinterpret_cast<const uint4*>(o8);
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -1095,6 +1189,15 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
     case MVLLM_BF16: return launch_decode<bf16_t>(a, int8, fast_ok, split, s);
     default: return launch_decode<f16_t>(a, int8, fast_ok, split, s);
   }
+}
+
+int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream) {
+  if (head_dim != 64 || dtype == MVLLM_F32) return MVLLM_ERR_UNSUPPORTED;
+  const int64_t tiles = a.total_tokens / kTile + a.num_seqs;      // upper bound on the 16-row tiles
+  const dim3 grid((unsigned)tiles, (unsigned)((a.num_heads + 3) / 4)), block(256);
+  if (dtype == MVLLM_BF16) prefill_rows16_kernel<bf16_t, 64><<<grid, block, 0, stream>>>(a, (int)tiles);
+  else prefill_rows16_kernel<f16_t, 64><<<grid, block, 0, stream>>>(a, (int)tiles);
+  return launch_status();
 }
 
 }  // namespace mvllm

@@ -34,44 +34,6 @@ struct PrefillArgs {
   int64_t num_blocks;
 };
 
-// Tile `tile` (global numbering) -> sequence and first row inside it.  Wave-parallel: 64 sequences
-// per step (tile counts, inclusive prefix sum by shuffles, ballot to pick the owner), so the cost is
-// a few hundred cycles per 64 sequences instead of one dependent load per sequence.  Every lane of
-// the calling wave must be active; all lanes return the same values.
-__device__ __forceinline__ bool locate_tile(const int32_t* __restrict__ cu, int num_seqs, int tile, int bm,
-                                            int& seq_start, int& seq_len, int& row0, int& seq_index) {
-  const int lane = threadIdx.x & 63;
-  int first = 0;
-  for (int base = 0; base < num_seqs; base += 64) {
-    const int s = base + lane;
-    int lo = 0, len = 0;
-    if (s < num_seqs) {
-      lo = cu[s];
-      len = cu[s + 1] - lo;
-    }
-    const int n = (len + bm - 1) / bm;
-    int incl = n;                                   // inclusive prefix sum of tile counts over the lanes
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int t = __shfl_up(incl, o, 64);
-      if (lane >= o) incl += t;
-    }
-    const int total = __shfl(incl, 63, 64);
-    if (tile < first + total) {
-      const unsigned long long owners = __ballot(tile < first + incl);   // first lane whose prefix passes the tile
-      const int owner = __ffsll((long long)owners) - 1;
-      const int start_tile = first + __shfl(incl - n, owner, 64);
-      seq_start = __shfl(lo, owner, 64);
-      seq_len = __shfl(len, owner, 64);
-      row0 = (tile - start_tile) * bm;
-      seq_index = base + owner;
-      return true;
-    }
-    first += total;
-  }
-  return false;
-}
-
 // ---------------------------------------------------------------------------
 // Generic path: any element type, head_dim <= 512.  One wave per query row,
 // lanes split head_dim, one key per step.  Correctness path (fp32 inputs and
@@ -675,6 +637,14 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 && (group == 1 || group == 2 || group % 4 == 0) &&
                        aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
                        num_kv_heads * group <= 65535;
+  // head_dim 64 in 16 bit: 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
+  if (!mfma_ok && dtype != MVLLM_F32 && head_dim == 64 && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
+      (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31)) {
+    PrefillRowsArgs r;
+    r.out = out; r.q = q; r.k = k; r.v = v; r.cu_seqlens = cu_seqlens; r.total_tokens = total_tokens;
+    r.num_seqs = num_seqs; r.num_heads = num_heads; r.num_kv_heads = num_kv_heads; r.scale_log2 = scale * kLog2e;
+    return launch_prefill_rows16(r, head_dim, dtype, (hipStream_t)stream);
+  }
   return prefill_dispatch<false>(a, dtype, mfma_ok, (hipStream_t)stream);
 }
 

@@ -97,3 +97,34 @@ def test_config2_full_size():
                                  torch.tensor(lengths, device=DEV), scale, hq, hkv, d, bs).cpu()
     mx, mean = error_stats(dec, out[last])
     assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,lengths", [
+    (16, 8, [64, 1, 130, 257, 31]),          # the reference demo's heads (main.py: 16 q / 8 kv heads of 64 dims)
+    (12, 12, [200, 15, 16, 17]),             # qwen3.py:333-339 self-test: 12 heads
+    (12, 1, [96, 33, 1000]),                 # one kv head
+    (6, 2, [17, 0, 5, 0, 48]),               # heads not a multiple of the four waves; empty sequences
+])
+def test_prefill_head_dim_64_vs_oracle(dtype, hq, hkv, lengths):
+    """head_dim 64 in 16 bit runs on 16-row tiles of the decode kernel's arithmetic (not on the generic kernel)."""
+    d = 64
+    case = make_varlen_case(56, lengths, hq, hkv, d, dtype=dtype)
+    scale = 1 / math.sqrt(d)
+    got = _run(*case, scale, hq, hkv, d)
+    want = _oracle32(*case, scale, hq, hkv, d)
+    mx, mean = error_stats(got, want)
+    assert got.dtype == dtype and got.shape == want.shape
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+    # first row of each sequence is exactly its own V row; rows do not depend on later sequences
+    q, k, v, cu = case
+    for s, n in enumerate(lengths):
+        if n:
+            lo = int(cu[s])
+            assert torch.equal(got[lo], v[lo].repeat_interleave(hq // hkv, dim=0))
+    k2, v2 = k.clone(), v.clone()
+    first = next(i for i, n in enumerate(lengths) if n)
+    cut = int(cu[first + 1])
+    k2[cut:] = 1.0
+    v2[cut:] = -1.0
+    assert torch.equal(_run(q, k2, v2, cu, scale, hq, hkv, d)[:cut], got[:cut])
