@@ -197,6 +197,13 @@ struct PrefillRowsArgs {
   int num_heads;
   int num_kv_heads;
   float scale_log2;
+  // paged mode (k, v are caches [num_blocks, block_size, Hkv, D] holding every key; cu_seqlens counts the query
+  // rows, cu_seqlens_k the keys): null / 0 otherwise
+  const int32_t* cu_seqlens_k;
+  const int32_t* block_tables;
+  int max_num_blocks;
+  int block_size;
+  int64_t num_blocks;
 };
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream);
 

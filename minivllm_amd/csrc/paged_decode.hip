@@ -505,7 +505,9 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
 // heads on the same rows, so with grouped heads they read the same K/V tiles at the same time.  No LDS and no
 // reuse of K/V across row tiles beyond the caches: tens of TFLOP/s, not hundreds.
 // ---------------------------------------------------------------------------
-template <typename T, int D>
+// PAGED: prefill of the rows that follow a cached prefix (mvllm_prefill_paged): row r of a sequence sits at key
+// position cached + r and every key is read from the paged cache through the block table, as in decode.
+template <typename T, int D, bool PAGED>
 __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsArgs a, int tiles_x) {
   int seq_start, seq_len, row0, seq_index;
   // latest (heaviest) tiles first
@@ -532,25 +534,56 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
 #pragma unroll
     for (int e = 0; e < 8; ++e) head.o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
   }
-  const int kv_end = row0 + rows;        // keys 0 .. kv_end - 1 are seen by at least one row of the tile
-  const int col_end = row0 + col + 1;    // keys seen by this lane's row
+  const int cached = PAGED ? max(a.cu_seqlens_k[seq_index + 1] - a.cu_seqlens_k[seq_index] - seq_len, 0) : 0;
+  const int kv_end = cached + row0 + rows;        // keys 0 .. kv_end - 1 are seen by at least one row of the tile
+  const int col_end = cached + row0 + col + 1;    // keys seen by this lane's row
   const int ntiles = (kv_end + kTile - 1) / kTile;
   const int64_t row = (int64_t)a.num_kv_heads * D;
-  const T* kc = reinterpret_cast<const T*>(a.k) + (int64_t)seq_start * row + (int64_t)g * D + cls * 8;
-  const T* vc = reinterpret_cast<const T*>(a.v) + (int64_t)seq_start * row + (int64_t)g * D + col * 8;
+  const T* kc = reinterpret_cast<const T*>(a.k) + (PAGED ? 0 : (int64_t)seq_start * row) + (int64_t)g * D + cls * 8;
+  const T* vc = reinterpret_cast<const T*>(a.v) + (PAGED ? 0 : (int64_t)seq_start * row) + (int64_t)g * D + col * 8;
+  // paged: block-table window, lane i holds entry win_base + i of this sequence (as in the decode kernel)
+  const int bs = PAGED ? a.block_size : 1;
+  const int32_t* table = PAGED ? a.block_tables + (int64_t)seq_index * a.max_num_blocks : nullptr;
+  int bi = 0, off = 0, win_base = 0, win = -1;
+  if (PAGED) win = lane < a.max_num_blocks ? table[lane] : -1;
 
-  // Tokens past kv_end are masked by consume(); their loads are redirected to the last visible row so that
-  // nothing past the end of the packed tensors is touched.
+  // Tokens past kv_end are masked by consume(); in the packed tensors their loads are redirected to the last
+  // visible row so that nothing past the end is touched (in a cache block they are rows of the same block).
   auto load_tile = [&](KVTile<T>& t, int tile) __attribute__((always_inline)) {
     t.t0 = tile * kTile;
     t.ok = true;
-    const T* kp = kc + (int64_t)min(t.t0 + col, kv_end - 1) * row;
+    int64_t k_tok, v_tok[4];
+    if constexpr (PAGED) {
+      if (bi - win_base >= 64) {
+        win_base = bi;
+        win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
+      }
+      const int phys = __builtin_amdgcn_readlane(win, bi - win_base);
+      t.ok = (bi < a.max_num_blocks) && phys >= 0 && (int64_t)phys < a.num_blocks;
+      const int64_t tok0 = (int64_t)(t.ok ? phys : 0) * bs + off;
+      k_tok = tok0 + col;
 #pragma unroll
-    for (int j = 0; j < D / 32; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
+      for (int i = 0; i < 4; ++i) v_tok[i] = tok0 + 4 * cls + i;
+      off += kTile;
+      if (off >= bs) { off = 0; ++bi; }
+    } else {
+      k_tok = min(t.t0 + col, kv_end - 1);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      t.v[i] = (D == 128 || col < D / 8) ? *reinterpret_cast<const uint4*>(vc + (int64_t)min(t.t0 + 4 * cls + i, kv_end - 1) * row)
-                                         : make_uint4(0u, 0u, 0u, 0u);
+      for (int i = 0; i < 4; ++i) v_tok[i] = min(t.t0 + 4 * cls + i, kv_end - 1);
+    }
+    if (t.ok) {
+      const T* kp = kc + k_tok * row;
+#pragma unroll
+      for (int j = 0; j < D / 32; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        t.v[i] = (D == 128 || col < D / 8) ? *reinterpret_cast<const uint4*>(vc + v_tok[i] * row) : make_uint4(0u, 0u, 0u, 0u);
+    } else {
+#pragma unroll
+      for (int j = 0; j < D / 32; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
   };
   KVTile<T> ta, tb;
   if (ntiles > 0) load_tile(ta, 0);
@@ -1195,8 +1228,15 @@ int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hip
   if (head_dim != 64 || dtype == MVLLM_F32) return MVLLM_ERR_UNSUPPORTED;
   const int64_t tiles = a.total_tokens / kTile + a.num_seqs;      // upper bound on the 16-row tiles
   const dim3 grid((unsigned)tiles, (unsigned)((a.num_heads + 3) / 4)), block(256);
-  if (dtype == MVLLM_BF16) prefill_rows16_kernel<bf16_t, 64><<<grid, block, 0, stream>>>(a, (int)tiles);
-  else prefill_rows16_kernel<f16_t, 64><<<grid, block, 0, stream>>>(a, (int)tiles);
+  const bool paged = a.block_tables != nullptr;
+  if (paged && a.block_size % kTile != 0) return MVLLM_ERR_UNSUPPORTED;
+  if (dtype == MVLLM_BF16) {
+    if (paged) prefill_rows16_kernel<bf16_t, 64, true><<<grid, block, 0, stream>>>(a, (int)tiles);
+    else prefill_rows16_kernel<bf16_t, 64, false><<<grid, block, 0, stream>>>(a, (int)tiles);
+  } else {
+    if (paged) prefill_rows16_kernel<f16_t, 64, true><<<grid, block, 0, stream>>>(a, (int)tiles);
+    else prefill_rows16_kernel<f16_t, 64, false><<<grid, block, 0, stream>>>(a, (int)tiles);
+  }
   return launch_status();
 }
 

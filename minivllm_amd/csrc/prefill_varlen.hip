@@ -643,6 +643,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
     PrefillRowsArgs r;
     r.out = out; r.q = q; r.k = k; r.v = v; r.cu_seqlens = cu_seqlens; r.total_tokens = total_tokens;
     r.num_seqs = num_seqs; r.num_heads = num_heads; r.num_kv_heads = num_kv_heads; r.scale_log2 = scale * kLog2e;
+    r.cu_seqlens_k = nullptr; r.block_tables = nullptr; r.max_num_blocks = 0; r.block_size = 0; r.num_blocks = 0;
     return launch_prefill_rows16(r, head_dim, dtype, (hipStream_t)stream);
   }
   return prefill_dispatch<false>(a, dtype, mfma_ok, (hipStream_t)stream);
@@ -675,5 +676,14 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
                        block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) &&
                        aligned16(out) && num_kv_heads * group <= 65535 &&
                        (int64_t)block_size * num_kv_heads * head_dim * 2 < ((int64_t)1 << 31);
+  if (!mfma_ok && dtype != MVLLM_F32 && head_dim == 64 && block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) &&
+      aligned16(v_cache) && aligned16(out) && (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31)) {
+    PrefillRowsArgs r;
+    r.out = out; r.q = q; r.k = k_cache; r.v = v_cache; r.cu_seqlens = cu_seqlens_q; r.total_tokens = total_q_tokens;
+    r.num_seqs = num_seqs; r.num_heads = num_heads; r.num_kv_heads = num_kv_heads; r.scale_log2 = scale * kLog2e;
+    r.cu_seqlens_k = cu_seqlens_k; r.block_tables = block_tables; r.max_num_blocks = max_num_blocks;
+    r.block_size = block_size; r.num_blocks = num_blocks;
+    return launch_prefill_rows16(r, head_dim, dtype, (hipStream_t)stream);
+  }
   return prefill_dispatch<true>(a, dtype, mfma_ok, (hipStream_t)stream);
 }

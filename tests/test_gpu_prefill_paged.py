@@ -48,7 +48,11 @@ def _check(got, want, dtype):
     (8, 8, 128, 32, [150], [96]),                                  # no grouping
     (32, 8, 128, 16, [131, 77, 260], [50, 1, 259]),                # prefixes at arbitrary token counts, 1 new token
     (6, 2, 80, 8, [40, 23], [16, 8]),                              # generic kernel (head_dim 80)
-    (4, 4, 64, 16, [70], [32]),                                    # generic kernel (head_dim 64)
+    (4, 4, 64, 16, [70], [32]),                                    # head_dim 64: 16-row tiles (fp32: generic kernel)
+    (16, 8, 64, 16, [300, 64, 129, 500], [256, 0, 17, 48]),        # head_dim 64, the reference demo's heads
+    (12, 1, 64, 256, [700, 30, 257], [512, 29, 0]),                # head_dim 64, one kv head, the engine's block size
+    (6, 2, 64, 48, [131, 77, 260], [50, 1, 259]),                  # head_dim 64, heads not a multiple of four
+    (4, 4, 64, 8, [70], [32]),                                     # head_dim 64 with a block size of 8: generic kernel
 ])
 def test_paged_prefill_vs_oracle(dtype, hq, hkv, d, bs, lengths, cached):
     c = make_paged_prefill_case(61, lengths, cached, hq, hkv, d, bs, dtype=dtype)
@@ -127,3 +131,11 @@ def test_attention_module_uses_the_paged_prefill_when_block_tables_are_set():
     want = _oracle32(c, 1 / math.sqrt(d), hq, hkv, d, bs).reshape(out.shape[0], -1)
     mx, mean = error_stats(out, want)
     assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16
+
+
+def test_paged_prefill_head_dim_64_without_prefix_matches_plain_prefill_bitwise():
+    hq, hkv, d, bs = 16, 8, 64, 16
+    c = make_paged_prefill_case(66, [90, 1, 257, 33], [0, 0, 0, 0], hq, hkv, d, bs, dtype=torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    plain = flash_attention_prefill(c["q"].to(DEV), c["k"].to(DEV), c["v"].to(DEV), c["cu_k"].to(DEV), scale, hq, hkv, d).cpu()
+    assert torch.equal(_run(c, scale, hq, hkv, d, bs), plain)
