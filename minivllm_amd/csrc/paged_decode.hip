@@ -498,7 +498,8 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
 
 // ---------------------------------------------------------------------------
 // Varlen causal prefill on the same tile arithmetic (flash_attention_prefill, attention.py:212-280, for 16-bit
-// head dims the LDS-tiled kernel of prefill_varlen.hip is not built for: head_dim 64, the reference demo's model).
+// shapes the LDS-tiled kernel of prefill_varlen.hip is not built for: head_dim 64, the reference demo's model, and
+// head_dim 128 with 3, 5, 6, 7, ... query heads per kv head).
 // One wave = 16 consecutive query rows of one query head: the rows take the place of the heads of a group
 // (column n of the first product = row n), the keys 0 .. row are walked in 16-token tiles straight from the
 // packed k / v tensors, and the causal limit is applied per column.  The four waves of a workgroup are four query
@@ -1224,18 +1225,22 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
   }
 }
 
+template <typename T, int D>
+static void launch_rows16(const PrefillRowsArgs& a, dim3 grid, int tiles, hipStream_t stream) {
+  if (a.block_tables) prefill_rows16_kernel<T, D, true><<<grid, dim3(256), 0, stream>>>(a, tiles);
+  else prefill_rows16_kernel<T, D, false><<<grid, dim3(256), 0, stream>>>(a, tiles);
+}
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream) {
-  if (head_dim != 64 || dtype == MVLLM_F32) return MVLLM_ERR_UNSUPPORTED;
+  if ((head_dim != 64 && head_dim != 128) || dtype == MVLLM_F32) return MVLLM_ERR_UNSUPPORTED;
+  if (a.block_tables && a.block_size % kTile != 0) return MVLLM_ERR_UNSUPPORTED;
   const int64_t tiles = a.total_tokens / kTile + a.num_seqs;      // upper bound on the 16-row tiles
-  const dim3 grid((unsigned)tiles, (unsigned)((a.num_heads + 3) / 4)), block(256);
-  const bool paged = a.block_tables != nullptr;
-  if (paged && a.block_size % kTile != 0) return MVLLM_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)tiles, (unsigned)((a.num_heads + 3) / 4));
   if (dtype == MVLLM_BF16) {
-    if (paged) prefill_rows16_kernel<bf16_t, 64, true><<<grid, block, 0, stream>>>(a, (int)tiles);
-    else prefill_rows16_kernel<bf16_t, 64, false><<<grid, block, 0, stream>>>(a, (int)tiles);
+    if (head_dim == 64) launch_rows16<bf16_t, 64>(a, grid, (int)tiles, stream);
+    else launch_rows16<bf16_t, 128>(a, grid, (int)tiles, stream);
   } else {
-    if (paged) prefill_rows16_kernel<f16_t, 64, true><<<grid, block, 0, stream>>>(a, (int)tiles);
-    else prefill_rows16_kernel<f16_t, 64, false><<<grid, block, 0, stream>>>(a, (int)tiles);
+    if (head_dim == 64) launch_rows16<f16_t, 64>(a, grid, (int)tiles, stream);
+    else launch_rows16<f16_t, 128>(a, grid, (int)tiles, stream);
   }
   return launch_status();
 }
