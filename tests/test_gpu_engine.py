@@ -134,3 +134,22 @@ def test_prefix_cache_hits_are_read_from_the_paged_cache():
     assert skipped[0] >= 48 + 48 + 16, skipped            # the 2nd step reuses 3 blocks twice, the 3rd at least 1
     same = sum(a == b for a, b in zip(*outs))
     assert same >= 4, outs                                # a 1-ulp difference may flip a sampling tie, rarely
+
+
+def test_reference_demo_model_shape_head_dim_64():
+    """The reference's demo model (main.py:18-30: 16 query / 8 kv heads of 64 dims) in bf16: generation with the
+    hipGraph decode path agrees with the eager path, prefix-cache hits are read from the paged cache, and both runs
+    use the MFMA decode kernels and the 16-row tile prefill (head_dim 64 has no generic-kernel fallback in 16 bit)."""
+    from minivllm_amd.layers.attention import paged_decode_plan
+    cfg = dict(SMALL, hidden_size=1024, num_heads=16, num_kv_heads=8, head_dim=64, num_layers=2,
+               max_num_sequences=4, max_cached_blocks=96, max_model_length=128)
+    assert paged_decode_plan(4, 16, 8, 64, 128 // 16, 16)[2] > 0
+    g = torch.Generator().manual_seed(21)
+    shared = torch.randint(0, 2048, (32,), generator=g).tolist()
+    prompts = [shared + torch.randint(0, 2048, (n,), generator=g).tolist() for n in (7, 20, 1)] + _prompts(3, 3, 40, seed=22)
+    sp = SamplingParams(temperature=0.7, max_tokens=16, ignore_eos=True)
+    eager = LLMEngine(dict(cfg, enforce_eager=True, prefix_caching=False)).generate(prompts, sp)["token_ids"]
+    graphed = LLMEngine(dict(cfg, enforce_eager=False, prefix_caching=True)).generate(prompts, sp)["token_ids"]
+    assert [len(t) for t in graphed] == [16] * 6
+    same = sum(a == b for a, b in zip(eager, graphed))
+    assert same >= 4, (same, eager, graphed)          # a 1-ulp difference may flip a sampling tie, rarely
