@@ -655,10 +655,12 @@ __device__ __forceinline__ uint2 load8_stream(const void* p) {
 }
 
 // W as in decode_mfma_item: 1 = the wave walks its partition, > 1 = W waves of the workgroup share it.
-template <typename T, int NCH, int W>
+template <typename T, int NCH, int W, int D>
 __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b, int p, int g, int w) {   // g: kv head
   static_assert(NCH == 1, "one chunk of up to 16 heads");
-  constexpr int D = 128;
+  static_assert(D == 128 || D == 64, "one or two 64-dim steps");
+  constexpr int kSteps = D / 64;               // 64-dim steps of the first product
+  const bool owns = D == 128 || (threadIdx.x & 15) < D / 8;   // this lane's 8 output dims exist
   const int lane = threadIdx.x & 63;
   const int group = a.num_heads / a.num_kv_heads;
   const int q4 = lane >> 4;            // token class: tokens 4*q4 .. 4*q4+3 of a tile
@@ -683,16 +685,16 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
   if constexpr (W == 1) win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
 
   // ---- query -> int8 hi/lo planes (B operand: column lane%16 -> head, bytes 16*q4.. of each 64-dim step)
-  v4i qhi[2], qlo[2];
+  v4i qhi[kSteps], qlo[kSteps];
   float qscale;                        // amax/16256 * scale*log2e of this lane's head
   {
     const T* q = reinterpret_cast<const T*>(a.q);
     const bool live = col < group;
     const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D;
-    float x[2][16];
+    float x[kSteps][16];
     float amax = 0.f;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < kSteps; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         x[j][e] = live ? to_float(src[64 * j + 16 * q4 + e]) : 0.f;
@@ -703,7 +705,7 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
     const float to_fix = amax > 0.f ? 16256.f / amax : 0.f;
     qscale = amax * (1.f / 16256.f) * a.scale_log2;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < kSteps; ++j) {
       int hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
@@ -744,15 +746,16 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
       const int64_t tok0 = (int64_t)phys * bs + off;
       const char* kp = kc + tok0 * row + k_lane_off;
       const char* vp = vc + tok0 * row + v_lane_off;
-      t.k[0] = *reinterpret_cast<const uint4*>(kp);
-      t.k[1] = *reinterpret_cast<const uint4*>(kp + 64);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) t.v[i] = load8_stream(vp + i * row);
+      for (int j = 0; j < kSteps; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 64 * j);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.v[i] = owns ? load8_stream(vp + i * row) : make_uint2(0u, 0u);
       const int64_t sidx = (tok0 + s_lane_tok) * a.num_kv_heads + g;
       t.ks = a.k_scale[sidx];
       t.vs = a.v_scale[sidx];
     } else {
-      t.k[0] = t.k[1] = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int j = 0; j < kSteps; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
       for (int i = 0; i < 4; ++i) t.v[i] = make_uint2(0u, 0u);
       t.ks = t.vs = 0.f;
@@ -784,7 +787,7 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
     for (int r = 0; r < 4; ++r) lv4[r] = __log2f(fmaxf(vs4[r], 9.094947e-13f));
     v4i shi = {0, 0, 0, 0}, slo = {0, 0, 0, 0};
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < kSteps; ++j) {
       const v4i kf = (v4i){(int)t.k[j].x, (int)t.k[j].y, (int)t.k[j].z, (int)t.k[j].w};
       shi = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qhi[j], shi, 0, 0, 0);
       slo = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qlo[j], slo, 0, 0, 0);
@@ -906,7 +909,7 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
     const int h = 4 * q4 + j;
     const float bias = 1152.f * __shfl(wsum, h, 64);          // lane h (class 0) holds head h
     const float lj = __shfl(linv, h, 64);
-    if (h < group) {
+    if (h < group && owns) {
       if (direct) {
         T r[8];
 #pragma unroll
@@ -941,17 +944,17 @@ __global__ __launch_bounds__(64 * W, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma
   const int p = (int)((blockIdx.y + (unsigned)b) % (unsigned)a.num_parts);
   decode_mfma_item<T, W, D>(a, b, p, g, threadIdx.x >> 6);
 }
-template <typename T, int NCH>
+template <typename T, int NCH, int D>
 __global__ __launch_bounds__(MVLLM_DECODE_I8_THREADS, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
   int b, p, hg;
   if (!decode_item<true>(a, b, p, hg)) return;
-  decode_mfma_int8_item<T, NCH, 1>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
+  decode_mfma_int8_item<T, NCH, 1, D>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
 }
-template <typename T, int W>
+template <typename T, int W, int D>
 __global__ __launch_bounds__(64 * W, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_split_kernel(const DecodeArgs a) {
   const int g = blockIdx.x, b = blockIdx.z;
   const int p = (int)((blockIdx.y + (unsigned)b) % (unsigned)a.num_parts);
-  decode_mfma_int8_item<T, 1, W>(a, b, p, g, threadIdx.x >> 6);
+  decode_mfma_int8_item<T, 1, W, D>(a, b, p, g, threadIdx.x >> 6);
 }
 
 // ---------------------------------------------------------------------------
@@ -1118,7 +1121,8 @@ static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int ma
 
 // shapes the MFMA kernels are built for (pointer alignment is checked by the caller)
 static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool int8) {
-  const bool dim_ok = head_dim == 128 || (head_dim == 64 && !int8);     // the INT8 kernel is built for 128 only
+  (void)int8;
+  const bool dim_ok = head_dim == 128 || head_dim == 64;
   return dtype != MVLLM_F32 && dim_ok && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
          (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
 }
@@ -1146,7 +1150,8 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
   if constexpr (IsSixteenBit<T>::value) {
     if (fast_ok && split) {
       const dim3 grid((unsigned)a.num_kv_heads, (unsigned)a.num_parts, (unsigned)a.batch), block(64 * kSplitWaves);
-      if (int8) decode_mfma_int8_split_kernel<T, kSplitWaves><<<grid, block, 0, stream>>>(a);
+      if (int8 && a.head_dim == 64) decode_mfma_int8_split_kernel<T, kSplitWaves, 64><<<grid, block, 0, stream>>>(a);
+      else if (int8) decode_mfma_int8_split_kernel<T, kSplitWaves, 128><<<grid, block, 0, stream>>>(a);
       else if (a.head_dim == 64) decode_mfma_split_kernel<T, kSplitWaves, 64><<<grid, block, 0, stream>>>(a);
       else decode_mfma_split_kernel<T, kSplitWaves, 128><<<grid, block, 0, stream>>>(a);
       launched = true;
@@ -1158,7 +1163,8 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
         wpb = largest_divisor_le(a.num_kv_heads, wpb - 1);
       const unsigned groups = (unsigned)(a.num_kv_heads / wpb);
       dim3 block(64 * wpb);
-      if (int8) decode_mfma_int8_kernel<T, 1><<<dim3((unsigned)a.num_parts, groups, (unsigned)a.batch), block, 0, stream>>>(a);
+      if (int8 && a.head_dim == 64) decode_mfma_int8_kernel<T, 1, 64><<<dim3((unsigned)a.num_parts, groups, (unsigned)a.batch), block, 0, stream>>>(a);
+      else if (int8) decode_mfma_int8_kernel<T, 1, 128><<<dim3((unsigned)a.num_parts, groups, (unsigned)a.batch), block, 0, stream>>>(a);
       else if (a.head_dim == 64) decode_mfma_kernel<T, 64><<<dim3((unsigned)a.num_parts, (unsigned)a.batch, groups), block, 0, stream>>>(a);
       else decode_mfma_kernel<T, 128><<<dim3((unsigned)a.num_parts, (unsigned)a.batch, groups), block, 0, stream>>>(a);
       launched = true;

@@ -70,8 +70,9 @@ def test_decode_plan_is_host_arithmetic():
     # INT8 caches, and shapes outside the MFMA kernels
     assert paged_decode_plan(64, 32, 8, 128, 256, 16, int8_cache=True) == (4096, 1, 4)
     assert paged_decode_plan(256, 32, 8, 128, 256, 16, int8_cache=True) == (1024, 4, 1)     # large INT8 batch: first form
-    assert paged_decode_plan(64, 16, 16, 64, 256, 16)[2] == 4                 # head_dim 64: MFMA kernels, 16-bit caches
-    assert paged_decode_plan(64, 16, 16, 64, 256, 16, int8_cache=True)[2] == 0
+    assert paged_decode_plan(64, 16, 16, 64, 256, 16)[2] == 4                 # head_dim 64: MFMA kernels, both cache types
+    assert paged_decode_plan(64, 16, 16, 64, 256, 16, int8_cache=True)[2] == 1      # 1024 (sequence, head) pairs: first form
+    assert paged_decode_plan(64, 16, 16, 96, 256, 16, int8_cache=True)[2] == 0
     assert paged_decode_plan(64, 16, 16, 96, 256, 16)[2] == 0                 # other head dims
     import torch
     assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32)[2] == 0

@@ -60,9 +60,9 @@ def test_int8_context_boundaries(ctx_list):
     _check(_quantised_case(62, 0, 0, 0, hq, hkv, d, bs, ctx_list=ctx_list), hq, hkv, d, bs, 0.1, torch.int32)
 
 
-@pytest.mark.parametrize("hq,hkv,d,bs", [(16, 16, 64, 16), (34, 2, 128, 16), (4, 2, 128, 8)])
+@pytest.mark.parametrize("hq,hkv,d,bs", [(16, 16, 96, 16), (34, 2, 128, 16), (4, 2, 128, 8), (8, 4, 64, 8)])
 def test_int8_generic_path(hq, hkv, d, bs):
-    """head_dim 64, GQA 17 and block_size 8 run on the generic kernel."""
+    """head_dim 96, GQA 17 and block_size 8 run on the generic kernel."""
     _check(_quantised_case(63, 5, 1, 300, hq, hkv, d, bs), hq, hkv, d, bs, 1 / math.sqrt(d))
 
 
@@ -90,11 +90,11 @@ def test_config4_subset():
     _check(case, hq, hkv, d, bs, 1 / math.sqrt(d))
 
 
-@pytest.mark.parametrize("hq,hkv,bs", [(32, 8, 16), (16, 8, 256), (16, 1, 32), (24, 2, 16), (5, 1, 64)])
+@pytest.mark.parametrize("hq,hkv,bs,d", [(32, 8, 16, 128), (16, 8, 256, 128), (16, 1, 32, 128), (24, 2, 16, 128),
+                                         (5, 1, 64, 128), (16, 8, 16, 64), (12, 1, 32, 64), (8, 4, 256, 64)])
 @pytest.mark.parametrize("form", ["one wave per head", "waves share a head", "waves share a head, one partition"])
-def test_int8_both_grid_forms(hq, hkv, bs, form):
+def test_int8_both_grid_forms(hq, hkv, bs, d, form):
     """As test_both_grid_forms_vs_oracle of the 16-bit cache: the table width and the batch size pick the form."""
-    d = 128
     batch = 7 if form == "waves share a head" else 64
     width = {"one wave per head": 32768, "waves share a head": 8192}.get(form, 4096) // bs * bs
     g = torch.Generator().manual_seed(66)
