@@ -97,8 +97,9 @@ size_t mvllm_paged_decode_workspace_bytes(int batch, int num_heads, int head_dim
  *   *num_parts        partitions per sequence (1: no workspace is touched and no merge kernel is launched)
  *   *waves_per_head   1: a workgroup holds up to 4 kv heads, one wave each, and every wave walks its partition;
  *                     >1: small-batch form, a workgroup is that many waves on one kv head that share the
- *                     partition's 16-token tiles and merge in LDS; 0: the generic kernel (fp32, head_dim other
- *                     than 128 or 64, block_size % 16 != 0 or more than 16 query heads per kv head)
+ *                     partition's 16-token tiles and merge in LDS; 0: the generic kernel (head_dim other than
+ *                     128 or 64, block_size % 16 != 0, more than 16 query heads per kv head, or fp32 queries over
+ *                     an INT8 cache)
  * Returns MVLLM_OK or MVLLM_ERR_BAD_SHAPE / MVLLM_ERR_BAD_DTYPE.
  */
 int mvllm_paged_decode_plan(int batch, int num_heads, int num_kv_heads, int head_dim,

@@ -184,11 +184,71 @@ __device__ __forceinline__ bool decode_item(const DecodeArgs& a, int& b, int& p,
 // Fast path
 // ---------------------------------------------------------------------------
 template <typename T>
-struct KVTile {
+struct KVTile {          // 16-bit elements: lane l holds 8 dims (16 B) of token l%16 per 32-dim step, and of its four V tokens
   uint4 k[4];
   uint4 v[4];
   int t0;
   bool ok;
+};
+template <>
+struct KVTile<float> {   // fp32: 4 dims (16 B) of token l%16 per 16-dim step; of each V token 4 dims per 64-dim step
+  float4 k[8];
+  float4 v[4][2];
+  int t0;
+  bool ok;
+};
+
+// How a lane's share of a tile is addressed and loaded.  kp points at (token lane%16, first dim of class lane/16),
+// vp at (one of the lane's four tokens, first dim of column lane%16).
+template <typename T, int D>
+struct TileIO {
+  static constexpr int kKLane = 8;     // dims between the classes (lane/16) of the first product
+  static constexpr int kVLane = 8;     // dims per column (lane%16) of the second product
+  static __device__ __forceinline__ bool owns(int col) { return D == 128 || col < D / 8; }
+  static __device__ __forceinline__ void load_k(KVTile<T>& t, const T* kp) {
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
+  }
+  template <bool STREAM>
+  static __device__ __forceinline__ void load_v(KVTile<T>& t, int i, const T* vp, bool own) {
+    t.v[i] = !own ? make_uint4(0u, 0u, 0u, 0u) : STREAM ? load16_stream(vp) : *reinterpret_cast<const uint4*>(vp);
+  }
+  static __device__ __forceinline__ void zero(KVTile<T>& t) {
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
+  }
+};
+template <int D>
+struct TileIO<float, D> {
+  static constexpr int kKLane = 4;
+  static constexpr int kVLane = 4;
+  static __device__ __forceinline__ bool owns(int) { return true; }     // 16 columns x 4 dims per 64-dim step
+  static __device__ __forceinline__ void load_k(KVTile<float>& t, const float* kp) {
+#pragma unroll
+    for (int j = 0; j < D / 16; ++j) t.k[j] = *reinterpret_cast<const float4*>(kp + 16 * j);
+  }
+  template <bool STREAM>
+  static __device__ __forceinline__ void load_v(KVTile<float>& t, int i, const float* vp, bool) {
+#pragma unroll
+    for (int jj = 0; jj < D / 64; ++jj) {
+      if (STREAM) {
+        const uint4 x = load16_stream(vp + 64 * jj);
+        t.v[i][jj] = make_float4(__uint_as_float(x.x), __uint_as_float(x.y), __uint_as_float(x.z), __uint_as_float(x.w));
+      } else {
+        t.v[i][jj] = *reinterpret_cast<const float4*>(vp + 64 * jj);
+      }
+    }
+  }
+  static __device__ __forceinline__ void zero(KVTile<float>& t) {
+#pragma unroll
+    for (int j = 0; j < D / 16; ++j) t.k[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int jj = 0; jj < D / 64; ++jj) t.v[i][jj] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
 };
 
 // 16-bit pair (a, b) in the element type
@@ -205,6 +265,36 @@ template <> __device__ __forceinline__ v4f mfma16x16x16<bf16_t>(uint2 x, uint2 y
 }
 template <> __device__ __forceinline__ v4f mfma16x16x16<f16_t>(uint2 x, uint2 y, v4f c) {
   return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(v4f16, x), __builtin_bit_cast(v4f16, y), c, 0, 0, 0);
+}
+
+// Shared by the 16-bit and fp32 heads (HEAD has m, l, o[kAcc], write_row, write_partial).
+template <typename HEAD>
+__device__ __forceinline__ void finish_head(HEAD& hd, const DecodeArgs& a, int b, int p, int g, int group, bool direct, int lane) {
+  using T = typename HEAD::Elem;
+  constexpr int D = HEAD::kDim;
+  const int cls = lane >> 4;
+  // denominators: add the four token classes (every lane of a head then holds the head's total)
+  hd.l += __shfl_xor(hd.l, 16, 64);
+  hd.l += __shfl_xor(hd.l, 32, 64);
+  const int head0 = g * group;
+  if (direct) {
+    T* out = reinterpret_cast<T*>(a.out);
+    const float linv = hd.l > 0.f ? 1.f / hd.l : 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int h = 4 * cls + j;
+      const float lj = __shfl(linv, h, 64);               // lane h (class 0) holds head h
+      if (h < group) hd.write_row(out + ((int64_t)b * a.num_heads + head0 + h) * D, j, lj, lane);
+    }
+  } else {
+    const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int h = 4 * cls + j;
+      if (h < group) hd.write_partial(a.ws_acc + (slot + h) * D, j, lane);
+    }
+    if (lane < group && lane < 16) *reinterpret_cast<float2*>(a.ws_ml + (slot + lane) * 2) = make_float2(hd.m, hd.l);
+  }
 }
 
 // One wave = one kv head of one (sequence, partition); both products run on the matrix unit.
@@ -226,6 +316,8 @@ template <> __device__ __forceinline__ v4f mfma16x16x16<f16_t>(uint2 x, uint2 y,
 // nothing.
 template <typename T, int D>
 struct DecodeHead {
+  using Elem = T;
+  static constexpr int kDim = D;
   static constexpr int kSteps = D / 32;     // 32-dim steps of the first product
   static constexpr int kCols = D / 8;       // lanes (l%16) that own 8 dims of the output
   uint4 qf[kSteps];           // Q fragments: B operand, column n = head n, k = 8*cls + 32 j
@@ -233,11 +325,9 @@ struct DecodeHead {
   float l;                    // this lane's share of the head's denominator
   v4f o[8];                   // o[e][j] = O[head 4*cls + j][dim 8*col + e]
 
-  __device__ __forceinline__ void start(const DecodeArgs& a, int b, int g, int group, int lane) {
-    const int col = lane & 15, cls = lane >> 4;
-    const T* q = reinterpret_cast<const T*>(a.q);
-    const bool live = col < group;
-    const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D + cls * 8;
+  // column lane%16 of the first product is the row of D elements at `row_ptr` (zero when not live)
+  __device__ __forceinline__ void load_q(const T* row_ptr, bool live, int lane) {
+    const T* src = row_ptr + (lane >> 4) * 8;
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
       const uint4 x = *reinterpret_cast<const uint4*>(src + 32 * j);
@@ -247,6 +337,29 @@ struct DecodeHead {
     l = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
+  }
+  __device__ __forceinline__ void start(const DecodeArgs& a, int b, int g, int group, int lane) {
+    const int col = lane & 15;
+    const bool live = col < group;
+    load_q(reinterpret_cast<const T*>(a.q) + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D, live, lane);
+  }
+  // this lane's dims of accumulator row j (head or query row 4*(lane/16) + j), scaled, into the row of D elements
+  __device__ __forceinline__ void write_row(T* row_ptr, int j, float scale, int lane) const {
+    const int col = lane & 15;
+    if (D == 128 || col < kCols) {
+      T r[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r[e] = from_float<T>(o[e][j] * scale);
+      *reinterpret_cast<uint4*>(row_ptr + col * 8) = *reinterpret_cast<const uint4*>(r);
+    }
+  }
+  __device__ __forceinline__ void write_partial(float* row_ptr, int j, int lane) const {
+    const int col = lane & 15;
+    if (D == 128 || col < kCols) {
+      float* dst = row_ptr + col * 8;
+      *reinterpret_cast<float4*>(dst) = make_float4(o[0][j], o[1][j], o[2][j], o[3][j]);
+      *reinterpret_cast<float4*>(dst + 4) = make_float4(o[4][j], o[5][j], o[6][j], o[7][j]);
+    }
   }
 
   // one tile of 16 tokens starting at token t0 of the sequence; tokens at or past part_end do not count
@@ -360,40 +473,166 @@ struct DecodeHead {
 
   // write the output row (direct) or this partition's partial result
   __device__ __forceinline__ void finish(const DecodeArgs& a, int b, int p, int g, int group, bool direct, int lane) {
-    const int col = lane & 15, cls = lane >> 4;
-    const bool owns = D == 128 || col < kCols;          // this lane's 8 dims exist
-    // denominators: add the four token classes (every lane of a head then holds the head's total)
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    const int head0 = g * group;
-    if (direct) {
-      T* out = reinterpret_cast<T*>(a.out);
-      const float linv = l > 0.f ? 1.f / l : 0.f;
+    finish_head(*this, a, b, p, g, group, direct, lane);
+  }
+};
+
+// fp32 caches and queries: the same decomposition on v_mfma_f32_16x16x4_f32 (one fp32 value per lane and operand,
+// k = lane/16), products and sums in fp32 throughout, the weights P are not rounded.
+//   S[token][head]      A = K: lane l holds 4 dims (16 B) of token l%16 per 16-dim step, dims 16 j + 4 (l/16) + e;
+//                       product (j, e) contracts exactly those dims; B = Q with the same dims of head l%16.
+//   O[head][dim] += P V A = P as it came out (row = head l%16, k = token 4 (l/16) + i for product i); B = V: the
+//                       lane's 4 dims (16 B) of that token per 64-dim step, so column n of product (i, jj, e) is dim
+//                       64 jj + 4 n + e.  Lane l ends with O[head 4 (l/16) + j][dims 64 jj + 4 (l%16) + e].
+template <int D>
+struct DecodeHead<float, D> {
+  using Elem = float;
+  static constexpr int kDim = D;
+  static constexpr int kSteps = D / 16;      // 16-dim steps of the first product (4 MFMAs each)
+  static constexpr int kVSteps = D / 64;     // 64-dim steps of the second
+  static constexpr int kAcc = 4 * kVSteps;
+  float4 qf[kSteps];
+  float m;
+  float l;
+  v4f o[kAcc];                // o[4 jj + e][j] = O[head 4*cls + j][dim 64 jj + 4 col + e]
+
+  __device__ __forceinline__ void load_q(const float* row_ptr, bool live, int lane) {
+    const float* src = row_ptr + (lane >> 4) * 4;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int h = 4 * cls + j;
-        const float lj = __shfl(linv, h, 64);               // lane h (class 0) holds head h
-        if (h < group && owns) {
-          T r[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) r[e] = from_float<T>(o[e][j] * lj);
-          *reinterpret_cast<uint4*>(out + ((int64_t)b * a.num_heads + head0 + h) * D + col * 8) =
-              *reinterpret_cast<const uint4*>(r);
-        }
-      }
-    } else {
-      const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int h = 4 * cls + j;
-        if (h < group && owns) {
-          float* dst = a.ws_acc + (slot + h) * D + col * 8;
-          *reinterpret_cast<float4*>(dst) = make_float4(o[0][j], o[1][j], o[2][j], o[3][j]);
-          *reinterpret_cast<float4*>(dst + 4) = make_float4(o[4][j], o[5][j], o[6][j], o[7][j]);
-        }
-      }
-      if (lane < group && lane < 16) *reinterpret_cast<float2*>(a.ws_ml + (slot + lane) * 2) = make_float2(m, l);
+    for (int j = 0; j < kSteps; ++j) {
+      const float4 x = *reinterpret_cast<const float4*>(src + 16 * j);
+      qf[j] = live ? x : make_float4(0.f, 0.f, 0.f, 0.f);
     }
+    m = -INFINITY;
+    l = 0.f;
+#pragma unroll
+    for (int e = 0; e < kAcc; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
+  }
+  __device__ __forceinline__ void start(const DecodeArgs& a, int b, int g, int group, int lane) {
+    const int col = lane & 15;
+    const bool live = col < group;
+    load_q(reinterpret_cast<const float*>(a.q) + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D, live, lane);
+  }
+
+  __device__ __forceinline__ void consume(const KVTile<float>& t, int part_end, float scale_log2, int lane,
+                                          int col_end = 0x7fffffff) {
+    const int cls = lane >> 4;
+    const int tok_base = t.t0 + 4 * cls;
+    const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
+    v4f s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < kSteps; ++j) {
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(t.k[j].x, qf[j].x, s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(t.k[j].y, qf[j].y, s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(t.k[j].z, qf[j].z, s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(t.k[j].w, qf[j].w, s, 0, 0, 0);
+    }
+    float s2[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s2[i] = s[i] * scale_log2;
+    float4 v[4][kVSteps];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int jj = 0; jj < kVSteps; ++jj) v[i][jj] = t.v[i][jj];
+    if (partial) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (!t.ok || tok_base + i >= part_end) {
+          s2[i] = -INFINITY;
+#pragma unroll
+          for (int jj = 0; jj < kVSteps; ++jj) v[i][jj] = make_float4(0.f, 0.f, 0.f, 0.f);   // must not meet p = 0 as NaN or Inf
+        }
+    }
+    if (col_end != 0x7fffffff) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (tok_base + i >= col_end) s2[i] = -INFINITY;
+    }
+    const float tile_max = fmaxf(fmaxf(s2[0], s2[1]), fmaxf(s2[2], s2[3]));
+    const bool grow = tile_max > m + kLazyRescale || (m == -INFINITY && tile_max > -INFINITY);
+    if (__any(grow)) {
+      float mh = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+      mh = fmaxf(mh, __shfl_xor(mh, 32, 64));
+      const bool grow_h = mh > m + kLazyRescale || (m == -INFINITY && mh > -INFINITY);
+      const float m_new = grow_h ? mh : m;
+      const float al = (m_new == m) ? 1.f : safe_exp2_diff(m, m_new);
+      l *= al;
+      m = m_new;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float aj = __shfl(al, 4 * cls + j, 64);
+#pragma unroll
+        for (int e = 0; e < kAcc; ++e) o[e][j] *= aj;
+      }
+    }
+    const float m_eff = (m == -INFINITY) ? 0.f : m;
+    float pr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pr[i] = fast_exp2(s2[i] - m_eff);
+      l += pr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int jj = 0; jj < kVSteps; ++jj) {
+        o[4 * jj + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(pr[i], v[i][jj].x, o[4 * jj + 0], 0, 0, 0);
+        o[4 * jj + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(pr[i], v[i][jj].y, o[4 * jj + 1], 0, 0, 0);
+        o[4 * jj + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(pr[i], v[i][jj].z, o[4 * jj + 2], 0, 0, 0);
+        o[4 * jj + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(pr[i], v[i][jj].w, o[4 * jj + 3], 0, 0, 0);
+      }
+  }
+
+  template <int W>
+  __device__ __forceinline__ bool merge(int w, int lane) {
+    __shared__ float4 part[(W - 1) * (1 + kAcc) * 64];
+    const int cls = lane >> 4;
+    if (w > 0) {
+      float4* dst = part + (w - 1) * (1 + kAcc) * 64 + lane;
+      dst[0] = make_float4(m, l, 0.f, 0.f);
+#pragma unroll
+      for (int e = 0; e < kAcc; ++e) dst[(1 + e) * 64] = make_float4(o[e][0], o[e][1], o[e][2], o[e][3]);
+    }
+    __syncthreads();
+    if (w > 0) return false;
+#pragma unroll 1
+    for (int x = 0; x < W - 1; ++x) {
+      const float4* src = part + x * (1 + kAcc) * 64 + lane;
+      const float4 ml = src[0];
+      const float m_new = fmaxf(m, ml.x);
+      const float f0 = safe_exp2_diff(m, m_new);
+      const float f1 = safe_exp2_diff(ml.x, m_new);
+      m = m_new;
+      l = l * f0 + ml.y * f1;
+      float a0[4], a1[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        a0[j] = __shfl(f0, 4 * cls + j, 64);
+        a1[j] = __shfl(f1, 4 * cls + j, 64);
+      }
+#pragma unroll
+      for (int e = 0; e < kAcc; ++e) {
+        const float4 ow = src[(1 + e) * 64];
+        o[e][0] = o[e][0] * a0[0] + ow.x * a1[0];
+        o[e][1] = o[e][1] * a0[1] + ow.y * a1[1];
+        o[e][2] = o[e][2] * a0[2] + ow.z * a1[2];
+        o[e][3] = o[e][3] * a0[3] + ow.w * a1[3];
+      }
+    }
+    return true;
+  }
+
+  __device__ __forceinline__ void write_row(float* row_ptr, int j, float scale, int lane) const {
+    const int col = lane & 15;
+#pragma unroll
+    for (int jj = 0; jj < kVSteps; ++jj)
+      *reinterpret_cast<float4*>(row_ptr + 64 * jj + 4 * col) =
+          make_float4(o[4 * jj][j] * scale, o[4 * jj + 1][j] * scale, o[4 * jj + 2][j] * scale, o[4 * jj + 3][j] * scale);
+  }
+  __device__ __forceinline__ void write_partial(float* row_ptr, int j, int lane) const { write_row(row_ptr, j, 1.f, lane); }
+  __device__ __forceinline__ void finish(const DecodeArgs& a, int b, int p, int g, int group, bool direct, int lane) {
+    finish_head(*this, a, b, p, g, group, direct, lane);
   }
 };
 
@@ -438,8 +677,9 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
   const T* kc = reinterpret_cast<const T*>(a.k_cache) + (int64_t)g * D;
   const T* vc = reinterpret_cast<const T*>(a.v_cache) + (int64_t)g * D;
 
-  const int k_lane_off = col * (int)row + cls * 8;        // token lane%16, dims 8*(lane/16)
-  const int v_lane_off = 4 * cls * (int)row + col * 8;    // token 4*(lane/16), dims 8*(lane%16)
+  using IO = TileIO<T, D>;
+  const int k_lane_off = col * (int)row + cls * IO::kKLane;        // token lane%16, first dim of class lane/16
+  const int v_lane_off = 4 * cls * (int)row + col * IO::kVLane;    // token 4*(lane/16), first dim of column lane%16
 
   auto load_tile = [&](KVTile<T>& t, int tile) {
     t.t0 = first + tile * (W * kTile);
@@ -457,16 +697,11 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
       // K is read in the MFMA operand layout, 64 bytes of a row per instruction, so the second half of each
       // 128-byte line has to survive in cache until the next instruction: ordinary loads (the hint costs 7 %
       // there).
+      IO::load_k(t, kp);
 #pragma unroll
-      for (int j = 0; j < D / 32; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        t.v[i] = (D == 128 || col < D / 8) ? load16_stream(vp + (int64_t)i * row) : make_uint4(0u, 0u, 0u, 0u);
+      for (int i = 0; i < 4; ++i) IO::template load_v<true>(t, i, vp + (int64_t)i * row, IO::owns(col));
     } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
+      IO::zero(t);
     }
     if constexpr (W == 1) {
       off += kTile;
@@ -520,28 +755,20 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
   const int g = h / (a.num_heads / a.num_kv_heads);
   const int rows = min(kTile, seq_len - row0);          // live query rows of the tile
 
+  using IO = TileIO<T, D>;
   DecodeHead<T, D> head;
   {
     const bool live = col < rows;
-    const T* src = reinterpret_cast<const T*>(a.q) +
-                   ((int64_t)(seq_start + row0 + (live ? col : 0)) * a.num_heads + h) * D + cls * 8;
-#pragma unroll
-    for (int j = 0; j < D / 32; ++j) {
-      const uint4 x = *reinterpret_cast<const uint4*>(src + 32 * j);
-      head.qf[j] = live ? x : make_uint4(0u, 0u, 0u, 0u);
-    }
-    head.m = -INFINITY;
-    head.l = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) head.o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
+    head.load_q(reinterpret_cast<const T*>(a.q) + ((int64_t)(seq_start + row0 + (live ? col : 0)) * a.num_heads + h) * D,
+                live, lane);
   }
   const int cached = PAGED ? max(a.cu_seqlens_k[seq_index + 1] - a.cu_seqlens_k[seq_index] - seq_len, 0) : 0;
   const int kv_end = cached + row0 + rows;        // keys 0 .. kv_end - 1 are seen by at least one row of the tile
   const int col_end = cached + row0 + col + 1;    // keys seen by this lane's row
   const int ntiles = (kv_end + kTile - 1) / kTile;
   const int64_t row = (int64_t)a.num_kv_heads * D;
-  const T* kc = reinterpret_cast<const T*>(a.k) + (PAGED ? 0 : (int64_t)seq_start * row) + (int64_t)g * D + cls * 8;
-  const T* vc = reinterpret_cast<const T*>(a.v) + (PAGED ? 0 : (int64_t)seq_start * row) + (int64_t)g * D + col * 8;
+  const T* kc = reinterpret_cast<const T*>(a.k) + (PAGED ? 0 : (int64_t)seq_start * row) + (int64_t)g * D + cls * IO::kKLane;
+  const T* vc = reinterpret_cast<const T*>(a.v) + (PAGED ? 0 : (int64_t)seq_start * row) + (int64_t)g * D + col * IO::kVLane;
   // paged: block-table window, lane i holds entry win_base + i of this sequence (as in the decode kernel)
   const int bs = PAGED ? a.block_size : 1;
   const int32_t* table = PAGED ? a.block_tables + (int64_t)seq_index * a.max_num_blocks : nullptr;
@@ -553,6 +780,9 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
   auto load_tile = [&](KVTile<T>& t, int tile) __attribute__((always_inline)) {
     t.t0 = tile * kTile;
     t.ok = true;
+    // An unmapped block reads as zero keys and values that still count (score 0), as in the other prefill
+    // kernels and unlike decode, where such tokens contribute nothing.
+    bool mapped = true;
     int64_t k_tok, v_tok[4];
     if constexpr (PAGED) {
       if (bi - win_base >= 64) {
@@ -560,8 +790,8 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
         win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
       }
       const int phys = __builtin_amdgcn_readlane(win, bi - win_base);
-      t.ok = (bi < a.max_num_blocks) && phys >= 0 && (int64_t)phys < a.num_blocks;
-      const int64_t tok0 = (int64_t)(t.ok ? phys : 0) * bs + off;
+      mapped = (bi < a.max_num_blocks) && phys >= 0 && (int64_t)phys < a.num_blocks;
+      const int64_t tok0 = (int64_t)(mapped ? phys : 0) * bs + off;
       k_tok = tok0 + col;
 #pragma unroll
       for (int i = 0; i < 4; ++i) v_tok[i] = tok0 + 4 * cls + i;
@@ -572,18 +802,12 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
 #pragma unroll
       for (int i = 0; i < 4; ++i) v_tok[i] = min(t.t0 + 4 * cls + i, kv_end - 1);
     }
-    if (t.ok) {
-      const T* kp = kc + k_tok * row;
+    if (mapped) {
+      IO::load_k(t, kc + k_tok * row);
 #pragma unroll
-      for (int j = 0; j < D / 32; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        t.v[i] = (D == 128 || col < D / 8) ? *reinterpret_cast<const uint4*>(vc + v_tok[i] * row) : make_uint4(0u, 0u, 0u, 0u);
+      for (int i = 0; i < 4; ++i) IO::template load_v<false>(t, i, vc + v_tok[i] * row, IO::owns(col));
     } else {
-#pragma unroll
-      for (int j = 0; j < D / 32; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
+      IO::zero(t);
     }
   };
   KVTile<T> ta, tb;
@@ -607,13 +831,7 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
   for (int j = 0; j < 4; ++j) {
     const int r = 4 * cls + j;
     const float lj = __shfl(linv, r, 64);                 // lane r (class 0) holds column r
-    if (r < rows && (D == 128 || col < D / 8)) {
-      T o8[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) o8[e] = from_float<T>(head.o[e][j] * lj);
-      *reinterpret_cast<uint4*>(out + ((int64_t)(seq_start + row0 + r) * a.num_heads + h) * D + col * 8) =
-          *reinterpret_cast<const uint4*>(o8);
-    }
+    if (r < rows) head.write_row(out + ((int64_t)(seq_start + row0 + r) * a.num_heads + h) * D, j, lj, lane);
   }
 }
 
@@ -1121,9 +1339,8 @@ static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int ma
 
 // shapes the MFMA kernels are built for (pointer alignment is checked by the caller)
 static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool int8) {
-  (void)int8;
   const bool dim_ok = head_dim == 128 || head_dim == 64;
-  return dtype != MVLLM_F32 && dim_ok && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
+  return (dtype != MVLLM_F32 || !int8) && dim_ok && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
          (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
 }
 
@@ -1145,28 +1362,30 @@ template <> struct IsSixteenBit<float> { static constexpr bool value = false; };
 
 template <typename T>
 static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipStream_t stream) {
-  const int group = a.num_heads / a.num_kv_heads;
   bool launched = false;
-  if constexpr (IsSixteenBit<T>::value) {
-    if (fast_ok && split) {
-      const dim3 grid((unsigned)a.num_kv_heads, (unsigned)a.num_parts, (unsigned)a.batch), block(64 * kSplitWaves);
-      if (int8 && a.head_dim == 64) decode_mfma_int8_split_kernel<T, kSplitWaves, 64><<<grid, block, 0, stream>>>(a);
-      else if (int8) decode_mfma_int8_split_kernel<T, kSplitWaves, 128><<<grid, block, 0, stream>>>(a);
-      else if (a.head_dim == 64) decode_mfma_split_kernel<T, kSplitWaves, 64><<<grid, block, 0, stream>>>(a);
-      else decode_mfma_split_kernel<T, kSplitWaves, 128><<<grid, block, 0, stream>>>(a);
-      launched = true;
-    } else if (fast_ok) {
-      // kv heads (waves) per workgroup: as many as allowed, so that a workgroup streams whole token rows;
-      // fewer when the grid would otherwise leave most CUs without a workgroup
-      int wpb = largest_divisor_le(a.num_kv_heads, int8 ? MVLLM_DECODE_I8_WPB : MVLLM_DECODE_WPB);
-      while (wpb > 1 && (int64_t)a.num_parts * a.batch * (a.num_kv_heads / wpb) < MVLLM_DECODE_SMALL_GRID)
-        wpb = largest_divisor_le(a.num_kv_heads, wpb - 1);
-      const unsigned groups = (unsigned)(a.num_kv_heads / wpb);
-      dim3 block(64 * wpb);
-      if (int8 && a.head_dim == 64) decode_mfma_int8_kernel<T, 1, 64><<<dim3((unsigned)a.num_parts, groups, (unsigned)a.batch), block, 0, stream>>>(a);
-      else if (int8) decode_mfma_int8_kernel<T, 1, 128><<<dim3((unsigned)a.num_parts, groups, (unsigned)a.batch), block, 0, stream>>>(a);
-      else if (a.head_dim == 64) decode_mfma_kernel<T, 64><<<dim3((unsigned)a.num_parts, (unsigned)a.batch, groups), block, 0, stream>>>(a);
-      else decode_mfma_kernel<T, 128><<<dim3((unsigned)a.num_parts, (unsigned)a.batch, groups), block, 0, stream>>>(a);
+  // kv heads (waves) per workgroup of the one-wave-per-head form: as many as allowed, so that a workgroup streams
+  // whole token rows; fewer when the grid would otherwise leave most CUs without a workgroup
+  int wpb = largest_divisor_le(a.num_kv_heads, int8 ? MVLLM_DECODE_I8_WPB : MVLLM_DECODE_WPB);
+  while (wpb > 1 && (int64_t)a.num_parts * a.batch * (a.num_kv_heads / wpb) < MVLLM_DECODE_SMALL_GRID)
+    wpb = largest_divisor_le(a.num_kv_heads, wpb - 1);
+  const unsigned groups = (unsigned)(a.num_kv_heads / wpb);
+  const dim3 split_grid((unsigned)a.num_kv_heads, (unsigned)a.num_parts, (unsigned)a.batch), split_block(64 * kSplitWaves);
+  const dim3 block(64 * wpb);
+  if (fast_ok && !int8) {
+    const dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, groups);
+    if (split && a.head_dim == 64) decode_mfma_split_kernel<T, kSplitWaves, 64><<<split_grid, split_block, 0, stream>>>(a);
+    else if (split) decode_mfma_split_kernel<T, kSplitWaves, 128><<<split_grid, split_block, 0, stream>>>(a);
+    else if (a.head_dim == 64) decode_mfma_kernel<T, 64><<<grid, block, 0, stream>>>(a);
+    else decode_mfma_kernel<T, 128><<<grid, block, 0, stream>>>(a);
+    launched = true;
+  }
+  if constexpr (IsSixteenBit<T>::value) {           // the INT8 kernels take 16-bit queries
+    if (fast_ok && int8) {
+      const dim3 grid((unsigned)a.num_parts, groups, (unsigned)a.batch);
+      if (split && a.head_dim == 64) decode_mfma_int8_split_kernel<T, kSplitWaves, 64><<<split_grid, split_block, 0, stream>>>(a);
+      else if (split) decode_mfma_int8_split_kernel<T, kSplitWaves, 128><<<split_grid, split_block, 0, stream>>>(a);
+      else if (a.head_dim == 64) decode_mfma_int8_kernel<T, 1, 64><<<grid, block, 0, stream>>>(a);
+      else decode_mfma_int8_kernel<T, 1, 128><<<grid, block, 0, stream>>>(a);
       launched = true;
     }
   }
@@ -1225,7 +1444,7 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
   }
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case MVLLM_F32: return launch_decode<float>(a, int8, false, false, s);
+    case MVLLM_F32: return launch_decode<float>(a, int8, fast_ok, split, s);
     case MVLLM_BF16: return launch_decode<bf16_t>(a, int8, fast_ok, split, s);
     default: return launch_decode<f16_t>(a, int8, fast_ok, split, s);
   }
@@ -1237,11 +1456,14 @@ static void launch_rows16(const PrefillRowsArgs& a, dim3 grid, int tiles, hipStr
   else prefill_rows16_kernel<T, D, false><<<grid, dim3(256), 0, stream>>>(a, tiles);
 }
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream) {
-  if ((head_dim != 64 && head_dim != 128) || dtype == MVLLM_F32) return MVLLM_ERR_UNSUPPORTED;
+  if (head_dim != 64 && head_dim != 128) return MVLLM_ERR_UNSUPPORTED;
   if (a.block_tables && a.block_size % kTile != 0) return MVLLM_ERR_UNSUPPORTED;
   const int64_t tiles = a.total_tokens / kTile + a.num_seqs;      // upper bound on the 16-row tiles
   const dim3 grid((unsigned)tiles, (unsigned)((a.num_heads + 3) / 4));
-  if (dtype == MVLLM_BF16) {
+  if (dtype == MVLLM_F32) {
+    if (head_dim == 64) launch_rows16<float, 64>(a, grid, (int)tiles, stream);
+    else launch_rows16<float, 128>(a, grid, (int)tiles, stream);
+  } else if (dtype == MVLLM_BF16) {
     if (head_dim == 64) launch_rows16<bf16_t, 64>(a, grid, (int)tiles, stream);
     else launch_rows16<bf16_t, 128>(a, grid, (int)tiles, stream);
   } else {

@@ -637,8 +637,8 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 && (group == 1 || group == 2 || group % 4 == 0) &&
                        aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
                        num_kv_heads * group <= 65535;
-  // other 16-bit shapes with head_dim 64 or 128: 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
-  if (!mfma_ok && dtype != MVLLM_F32 && (head_dim == 64 || head_dim == 128) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
+  // other shapes with head_dim 64 or 128 (fp32 included): 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
+  if (!mfma_ok && (head_dim == 64 || head_dim == 128) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
       (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31)) {
     PrefillRowsArgs r;
     r.out = out; r.q = q; r.k = k; r.v = v; r.cu_seqlens = cu_seqlens; r.total_tokens = total_tokens;
@@ -676,7 +676,7 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
                        block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) &&
                        aligned16(out) && num_kv_heads * group <= 65535 &&
                        (int64_t)block_size * num_kv_heads * head_dim * 2 < ((int64_t)1 << 31);
-  if (!mfma_ok && dtype != MVLLM_F32 && (head_dim == 64 || head_dim == 128) && block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) &&
+  if (!mfma_ok && (head_dim == 64 || head_dim == 128) && block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) &&
       aligned16(v_cache) && aligned16(out) && (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31)) {
     PrefillRowsArgs r;
     r.out = out; r.q = q; r.k = k_cache; r.v = v_cache; r.cu_seqlens = cu_seqlens_q; r.total_tokens = total_q_tokens;

@@ -75,7 +75,8 @@ def test_decode_plan_is_host_arithmetic():
     assert paged_decode_plan(64, 16, 16, 96, 256, 16, int8_cache=True)[2] == 0
     assert paged_decode_plan(64, 16, 16, 96, 256, 16)[2] == 0                 # other head dims
     import torch
-    assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32)[2] == 0
+    assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32)[2] == 4       # fp32 caches: fp32 MFMA
+    assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32, int8_cache=True)[2] == 0
     assert paged_decode_plan(8, 34, 2, 128, 64, 16)[2] == 0                   # 17 query heads per kv head
     # the advertised workspace covers whatever form is chosen
     for batch in (1, 3, 16, 64, 200, 1000):

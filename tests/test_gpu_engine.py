@@ -136,14 +136,15 @@ def test_prefix_cache_hits_are_read_from_the_paged_cache():
     assert same >= 4, outs                                # a 1-ulp difference may flip a sampling tie, rarely
 
 
-def test_reference_demo_model_shape_head_dim_64():
-    """The reference's demo model (main.py:18-30: 16 query / 8 kv heads of 64 dims) in bf16: generation with the
-    hipGraph decode path agrees with the eager path, prefix-cache hits are read from the paged cache, and both runs
-    use the MFMA decode kernels and the 16-row tile prefill (head_dim 64 has no generic-kernel fallback in 16 bit)."""
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_reference_demo_model_shape_head_dim_64(dtype):
+    """The reference's demo model (main.py:18-30: 16 query / 8 kv heads of 64 dims), in bf16 and in main.py's own
+    fp32: generation with the hipGraph decode path agrees with the eager path, prefix-cache hits are read from the
+    paged cache, and both runs use the MFMA decode kernels and the 16-row tile prefill, not the generic kernels."""
     from minivllm_amd.layers.attention import paged_decode_plan
     cfg = dict(SMALL, hidden_size=1024, num_heads=16, num_kv_heads=8, head_dim=64, num_layers=2,
-               max_num_sequences=4, max_cached_blocks=96, max_model_length=128)
-    assert paged_decode_plan(4, 16, 8, 64, 128 // 16, 16)[2] > 0
+               max_num_sequences=4, max_cached_blocks=96, max_model_length=128, dtype=dtype)
+    assert paged_decode_plan(4, 16, 8, 64, 128 // 16, 16, torch.float32 if dtype == "fp32" else torch.bfloat16)[2] > 0
     g = torch.Generator().manual_seed(21)
     shared = torch.randint(0, 2048, (32,), generator=g).tolist()
     prompts = [shared + torch.randint(0, 2048, (n,), generator=g).tolist() for n in (7, 20, 1)] + _prompts(3, 3, 40, seed=22)
