@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,decode_small,fused_qk,sampler,engine,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,decode_small,demo_shape,fused_qk,sampler,engine,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -380,6 +380,36 @@ def bench_decode_small(args):
             "int8_us_per_call": us8, "int8_gbs": tokens * hkv * (2 * d + 8) / (us8 * 1e-6) / 1e9}
 
 
+def bench_demo_shape(args):
+    """The reference demo's attention shape (main.py:18-30: 16 query / 8 kv heads of 64 dims) in main.py's fp32 and
+    in bf16: decode of 64 sequences of 1000-3000 tokens and prefill of 16 prompts of 64-2048 tokens."""
+    import torch
+    from helpers import make_paged_case_on_device, make_varlen_case
+    from minivllm_amd.layers.attention import flash_attention_prefill, paged_attention_decode
+
+    dev = "cuda:0"
+    hq, hkv, d, bs = 16, 8, 64, 16
+    out = {"workload": "Hq16 Hkv8 D64: decode B64 ctx~U[1000,3000] block_size 16; prefill 16 prompts L~U[64,2048]"}
+    g = torch.Generator().manual_seed(args.seed)
+    lengths = torch.randint(64, 2049, (16,), generator=g).tolist()
+    flops = 4 * hq * d * sum(n * (n + 1) // 2 for n in lengths)
+    for name, dtype in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        q, kc, vc, tables, ctx = make_paged_case_on_device(args.seed, dev, 64, 1000, 3000, hq, hkv, d, bs, dtype=dtype,
+                                                           log_uniform=False)
+        td, cd = tables.to(dev), ctx.to(dev)
+        _, ms = time_steps(lambda: paged_attention_decode(q, kc, vc, td, cd, 1 / math.sqrt(d), hq, hkv, d, bs),
+                           args.steps, args.warmup)
+        nbytes = int(ctx.sum()) * hkv * d * 2 * kc.element_size()
+        out[f"decode_{name}_us"] = ms * 1e3
+        out[f"decode_{name}_gbs"] = nbytes / (ms * 1e-3) / 1e9
+        qq, kk, vv, cu = (t.to(dev) for t in make_varlen_case(args.seed + 1, lengths, hq, hkv, d, dtype=dtype))
+        _, ms = time_steps(lambda: flash_attention_prefill(qq, kk, vv, cu, 1 / math.sqrt(d), hq, hkv, d),
+                           max(3, args.steps // 3), max(1, args.warmup // 2))
+        out[f"prefill_{name}_ms"] = ms
+        out[f"prefill_{name}_tflops"] = flops / (ms * 1e-3) / 1e12
+    return out
+
+
 def bench_engine(args, max_num_sequences, graph):
     """BASELINE.json config 5: random-init Qwen3-style decoder (hidden 1024, 8 layers, Hq16/Hkv8/D128, FFN 3072,
     vocab 151936, bf16), 60 prompts of random ids with lengths U[32,96], 256 new tokens each, T 0.6."""
@@ -449,6 +479,8 @@ def main():
         extra["int8"] = bench_int8(args)
     if want("decode_small"):
         extra["decode_small_batch"] = bench_decode_small(args)
+    if want("demo_shape"):
+        extra["reference_demo_shape"] = bench_demo_shape(args)
     if want("fused_qk"):
         extra["fused_qk"] = bench_fused_qk(args)
     if want("sampler"):
