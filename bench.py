@@ -127,7 +127,7 @@ def bench_decode(args, block_size, want_cpu):
         while True:
             ref = oracle.decode_naive_oracle(qcpu, kcpu, vcpu, tcpu, ccpu, scale, hq, hkv, d, block_size)
             reps += 1
-            if time.perf_counter() - t0 > 10.0 or reps >= 20:
+            if time.perf_counter() - t0 > 10.0 or reps >= 60:
                 break
         cpu_s = (time.perf_counter() - t0) / reps
         sub_bytes = decode_bytes(ccpu, block_size, hq, hkv, d, 2, 2, 8)
