@@ -580,7 +580,9 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
 template <typename T, bool PAGED>
 static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   const int group = a.num_heads / a.num_kv_heads;
-  const int hpw = group >= 4 ? 4 : group;              // 1, 2 or 4 (group is 1, 2 or a multiple of 4)
+  // query heads of a kv head per workgroup: 4 or 2 where they divide the group, else 1 (the workgroup is then four
+  // row tiles of one head)
+  const int hpw = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
   const int bm = kWaveRows * (kPfWaves / hpw);
   PrefillArgs b = a;
   b.tiles_x = (int)(a.total_tokens / bm + a.num_seqs);
@@ -634,7 +636,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   a.tiles_x = 0; a.heads_y = 0;
   a.cu_seqlens_k = nullptr; a.block_tables = nullptr; a.max_num_blocks = 0; a.block_size = 0; a.num_blocks = 0;
   const int group = num_heads / num_kv_heads;
-  const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 && (group == 1 || group == 2 || group % 4 == 0) &&
+  const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 &&
                        aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
                        num_kv_heads * group <= 65535;
   // other shapes with head_dim 64 or 128 (fp32 included): 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
@@ -672,7 +674,7 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
   a.cu_seqlens_k = cu_seqlens_k; a.block_tables = block_tables; a.max_num_blocks = max_num_blocks;
   a.block_size = block_size; a.num_blocks = num_blocks;
   const int group = num_heads / num_kv_heads;
-  const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 && (group == 1 || group == 2 || group % 4 == 0) &&
+  const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 &&
                        block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) &&
                        aligned16(out) && num_kv_heads * group <= 65535 &&
                        (int64_t)block_size * num_kv_heads * head_dim * 2 < ((int64_t)1 << 31);

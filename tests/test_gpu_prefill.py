@@ -31,7 +31,7 @@ def _oracle32(q, k, v, cu, scale, hq, hkv, d):
     (8, 8, 128, [200]),
     (16, 16, 64, [60, 60]),             # the reference demo's head_dim
     (6, 2, 80, [17, 5]),
-    (6, 2, 128, [300, 17, 64]),         # three query heads per kv head: 16-row tiles instead of the LDS-tiled kernel
+    (6, 2, 128, [300, 17, 64]),         # three query heads per kv head: one head per workgroup
     (10, 2, 128, [33, 129]),            # five
 ])
 def test_prefill_vs_oracle(dtype, hq, hkv, d, lengths):

@@ -53,7 +53,7 @@ def _check(got, want, dtype):
     (12, 1, 64, 256, [700, 30, 257], [512, 29, 0]),                # head_dim 64, one kv head, the engine's block size
     (6, 2, 64, 48, [131, 77, 260], [50, 1, 259]),                  # head_dim 64, heads not a multiple of four
     (4, 4, 64, 8, [70], [32]),                                     # head_dim 64 with a block size of 8: generic kernel
-    (6, 2, 128, 16, [131, 77, 260], [50, 1, 259]),                 # head_dim 128, three query heads per kv head
+    (6, 2, 128, 16, [131, 77, 260], [50, 1, 259]),                 # head_dim 128, three query heads per kv head (one head per workgroup)
 ])
 def test_paged_prefill_vs_oracle(dtype, hq, hkv, d, bs, lengths, cached):
     c = make_paged_prefill_case(61, lengths, cached, hq, hkv, d, bs, dtype=dtype)
