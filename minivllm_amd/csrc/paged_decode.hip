@@ -732,8 +732,8 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
 }
 
 // ---------------------------------------------------------------------------
-// Varlen causal prefill on the same tile arithmetic (flash_attention_prefill, attention.py:212-280, for the shapes
-// the LDS-tiled kernel of prefill_varlen.hip is not built for: head_dim 64, the reference demo's model, and fp32).
+// Varlen causal prefill on the same tile arithmetic (flash_attention_prefill, attention.py:212-280), for fp32, which
+// the LDS-tiled kernel of prefill_varlen.hip does not take (the reference's main.py runs in fp32).
 // One wave = 16 consecutive query rows of one query head: the rows take the place of the heads of a group
 // (column n of the first product = row n), the keys 0 .. row are walked in 16-token tiles straight from the
 // packed k / v tensors, and the causal limit is applied per column.  The four waves of a workgroup are four query

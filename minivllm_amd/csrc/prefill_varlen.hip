@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs 
 }
 
 // ---------------------------------------------------------------------------
-// MFMA path: 16-bit inputs, head_dim 128.
+// MFMA path: 16-bit inputs, head_dim 128 or 64 (described for 128).
 //
 // Workgroup = 4 waves = (one kv head, HPW of the query heads that share it,
 // 4/HPW consecutive 32-row query tiles); every wave owns 32 query rows of one
@@ -153,7 +153,6 @@ constexpr unsigned kXcdChunk = MVLLM_PF_XCD_CHUNK;   // consecutive work items h
 constexpr int kPfWaves = MVLLM_PF_WAVES;             // waves per workgroup: 4, so that two workgroups share a CU
 constexpr int kBN = 64;                 // K/V rows per LDS tile
 constexpr int kWaveRows = 32;           // query rows per wave
-constexpr int kTileBytes = kBN * 256;   // one K (or V) tile, head_dim 128 x 2 B
 
 // v_max3_f32 without the canonicalising self-max the compiler puts in front of every fmaxf operand that
 // comes out of an MFMA (scores are finite or -inf here, never NaN).  The compiler does not know what the asm
@@ -213,9 +212,22 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
 
-template <typename T, int HPW, bool PAGED>
+// D = 128 or 64.  A row of a tile is D*2 bytes = kChunks 16-byte chunks; one copy instruction moves 1 KB = kCopyRows
+// rows.  The chunk swizzles (kswz for K, vswz for V) must not change when 8, 16 or 32 rows are added, because the
+// per-lane LDS offsets are computed once and the tile rows are reached through immediates.
+template <typename T, int HPW, bool PAGED, int D>
 __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const PrefillArgs a) {
-  constexpr int D = 128;
+  constexpr int kRowB = D * 2;                  // bytes per tile row
+  constexpr int kChunks = kRowB / 16;           // 16-byte chunks per row: 16 or 8
+  constexpr int kCopyRows = 1024 / kRowB;       // rows per copy instruction: 4 or 8
+  constexpr int kTileBytes = kBN * kRowB;       // one K (or V) tile
+  constexpr int kKS = D / 16;                   // 16-dim steps of the first product
+  constexpr int kTD = D / 32;                   // 32-dim blocks of the output
+  // K rows are read 16 at a time with the same logical chunk: the swizzle spreads them over the banks.  With 128-byte
+  // rows two rows share a 256-byte bank line, so the row index is halved first.
+  auto kswz = [](int row) __attribute__((always_inline)) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
+  // V is read by the transposing loads as 4 rows x 64 bytes per 16 lanes
+  auto vswz = [](int row) __attribute__((always_inline)) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
   constexpr int ROW_TILES = kPfWaves / HPW;     // 32-row query tiles per workgroup
   constexpr int ROWS_PER_WAVE = kBN / kPfWaves; // K/V tile rows one wave copies (4 per instruction)
   constexpr int BM = kWaveRows * ROW_TILES;     // query rows per workgroup
@@ -276,17 +288,17 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   // Addresses are a wave-uniform 64-bit base (tile start, SALU arithmetic) plus a per-lane 32-bit offset that
   // never changes, so a tile costs no VALU address math.  Only a tile that runs past the last packed token
   // (the tail of the last sequence) recomputes clamped offsets.
-  const int ld_row = lane >> 4;        // row inside the 4-row group
-  const int ld_chunk = lane & 15;      // destination chunk inside the row
-  constexpr int kCopies = ROWS_PER_WAVE / 4;
+  const int ld_row = lane / kChunks;   // row inside the group of rows one instruction copies
+  const int ld_chunk = lane % kChunks; // destination chunk inside the row
+  constexpr int kCopies = ROWS_PER_WAVE / kCopyRows;
   static_assert(!PAGED || ROWS_PER_WAVE == 16, "paged mode: one wave copies one 16-row piece of a cache block");
   uint32_t k_src_off[kCopies], v_src_off[kCopies];
 #pragma unroll
   for (int i = 0; i < kCopies; ++i) {
-    const int row = ROWS_PER_WAVE * wave + 4 * i + ld_row;   // row inside the tile (decides the swizzle)
-    const int src_row = PAGED ? 4 * i + ld_row : row;        // paged: the descriptor starts at the wave's own rows
-    k_src_off[i] = (uint32_t)(src_row * (int)kv_row_bytes + ((ld_chunk ^ (row & 15)) << 4));
-    v_src_off[i] = (uint32_t)(src_row * (int)kv_row_bytes + ((ld_chunk ^ ((row & 3) << 2)) << 4));
+    const int row = ROWS_PER_WAVE * wave + kCopyRows * i + ld_row;   // row inside the tile (decides the swizzle)
+    const int src_row = PAGED ? kCopyRows * i + ld_row : row;        // paged: the descriptor starts at the wave's own rows
+    k_src_off[i] = (uint32_t)(src_row * (int)kv_row_bytes + ((ld_chunk ^ kswz(row)) << 4));
+    v_src_off[i] = (uint32_t)(src_row * (int)kv_row_bytes + ((ld_chunk ^ vswz(row)) << 4));
   }
   // One tile's copy is 2 * kCopies instructions per wave (K copies first, then V).  Inside tile_step they are
   // issued one at a time, spread between the MFMAs of the tile before, because a wave that issues them back
@@ -345,12 +357,12 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   };
   // LDS byte address of this wave's first row in buffer 0 of K; V, buffer 1 and later copies are constants away
   // (the two arrays are laid out back to back by the struct below).
-  const uint32_t lds_wave_base = lds_address(&lds.k[0][0]) + (uint32_t)(ROWS_PER_WAVE * wave * 256);
+  const uint32_t lds_wave_base = lds_address(&lds.k[0][0]) + (uint32_t)(ROWS_PER_WAVE * wave * kRowB);
   auto issue_copy = [&](const TileSrc& t, auto BUF, auto C) {               // C < kCopies: K copy C, else V copy C - kCopies
     constexpr int c = decltype(C)::value;
     constexpr bool is_k = c < kCopies;
     constexpr int i = is_k ? c : c - kCopies;
-    constexpr int imm = (is_k ? 0 : 2 * kTileBytes) + decltype(BUF)::value * kTileBytes + 4 * i * 256;
+    constexpr int imm = (is_k ? 0 : 2 * kTileBytes) + decltype(BUF)::value * kTileBytes + i * 1024;
     dma16_to_lds<imm>(is_k ? t.k : t.v, is_k ? k_src_off[i] : v_src_off[i], lds_wave_base);
   };
   auto issue_tile = [&](int j, int buf) {                        // whole tile at once, buffer chosen at run time
@@ -358,29 +370,29 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     const uint32_t base = lds_wave_base + (uint32_t)buf * kTileBytes;
     static_for<kCopies>([&](auto I) {
       constexpr int i = decltype(I)::value;
-      dma16_to_lds<4 * i * 256>(t.k, k_src_off[i], base);
-      dma16_to_lds<2 * kTileBytes + 4 * i * 256>(t.v, v_src_off[i], base);
+      dma16_to_lds<i * 1024>(t.k, k_src_off[i], base);
+      dma16_to_lds<2 * kTileBytes + i * 1024>(t.v, v_src_off[i], base);
     });
   };
   issue_tile(0, 0);
 
   // Q fragments (B operand): column = query row l32, k = 16*ks + 8*hi ..
-  uint4 qf[8];
+  uint4 qf[kKS];
   {
     int64_t tok = (int64_t)seq_start + qrow;
     if (tok > last_token) tok = last_token;
     const T* src = q + (tok * a.num_heads + h) * D + 8 * hi;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
+    for (int ks = 0; ks < kKS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
   }
   // Make the compiler retire the Q loads here: otherwise it carries "Q may still be in flight" into
   // the loop and its vmcnt waits there would also wait for the tile prefetch.
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) asm volatile("" ::"v"(qf[ks].x), "v"(qf[ks].w));
+  for (int ks = 0; ks < kKS; ++ks) asm volatile("" ::"v"(qf[ks].x), "v"(qf[ks].w));
 
-  v16f o[4];
+  v16f o[kTD];
 #pragma unroll
-  for (int td = 0; td < 4; ++td)
+  for (int td = 0; td < kTD; ++td)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[td][r] = 0.f;
   float m = -INFINITY;
@@ -392,14 +404,14 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   //   V: row 4*hi + (lane&15)/4 (+8, +16*st, +32*tk rows), chunk (4*td + 2*half + ...) ^ 4*(row & 3)
   const int i16 = lane & 15;
   const int half = (lane >> 4) & 1;
-  int k_off[8];
+  int k_off[kKS];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) k_off[ks] = l32 * 256 + (((2 * ks + hi) ^ (l32 & 15)) << 4);
+  for (int ks = 0; ks < kKS; ++ks) k_off[ks] = l32 * kRowB + (((2 * ks + hi) ^ kswz(l32)) << 4);
   const int v_row = 4 * hi + (i16 >> 2);
-  int v_off[4];
+  int v_off[kTD];
 #pragma unroll
-  for (int td = 0; td < 4; ++td)
-    v_off[td] = v_row * 256 + (((4 * td + 2 * half + ((i16 & 3) >> 1)) ^ ((v_row & 3) << 2)) << 4) + ((i16 & 1) << 3);
+  for (int td = 0; td < kTD; ++td)
+    v_off[td] = v_row * kRowB + (((4 * td + 2 * half + ((i16 & 3) >> 1)) ^ vswz(v_row)) << 4) + ((i16 & 1) << 3);
 
   // One K/V tile: scores, softmax, P.V.  Compile-time parameters: BUF, the buffer index (so that all LDS
   // addresses are register + constant); DIAG, set for the wave's last tile, the one the causal diagonal runs
@@ -422,11 +434,11 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int tk = 0; tk < NH; ++tk) s[tk] = zero;
-      static_for<8>([&](auto KS) {
+      static_for<kKS>([&](auto KS) {
         constexpr int ks = decltype(KS)::value;
         uint4 kf[NH];
 #pragma unroll
-        for (int tk = 0; tk < NH; ++tk) kf[tk] = *reinterpret_cast<const uint4*>(kb + k_off[ks] + tk * 32 * 256);
+        for (int tk = 0; tk < NH; ++tk) kf[tk] = *reinterpret_cast<const uint4*>(kb + k_off[ks] + tk * 32 * kRowB);
 #pragma unroll
         for (int tk = 0; tk < NH; ++tk) s[tk] = mfma32x32x16<T>(kf[tk], qf[ks], s[tk]);
         if constexpr (ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);           // copies of the next tile, K first
@@ -464,7 +476,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       const float alpha = (m_new == m) ? 1.f : fast_exp2(m - m_new);   // exp2(-inf) = 0 on the first tile
       l *= alpha;
 #pragma unroll
-      for (int td = 0; td < 4; ++td)
+      for (int td = 0; td < kTD; ++td)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[td][r] *= alpha;
       m = m_new;
@@ -488,17 +500,17 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
       pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
       pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
-      uint4 af[4];
+      uint4 af[kTD];
 #pragma unroll
-      for (int td = 0; td < 4; ++td) {
-        const char* p0 = vb + v_off[td] + (32 * tk + 16 * st) * 256;
+      for (int td = 0; td < kTD; ++td) {
+        const char* p0 = vb + v_off[td] + (32 * tk + 16 * st) * kRowB;
         const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
-        const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * 256));
+        const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * kRowB));
         af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;
         af[td].z = __builtin_bit_cast(uint2, a1).x; af[td].w = __builtin_bit_cast(uint2, a1).y;
       }
 #pragma unroll
-      for (int td = 0; td < 4; ++td) o[td] = mfma32x32x16<T>(af[td], pf, o[td]);
+      for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(af[td], pf, o[td]);
     });
   };
 
@@ -551,27 +563,27 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   dma_wait_all();                                    // the zero fill issued during the last tile has landed
   __syncthreads();                                   // every wave is done reading K/V tiles
   if (!active) return;
-  char* ot = &lds.k[0][0] + wave * (kWaveRows * 256);   // 8 waves x 8 KB = both K buffers
+  char* ot = &lds.k[0][0] + wave * (kWaveRows * kRowB);   // 4 waves x 32 rows = both K buffers
   {
     const float lt = l + __shfl_xor(l, 32, 64);
     const float inv = 1.f / lt;
 #pragma unroll
-    for (int td = 0; td < 4; ++td)
+    for (int td = 0; td < kTD; ++td)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         uint2 w;
         w.x = pack2<T>(o[td][4 * r4 + 0] * inv, o[td][4 * r4 + 1] * inv);
         w.y = pack2<T>(o[td][4 * r4 + 2] * inv, o[td][4 * r4 + 3] * inv);
-        *reinterpret_cast<uint2*>(ot + l32 * 256 + (((4 * td + r4) ^ (l32 & 15)) << 4) + 8 * hi) = w;
+        *reinterpret_cast<uint2*>(ot + l32 * kRowB + (((4 * td + r4) ^ kswz(l32)) << 4) + 8 * hi) = w;
       }
   }
   // wave-private tile: the writes above and the reads below are ordered by the LDS queue of this wave
   T* out = reinterpret_cast<T*>(a.out);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = 4 * i + (lane >> 4);
-    const int c = lane & 15;
-    const uint4 w = *reinterpret_cast<const uint4*>(ot + row * 256 + ((c ^ (row & 15)) << 4));
+  for (int i = 0; i < kWaveRows / kCopyRows; ++i) {
+    const int row = kCopyRows * i + lane / kChunks;
+    const int c = lane % kChunks;
+    const uint4 w = *reinterpret_cast<const uint4*>(ot + row * kRowB + ((c ^ kswz(row)) << 4));
     if (r0 + row < seq_len)
       store16_stream(out + ((int64_t)(seq_start + r0 + row) * a.num_heads + h) * D + 8 * c, w);   // +2.5 % at config 2
   }
@@ -590,9 +602,16 @@ static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   const int64_t items = (int64_t)b.tiles_x * b.heads_y;
   const int64_t span = 8 * (int64_t)kXcdChunk;
   dim3 grid((unsigned)((items + span - 1) / span * span));
-  if (hpw == 4) prefill_mfma_kernel<T, 4, PAGED><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
-  else if (hpw == 2) prefill_mfma_kernel<T, 2, PAGED><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
-  else prefill_mfma_kernel<T, 1, PAGED><<<grid, dim3(64 * kPfWaves), 0, stream>>>(b);
+  const dim3 block(64 * kPfWaves);
+  if (a.head_dim == 64) {
+    if (hpw == 4) prefill_mfma_kernel<T, 4, PAGED, 64><<<grid, block, 0, stream>>>(b);
+    else if (hpw == 2) prefill_mfma_kernel<T, 2, PAGED, 64><<<grid, block, 0, stream>>>(b);
+    else prefill_mfma_kernel<T, 1, PAGED, 64><<<grid, block, 0, stream>>>(b);
+  } else {
+    if (hpw == 4) prefill_mfma_kernel<T, 4, PAGED, 128><<<grid, block, 0, stream>>>(b);
+    else if (hpw == 2) prefill_mfma_kernel<T, 2, PAGED, 128><<<grid, block, 0, stream>>>(b);
+    else prefill_mfma_kernel<T, 1, PAGED, 128><<<grid, block, 0, stream>>>(b);
+  }
   return launch_status();
 }
 template <typename T, bool PAGED>
@@ -636,10 +655,10 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   a.tiles_x = 0; a.heads_y = 0;
   a.cu_seqlens_k = nullptr; a.block_tables = nullptr; a.max_num_blocks = 0; a.block_size = 0; a.num_blocks = 0;
   const int group = num_heads / num_kv_heads;
-  const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 &&
+  const bool mfma_ok = dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64) &&
                        aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
                        num_kv_heads * group <= 65535;
-  // other shapes with head_dim 64 or 128 (fp32 included): 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
+  // fp32 with head_dim 64 or 128: 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
   if (!mfma_ok && (head_dim == 64 || head_dim == 128) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
       (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31)) {
     PrefillRowsArgs r;
@@ -674,7 +693,7 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
   a.cu_seqlens_k = cu_seqlens_k; a.block_tables = block_tables; a.max_num_blocks = max_num_blocks;
   a.block_size = block_size; a.num_blocks = num_blocks;
   const int group = num_heads / num_kv_heads;
-  const bool mfma_ok = dtype != MVLLM_F32 && head_dim == 128 &&
+  const bool mfma_ok = dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64) &&
                        block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) &&
                        aligned16(out) && num_kv_heads * group <= 65535 &&
                        (int64_t)block_size * num_kv_heads * head_dim * 2 < ((int64_t)1 << 31);
