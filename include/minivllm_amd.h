@@ -180,6 +180,22 @@ int mvllm_prefill_paged(void* out, const void* q, const void* k_cache, const voi
                         int64_t num_blocks, float scale, int dtype, void* stream);
 
 /*
+ * The same prefill over an INT8 cache (codes + fp32 scales per (token, kv head), as mvllm_store_kvcache_int8 writes
+ * them; no counterpart in the reference, which has neither an INT8 cache nor a consumer of its prefix-cache
+ * metadata).  Every key, the new tokens' included, is read from the cache and dequantised (code * scale, rounded
+ * to `dtype`) on the way into the matrix unit, which is what decode will see for the same tokens.
+ * bf16 / fp16 queries, head_dim 128 or 64, block_size a multiple of 16; else MVLLM_ERR_UNSUPPORTED.
+ */
+int mvllm_prefill_paged_int8(void* out, const void* q,
+                             const int8_t* k_cache, const int8_t* v_cache,
+                             const float* k_scale, const float* v_scale,
+                             const int32_t* block_tables, int max_num_blocks,
+                             const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                             int num_seqs, int64_t total_q_tokens,
+                             int num_heads, int num_kv_heads, int head_dim, int block_size,
+                             int64_t num_blocks, float scale, int dtype, void* stream);
+
+/*
  * The caller's per-layer chain between the QKV projection and the attention kernels, fused:
  *   q = rms_norm(q); k = rms_norm(k)      src/myvllm/models/qwen3.py:104-106, layers/layernorm.py:9-17
  *   q, k = rotary_emb(positions, q, k)    qwen3.py:108, layers/rotary_embedding.py:4-23, 77-83

@@ -204,6 +204,10 @@ struct PrefillRowsArgs {
   int max_num_blocks;
   int block_size;
   int64_t num_blocks;
+  // INT8 cache (paged mode only; k, v are the int8 codes [num_blocks, block_size, Hkv, D]): fp32 scales
+  // [num_blocks, block_size, Hkv], else null
+  const float* k_scale;
+  const float* v_scale;
 };
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream);
 

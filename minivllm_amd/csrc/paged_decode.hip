@@ -742,8 +742,25 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
 // ---------------------------------------------------------------------------
 // PAGED: prefill of the rows that follow a cached prefix (mvllm_prefill_paged): row r of a sequence sits at key
 // position cached + r and every key is read from the paged cache through the block table, as in decode.
-template <typename T, int D, bool PAGED>
+// I8 (paged only): the cache holds int8 codes and per-(token, kv head) fp32 scales (the format store_kvcache_int8
+// writes); a lane dequantises its share of a tile to the query's 16-bit type as it loads it (code * scale, rounded
+// once), after which the tile is an ordinary 16-bit tile.
+template <typename T>
+__device__ __forceinline__ uint4 dequant8(uint2 codes, float scale) {
+  const uint32_t w[2] = {codes.x, codes.y};
+  uint32_t out[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float x0 = (float)(int)(int8_t)(w[e >> 1] >> (16 * (e & 1))) * scale;
+    const float x1 = (float)(int)(int8_t)(w[e >> 1] >> (16 * (e & 1) + 8)) * scale;
+    out[e] = pack_pair<T>(x0, x1);
+  }
+  return make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+template <typename T, int D, bool PAGED, bool I8 = false>
 __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsArgs a, int tiles_x) {
+  static_assert(!I8 || (PAGED && sizeof(T) == 2), "INT8 caches: paged mode, 16-bit queries");
   int seq_start, seq_len, row0, seq_index;
   // latest (heaviest) tiles first
   if (!locate_tile(a.cu_seqlens, a.num_seqs, tiles_x - 1 - (int)blockIdx.x, kTile, seq_start, seq_len, row0, seq_index)) return;
@@ -768,6 +785,9 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
   const int64_t row = (int64_t)a.num_kv_heads * D;
   const T* kc = reinterpret_cast<const T*>(a.k) + (PAGED ? 0 : (int64_t)seq_start * row) + (int64_t)g * D + cls * IO::kKLane;
   const T* vc = reinterpret_cast<const T*>(a.v) + (PAGED ? 0 : (int64_t)seq_start * row) + (int64_t)g * D + col * IO::kVLane;
+  // INT8: the same element offsets in bytes
+  const int8_t* kc8 = reinterpret_cast<const int8_t*>(a.k) + (int64_t)g * D + cls * 8;
+  const int8_t* vc8 = reinterpret_cast<const int8_t*>(a.v) + (int64_t)g * D + col * 8;
   // paged: block-table window, lane i holds entry win_base + i of this sequence (as in the decode kernel)
   const int bs = PAGED ? a.block_size : 1;
   const int32_t* table = PAGED ? a.block_tables + (int64_t)seq_index * a.max_num_blocks : nullptr;
@@ -801,7 +821,20 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
 #pragma unroll
       for (int i = 0; i < 4; ++i) v_tok[i] = min(t.t0 + 4 * cls + i, kv_end - 1);
     }
-    if (mapped) {
+    if constexpr (I8) {
+      if (mapped) {
+        const float ks = a.k_scale[k_tok * a.num_kv_heads + g];
+#pragma unroll
+        for (int j = 0; j < D / 32; ++j) t.k[j] = dequant8<T>(*reinterpret_cast<const uint2*>(kc8 + k_tok * row + 32 * j), ks);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          t.v[i] = IO::owns(col) ? dequant8<T>(*reinterpret_cast<const uint2*>(vc8 + v_tok[i] * row),
+                                               a.v_scale[v_tok[i] * a.num_kv_heads + g])
+                                 : make_uint4(0u, 0u, 0u, 0u);
+      } else {
+        IO::zero(t);
+      }
+    } else if (mapped) {
       IO::load_k(t, kc + k_tok * row);
 #pragma unroll
       for (int i = 0; i < 4; ++i) IO::template load_v<false>(t, i, vc + v_tok[i] * row, IO::owns(col));
@@ -1451,12 +1484,19 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
 
 template <typename T, int D>
 static void launch_rows16(const PrefillRowsArgs& a, dim3 grid, int tiles, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    if (a.k_scale) {
+      prefill_rows16_kernel<T, D, true, true><<<grid, dim3(256), 0, stream>>>(a, tiles);
+      return;
+    }
+  }
   if (a.block_tables) prefill_rows16_kernel<T, D, true><<<grid, dim3(256), 0, stream>>>(a, tiles);
   else prefill_rows16_kernel<T, D, false><<<grid, dim3(256), 0, stream>>>(a, tiles);
 }
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream) {
   if (head_dim != 64 && head_dim != 128) return MVLLM_ERR_UNSUPPORTED;
   if (a.block_tables && a.block_size % kTile != 0) return MVLLM_ERR_UNSUPPORTED;
+  if (a.k_scale && (!a.v_scale || !a.block_tables || dtype == MVLLM_F32)) return MVLLM_ERR_UNSUPPORTED;
   const int64_t tiles = a.total_tokens / kTile + a.num_seqs;      // upper bound on the 16-row tiles
   const dim3 grid((unsigned)tiles, (unsigned)((a.num_heads + 3) / 4));
   if (dtype == MVLLM_F32) {

@@ -665,6 +665,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
     r.out = out; r.q = q; r.k = k; r.v = v; r.cu_seqlens = cu_seqlens; r.total_tokens = total_tokens;
     r.num_seqs = num_seqs; r.num_heads = num_heads; r.num_kv_heads = num_kv_heads; r.scale_log2 = scale * kLog2e;
     r.cu_seqlens_k = nullptr; r.block_tables = nullptr; r.max_num_blocks = 0; r.block_size = 0; r.num_blocks = 0;
+    r.k_scale = nullptr; r.v_scale = nullptr;
     return launch_prefill_rows16(r, head_dim, dtype, (hipStream_t)stream);
   }
   return prefill_dispatch<false>(a, dtype, mfma_ok, (hipStream_t)stream);
@@ -703,8 +704,34 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
     r.out = out; r.q = q; r.k = k_cache; r.v = v_cache; r.cu_seqlens = cu_seqlens_q; r.total_tokens = total_q_tokens;
     r.num_seqs = num_seqs; r.num_heads = num_heads; r.num_kv_heads = num_kv_heads; r.scale_log2 = scale * kLog2e;
     r.cu_seqlens_k = cu_seqlens_k; r.block_tables = block_tables; r.max_num_blocks = max_num_blocks;
-    r.block_size = block_size; r.num_blocks = num_blocks;
+    r.block_size = block_size; r.num_blocks = num_blocks; r.k_scale = nullptr; r.v_scale = nullptr;
     return launch_prefill_rows16(r, head_dim, dtype, (hipStream_t)stream);
   }
   return prefill_dispatch<true>(a, dtype, mfma_ok, (hipStream_t)stream);
+}
+
+extern "C" int mvllm_prefill_paged_int8(void* out, const void* q, const int8_t* k_cache, const int8_t* v_cache,
+                                        const float* k_scale, const float* v_scale, const int32_t* block_tables,
+                                        int max_num_blocks, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                        int num_seqs, int64_t total_q_tokens, int num_heads, int num_kv_heads,
+                                        int head_dim, int block_size, int64_t num_blocks, float scale, int dtype,
+                                        void* stream) {
+  if (dtype_size(dtype) == 0) return MVLLM_ERR_BAD_DTYPE;
+  if (num_seqs < 0 || total_q_tokens < 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 ||
+      block_size <= 0 || num_blocks < 0 || max_num_blocks < 0)
+    return MVLLM_ERR_BAD_SHAPE;
+  if (num_heads % num_kv_heads != 0) return MVLLM_ERR_BAD_SHAPE;
+  if (num_seqs == 0 || total_q_tokens == 0) return MVLLM_OK;
+  if (!out || !q || !k_cache || !v_cache || !k_scale || !v_scale || !block_tables || !cu_seqlens_q || !cu_seqlens_k)
+    return MVLLM_ERR_NULL_POINTER;
+  if (dtype == MVLLM_F32 || (head_dim != 128 && head_dim != 64) || block_size % 16 != 0 || num_heads > 65535 ||
+      total_q_tokens > ((int64_t)1 << 30) || (int64_t)num_kv_heads * head_dim * 64 >= ((int64_t)1 << 31))
+    return MVLLM_ERR_UNSUPPORTED;
+  if (!aligned16(q) || !aligned16(out) || !aligned16(k_cache) || !aligned16(v_cache)) return MVLLM_ERR_MISALIGNED;
+  PrefillRowsArgs r;
+  r.out = out; r.q = q; r.k = k_cache; r.v = v_cache; r.cu_seqlens = cu_seqlens_q; r.total_tokens = total_q_tokens;
+  r.num_seqs = num_seqs; r.num_heads = num_heads; r.num_kv_heads = num_kv_heads; r.scale_log2 = scale * kLog2e;
+  r.cu_seqlens_k = cu_seqlens_k; r.block_tables = block_tables; r.max_num_blocks = max_num_blocks;
+  r.block_size = block_size; r.num_blocks = num_blocks; r.k_scale = k_scale; r.v_scale = v_scale;
+  return launch_prefill_rows16(r, head_dim, dtype, (hipStream_t)stream);
 }

@@ -81,9 +81,12 @@ class ModelRunner:
 
     def prepare_prefill(self, seqs):
         """Packed prompt tokens and their metadata (model_runner.py:180-227).  Tokens covered by prefix-cache hits
-        are left out and read from the paged cache by the attention kernel; with an int8 cache (no paged prefill
-        for it) or ``prefix_caching=False`` they are recomputed into the shared blocks instead."""
-        reuse = self.kv_cache_dtype != "int8" and self.config.get("prefix_caching", True)
+        are left out and read from the paged cache by the attention kernel (also from an int8 cache, for 16-bit
+        models with head_dim 128 or 64 and blocks of a multiple of 16 tokens); with ``prefix_caching=False`` they are
+        recomputed into the shared blocks instead."""
+        head_dim = self.config.get("head_dim") or self.config["hidden_size"] // self.config["num_heads"]
+        int8_ok = self.dtype != torch.float32 and head_dim in (64, 128) and self.block_size % 16 == 0
+        reuse = (self.kv_cache_dtype != "int8" or int8_ok) and self.config.get("prefix_caching", True)
         md = prefill_metadata(seqs, self.block_size, reuse_cached_kv=reuse)
         positions = [p for seq in seqs for p in range(seq.num_cached_tokens if reuse else 0, len(seq))]
         tables = md["block_tables"]

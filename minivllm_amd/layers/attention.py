@@ -22,6 +22,7 @@ from minivllm_amd.utils.context import get_context
 
 __all__ = [
     "store_kvcache", "store_kvcache_int8", "flash_attention_prefill", "flash_attention_prefill_paged",
+    "flash_attention_prefill_paged_int8",
     "paged_attention_decode", "paged_attention_decode_int8", "Attention",
 ]
 
@@ -191,6 +192,44 @@ def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cach
                                  q.shape[0], num_heads, num_kv_heads, head_dim, block_size, k_cache.shape[0],
                                  float(scale), _C.dtype_code(q.dtype), _C.current_stream_ptr(q.device))
     _C.check(st, "flash_attention_prefill_paged")
+    return output
+
+
+def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                                       k_scale: torch.Tensor, v_scale: torch.Tensor, block_tables: torch.Tensor,
+                                       cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, scale: float,
+                                       num_heads: int, num_kv_heads: int, head_dim: int, block_size: int) -> torch.Tensor:
+    """``flash_attention_prefill_paged`` over an INT8 cache written by ``store_kvcache_int8``: every key, the new
+    tokens' included, is read from the cache and dequantised in the kernel, as decode does for the same tokens.
+    q bf16 / fp16; caches int8 (num_blocks, block_size, Hkv, D); scales float32 (num_blocks, block_size, Hkv)."""
+    _C.require_cuda(q, k_cache, v_cache, k_scale, v_scale, block_tables, cu_seqlens_q, cu_seqlens_k)
+    if q.dim() != 3 or tuple(q.shape[1:]) != (num_heads, head_dim):
+        raise ValueError(f"q must be (total_tokens, {num_heads}, {head_dim}), got {tuple(q.shape)}")
+    if k_cache.dtype != torch.int8 or v_cache.dtype != torch.int8:
+        raise ValueError("int8 caches expected")
+    _check_cache("k_cache", k_cache, num_kv_heads, head_dim)
+    _check_cache("v_cache", v_cache, num_kv_heads, head_dim)
+    if k_cache.shape != v_cache.shape or k_cache.shape[1] != block_size:
+        raise ValueError("K and V cache shapes must match and have block_size rows per block")
+    for name, sc in (("k_scale", k_scale), ("v_scale", v_scale)):
+        if sc.dtype != torch.float32 or tuple(sc.shape) != tuple(k_cache.shape[:3]) or not sc.is_contiguous():
+            raise ValueError(f"{name} must be contiguous float32 {tuple(k_cache.shape[:3])}")
+    num_seqs = cu_seqlens_q.shape[0] - 1
+    if cu_seqlens_k.shape[0] != num_seqs + 1:
+        raise ValueError("cu_seqlens_q and cu_seqlens_k must have the same length")
+    if block_tables.dim() != 2 or block_tables.shape[0] != num_seqs:
+        raise ValueError(f"block_tables must be ({num_seqs}, max_num_blocks), got {tuple(block_tables.shape)}")
+    q = q.contiguous()
+    block_tables = block_tables.to(torch.int32).contiguous()
+    cu_seqlens_q = cu_seqlens_q.to(torch.int32).contiguous()
+    cu_seqlens_k = cu_seqlens_k.to(torch.int32).contiguous()
+    output = torch.empty_like(q)
+    st = _C.load().mvllm_prefill_paged_int8(_ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale),
+                                            _ptr(v_scale), _ptr(block_tables), block_tables.shape[1],
+                                            _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), num_seqs, q.shape[0], num_heads,
+                                            num_kv_heads, head_dim, block_size, k_cache.shape[0], float(scale),
+                                            _C.dtype_code(q.dtype), _C.current_stream_ptr(q.device))
+    _C.check(st, "flash_attention_prefill_paged_int8")
     return output
 
 
@@ -370,13 +409,17 @@ class Attention(nn.Module):
             if context.block_tables is not None:
                 # some sequence starts after a cached prefix: every key comes from the paged cache, which the
                 # store above has just completed with the new tokens (model_runner.py:206-215)
-                if int8:
-                    raise ValueError("prefill over a cached prefix needs a cache in the model dtype, not int8")
                 if context.cu_seqlens_k is None or k_cache.numel() == 0:
                     raise ValueError("cu_seqlens_k and the KV cache must be provided for prefill over a cached prefix")
-                o = flash_attention_prefill_paged(q, k_cache, v_cache, context.block_tables, cu_seqlens,
-                                                  context.cu_seqlens_k, scale, self.num_heads, self.num_kv_heads,
-                                                  self.head_dim, self.block_size)
+                if int8:
+                    o = flash_attention_prefill_paged_int8(q, k_cache, v_cache, self.k_scale, self.v_scale,
+                                                           context.block_tables, cu_seqlens, context.cu_seqlens_k,
+                                                           scale, self.num_heads, self.num_kv_heads, self.head_dim,
+                                                           self.block_size)
+                else:
+                    o = flash_attention_prefill_paged(q, k_cache, v_cache, context.block_tables, cu_seqlens,
+                                                      context.cu_seqlens_k, scale, self.num_heads, self.num_kv_heads,
+                                                      self.head_dim, self.block_size)
                 return o.reshape(o.shape[0], self.num_heads * self.head_dim)
             o = flash_attention_prefill(q, k, v, cu_seqlens, scale, self.num_heads, self.num_kv_heads,
                                         self.head_dim)

@@ -28,7 +28,7 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_varlen",
-              "mvllm_prefill_paged", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_workspace_bytes",
+              "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_workspace_bytes",
               "mvllm_add_rms_norm",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
         assert n in names

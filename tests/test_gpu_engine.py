@@ -108,7 +108,8 @@ def test_fused_qk_path_matches_unfused_modules(kv_cache_dtype):
         assert (a - b).abs().max() <= 6e-2 and (a - b).abs().mean() <= 1e-3
 
 
-def test_prefix_cache_hits_are_read_from_the_paged_cache():
+@pytest.mark.parametrize("kv_cache_dtype", ["auto", "int8"])
+def test_prefix_cache_hits_are_read_from_the_paged_cache(kv_cache_dtype):
     """Prompts that share whole blocks with an earlier request skip those tokens in prefill (the attention
     kernel reads their keys from the paged cache).  The generated tokens must match a run that recomputes them."""
     g = torch.Generator().manual_seed(12)
@@ -116,7 +117,7 @@ def test_prefix_cache_hits_are_read_from_the_paged_cache():
     prompts = [shared + torch.randint(0, 2048, (n,), generator=g).tolist() for n in (5, 21, 0, 16)]
     prompts.append(shared[:32])                                            # exactly two cached blocks, nothing new
     sp = SamplingParams(temperature=0.6, max_tokens=8, ignore_eos=True)
-    cfg = dict(SMALL, max_num_sequences=2, max_cached_blocks=64)           # two per step: later steps hit the cache
+    cfg = dict(SMALL, max_num_sequences=2, max_cached_blocks=64, kv_cache_dtype=kv_cache_dtype)   # two per step: later steps hit the cache
     outs, skipped = [], []
     for reuse in (True, False):
         eng = LLMEngine(dict(cfg, prefix_caching=reuse))
@@ -133,7 +134,9 @@ def test_prefix_cache_hits_are_read_from_the_paged_cache():
     assert skipped[1] == 0
     assert skipped[0] >= 48 + 48 + 16, skipped            # the 2nd step reuses 3 blocks twice, the 3rd at least 1
     same = sum(a == b for a, b in zip(*outs))
-    assert same >= 4, outs                                # a 1-ulp difference may flip a sampling tie, rarely
+    # a 1-ulp difference may flip a sampling tie, rarely; with an int8 cache the run that recomputes a prefix attends
+    # to its exact keys where the run that reuses it reads the quantised ones, so more samples may differ
+    assert same >= (4 if kv_cache_dtype == "auto" else 2), outs
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])

@@ -140,3 +140,40 @@ def test_paged_prefill_head_dim_64_without_prefix_matches_plain_prefill_bitwise(
     scale = 1 / math.sqrt(d)
     plain = flash_attention_prefill(c["q"].to(DEV), c["k"].to(DEV), c["v"].to(DEV), c["cu_k"].to(DEV), scale, hq, hkv, d).cpu()
     assert torch.equal(_run(c, scale, hq, hkv, d, bs), plain)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,d,bs,lengths,cached", [
+    (32, 8, 128, 16, [300, 64, 129, 500], [256, 0, 17, 48]),
+    (16, 8, 64, 16, [200, 90, 33], [160, 80, 0]),                  # the reference demo's heads
+    (12, 1, 128, 256, [700, 30, 257], [512, 29, 0]),               # one kv head, the engine's block size
+    (6, 2, 64, 48, [131, 77, 260], [50, 1, 259]),                  # three query heads per kv head
+])
+def test_paged_prefill_over_an_int8_cache(dtype, hq, hkv, d, bs, lengths, cached):
+    """Every key comes from the INT8 cache: the oracle is the paged prefill over the dequantised cache (code * scale
+    in fp32).  Tolerance as for INT8 decode: mean-abs 2e-3, |err| <= 2e-2 + |want| * 2^-8."""
+    from minivllm_amd.layers.attention import flash_attention_prefill_paged_int8, store_kvcache_int8
+    c = make_paged_prefill_case(67, lengths, cached, hq, hkv, d, bs, dtype=dtype, poison=0.0)
+    nb = c["k_cache"].shape[0]
+    ck, cv = (torch.zeros(nb, bs, hkv, d, dtype=torch.int8, device=DEV) for _ in range(2))
+    sk, sv = (torch.zeros(nb, bs, hkv, device=DEV) for _ in range(2))
+    store_kvcache_int8(c["k_cache"].view(-1, hkv, d).to(DEV), c["v_cache"].view(-1, hkv, d).to(DEV), ck, cv, sk, sv,
+                       torch.arange(nb * bs, device=DEV), bs)
+    scale = 1 / math.sqrt(d)
+    got = flash_attention_prefill_paged_int8(c["q_new"].to(DEV), ck, cv, sk, sv, c["block_tables"].to(DEV),
+                                             c["cu_q"].to(DEV), c["cu_k"].to(DEV), scale, hq, hkv, d, bs).cpu()
+    kd = oracle.dequantize_cache_oracle(ck.cpu(), sk.cpu())
+    vd = oracle.dequantize_cache_oracle(cv.cpu(), sv.cpu())
+    want = oracle.prefill_paged_oracle(c["q_new"].float(), kd, vd, c["block_tables"], c["cu_q"], c["cu_k"], scale,
+                                       hq, hkv, d, bs)
+    assert got.dtype == dtype and got.shape == want.shape and torch.isfinite(got.float()).all()
+    mx, mean = error_stats(got, want)
+    excess = ((got.float() - want).abs() - want.abs() * 2.0 ** -8).max().item()
+    assert excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
+    # one new token per sequence: the same rows as INT8 decode over the same cache
+    from minivllm_amd.layers.attention import paged_attention_decode_int8
+    last = torch.tensor([int(c["cu_q"][i + 1]) - 1 for i in range(len(lengths))])
+    dec = paged_attention_decode_int8(c["q_new"][last].to(DEV), ck, cv, sk, sv, c["block_tables"].to(DEV),
+                                      torch.tensor(lengths, device=DEV), scale, hq, hkv, d, bs).cpu()
+    mx, mean = error_stats(got[last], dec.float())
+    assert mx <= 3e-2 and mean <= 3e-3, (mx, mean)
