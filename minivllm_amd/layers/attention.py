@@ -169,7 +169,7 @@ def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cach
     if q.dim() != 3 or tuple(q.shape[1:]) != (num_heads, head_dim):
         raise ValueError(f"q must be (total_tokens, {num_heads}, {head_dim}), got {tuple(q.shape)}")
     if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
-        raise ValueError(f"q {q.dtype} and cache {k_cache.dtype} dtypes differ (no int8 cache in paged prefill)")
+        raise ValueError(f"q {q.dtype} and cache {k_cache.dtype} dtypes differ (for an int8 cache use flash_attention_prefill_paged_int8)")
     _check_cache("k_cache", k_cache, num_kv_heads, head_dim)
     _check_cache("v_cache", v_cache, num_kv_heads, head_dim)
     if k_cache.shape != v_cache.shape:
