@@ -21,9 +21,21 @@ class LLMEngine:
             block_size=self.block_size,
             eos=config.get("eos", 50256))
         self.model_runner = model_runner if model_runner is not None else ModelRunner(config)
+        # longest sequence (prompt + new tokens) the rotary table and the graph's block-table buffer are sized for
+        self.max_model_length = min(config.get("max_model_length", config.get("max_position", 4096)),
+                                    config.get("max_position", 4096))
         self.stats = {"prefill_tokens": 0, "decode_tokens": 0, "prefill_s": 0.0, "decode_s": 0.0, "steps": 0}
 
     def add_prompt(self, prompt_token_ids: list[int], sampling_params: SamplingParams) -> None:
+        """Queue a prompt.  A request that could outgrow ``max_model_length`` / ``max_position`` is refused here:
+        the reference's demo exceeds its own limit silently (main.py:35,38,49) and would index the rotary table
+        out of range (rotary_embedding.py:78)."""
+        if not prompt_token_ids:
+            raise ValueError("empty prompt")
+        longest = len(prompt_token_ids) + sampling_params.max_tokens
+        if longest > self.max_model_length:
+            raise ValueError(f"prompt of {len(prompt_token_ids)} tokens + max_tokens {sampling_params.max_tokens} "
+                             f"exceeds max_model_length / max_position {self.max_model_length}")
         self.scheduler.add_sequence(Sequence(prompt_token_ids, sampling_params, self.block_size))
 
     def step(self):

@@ -12,6 +12,7 @@ from __future__ import annotations
 import torch
 
 from minivllm_amd.engine.metadata import decode_metadata, prefill_metadata
+from minivllm_amd.layers.attention import decode_workspace_bytes
 from minivllm_amd.layers.basic import Sampler
 from minivllm_amd.layers.fused import sample_tokens
 from minivllm_amd.models.qwen3 import Qwen3ForCausalLM
@@ -130,6 +131,7 @@ class ModelRunner:
             outputs=torch.zeros(max_bs, cfg["hidden_size"], dtype=self.dtype, device=dev))
         v = self.graph_vars
         buckets = sorted({b for b in [1, 2, 4, 8] + list(range(16, max_bs + 1, 16)) + [max_bs] if b <= max_bs})
+        self._own_decode_workspace(buckets, max_blocks)
         pool = None
         for bs in reversed(buckets):
             set_context(False, slot_mapping=v["slot_mapping"][:bs], context_lens=v["context_lens"][:bs],
@@ -139,7 +141,7 @@ class ModelRunner:
                 positions = (v["context_lens"][:bs] - 1).clamp_min(0)
                 v["outputs"][:bs] = self.model(v["input_ids"][:bs], positions)
 
-            forward()                                    # warm-up: sizes the attention workspace before capture
+            forward()                                    # warm-up outside the capture (library handles, lazy loads)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool):
@@ -148,6 +150,19 @@ class ModelRunner:
             self.graphs[bs] = graph
             torch.cuda.synchronize()
             reset_context()
+
+    def _own_decode_workspace(self, buckets, max_blocks):
+        """One split-K scratch buffer for every decode call of this runner, allocated before any graph is
+        captured and sized for the largest need over the batch buckets.  The need is not monotonic in the batch
+        (a smaller batch is cut into more partitions), so a buffer grown bucket by bucket would be replaced,
+        and freed, after a graph that holds its address had been captured."""
+        cfg = self.config
+        head_dim = cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_heads"]
+        need = max(decode_workspace_bytes(b, cfg["num_heads"], head_dim, max_blocks, self.block_size) for b in buckets)
+        self.decode_workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=self.device)
+        for module in self.model.modules():
+            if hasattr(module, "decode_workspace"):
+                module.decode_workspace = self.decode_workspace
 
     def _fill_decode_buffers(self, seqs, gbs):
         """Full refill of the static decode buffers from the host-side metadata (model_runner.py:231-256)."""

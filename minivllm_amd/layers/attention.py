@@ -23,22 +23,34 @@ from minivllm_amd.utils.context import get_context
 __all__ = [
     "store_kvcache", "store_kvcache_int8", "flash_attention_prefill", "flash_attention_prefill_paged",
     "flash_attention_prefill_paged_int8",
-    "paged_attention_decode", "paged_attention_decode_int8", "Attention",
+    "paged_attention_decode", "paged_attention_decode_int8", "decode_workspace_bytes", "Attention",
 ]
 
-_workspaces: dict = {}   # device index -> uint8 tensor reused by every decode call on that device
+_workspaces: dict = {}   # device index -> uint8 tensor reused by decode calls on that device that bring no workspace
+_retired: list = []      # outgrown workspaces: kept alive, because a captured hipGraph may hold their address
 
 
-def _decode_workspace(device: torch.device, nbytes: int):
-    """Split-K scratch for paged decode: grown on demand, never shrunk, one per device."""
+def _decode_workspace(device: torch.device, nbytes: int, own: torch.Tensor | None = None):
+    """Split-K scratch for paged decode.  ``own`` (a caller-owned uint8 tensor, e.g. the model runner's, sized
+    before its graphs were captured) is used when it is large enough; otherwise one buffer per device, grown on
+    demand and never freed: a buffer that has been handed out may be referenced by a captured graph."""
     if nbytes == 0:
         return None
+    if own is not None and own.numel() >= nbytes:
+        return own
     key = device.index if device.index is not None else torch.cuda.current_device()
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is not None:
+            _retired.append(ws)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def decode_workspace_bytes(batch: int, num_heads: int, head_dim: int, max_num_blocks: int, block_size: int) -> int:
+    """Bytes of split-K scratch a decode call of these static sizes may use (host arithmetic only)."""
+    return int(_C.load().mvllm_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_num_blocks, block_size))
 
 
 def _ptr(t):
@@ -274,12 +286,15 @@ def paged_decode_plan(batch: int, num_heads: int, num_kv_heads: int, head_dim: i
 
 def paged_attention_decode(query: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                            block_tables: torch.Tensor, context_lens: torch.Tensor, scale: float,
-                           num_heads: int, num_kv_heads: int, head_dim: int, block_size: int) -> torch.Tensor:
+                           num_heads: int, num_kv_heads: int, head_dim: int, block_size: int, *,
+                           workspace: torch.Tensor | None = None) -> torch.Tensor:
     """One query token per sequence over its paged KV.  Reference: attention.py:418-473.
 
     query: (batch, num_heads, head_dim); caches (num_blocks, block_size, Hkv, D);
     block_tables int32 (batch, max_num_blocks), -1 padded; context_lens int32 or
     int64 (batch,).  Returns a tensor like query; rows with context_len 0 are zeros.
+    ``workspace`` (optional, not in the reference): a uint8 device tensor the caller owns for the split-K
+    partials; without it, or when it is too small, a per-device buffer of this module is used.
     """
     _C.require_cuda(query, k_cache, v_cache, block_tables, context_lens)
     if k_cache.dtype != query.dtype or v_cache.dtype != query.dtype:
@@ -292,7 +307,7 @@ def paged_attention_decode(query: torch.Tensor, k_cache: torch.Tensor, v_cache: 
         return output
     lib = _C.load()
     nbytes = lib.mvllm_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks, block_size)
-    ws = _decode_workspace(query.device, nbytes)
+    ws = _decode_workspace(query.device, nbytes, workspace)
     st = lib.mvllm_paged_decode(_ptr(output), _ptr(query), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                 max_blocks, _ptr(context_lens), int(context_lens.dtype == torch.int64), batch,
                                 num_heads, num_kv_heads, head_dim, block_size, k_cache.shape[0], float(scale),
@@ -305,8 +320,10 @@ def paged_attention_decode(query: torch.Tensor, k_cache: torch.Tensor, v_cache: 
 def paged_attention_decode_int8(query: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                                 k_scale: torch.Tensor, v_scale: torch.Tensor, block_tables: torch.Tensor,
                                 context_lens: torch.Tensor, scale: float, num_heads: int, num_kv_heads: int,
-                                head_dim: int, block_size: int) -> torch.Tensor:
-    """Paged decode over an int8 cache written by ``store_kvcache_int8``."""
+                                head_dim: int, block_size: int, *,
+                                workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """Paged decode over an int8 cache written by ``store_kvcache_int8`` (``workspace`` as in
+    ``paged_attention_decode``)."""
     _C.require_cuda(query, k_cache, v_cache, k_scale, v_scale, block_tables, context_lens)
     if k_cache.dtype != torch.int8 or v_cache.dtype != torch.int8:
         raise ValueError("int8 caches expected")
@@ -321,7 +338,7 @@ def paged_attention_decode_int8(query: torch.Tensor, k_cache: torch.Tensor, v_ca
         return output
     lib = _C.load()
     nbytes = lib.mvllm_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks, block_size)
-    ws = _decode_workspace(query.device, nbytes)
+    ws = _decode_workspace(query.device, nbytes, workspace)
     st = lib.mvllm_paged_decode_int8(_ptr(output), _ptr(query), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale),
                                      _ptr(v_scale), _ptr(block_tables), max_blocks, _ptr(context_lens),
                                      int(context_lens.dtype == torch.int64), batch, num_heads, num_kv_heads,
@@ -356,6 +373,7 @@ class Attention(nn.Module):
         self.kv_cache_dtype = kv_cache_dtype
         self.k_cache = self.v_cache = torch.tensor([])
         self.k_scale = self.v_scale = torch.tensor([])
+        self.decode_workspace = None      # optional split-K scratch assigned from outside, like the caches
 
     def forward_fused(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor,
                       cos_sin_cache: torch.Tensor, gamma: torch.Tensor | None, eps: float) -> torch.Tensor:
@@ -430,8 +448,10 @@ class Attention(nn.Module):
         if int8:
             o = paged_attention_decode_int8(q, k_cache, v_cache, self.k_scale, self.v_scale,
                                             context.block_tables, context.context_lens, scale,
-                                            self.num_heads, self.num_kv_heads, self.head_dim, self.block_size)
+                                            self.num_heads, self.num_kv_heads, self.head_dim, self.block_size,
+                                            workspace=self.decode_workspace)
         else:
             o = paged_attention_decode(q, k_cache, v_cache, context.block_tables, context.context_lens, scale,
-                                       self.num_heads, self.num_kv_heads, self.head_dim, self.block_size)
+                                       self.num_heads, self.num_kv_heads, self.head_dim, self.block_size,
+                                       workspace=self.decode_workspace)
         return o.reshape(o.shape[0], self.num_heads * self.head_dim)

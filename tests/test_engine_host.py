@@ -190,3 +190,30 @@ def test_full_prefix_hit_still_leaves_one_block_to_compute():
     assert md["input_ids"] == [4, 5, 6, 7] and md["cu_seqlens_q"] == [0, 4] and md["cu_seqlens_k"] == [0, 8]
     assert md["slot_mapping"] == [again.block_table[1] * 4 + i for i in range(4)]
     assert md["block_tables"] == [again.block_table]
+
+
+def test_requests_longer_than_the_model_length_are_refused_at_admission():
+    import pytest
+    cfg = dict(max_num_sequences=2, max_num_batched_tokens=64, max_cached_blocks=16, block_size=4, eos=-1,
+               max_position=32, max_model_length=24)
+    eng = LLMEngine(cfg, model_runner=FakeRunner())
+    eng.add_prompt(list(range(20)), SamplingParams(max_tokens=4))          # 24: fits exactly
+    with pytest.raises(ValueError):
+        eng.add_prompt(list(range(21)), SamplingParams(max_tokens=4))
+    with pytest.raises(ValueError):
+        eng.add_prompt([], SamplingParams(max_tokens=4))
+    assert len(eng.scheduler.waiting) == 1
+
+
+def test_decode_workspace_need_is_not_monotonic_and_the_runner_sizes_for_the_maximum():
+    """The split-K scratch a decode call may use is not monotonic in the batch size (a smaller batch is cut into
+    more partitions), so the model runner sizes one buffer for the maximum over its batch buckets before it
+    captures any graph; every bucket then fits that buffer."""
+    from minivllm_amd.layers.attention import decode_workspace_bytes
+    hq, d, bs = 16, 128, 16
+    for max_len in (4096, 8192):
+        blocks = max_len // bs
+        need = {b: decode_workspace_bytes(b, hq, d, blocks, bs) for b in [1, 2, 4, 8, 16, 32, 48, 64]}
+        assert need[48] > need[64] > 0                 # 48 x 32 partitions against 64 x 16
+        sized = max(need.values())
+        assert all(n <= sized for n in need.values())

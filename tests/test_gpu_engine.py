@@ -157,3 +157,88 @@ def test_reference_demo_model_shape_head_dim_64(dtype):
     assert [len(t) for t in graphed] == [16] * 6
     same = sum(a == b for a, b in zip(eager, graphed))
     assert same >= 4, (same, eager, graphed)          # a 1-ulp difference may flip a sampling tie, rarely
+
+
+CONFIG5 = dict(vocab_size=151936, hidden_size=1024, num_layers=8, num_heads=16, num_kv_heads=8, head_dim=128,
+               intermediate_size=3072, base=1_000_000, rms_norm_epsilon=1e-6, qkv_bias=False, ffn_bias=True,
+               scale=1.0, tie_word_embeddings=True, block_size=256, max_num_batched_tokens=16384,
+               max_cached_blocks=256, max_position=512, max_model_length=512, dtype="bf16", eos=-1, seed=0)
+
+
+def test_config5_full_shape():
+    """BASELINE.json config 5 at its own shape (llm_engine.py:71-88 driven as main.py:15-41 does): Qwen3-style
+    decoder 8 x 1024, 16 query / 8 kv heads of 128 dims, vocabulary 151 936, blocks of 256 tokens, 60 prompts of
+    32-96 random ids, 256 new tokens each at temperature 0.6.  Checked: the run completes with every id in range;
+    the hipGraph decode run and the eager run (same seed, so the same sampler noise) agree on at least 90 % of the
+    sequences' first 32 new tokens and on at least half of the whole sequences (one flipped sampling tie changes
+    everything after it); and the paged cache that 60 decode steps leave behind equals the K/V of one varlen
+    prefill over the same tokens."""
+    vocab = CONFIG5["vocab_size"]
+    prompts = _prompts(60, 32, 96, seed=50, vocab=vocab)
+    sp = SamplingParams(temperature=0.6, max_tokens=256, ignore_eos=True)
+    runs = {}
+    for graph in (True, False):
+        eng = LLMEngine(dict(CONFIG5, max_num_sequences=64, enforce_eager=not graph))
+        out = eng.generate(prompts, sp)["token_ids"]
+        assert [len(t) for t in out] == [256] * 60
+        assert all(0 <= t < vocab for seq in out for t in seq)
+        assert len(eng.scheduler.block_manager.free_block_ids) == CONFIG5["max_cached_blocks"]   # every block released
+        runs[graph] = out
+        del eng
+        torch.cuda.empty_cache()
+    head = sum(a[:32] == b[:32] for a, b in zip(runs[True], runs[False]))
+    whole = sum(a == b for a, b in zip(runs[True], runs[False]))
+    assert head >= 54 and whole >= 30, (head, whole)
+
+    # the cache after 60 decode steps == one prefill of the same tokens, at this shape; prompts of 200-250 tokens,
+    # so that sequences open their second 256-token block while decoding
+    eng = LLMEngine(dict(CONFIG5, max_num_sequences=16, enforce_eager=True))
+    long_prompts = _prompts(12, 200, 250, seed=51, vocab=vocab)
+    for p in long_prompts:
+        eng.add_prompt(p, sp)
+    for _ in range(1 + 60):
+        eng.step()
+    seqs = list(eng.scheduler.running)
+    assert len(seqs) == 12 and all(s.num_completion_tokens == 61 for s in seqs)
+    assert any(len(s.block_table) == 2 for s in seqs)              # the block boundary was crossed in decode
+    runner = eng.model_runner
+    bs = runner.block_size
+    flat = lambda: runner.kv_cache.view(2, runner.kv_cache.shape[1], -1, *runner.kv_cache.shape[-2:])
+    rows_of = lambda s: torch.tensor([s.block_table[i // bs] * bs + i % bs for i in range(len(s) - 1)], device=DEV)
+    paged = [flat()[:, :, rows_of(s)].clone() for s in seqs]
+    runner.kv_cache.zero_()
+    tokens = [s.token_ids[:-1] for s in seqs]
+    cu = torch.tensor([0] + [len(t) for t in tokens]).cumsum(0).to(torch.int32)
+    slots = torch.cat([rows_of(s) for s in seqs])
+    set_context(True, cu.to(DEV), cu.to(DEV), max(map(len, tokens)), max(map(len, tokens)), slots, None, None)
+    with torch.inference_mode():
+        runner.model(torch.tensor([x for t in tokens for x in t], device=DEV),
+                     torch.tensor([i for t in tokens for i in range(len(t))], device=DEV))
+    reset_context()
+    for s, old in zip(seqs, paged):
+        new = flat()[:, :, rows_of(s)]
+        assert (old[:, 0].float() - new[:, 0].float()).abs().max() <= 3.2e-2
+        diff = (old.float() - new.float()).abs()
+        assert diff.max() <= 0.25 and diff.mean() <= 4e-3, (diff.max().item(), diff.mean().item())
+
+
+def test_graph_decode_with_split_partitions_in_every_bucket():
+    """64 sequences and a 4096-token model length with 2 kv heads: every batch bucket decodes in several partitions
+    through the split-K scratch, whose need is largest at bucket 48, not 64.  The runner owns one buffer sized
+    before any capture, so the graphs captured first keep a valid address; graph and eager runs must agree."""
+    from minivllm_amd.layers.attention import paged_decode_plan
+    cfg = dict(SMALL, max_num_sequences=64, max_cached_blocks=640, max_model_length=4096, max_position=4096,
+               max_num_batched_tokens=8192)
+    assert all(paged_decode_plan(b, 4, 2, 128, 256, 16)[1] > 1 for b in (1, 16, 48, 64))
+    prompts = _prompts(64, 20, 120, seed=31)
+    sp = SamplingParams(temperature=0.7, max_tokens=20, ignore_eos=True)
+    eager = LLMEngine(dict(cfg, enforce_eager=True)).generate(prompts, sp)["token_ids"]
+    eng = LLMEngine(dict(cfg, enforce_eager=False))
+    runner = eng.model_runner
+    assert sorted(runner.graphs) == [1, 2, 4, 8, 16, 32, 48, 64]
+    attn = [m for m in runner.model.modules() if hasattr(m, "decode_workspace")]
+    assert attn and all(m.decode_workspace is runner.decode_workspace for m in attn)
+    graphed = eng.generate(prompts, sp)["token_ids"]
+    assert [len(t) for t in graphed] == [20] * 64
+    same = sum(a == b for a, b in zip(eager, graphed))
+    assert same >= 58, (same,)                        # a 1-ulp GEMM difference between buckets may flip a tie, rarely

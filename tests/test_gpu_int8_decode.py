@@ -116,3 +116,57 @@ def test_int8_both_grid_forms(hq, hkv, bs, d, form):
     mx, mean = error_stats(got, want)
     excess = ((got.float() - want).abs() - want.abs() * 2.0 ** -8).max().item()
     assert torch.isfinite(got).all() and excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
+
+
+def test_config4_full_size_on_its_own_plan():
+    """BASELINE.json config 4 in full: B 128, ctx U[256,16384], Hq32/Hkv8/D128, block 16, N(0,1) inputs with 1 % of
+    the entries at 8 sigma, INT8 store then INT8 decode.  At this size the host picks the one-wave-per-head kernel
+    with 16 partitions of 1024 tokens and the merge kernel (a smaller batch would take the other form).  The cache
+    (2.2 GB of codes) is written on the device by the INT8 store in chunks; the oracle runs on picked sequences."""
+    hq, hkv, d, bs, batch = 32, 8, 128, 16, 128
+    scale = 1 / math.sqrt(d)
+    g = torch.Generator().manual_seed(165)
+    ctx = torch.randint(256, 16385, (batch,), generator=g)
+    ctx[7], ctx[99] = 16384, 256                                   # both ends of the range are present
+    need = [-(-int(c) // bs) for c in ctx.tolist()]
+    nb = sum(need)
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.full((batch, 16384 // bs), -1, dtype=torch.int32)
+    at = 0
+    for b, n in enumerate(need):
+        tables[b, :n] = perm[at:at + n].to(torch.int32)
+        at += n
+    assert paged_decode_plan(batch, hq, hkv, d, tables.shape[1], bs, torch.bfloat16, int8_cache=True) == (1024, 16, 1)
+    ck = torch.empty(nb, bs, hkv, d, dtype=torch.int8, device=DEV)
+    cv = torch.empty_like(ck)
+    sk = torch.empty(nb, bs, hkv, device=DEV)
+    sv = torch.empty_like(sk)
+    dg = torch.Generator(device=DEV).manual_seed(166)
+    step = 4096                                                    # blocks per chunk: 64 K tokens, 134 MB of bf16 each
+    for lo in range(0, nb, step):
+        n = min(step, nb - lo) * bs
+        kv = []
+        for _ in range(2):
+            x = torch.randn(n, hkv, d, generator=dg, device=DEV)
+            x = torch.where(torch.rand(x.shape, generator=dg, device=DEV) < 0.01, x * 8.0, x)
+            kv.append(x.to(torch.bfloat16))
+        store_kvcache_int8(kv[0], kv[1], ck, cv, sk, sv, torch.arange(lo * bs, lo * bs + n, device=DEV), bs)
+    q = torch.randn(batch, hq, d, generator=dg, device=DEV).to(torch.bfloat16)
+    td, cd = tables.to(DEV), ctx.to(DEV)
+    got = paged_attention_decode_int8(q, ck, cv, sk, sv, td, cd, scale, hq, hkv, d, bs).cpu()
+    assert torch.isfinite(got).all()
+    order = torch.argsort(ctx)
+    pick = sorted({int(order[0]), int(order[1]), int(order[-1]), int(order[-2]), int(order[batch // 2]), 0, 64, 127})
+    assert len(pick) >= 8
+    for b in pick:
+        ids = tables[b, :need[b]].long().to(DEV)
+        table = torch.arange(need[b], dtype=torch.int32).unsqueeze(0)
+        want = oracle.decode_int8_oracle(q[b:b + 1].cpu().float(), ck[ids].cpu(), cv[ids].cpu(), sk[ids].cpu(),
+                                         sv[ids].cpu(), table, ctx[b:b + 1], scale, hq, hkv, d, bs)
+        mx, mean = error_stats(got[b:b + 1], want)
+        excess = ((got[b:b + 1].float() - want).abs() - want.abs() * 2.0 ** -8).max().item()
+        assert excess <= 2e-2 and mean <= 2e-3, (b, int(ctx[b]), mx, excess, mean)
+    # size-independent property over the whole batch: the output is linear in the V scales
+    sv *= 2
+    got2 = paged_attention_decode_int8(q, ck, cv, sk, sv, td, cd, scale, hq, hkv, d, bs).cpu()
+    assert (got2.float() - 2 * got.float()).abs().max() <= 2e-2 + 2.0 ** -7 * got.float().abs().max()
