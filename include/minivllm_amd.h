@@ -144,6 +144,25 @@ int mvllm_paged_decode_int8(void* out, const void* q,
                             void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * mvllm_paged_decode for callers that cannot allocate device memory (code under hipGraph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * mvllm_paged_decode without the workspace: the split-K partials go to a static device array inside the library
+ * (MVLLM_PAGED_DECODE_NOALLOC_MAX_BYTES per GPU, held until the process ends).  Shapes for which
+ * mvllm_paged_decode_workspace_bytes() exceeds that size return MVLLM_ERR_WORKSPACE.  The call allocates and frees
+ * nothing; the first call on a device looks up the array's address (make it outside graph capture).  All calls on
+ * one GPU share the array: calls that overlap on one GPU (two streams, two threads) race on it.  Nothing in it
+ * has to be cleared between calls: a merge reads only partials that the same call has written.
+ */
+#define MVLLM_PAGED_DECODE_NOALLOC_MAX_BYTES (32u << 20)
+int mvllm_paged_decode_noalloc(void* out, const void* q,
+                               const void* k_cache, const void* v_cache,
+                               const int32_t* block_tables, int max_num_blocks,
+                               const void* context_lens, int ctx_is_i64,
+                               int batch, int num_heads, int num_kv_heads, int head_dim,
+                               int block_size, int64_t num_blocks, float scale, int dtype,
+                               void* stream);
+
+/*
  * flash_attention_prefill -- src/myvllm/layers/attention.py:212-280 (kernel :111-209).
  * Packed ragged batch: sequence s owns rows [cu_seqlens[s], cu_seqlens[s+1]).
  * out[i,h,:] = softmax_{j<=i, same sequence}( scale * q[i,h,:] . k[j,g(h),:] ) v[j,g(h),:].

@@ -29,6 +29,8 @@ SIGNATURES = {
     "mvllm_paged_decode_plan": (c_int, [c_int] * 8 + [ctypes.POINTER(c_int)] * 3),
     "mvllm_paged_decode": (c_int, [c_void_p] * 5 + [c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                                      c_int64, c_float, c_int, c_void_p, c_size_t, c_void_p]),
+    "mvllm_paged_decode_noalloc": (c_int, [c_void_p] * 5 + [c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                                             c_int64, c_float, c_int, c_void_p]),
     "mvllm_paged_decode_int8": (c_int, [c_void_p] * 7 + [c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                                           c_int, c_int64, c_float, c_int, c_void_p, c_size_t,
                                                           c_void_p]),

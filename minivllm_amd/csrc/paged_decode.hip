@@ -17,6 +17,7 @@
 //   See DecodeHead for the operand layouts.
 // The kernel is HBM-bound: a kernel that only issues the same loads (no arithmetic) reaches
 // 6.25 TB/s on this access pattern, this one about 6.05.
+#include <atomic>
 #include "common.h"
 
 namespace mvllm {
@@ -1435,12 +1436,11 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
   return st;
 }
 
-static int decode_entry(void* out, const void* q, const void* k_cache, const void* v_cache,
-                        const float* k_scale, const float* v_scale, bool int8,
-                        const int32_t* block_tables, int max_num_blocks, const void* context_lens,
-                        int ctx_is_i64, int batch, int num_heads, int num_kv_heads, int head_dim,
-                        int block_size, int64_t num_blocks, float scale, int dtype, void* workspace,
-                        size_t workspace_bytes, void* stream) {
+// Argument checks of the decode entry points (host only; nothing touches the device).
+static int decode_check(const void* out, const void* q, const void* k_cache, const void* v_cache, const float* k_scale,
+                        const float* v_scale, bool int8, const int32_t* block_tables, int max_num_blocks,
+                        const void* context_lens, int batch, int num_heads, int num_kv_heads, int head_dim,
+                        int block_size, int64_t num_blocks, int dtype) {
   if (dtype_size(dtype) == 0) return MVLLM_ERR_BAD_DTYPE;
   if (batch < 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 ||
       max_num_blocks <= 0 || num_blocks < 0)
@@ -1452,6 +1452,19 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
   if (head_dim > 64 * kGenericMaxR) return MVLLM_ERR_UNSUPPORTED;
   if ((int64_t)max_num_blocks * block_size > (int64_t)1 << 30) return MVLLM_ERR_UNSUPPORTED;
   if (batch > 65535 || num_heads > 65535) return MVLLM_ERR_UNSUPPORTED;
+  return MVLLM_OK;
+}
+
+static int decode_entry(void* out, const void* q, const void* k_cache, const void* v_cache,
+                        const float* k_scale, const float* v_scale, bool int8,
+                        const int32_t* block_tables, int max_num_blocks, const void* context_lens,
+                        int ctx_is_i64, int batch, int num_heads, int num_kv_heads, int head_dim,
+                        int block_size, int64_t num_blocks, float scale, int dtype, void* workspace,
+                        size_t workspace_bytes, void* stream) {
+  const int bad = decode_check(out, q, k_cache, v_cache, k_scale, v_scale, int8, block_tables, max_num_blocks,
+                               context_lens, batch, num_heads, num_kv_heads, head_dim, block_size, num_blocks, dtype);
+  if (bad != MVLLM_OK) return bad;
+  if (batch == 0) return MVLLM_OK;
 
   DecodeArgs a;
   a.out = out; a.q = q; a.k_cache = k_cache; a.v_cache = v_cache;
@@ -1544,6 +1557,49 @@ extern "C" int mvllm_paged_decode(void* out, const void* q, const void* k_cache,
   return decode_entry(out, q, k_cache, v_cache, nullptr, nullptr, false, block_tables, max_num_blocks,
                       context_lens, ctx_is_i64, batch, num_heads, num_kv_heads, head_dim, block_size,
                       num_blocks, scale, dtype, workspace, workspace_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------
+// Entry point for callers that cannot allocate: the split-K partials go to a static device array instead of a
+// caller-owned workspace.  The array's name is only a host-side handle; its device address is looked up once per
+// device (hipGetSymbolAddress with that device current) and kept.
+// ---------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = MVLLM_PAGED_DECODE_NOALLOC_MAX_BYTES;   // 32 MiB per GPU
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device; null (and *status set) when the lookup fails.
+static void* static_scratch(int* status) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { *status = (int)e; return nullptr; }
+  if (dev < 0 || dev >= kMaxDevices) { *status = MVLLM_ERR_UNSUPPORTED; return nullptr; }
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !p) { *status = e != hipSuccess ? (int)e : MVLLM_ERR_WORKSPACE; return nullptr; }
+  g_scratch_ptr[dev].store(p, std::memory_order_release);   // two threads racing here store the same address
+  return p;
+}
+
+extern "C" int mvllm_paged_decode_noalloc(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                          const int32_t* block_tables, int max_num_blocks, const void* context_lens,
+                                          int ctx_is_i64, int batch, int num_heads, int num_kv_heads, int head_dim,
+                                          int block_size, int64_t num_blocks, float scale, int dtype, void* stream) {
+  // arguments and sizes first, so that a bad call is refused before anything touches the device
+  int status = decode_check(out, q, k_cache, v_cache, nullptr, nullptr, false, block_tables, max_num_blocks,
+                            context_lens, batch, num_heads, num_kv_heads, head_dim, block_size, num_blocks, dtype);
+  if (status != MVLLM_OK || batch == 0) return status;
+  const size_t need = workspace_bytes_for(batch, num_heads, head_dim, max_num_blocks, block_size);
+  if (need > kStaticScratchBytes) return MVLLM_ERR_WORKSPACE;
+  void* ws = static_scratch(&status);
+  if (!ws) return status;
+  // Every partial a merge reads has been written by a workgroup of the same call (a sequence's live partitions
+  // all run), so nothing in the array has to start at zero.
+  return decode_entry(out, q, k_cache, v_cache, nullptr, nullptr, false, block_tables, max_num_blocks,
+                      context_lens, ctx_is_i64, batch, num_heads, num_kv_heads, head_dim, block_size,
+                      num_blocks, scale, dtype, ws, kStaticScratchBytes, stream);
 }
 
 extern "C" int mvllm_paged_decode_int8(void* out, const void* q, const int8_t* k_cache, const int8_t* v_cache,

@@ -27,7 +27,7 @@ def _lib():
 def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
-              "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_varlen",
+              "mvllm_paged_decode_int8", "mvllm_paged_decode_noalloc", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_varlen",
               "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_workspace_bytes",
               "mvllm_add_rms_norm",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
@@ -98,6 +98,9 @@ def test_argument_validation_without_gpu():
     assert lib.mvllm_store_kvcache(0, 0, 0, 0, 0, 0, 16, 2, 8, 1, 0) == 0       # empty is a no-op
     assert lib.mvllm_store_kvcache_int8(0, 0, 0, 0, 0, 0, 0, 4, 16, 2, 12, 1, 0) == -4   # D % 8 != 0
     assert lib.mvllm_paged_decode(0, 0, 0, 0, 0, 4, 0, 1, 2, 6, 4, 128, 16, 8, 1.0, 1, 0, 0, 0) == -3  # Hq % Hkv
+    noalloc = lib.mvllm_paged_decode_noalloc
+    assert noalloc(0, 0, 0, 0, 0, 4, 0, 1, 2, 6, 4, 128, 16, 8, 1.0, 1, 0) == -3                       # Hq % Hkv
+    assert noalloc(1, 1, 1, 1, 1, 2048, 1, 1, 256, 32, 8, 128, 16, 8, 1.0, 1, 0) == -5                 # beyond the static array: refused before any launch
     assert lib.mvllm_prefill_varlen(0, 0, 0, 0, 0, 0, 0, 4, 2, 128, 1.0, 1, 0) == 0      # empty batch
     assert lib.mvllm_prefill_varlen(0, 0, 0, 0, 0, 1, 5, 4, 2, 128, 1.0, 1, 0) == -1
     paged = lib.mvllm_prefill_paged
