@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,decode_small,demo_shape,fused_qk,sampler,engine,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,engine,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -46,12 +46,22 @@ def parse_args():
     return ap.parse_args()
 
 
-def time_steps(fn, steps, warmup):
+def time_steps(fn, steps, warmup, min_warm_ms=0.0):
     """W untimed calls, then K calls timed by wall clock (synchronised both sides) and by HIP events on the
-    current torch stream (the stream the kernels are launched on).  Returns (wall ms/step, event ms/step)."""
+    current torch stream (the stream the kernels are launched on).  Returns (wall ms/step, event ms/step).
+    min_warm_ms > 0 (the `extra` legs, never the headline): warm-up calls continue until that much wall time has
+    passed, because the GPU needs about 25 ms under load before its clock settles (a 0.2 ms kernel measured
+    after 5 warm-up launches is 15 % slower than in steady state)."""
     import torch
     for _ in range(warmup):
         fn()
+    if min_warm_ms > 0:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < min_warm_ms:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -62,6 +72,15 @@ def time_steps(fn, steps, warmup):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
     return wall, start.elapsed_time(stop) / steps
+
+
+EXTRA_WARM_MS = 50.0     # minimum warm-up of the legs under `extra` (the headline uses exactly --warmup steps)
+
+
+def roofline(bound, achieved, kernel):
+    """The same shape as the headline's `roofline` object, for a leg under `extra`."""
+    peak, unit = (HBM_PEAK_GBS, "GB/s") if bound == "hbm" else (MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
+    return {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak, "kernel": kernel}
 
 
 def decode_bytes(ctx, block_size, num_heads, num_kv_heads, head_dim, kv_elem, q_elem, ctx_elem, int8_scales=False):
@@ -132,6 +151,15 @@ def bench_decode(args, block_size, want_cpu):
         cpu_s = (time.perf_counter() - t0) / reps
         sub_bytes = decode_bytes(ccpu, block_size, hq, hkv, d, 2, 2, 8)
         got = step()[picked].float().cpu()
+        # the reference's second PyTorch path (decode_torch_optimized, benchmark_decoding.py:136-189) on the same sample
+        oracle.decode_vectorised_oracle(qcpu[:1], kcpu, vcpu, tcpu[:1], ccpu[:1], scale, hq, hkv, d, block_size)
+        vreps, t1 = 0, time.perf_counter()
+        while True:
+            ref2 = oracle.decode_vectorised_oracle(qcpu, kcpu, vcpu, tcpu, ccpu, scale, hq, hkv, d, block_size)
+            vreps += 1
+            if time.perf_counter() - t1 > 5.0 or vreps >= 60:
+                break
+        vec_s = (time.perf_counter() - t1) / vreps
         cpu = {
             "value": sub_bytes / cpu_s / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"oracle naive decode (fp32, torch-CPU) on the first {len(picked)} sequences of the same "
@@ -139,13 +167,36 @@ def bench_decode(args, block_size, want_cpu):
                       f"algorithmic bytes",
             "host_cpu_count": os.cpu_count(),
             "gpu_vs_oracle_max_abs": (got - ref).abs().max().item(),
+            "vectorised_oracle": {"value": sub_bytes / vec_s / 1e9, "unit": "GB/s", "reps": vreps,
+                                  "ms_each": vec_s * 1e3, "gpu_vs_oracle_max_abs": (got - ref2).abs().max().item()},
         }
     del kc, vc
     torch.cuda.empty_cache()
     return res, cpu
 
 
-def bench_prefill_store(args, which):
+def cpu_prefill_baseline(q, k, v, cu, lengths, scale, hq, hkv, d, flops, gpu_fn):
+    """The oracle's O(N^2) prefill (benchmark_prefilling.py:9-52 restated) on the whole config-2 batch on the host
+    cores, fp32, timed beside the GPU; also the value check of the GPU result at full size."""
+    import torch
+    import oracle
+    qc, kc, vc, cuc = q.float().cpu(), k.float().cpu(), v.float().cpu(), cu.cpu()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        ref = oracle.prefill_standard_oracle(qc, kc, vc, cuc, scale, hq, hkv, d)
+        reps += 1
+        if time.perf_counter() - t0 > 10.0 or reps >= 5:
+            break
+    cpu_s = (time.perf_counter() - t0) / reps
+    got = gpu_fn(q, k, v, cu, scale, hq, hkv, d).float().cpu()
+    err = (got - ref).abs()
+    return {"value": flops / cpu_s / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle O(N^2) prefill (fp32, torch-CPU) on the whole batch of {len(lengths)} prompts, "
+                      f"{reps} reps, {cpu_s:.2f} s each; causal flops only",
+            "gpu_vs_oracle_max_abs": err.max().item(), "gpu_vs_oracle_mean_abs": err.mean().item()}
+
+
+def bench_prefill_store(args, which, want_cpu=False):
     """BASELINE.json config 2: 16 prompts L~U[64,2048], Hq32/Hkv8/D128 bf16; store into a block-256 paged cache."""
     import torch
     from helpers import make_slot_mapping
@@ -167,14 +218,19 @@ def bench_prefill_store(args, which):
     if "prefill" in which:
         scale = 1.0 / math.sqrt(d)
         wall_ms, event_ms = time_steps(lambda: flash_attention_prefill(q, k, v, cu, scale, hq, hkv, d),
-                                       max(3, args.steps // 3), max(1, args.warmup // 2))
+                                       args.steps, args.warmup, EXTRA_WARM_MS)
         flops = 4 * hq * d * sum(n * (n + 1) // 2 for n in lengths)
         out["prefill"] = {
             "workload": "varlen causal prefill, 16 prompts L~U[64,2048], Hq32 Hkv8 D128 bf16",
             "tokens": total, "algorithmic_flops": flops, "ms_per_step": wall_ms, "event_ms_per_step": event_ms,
+            "steps": args.steps, "warmup": f"{args.warmup} launches, then at least {EXTRA_WARM_MS:.0f} ms of launches",
             "tflops": flops / (event_ms * 1e-3) / 1e12,
             "frac_of_bf16_mfma_peak": flops / (event_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+            "roofline": roofline("mfma", flops / (event_ms * 1e-3) / 1e12, "prefill_mfma_kernel (one launch = the whole ragged batch)"),
         }
+        if want_cpu:
+            out["prefill"]["cpu_baseline"] = cpu_prefill_baseline(q, k, v, cu, lengths, scale, hq, hkv, d, flops,
+                                                                  flash_attention_prefill)
     if "prefill" in which:
         # the same prompts with the first half (whole 16-token blocks) already cached: only the second half is
         # computed, every key comes from a block-16 paged cache
@@ -195,30 +251,48 @@ def bench_prefill_store(args, which):
         scale = 1.0 / math.sqrt(d)
         _, event_ms = time_steps(lambda: flash_attention_prefill_paged(q_new, kc16, vc16, bt, cu_q, cu, scale, hq, hkv,
                                                                        d, pbs),
-                                 max(3, args.steps // 3), max(1, args.warmup // 2))
+                                 args.steps, args.warmup, EXTRA_WARM_MS)
         flops = 4 * hq * d * sum((n - c) * c + (n - c) * (n - c + 1) // 2 for n, c in zip(lengths, cached))
         out["prefill_cached_prefix"] = {
             "workload": "same prompts, first half of each (whole blocks) cached: paged prefill of the rest, block_size 16",
             "new_tokens": int(cu_q[-1]), "algorithmic_flops": flops, "event_ms_per_step": event_ms,
             "tflops": flops / (event_ms * 1e-3) / 1e12,
             "frac_of_bf16_mfma_peak": flops / (event_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+            "roofline": roofline("mfma", flops / (event_ms * 1e-3) / 1e12, "prefill_mfma_kernel, paged mode"),
+        }
+        # ... and over an INT8 cache holding the same keys (codes + scales written by the INT8 store)
+        from minivllm_amd.layers.attention import flash_attention_prefill_paged_int8, store_kvcache_int8
+        ck8 = torch.zeros(nb16, pbs, hkv, d, dtype=torch.int8, device=dev)
+        cv8 = torch.zeros_like(ck8)
+        sk8 = torch.zeros(nb16, pbs, hkv, dtype=torch.float32, device=dev)
+        sv8 = torch.zeros_like(sk8)
+        store_kvcache_int8(k, v, ck8, cv8, sk8, sv8, slots16.to(dev), pbs)
+        _, event_ms8 = time_steps(lambda: flash_attention_prefill_paged_int8(q_new, ck8, cv8, sk8, sv8, bt, cu_q, cu,
+                                                                             scale, hq, hkv, d, pbs),
+                                  args.steps, args.warmup, EXTRA_WARM_MS)
+        out["prefill_cached_prefix_int8"] = {
+            "workload": "the same paged prefill over an INT8 cache (codes + fp32 scales per token and kv head), block_size 16",
+            "new_tokens": int(cu_q[-1]), "algorithmic_flops": flops, "event_ms_per_step": event_ms8,
+            "tflops": flops / (event_ms8 * 1e-3) / 1e12,
+            "roofline": roofline("mfma", flops / (event_ms8 * 1e-3) / 1e12, "mvllm_prefill_paged_int8"),
         }
     if "store" in which:
         slots, _, nb = make_slot_mapping(args.seed + 2, lengths, bs)
         kc = torch.zeros(nb, bs, hkv, d, dtype=torch.bfloat16, device=dev)
         vc = torch.zeros_like(kc)
         sl = slots.to(dev)
-        wall_ms, event_ms = time_steps(lambda: store_kvcache(k, v, kc, vc, sl, bs), args.steps, args.warmup)
+        wall_ms, event_ms = time_steps(lambda: store_kvcache(k, v, kc, vc, sl, bs), args.steps, args.warmup, EXTRA_WARM_MS)
         nbytes = 2 * total * hkv * d * (2 + 2) + 8 * total
         out["store"] = {
             "workload": "store_kvcache of the same batch into a block-256 bf16 cache, shuffled blocks",
             "tokens": total, "algorithmic_bytes": nbytes, "ms_per_step": wall_ms, "event_ms_per_step": event_ms,
             "gbs": nbytes / (event_ms * 1e-3) / 1e9,
+            "roofline": roofline("hbm", nbytes / (event_ms * 1e-3) / 1e9, "store_rows_kernel"),
         }
     return out
 
 
-def bench_int8(args):
+def bench_int8(args, want_cpu=True):
     """BASELINE.json config 4: B 128, ctx U[256,16384], Hq32/Hkv8/D128; K/V ~ N(0,1) with 1 % outliers at 8 sigma are
     quantised by store_kvcache_int8 into a block-16 int8 cache, then decoded with in-kernel dequantisation."""
     import torch
@@ -251,7 +325,8 @@ def bench_int8(args):
         v = torch.where(torch.rand(v.shape, generator=dg, device=dev) < 0.01, v * 8, v).to(torch.bfloat16)
         slots = torch.arange(lo, lo + n, device=dev)
         if lo == 0:
-            _, ms = time_steps(lambda: store_kvcache_int8(k, v, kc, vc, ks, vs, slots, bs), 10, 2)
+            _, ms = time_steps(lambda: store_kvcache_int8(k, v, kc, vc, ks, vs, slots, bs), args.steps, args.warmup,
+                               EXTRA_WARM_MS)
             store_ms.append(ms)
             store_bytes = 2 * n * hkv * d * (2 + 1) + 8 * n + 2 * n * hkv * 4
         store_kvcache_int8(k, v, kc, vc, ks, vs, slots, bs)
@@ -260,9 +335,27 @@ def bench_int8(args):
     scale = 1.0 / math.sqrt(d)
     wall_ms, event_ms = time_steps(
         lambda: paged_attention_decode_int8(q, kc, vc, ks, vs, td, cd, scale, hq, hkv, d, bs),
-        max(3, args.steps // 3), max(1, args.warmup // 2))
+        args.steps, args.warmup, EXTRA_WARM_MS)
     nbytes = decode_bytes(ctx, bs, hq, hkv, d, 1, 2, 8, int8_scales=True)
+    check = {}
+    if want_cpu:
+        # value check at full size on the launch plan of the full batch: the longest, the shortest and six more
+        # sequences against the INT8 oracle (dequantise in fp32, naive decode)
+        import oracle
+        got = paged_attention_decode_int8(q, kc, vc, ks, vs, td, cd, scale, hq, hkv, d, bs).float().cpu()
+        order = torch.argsort(ctx)
+        worst = 0.0
+        for b in sorted({int(order[0]), int(order[-1]), 0, 17, 42, 64, 99, 127}):
+            ids = tables[b, :need[b]].long().to(dev)
+            want = oracle.decode_int8_oracle(q[b:b + 1].float().cpu(), kc[ids].cpu(), vc[ids].cpu(), ks[ids].cpu(),
+                                             vs[ids].cpu(), torch.arange(need[b], dtype=torch.int32).unsqueeze(0),
+                                             ctx[b:b + 1], scale, hq, hkv, d, bs)
+            worst = max(worst, (got[b:b + 1] - want).abs().max().item())
+        check = {"gpu_vs_oracle_max_abs": worst, "oracle_sequences": 8}
     return {
+        **check,
+        "roofline": roofline("hbm", nbytes / (event_ms * 1e-3) / 1e9, "decode_mfma_int8_kernel + decode_reduce_kernel"),
+        "store_roofline": roofline("hbm", store_bytes / (store_ms[0] * 1e-3) / 1e9, "store_int8_kernel"),
         "workload": "INT8 KV cache: decode B128 ctx~U[256,16384] Hq32 Hkv8 D128 block_size 16, bf16 q",
         "tokens": int(ctx.sum()), "algorithmic_bytes": nbytes, "ms_per_step": wall_ms,
         "event_ms_per_step": event_ms, "gbs": nbytes / (event_ms * 1e-3) / 1e9,
@@ -306,14 +399,15 @@ def bench_fused_qk(args):
 
     fused = lambda: qk_norm_rope_store(q, k, v, pos, rotary.cos_sin_cache, gamma, 1e-6, sl, kc, vc)
     with torch.inference_mode():
-        _, fused_ms = time_steps(fused, args.steps, args.warmup)
-        _, unfused_ms = time_steps(unfused, max(3, args.steps // 3), max(1, args.warmup // 2))
+        _, fused_ms = time_steps(fused, args.steps, args.warmup, EXTRA_WARM_MS)
+        _, unfused_ms = time_steps(unfused, args.steps, args.warmup, EXTRA_WARM_MS)
     # read q, k, v once; write q_out, k_out, v_out and the two cache rows; per token: position, slot, table row
     nbytes = total * ((hq + 2 * hkv) * d * 2 * 2 + 2 * hkv * d * 2 + 8 + 8 + d * 4)
     return {
         "workload": "q/k RMSNorm + rotary + store_kvcache on the config-2 prefill batch, Hq32 Hkv8 D128 bf16, block 256",
         "tokens": total, "algorithmic_bytes": nbytes, "event_ms_per_step": fused_ms,
         "gbs": nbytes / (fused_ms * 1e-3) / 1e9, "unfused_modules_event_ms": unfused_ms,
+        "roofline": roofline("hbm", nbytes / (fused_ms * 1e-3) / 1e9, "qk_norm_rope_store_kernel"),
     }
 
 
@@ -330,8 +424,8 @@ def bench_sampler(args):
     logits = (torch.randn(batch, vocab, generator=dg, device=dev) * 2).to(torch.bfloat16)
     temps = torch.full((batch,), 0.6, device=dev)
     sampler = Sampler()
-    _, fused_ms = time_steps(lambda: sample_tokens(logits, temps, 0, 0), args.steps, args.warmup)
-    _, modules_ms = time_steps(lambda: sampler(logits, temps, dg), max(3, args.steps // 3), max(1, args.warmup // 2))
+    _, fused_ms = time_steps(lambda: sample_tokens(logits, temps, 0, 0), args.steps, args.warmup, EXTRA_WARM_MS)
+    _, modules_ms = time_steps(lambda: sampler(logits, temps, dg), args.steps, args.warmup, EXTRA_WARM_MS)
     nbytes = batch * vocab * 2 + batch * 12
     return {"workload": "sampler: 64 x 151936 bf16 logits, T 0.6", "algorithmic_bytes": nbytes,
             "event_ms_per_step": fused_ms, "gbs": nbytes / (fused_ms * 1e-3) / 1e9, "unfused_modules_event_ms": modules_ms}
@@ -367,7 +461,7 @@ def bench_decode_small(args):
         with torch.cuda.graph(g):
             for _ in range(calls):
                 fn()
-        _, ms = time_steps(g.replay, max(5, args.steps // 3), 2)
+        _, ms = time_steps(g.replay, args.steps, 2, EXTRA_WARM_MS)
         return ms * 1e3 / calls
 
     us16 = graph_us(lambda: paged_attention_decode(q, kc, vc, td, cd, scale, hq, hkv, d, bs))
@@ -398,16 +492,140 @@ def bench_demo_shape(args):
                                                            log_uniform=False)
         td, cd = tables.to(dev), ctx.to(dev)
         _, ms = time_steps(lambda: paged_attention_decode(q, kc, vc, td, cd, 1 / math.sqrt(d), hq, hkv, d, bs),
-                           args.steps, args.warmup)
+                           args.steps, args.warmup, EXTRA_WARM_MS)
         nbytes = int(ctx.sum()) * hkv * d * 2 * kc.element_size()
         out[f"decode_{name}_us"] = ms * 1e3
         out[f"decode_{name}_gbs"] = nbytes / (ms * 1e-3) / 1e9
         qq, kk, vv, cu = (t.to(dev) for t in make_varlen_case(args.seed + 1, lengths, hq, hkv, d, dtype=dtype))
         _, ms = time_steps(lambda: flash_attention_prefill(qq, kk, vv, cu, 1 / math.sqrt(d), hq, hkv, d),
-                           max(3, args.steps // 3), max(1, args.warmup // 2))
+                           args.steps, args.warmup, EXTRA_WARM_MS)
         out[f"prefill_{name}_ms"] = ms
         out[f"prefill_{name}_tflops"] = flops / (ms * 1e-3) / 1e12
     return out
+
+
+def bench_reference_shapes(args, want_cpu):
+    """The shapes the reference's own benchmark scripts run (fp16, 32 query / 8 kv heads of 128 dims, block 16,
+    identity block tables, every context the same length): decode (B, L) = (2,60) (1,512) (16,256) (4,2048)
+    (benchmark_decoding.py:298-374) and prefill (seqs, L) = (2,60) (4,64) (2,1024) (1,4096)
+    (benchmark_prefilling.py:427-495).  GPU time per call inside a hipGraph of 20 calls (these calls are latency,
+    not bandwidth), the CPU oracle beside it (the PyTorch functions those scripts time, restated), and the
+    difference between the two results."""
+    import torch
+    import oracle
+    from minivllm_amd.layers.attention import flash_attention_prefill, paged_attention_decode
+
+    dev = "cuda:0"
+    hq, hkv, d, bs = 32, 8, 128, 16
+    scale = 1.0 / math.sqrt(d)
+    calls = 20
+
+    def graph_us(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(calls):
+                fn()
+        _, ms = time_steps(g.replay, args.steps, 2, EXTRA_WARM_MS)
+        return ms * 1e3 / calls
+
+    def cpu_ms(fn, budget_s=2.0):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            ref = fn()
+            reps += 1
+            if time.perf_counter() - t0 > budget_s or reps >= 50:
+                return (time.perf_counter() - t0) / reps * 1e3, ref
+
+    rows = {"decode": [], "prefill": []}
+    gen = torch.Generator().manual_seed(args.seed)
+    for batch, length in ((2, 60), (1, 512), (16, 256), (4, 2048)):
+        mb = -(-length // bs)
+        q = torch.randn(batch, hq, d, generator=gen).to(torch.float16)
+        kc = torch.randn(batch * mb, bs, hkv, d, generator=gen).to(torch.float16)
+        vc = torch.randn(batch * mb, bs, hkv, d, generator=gen).to(torch.float16)
+        tables = torch.arange(batch * mb, dtype=torch.int32).reshape(batch, mb)
+        ctx = torch.full((batch,), length, dtype=torch.int32)
+        qd, kd, vd, td, cd = (t.to(dev) for t in (q, kc, vc, tables, ctx))
+        us = graph_us(lambda: paged_attention_decode(qd, kd, vd, td, cd, scale, hq, hkv, d, bs))
+        row = {"batch": batch, "context": length, "gpu_us_per_call": us}
+        if want_cpu:
+            got = paged_attention_decode(qd, kd, vd, td, cd, scale, hq, hkv, d, bs).float().cpu()
+            args32 = (q.float(), kc.float(), vc.float(), tables, ctx, scale, hq, hkv, d, bs)
+            row["cpu_naive_ms"], ref = cpu_ms(lambda: oracle.decode_naive_oracle(*args32))
+            row["cpu_vectorised_ms"], _ = cpu_ms(lambda: oracle.decode_vectorised_oracle(*args32))
+            row["gpu_vs_oracle_max_abs"] = (got - ref).abs().max().item()
+        rows["decode"].append(row)
+    for seqs, length in ((2, 60), (4, 64), (2, 1024), (1, 4096)):
+        total = seqs * length
+        q = torch.randn(total, hq, d, generator=gen).to(torch.float16)
+        k = torch.randn(total, hkv, d, generator=gen).to(torch.float16)
+        v = torch.randn(total, hkv, d, generator=gen).to(torch.float16)
+        cu = torch.arange(seqs + 1, dtype=torch.int32) * length
+        qd, kd, vd, cud = (t.to(dev) for t in (q, k, v, cu))
+        us = graph_us(lambda: flash_attention_prefill(qd, kd, vd, cud, scale, hq, hkv, d))
+        flops = 4 * hq * d * seqs * length * (length + 1) // 2
+        row = {"seqs": seqs, "length": length, "gpu_us_per_call": us, "gpu_tflops": flops / (us * 1e-6) / 1e12}
+        if want_cpu:
+            got = flash_attention_prefill(qd, kd, vd, cud, scale, hq, hkv, d).float().cpu()
+            row["cpu_standard_ms"], ref = cpu_ms(lambda: oracle.prefill_standard_oracle(q.float(), k.float(), v.float(), cu,
+                                                                                        scale, hq, hkv, d))
+            row["gpu_vs_oracle_max_abs"] = (got - ref).abs().max().item()
+        rows["prefill"].append(row)
+    rows["workload"] = ("the reference benchmark scripts' shapes: fp16, Hq32 Hkv8 D128, block_size 16, equal lengths; "
+                        f"GPU: {calls} calls per hipGraph replay; CPU: the oracle (fp32) on {torch.get_num_threads()} threads")
+    return rows
+
+
+def bench_mfma_probe(args):
+    """What the matrix unit sustains on this GPU (libmvllm_probe.so, csrc/mfma_probe.hip): register-only loops of
+    v_mfma_f32_32x32x16_bf16 alone, with n v_fma_f32 (+ one v_exp_f32) issued after every MFMA by the same wave, and
+    with the vector instructions on a second wave of the same SIMD.  The prefill tile body is 32 MFMAs and about 4
+    other vector instructions + 1 exp per MFMA; these loops give its ceiling at the clock the GPU holds under that
+    load.  Reported per mix: TFLOP/s of the MFMAs and the fraction of the 2.5 PFLOP/s data-sheet peak."""
+    import ctypes
+    import torch
+    lib = ctypes.CDLL(os.path.join(ROOT, "minivllm_amd", "libmvllm_probe.so"))
+    fn = lib.mvllm_probe_mfma_mix
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+    out = torch.zeros(16, device="cuda:0")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    iters = 100000
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run(nv, ne, role, wps, per_cu=1):
+        blocks = cus * per_cu
+
+        def launch():
+            st = fn(nv, ne, role, wps, blocks, out.data_ptr(), iters, stream)
+            assert st == 0, st
+        _, ms = time_steps(launch, 3, 1)
+        torch.cuda.synchronize()
+        clocks, ticks = out[1].item(), out[2].item()        # wave 0: shader clocks and 100 MHz ticks inside its loop
+        mfma_waves = blocks * 4 * (1 if role == 1 else wps)
+        flops = 0 if role == 2 else mfma_waves * iters * 4 * 32 * 32 * 16 * 2
+        slots = blocks * 4 * wps * iters * 4 if role != 1 else blocks * 4 * iters * 4
+        return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "frac_of_peak": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                "shader_ghz": clocks / (ticks * 10.0) if ticks else None,
+                # an MFMA alone is 32 clocks: 13.3 ns at 2.4 GHz
+                "ns_per_slot_per_simd": ms * 1e6 / (slots / (cus * 4)),
+                "clocks_per_slot_wave0": clocks / (iters * 4)}
+
+    res = {"workload": f"register-only loops, {cus} CUs, {iters} iterations x 4 slots per wave; slot = 1 MFMA 32x32x16 bf16 + "
+                       "nv v_fma_f32 + ne v_exp_f32", "mixes": {}}
+    for wps in (1, 2):
+        res["mixes"][f"mfma_only_{wps}wave_per_simd"] = run(0, 0, 0, wps)
+    for nv, ne in ((2, 0), (4, 0), (6, 0), (8, 0), (0, 1), (3, 1), (4, 1)):
+        res["mixes"][f"same_wave_nv{nv}_ne{ne}_2waves_per_simd"] = run(nv, ne, 0, 2)
+    res["mixes"]["same_wave_nv4_ne1_1wave_per_simd"] = run(4, 1, 0, 1)
+    for nv, ne in ((4, 0), (8, 0), (4, 1)):
+        res["mixes"][f"other_wave_nv{nv}_ne{ne}"] = run(nv, ne, 1, 2)
+        res["mixes"][f"vector_only_nv{nv}_ne{ne}_1wave_per_simd"] = run(nv, ne, 2, 1)
+    return res
 
 
 def bench_engine(args, max_num_sequences, graph):
@@ -472,11 +690,14 @@ def main():
     head, cpu = bench_decode(args, args.block_size, want_cpu=not args.no_cpu and want("cpu"))
     if want("decode256") and args.block_size != 256:
         extra["decode_block256"], _ = bench_decode(args, 256, want_cpu=False)
+    want_cpu = not args.no_cpu and want("cpu")
     which = [n for n in ("prefill", "store") if want(n)]
     if which:
-        extra.update(bench_prefill_store(args, which))
+        extra.update(bench_prefill_store(args, which, want_cpu))
     if want("int8"):
-        extra["int8"] = bench_int8(args)
+        extra["int8"] = bench_int8(args, want_cpu)
+    if want("reference_shapes"):
+        extra["reference_benchmark_shapes"] = bench_reference_shapes(args, want_cpu)
     if want("decode_small"):
         extra["decode_small_batch"] = bench_decode_small(args)
     if want("demo_shape"):
@@ -485,6 +706,8 @@ def main():
         extra["fused_qk"] = bench_fused_qk(args)
     if want("sampler"):
         extra["sampler"] = bench_sampler(args)
+    if want("mfma_probe"):
+        extra["mfma_probe"] = bench_mfma_probe(args)
     if want("engine"):
         extra["engine_16seq_eager"] = bench_engine(args, 16, False)
         extra["engine_16seq_graph"] = bench_engine(args, 16, True)
@@ -511,6 +734,8 @@ def main():
             "unit": "GB/s",
             "frac": head["gbs_event"] / HBM_PEAK_GBS,
             "traffic": DECODE_TRAFFIC_BYTES_DEFAULT if (args.seed == 0 and args.block_size == 16) else None,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload summarised in "
+                              "profiles/bench_hbm_traffic_pmc.txt (a counter run cannot time; not re-measured in this run)",
             "kernel": "decode_mfma_kernel + decode_reduce_kernel (one decode call, HIP events on the launch stream)",
         },
         "cpu_baseline": cpu,

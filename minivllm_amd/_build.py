@@ -14,6 +14,8 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libminivllm_amd.so")
+PROBE_LIB_PATH = os.path.join(PKG_DIR, "libmvllm_probe.so")      # measurement support for bench.py, not an operator
+PROBE_SOURCES = ["mfma_probe.hip"]
 SOURCES = ["capi.hip", "store_kvcache.hip", "paged_decode.hip", "prefill_varlen.hip", "qk_norm_rope_store.hip", "sampler.hip",
            "rms_norm.hip", "activation.hip"]
 
@@ -55,13 +57,14 @@ def build_library(verbose: bool = True, jobs: int = 4) -> str:
         return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(compile_one, SOURCES))
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"link failed:\n{res.stderr}")
+        objs = list(pool.map(compile_one, SOURCES + PROBE_SOURCES))
+    for lib, members in ((LIB_PATH, objs[:len(SOURCES)]), (PROBE_LIB_PATH, objs[len(SOURCES):])):
+        cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *members]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"link failed:\n{res.stderr}")
     return LIB_PATH
 
 

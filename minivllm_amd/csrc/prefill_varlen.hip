@@ -147,6 +147,12 @@ typedef __attribute__((ext_vector_type(2))) _Float16 v2f16;
 #define MVLLM_PF_XCD_CHUNK 32
 #endif
 constexpr unsigned kXcdChunk = MVLLM_PF_XCD_CHUNK;   // consecutive work items handed to one XCD
+#ifndef MVLLM_PF_BAND_ROWS
+#define MVLLM_PF_BAND_ROWS 256        // rows per band of the heaviest-first item order (a multiple of 128)
+#endif
+#ifndef MVLLM_PF_PIN_KREADS
+#define MVLLM_PF_PIN_KREADS 1
+#endif
 #ifndef MVLLM_PF_WAVES
 #define MVLLM_PF_WAVES 4
 #endif
@@ -162,6 +168,13 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
+}
+
+// max(x[l], x[l ^ 32]) in every lane l, by v_permlane32_swap.
+__device__ __forceinline__ float max_with_lane_xor32(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  // r[0] = (x[0..31], x[0..31]), r[1] = (x[32..63], x[32..63]): their maximum is max(x[l], x[l ^ 32]) in every lane
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
 // Compile-time loop: f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{}).
@@ -182,6 +195,21 @@ template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) 
 template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
   v2f x = {a, b};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, v2f16));
+}
+
+// (lo, hi) of a packed 16-bit pair, each multiplied by c and rounded back to the element type.
+template <typename T> __device__ __forceinline__ uint32_t scale_pair(uint32_t w, float c) {
+  return pack2<T>(lo_to_float<T>(w) * c, hi_to_float<T>(w) * c);
+}
+// acc + lo + hi of a packed 16-bit pair in one instruction (v_dot2_f32_bf16 / v_dot2_f32_f16 against (1, 1)).
+template <typename T> __device__ __forceinline__ float add_pair(uint32_t w, float acc);
+template <> __device__ __forceinline__ float add_pair<bf16_t>(uint32_t w, float acc) {
+  const v2bf16 ones = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf16, w), ones, acc, false);
+}
+template <> __device__ __forceinline__ float add_pair<f16_t>(uint32_t w, float acc) {
+  const v2f16 ones = {(_Float16)1.0f, (_Float16)1.0f};
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2f16, w), ones, acc, false);
 }
 
 // 16 bytes per lane from a buffer resource (wave-uniform descriptor + per-lane 32-bit byte offset) straight
@@ -210,6 +238,66 @@ __device__ __forceinline__ v4i make_rsrc(const char* base, uint32_t bytes) {
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+
+// Work item -> (head slice, sequence, first row) for batches of at most 64 sequences, heaviest items first.
+// A query tile's cost grows with its position in the sequence (causal: tile t walks t + 1 key tiles), so the items
+// are dealt in bands of kBandRows rows: band b of a sequence is its row tiles [b R, b R + R), R = kBandRows / BM.  The order is
+// band level descending (every sequence's last band comes before anybody's band below it), inside a level head
+// slice, then sequence, then the band's R tiles from the last (heaviest) down.  The launch then ends with the
+// level-0 bands of all sequences, whose items take a few key tiles each, instead of with whatever rows the last
+// sequence in memory order has: with 16 prompts of 64-2048 tokens the launch used to end with a single prompt's
+// 60-tile items running alone.  Consecutive items still share a sequence's keys (R tiles of one band, and
+// neighbouring bands of the same level), which keeps them in one XCD's L2.  Bands past a sequence's last tile are
+// padding: those workgroups return at once (at most R - 1 per sequence and head slice).
+// Every lane of the calling wave must be active; all lanes return the same values.
+constexpr int kBandRows = MVLLM_PF_BAND_ROWS;
+template <int BM>
+__device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, int num_seqs, unsigned item, int heads_y,
+                                              int& seq_start, int& seq_len, int& row0, int& seq_index, int& item_y) {
+  constexpr int R = kBandRows / BM;
+  const int lane = threadIdx.x & 63;
+  int lo = 0, len = 0;
+  if (lane < num_seqs) {
+    lo = cu[lane];
+    len = cu[lane + 1] - lo;
+  }
+  const int n = (len + BM - 1) / BM;            // row tiles of the lane's sequence
+  const int nb = (n + R - 1) / R;               // ... and bands
+  // highest band level in the batch: bit by bit from the top (lengths are below 2^30, bands below 2^23)
+  int top = 0;
+  for (int bit = 22; bit >= 0; --bit) {
+    const int trial = top | (1 << bit);
+    if (__ballot(nb >= trial) != 0ull) top = trial;
+  }
+  // walk the levels down from the top one until the item's level is found
+  unsigned base = 0;
+  int b = top - 1;
+  unsigned long long mask = 0ull;
+  unsigned per_y = 0;
+  for (; b >= 0; --b) {
+    mask = __ballot(nb > b);
+    per_y = (unsigned)__popcll(mask) * (unsigned)R;
+    const unsigned items = per_y * (unsigned)heads_y;
+    if (item - base < items) break;
+    base += items;
+  }
+  if (b < 0) return false;                      // past the last item: grid padding
+  const unsigned idx = item - base;
+  item_y = (int)(idx / per_y);
+  const unsigned rem = idx - (unsigned)item_y * per_y;
+  const int q = (int)(rem / (unsigned)R), r = (int)(rem % (unsigned)R);
+  // the q-th sequence of this level = the lane whose bit is set with q set bits below it
+  const int below = __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+  const unsigned long long pick = __ballot(((mask >> lane) & 1ull) != 0ull && below == q);
+  const int owner = __ffsll((long long)pick) - 1;
+  const int t = b * R + (R - 1 - r);            // row tile inside the sequence, last tile of the band first
+  if (t >= __shfl(n, owner, 64)) return false;  // the band's padding
+  seq_start = __shfl(lo, owner, 64);
+  seq_len = __shfl(len, owner, 64);
+  row0 = t * BM;
+  seq_index = owner;
+  return true;
 }
 
 // D = 128 or 64.  A row of a tile is D*2 bytes = kChunks 16-byte chunks; one copy instruction moves 1 KB = kCopyRows
@@ -244,12 +332,17 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   // a long sequence over all XCDs instead of always handing them to the same one
   const unsigned round = slot / kXcdChunk;
   const unsigned item = (round * 8 + ((xcd + round) & 7)) * kXcdChunk + slot % kXcdChunk;
-  if (item >= (unsigned)tiles_x * (unsigned)a.heads_y) return;
-  const int item_y = (int)(item / (unsigned)tiles_x);
-  const int item_x = (int)(item % (unsigned)tiles_x);
-  int seq_start, seq_len, row0, seq_index;
-  // latest (heaviest) tiles of a sequence first
-  if (!locate_tile(a.cu_seqlens, a.num_seqs, tiles_x - 1 - item_x, BM, seq_start, seq_len, row0, seq_index)) return;
+  int item_y, seq_start, seq_len, row0, seq_index;
+  if (a.num_seqs <= 64) {
+    if (!locate_banded<BM>(a.cu_seqlens, a.num_seqs, item, a.heads_y, seq_start, seq_len, row0, seq_index, item_y)) return;
+  } else {
+    // more sequences than one wave holds: memory order, inside a sequence the latest (heaviest) tiles first
+    if (item >= (unsigned)tiles_x * (unsigned)a.heads_y) return;
+    item_y = (int)(item / (unsigned)tiles_x);
+    const int item_x = (int)(item % (unsigned)tiles_x);
+    if (!locate_tile(a.cu_seqlens, a.num_seqs, tiles_x - 1 - item_x, BM, seq_start, seq_len, row0, seq_index)) return;
+  }
+  item_y = __builtin_amdgcn_readfirstlane(item_y);
   // Wave-uniform by construction; say so, so that everything derived from them (tile counts, loop bounds,
   // tile base addresses, branches) lives in scalar registers and runs on the scalar unit.
   seq_start = __builtin_amdgcn_readfirstlane(seq_start);
@@ -384,6 +477,16 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     const T* src = q + (tok * a.num_heads + h) * D + 8 * hi;
 #pragma unroll
     for (int ks = 0; ks < kKS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
+    // The softmax scale (times log2 e) goes into Q once, rounded to the element type, so that the scores leave
+    // the matrix unit as exp2 arguments: the tile loop has no multiply per score.  This runs while the first K/V
+    // tile is still on its way.
+#pragma unroll
+    for (int ks = 0; ks < kKS; ++ks) {
+      qf[ks].x = scale_pair<T>(qf[ks].x, a.scale_log2);
+      qf[ks].y = scale_pair<T>(qf[ks].y, a.scale_log2);
+      qf[ks].z = scale_pair<T>(qf[ks].z, a.scale_log2);
+      qf[ks].w = scale_pair<T>(qf[ks].w, a.scale_log2);
+    }
   }
   // Make the compiler retire the Q loads here: otherwise it carries "Q may still be in flight" into
   // the loop and its vmcnt waits there would also wait for the tile prefetch.
@@ -395,7 +498,14 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   for (int td = 0; td < kTD; ++td)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[td][r] = 0.f;
-  float m = -INFINITY;
+  // Running maximum of the lane's query row, kept negated in all 16 registers of an accumulator tuple: the score
+  // products start from it (C operand of their first MFMA), so a tile's scores arrive as  s * scale * log2 e - m,
+  // ready for exp2.  It only changes when a tile's maximum exceeds it by more than 2^8 (lazy rescale), which
+  // is rare after a row's first tile.
+  v16f neg_m;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) neg_m[r] = 0.f;
+  bool first = true;                                 // no tile seen yet: the maximum is still the placeholder 0
   float l = 0.f;
 
   // Per-lane LDS byte offsets, computed once: the xor swizzle keeps the compiler from folding them into
@@ -431,16 +541,22 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     v16f s[NH];
     const char* kb = &lds.k[buf][0];
     {
-      const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      // K fragments are read one step ahead of the MFMAs that use them.  The reads of step ks + 1 stand in front
+      // of step ks's copy instruction on purpose: the copy is an asm statement, which no LDS read is moved
+      // across, so reads placed after it would be issued right before their use and wait out the LDS latency.
+      uint4 kf[2][NH];
 #pragma unroll
-      for (int tk = 0; tk < NH; ++tk) s[tk] = zero;
+      for (int tk = 0; tk < NH; ++tk) kf[0][tk] = *reinterpret_cast<const uint4*>(kb + k_off[0] + tk * 32 * kRowB);
       static_for<kKS>([&](auto KS) {
         constexpr int ks = decltype(KS)::value;
-        uint4 kf[NH];
+        if constexpr (ks + 1 < kKS) {
 #pragma unroll
-        for (int tk = 0; tk < NH; ++tk) kf[tk] = *reinterpret_cast<const uint4*>(kb + k_off[ks] + tk * 32 * kRowB);
+          for (int tk = 0; tk < NH; ++tk)
+            kf[(ks + 1) & 1][tk] = *reinterpret_cast<const uint4*>(kb + k_off[ks + 1] + tk * 32 * kRowB);
+          if (MVLLM_PF_PIN_KREADS) __builtin_amdgcn_sched_barrier(0);   // keep the reads in front of this step's MFMAs
+        }
 #pragma unroll
-        for (int tk = 0; tk < NH; ++tk) s[tk] = mfma32x32x16<T>(kf[tk], qf[ks], s[tk]);
+        for (int tk = 0; tk < NH; ++tk) s[tk] = mfma32x32x16<T>(kf[ks & 1][tk], qf[ks], ks == 0 ? neg_m : s[tk]);
         if constexpr (ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);           // copies of the next tile, K first
       });
     }
@@ -459,37 +575,48 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     // distance an MFMA result needs before a vector instruction may read it only for instructions it knows,
     // not for the v_max3 asm, and every max3 below depends on this first value (MFMAs finish in issue order,
     // so once the last instruction of a chain has delivered, the chain's other registers are final too).
-    float mx = fmaxf(s[0][15], s[NH - 1][15]);
-#pragma unroll
-    for (int r = 0; r < 14; r += 2) mx = max3(mx, s[0][r], s[0][r + 1]);
+    // Two chains, one per half, so that the dependent maxima are half as deep; both start from mx0.
+    const float mx0 = fmaxf(s[0][15], s[NH - 1][15]);
+    float mx = mx0;
     if constexpr (NH == 2) {
-      mx = max3(mx, s[0][14], s[1][14]);
+      float mx1 = mx0;
 #pragma unroll
-      for (int r = 0; r < 14; r += 2) mx = max3(mx, s[1][r], s[1][r + 1]);
+      for (int r = 0; r < 14; r += 2) {
+        mx = max3(mx, s[0][r], s[0][r + 1]);
+        mx1 = max3(mx1, s[1][r], s[1][r + 1]);
+      }
+      mx = max3(mx, s[0][14], s[1][14]);
+      mx = fmaxf(mx, mx1);
     } else {
-      mx = max3(mx, s[0][14], s[0][14]);
+#pragma unroll
+      for (int r = 0; r < 14; r += 2) mx = max3(mx, s[0][r], s[0][r + 1]);
+      mx = fmaxf(mx, s[0][14]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * a.scale_log2;
-    const bool grow = mx > m + 8.f || m == -INFINITY;
+    // the other half of the row's keys sits in lane l ^ 32: exchange on the vector unit (no LDS round trip, and
+    // no wait behind the fragment reads queued there)
+    mx = max_with_lane_xor32(mx);                      // tile maximum of the row, relative to the running one
+    const bool grow = first || mx > 8.f;
     if (__any(grow)) {
-      const float m_new = grow ? mx : m;
-      const float alpha = (m_new == m) ? 1.f : fast_exp2(m - m_new);   // exp2(-inf) = 0 on the first tile
+      const float d = grow ? mx : 0.f;                 // the running maximum moves up by d (any finite d on the first tile)
+      const float alpha = first ? 1.f : fast_exp2(-d); // nothing is accumulated yet on the first tile
       l *= alpha;
 #pragma unroll
       for (int td = 0; td < kTD; ++td)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[td][r] *= alpha;
-      m = m_new;
+      const float nm = neg_m[0] - d;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) neg_m[r] = nm;
+#pragma unroll
+      for (int tk = 0; tk < NH; ++tk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[tk][r] -= d;
+      first = false;
     }
-    const float neg_m = -m;
 #pragma unroll
     for (int tk = 0; tk < NH; ++tk)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float pv = fast_exp2(fmaf(s[tk][r], a.scale_log2, neg_m));
-        s[tk][r] = pv;
-        l += pv;      // partial: this lane's kv rows only; lanes l and l^32 are added at the end
-      }
+      for (int r = 0; r < 16; ++r) s[tk][r] = fast_exp2(s[tk][r]);
 
     // ---- O^T += V^T P^T ----
     const char* vb = &lds.v[buf][0];
@@ -500,6 +627,9 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
       pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
       pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
+      // row sum from the rounded weights, the ones the numerator uses; partial: this lane's kv rows only
+      // (lanes l and l^32 are added at the end)
+      l = add_pair<T>(pf.w, add_pair<T>(pf.z, add_pair<T>(pf.y, add_pair<T>(pf.x, l))));
       uint4 af[kTD];
 #pragma unroll
       for (int td = 0; td < kTD; ++td) {
@@ -597,7 +727,10 @@ static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   const int hpw = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
   const int bm = kWaveRows * (kPfWaves / hpw);
   PrefillArgs b = a;
-  b.tiles_x = (int)(a.total_tokens / bm + a.num_seqs);
+  // upper bound on the query tiles: every sequence may end with a partial tile; in the banded order (at most 64
+  // sequences) every sequence may also end with a partial band of kBandRows / bm tiles
+  b.tiles_x = a.num_seqs <= 64 ? (int)(a.total_tokens / bm + (int64_t)a.num_seqs * (kBandRows / bm))
+                               : (int)(a.total_tokens / bm + a.num_seqs);
   b.heads_y = a.num_kv_heads * (group / hpw);
   const int64_t items = (int64_t)b.tiles_x * b.heads_y;
   const int64_t span = 8 * (int64_t)kXcdChunk;

@@ -66,6 +66,36 @@ def test_prefill_zero_length_sequences_and_independence():
     assert torch.equal(got[:70], got2[:70])
 
 
+@pytest.mark.parametrize("hq,hkv", [(4, 1), (4, 2), (3, 3)])        # 4, 2 and 1 query heads of a kv head per workgroup
+@pytest.mark.parametrize("num_seqs", [64, 65, 130])
+def test_prefill_item_order_covers_every_tile(hq, hkv, num_seqs):
+    """Up to 64 sequences the workgroups take their (sequence, row tile) from the heaviest-first banded order, beyond
+    that from the plain one.  Ragged lengths around the band and tile boundaries (0, 1, 31..33, 255..257, 511..513,
+    700) in a shuffled order: every row of every sequence must come out right, so no tile is skipped or doubled."""
+    d = 128
+    g = torch.Generator().manual_seed(500 + num_seqs)
+    pool = [0, 1, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 700]
+    lengths = [pool[i] for i in torch.randint(0, len(pool), (num_seqs,), generator=g).tolist()]
+    lengths[num_seqs // 2] = 700
+    lengths[-1] = 257
+    q, k, v, cu = make_varlen_case(53, lengths, hq, hkv, d, dtype=torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    poison = torch.full_like(q, float("nan"))                       # a skipped tile would leave its rows untouched
+    from minivllm_amd import _C
+    out = poison.to(DEV)
+    qd, kd, vd, cud = (t.to(DEV) for t in (q, k, v, cu))
+    st = _C.load().mvllm_prefill_varlen(out.data_ptr(), qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), cud.data_ptr(),
+                                        num_seqs, q.shape[0], hq, hkv, d, scale, _C.dtype_code(q.dtype),
+                                        _C.current_stream_ptr(out.device))
+    torch.cuda.synchronize()
+    assert st == 0
+    got = out.cpu()
+    assert torch.isfinite(got).all()
+    want = _oracle32(q, k, v, cu, scale, hq, hkv, d)
+    mx, mean = error_stats(got, want)
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
 def test_config2_full_size():
     """BASELINE.json config 2: 16 prompts L U[64,2048], Hq32/Hkv8/D128 bf16; store into block-256 cache; the last
     row of each prompt must agree with a paged decode of that token over the stored cache."""
