@@ -25,6 +25,7 @@ struct PrefillArgs {
   float scale_log2;
   int tiles_x;      // MFMA path: query-tile upper bound (total_tokens / BM + num_seqs)
   int heads_y;      // MFMA path: head slices (kv heads x query-head chunks)
+  int band_bits;    // MFMA path: bits that hold the band count of the longest possible sequence (total_tokens / kBandRows + 1)
   // Paged mode (k, v are caches [num_blocks, block_size, Hkv, D]; q holds only the tokens after each
   // sequence's cached prefix): cu_seqlens counts the query rows, cu_seqlens_k the keys (prefix + new).
   const int32_t* cu_seqlens_k;
@@ -254,7 +255,7 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 constexpr int kBandRows = MVLLM_PF_BAND_ROWS;
 template <int BM>
 __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, int num_seqs, unsigned item, int heads_y,
-                                              int& seq_start, int& seq_len, int& row0, int& seq_index, int& item_y) {
+                                              int band_bits, int& seq_start, int& seq_len, int& row0, int& seq_index, int& item_y) {
   constexpr int R = kBandRows / BM;
   const int lane = threadIdx.x & 63;
   int lo = 0, len = 0;
@@ -264,9 +265,9 @@ __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, in
   }
   const int n = (len + BM - 1) / BM;            // row tiles of the lane's sequence
   const int nb = (n + R - 1) / R;               // ... and bands
-  // highest band level in the batch: bit by bit from the top (lengths are below 2^30, bands below 2^23)
+  // highest band level in the batch: bit by bit from the top (band_bits: the host's bound from the token count)
   int top = 0;
-  for (int bit = 22; bit >= 0; --bit) {
+  for (int bit = band_bits - 1; bit >= 0; --bit) {
     const int trial = top | (1 << bit);
     if (__ballot(nb >= trial) != 0ull) top = trial;
   }
@@ -334,7 +335,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   const unsigned item = (round * 8 + ((xcd + round) & 7)) * kXcdChunk + slot % kXcdChunk;
   int item_y, seq_start, seq_len, row0, seq_index;
   if (a.num_seqs <= 64) {
-    if (!locate_banded<BM>(a.cu_seqlens, a.num_seqs, item, a.heads_y, seq_start, seq_len, row0, seq_index, item_y)) return;
+    if (!locate_banded<BM>(a.cu_seqlens, a.num_seqs, item, a.heads_y, a.band_bits, seq_start, seq_len, row0, seq_index, item_y)) return;
   } else {
     // more sequences than one wave holds: memory order, inside a sequence the latest (heaviest) tiles first
     if (item >= (unsigned)tiles_x * (unsigned)a.heads_y) return;
@@ -732,6 +733,8 @@ static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   b.tiles_x = a.num_seqs <= 64 ? (int)(a.total_tokens / bm + (int64_t)a.num_seqs * (kBandRows / bm))
                                : (int)(a.total_tokens / bm + a.num_seqs);
   b.heads_y = a.num_kv_heads * (group / hpw);
+  b.band_bits = 1;
+  while (((int64_t)1 << b.band_bits) <= a.total_tokens / kBandRows + 1) ++b.band_bits;
   const int64_t items = (int64_t)b.tiles_x * b.heads_y;
   const int64_t span = 8 * (int64_t)kXcdChunk;
   dim3 grid((unsigned)((items + span - 1) / span * span));
@@ -785,7 +788,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   a.out = out; a.q = q; a.k = k; a.v = v; a.cu_seqlens = cu_seqlens;
   a.total_tokens = total_tokens; a.num_seqs = num_seqs; a.num_heads = num_heads;
   a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
-  a.tiles_x = 0; a.heads_y = 0;
+  a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
   a.cu_seqlens_k = nullptr; a.block_tables = nullptr; a.max_num_blocks = 0; a.block_size = 0; a.num_blocks = 0;
   const int group = num_heads / num_kv_heads;
   const bool mfma_ok = dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64) &&
@@ -823,7 +826,7 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
   a.out = out; a.q = q; a.k = k_cache; a.v = v_cache; a.cu_seqlens = cu_seqlens_q;
   a.total_tokens = total_q_tokens; a.num_seqs = num_seqs; a.num_heads = num_heads;
   a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
-  a.tiles_x = 0; a.heads_y = 0;
+  a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
   a.cu_seqlens_k = cu_seqlens_k; a.block_tables = block_tables; a.max_num_blocks = max_num_blocks;
   a.block_size = block_size; a.num_blocks = num_blocks;
   const int group = num_heads / num_kv_heads;

@@ -418,9 +418,21 @@ class Attention(nn.Module):
         scale = self.scale / (self.head_dim ** 0.5)
 
         if context.is_prefill:
+            if q.dim() == 4:
+                # Batched mode (B, N, Hq, D): B sequences of N tokens each.  The reference dispatches to a function
+                # it never defines (attention.py:526-533); here the batch is the packed case with equal lengths.
+                if context.block_tables is not None:
+                    raise ValueError("batched 4-D prefill over a cached prefix is not provided; pack the new tokens")
+                bsz, n = q.shape[:2]
+                cu = torch.arange(bsz + 1, dtype=torch.int32, device=q.device) * n
+                o = flash_attention_prefill(q.reshape(bsz * n, self.num_heads, self.head_dim),
+                                            k.reshape(bsz * n, self.num_kv_heads, self.head_dim),
+                                            v.reshape(bsz * n, self.num_kv_heads, self.head_dim), cu, scale,
+                                            self.num_heads, self.num_kv_heads, self.head_dim)
+                return o.reshape(bsz, n, self.num_heads * self.head_dim)
             if q.dim() != 3:
-                raise ValueError("prefill expects packed varlen q of shape (total_tokens, num_heads, head_dim); "
-                                 "batched 4-D prefill is not provided")
+                raise ValueError("prefill expects q of shape (total_tokens, num_heads, head_dim) or "
+                                 "(batch, tokens, num_heads, head_dim)")
             cu_seqlens = context.cu_seqlens_q
             if cu_seqlens is None:
                 raise ValueError("cu_seqlens_q must be provided for varlen attention")

@@ -164,3 +164,26 @@ def test_prefill_head_dim_64_vs_oracle(dtype, hq, hkv, lengths):
     k2[cut:] = 1.0
     v2[cut:] = -1.0
     assert torch.equal(_run(q, k2, v2, cu, scale, hq, hkv, d)[:cut], got[:cut])
+
+
+def test_attention_module_batched_4d_prefill():
+    """Batched mode of Attention.forward (attention.py:526-533: q (B, N, Hq, D); the reference calls a function it
+    never defines): B sequences of N tokens, causal inside each, output (B, N, Hq * D); K/V rows are stored to
+    their slots on the way, as in the packed mode."""
+    from minivllm_amd.layers.attention import Attention
+    from minivllm_amd.utils import reset_context, set_context
+    hq, hkv, d, bs, bsz, n = 8, 2, 128, 16, 3, 70
+    q, k, v, cu = make_varlen_case(54, [n] * bsz, hq, hkv, d, dtype=torch.bfloat16)
+    layer = Attention(hq, d, 1.0, hkv, bs)
+    nb = bsz * (-(-n // bs))
+    layer.k_cache = torch.zeros(nb, bs, hkv, d, dtype=torch.bfloat16, device=DEV)
+    layer.v_cache = torch.zeros_like(layer.k_cache)
+    slots = torch.cat([torch.arange(n) + s * (-(-n // bs)) * bs for s in range(bsz)])
+    set_context(True, None, None, n, n, slots.to(DEV), None, None)          # no cu_seqlens: the shape carries it
+    out = layer(q.view(bsz, n, hq, d).to(DEV), k.view(bsz, n, hkv, d).to(DEV), v.view(bsz, n, hkv, d).to(DEV))
+    reset_context()
+    assert out.shape == (bsz, n, hq * d)
+    want = _oracle32(q, k, v, cu, 1 / math.sqrt(d), hq, hkv, d)
+    mx, mean = error_stats(out.cpu().view(bsz * n, hq, d), want)
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+    assert torch.equal(layer.k_cache.view(-1, hkv, d)[slots.to(DEV)].cpu(), k)
