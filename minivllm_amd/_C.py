@@ -34,6 +34,7 @@ SIGNATURES = {
     "mvllm_paged_decode_int8": (c_int, [c_void_p] * 7 + [c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                                           c_int, c_int64, c_float, c_int, c_void_p, c_size_t,
                                                           c_void_p]),
+    "mvllm_prefill_plan": (c_int, [c_int] * 6 + [ctypes.POINTER(c_int)]),
     "mvllm_prefill_varlen": (c_int, [c_void_p] * 5 + [c_int, c_int64, c_int, c_int, c_int, c_float, c_int,
                                                        c_void_p]),
     "mvllm_prefill_paged": (c_int, [c_void_p] * 5 + [c_int, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int,

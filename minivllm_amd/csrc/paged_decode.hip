@@ -18,6 +18,7 @@
 // The kernel is HBM-bound: a kernel that only issues the same loads (no arithmetic) reaches
 // 6.25 TB/s on this access pattern, this one about 6.05.
 #include <atomic>
+#include <type_traits>
 #include "common.h"
 
 namespace mvllm {
@@ -184,15 +185,17 @@ __device__ __forceinline__ bool decode_item(const DecodeArgs& a, int& b, int& p,
 // ---------------------------------------------------------------------------
 // Fast path
 // ---------------------------------------------------------------------------
-template <typename T>
+// head dims of the 16-bit kernels: 32, 64, 128 (one set of up to sixteen 8-dim output columns) and 256 (two sets)
+constexpr int dim_sets(int d) { return d > 128 ? d / 128 : 1; }
+template <typename T, int D = 128>
 struct KVTile {          // 16-bit elements: lane l holds 8 dims (16 B) of token l%16 per 32-dim step, and of its four V tokens
-  uint4 k[4];
-  uint4 v[4];
+  uint4 k[D > 128 ? D / 32 : 4];
+  uint4 v[4 * dim_sets(D)];     // v[4 s + i]: token i, dims 128 s + 8 (l%16) ..
   int t0;
   bool ok;
 };
-template <>
-struct KVTile<float> {   // fp32: 4 dims (16 B) of token l%16 per 16-dim step; of each V token 4 dims per 64-dim step
+template <int D>
+struct KVTile<float, D> {   // fp32: 4 dims (16 B) of token l%16 per 16-dim step; of each V token 4 dims per 64-dim step
   float4 k[8];
   float4 v[4][2];
   int t0;
@@ -205,20 +208,24 @@ template <typename T, int D>
 struct TileIO {
   static constexpr int kKLane = 8;     // dims between the classes (lane/16) of the first product
   static constexpr int kVLane = 8;     // dims per column (lane%16) of the second product
-  static __device__ __forceinline__ bool owns(int col) { return D == 128 || col < D / 8; }
-  static __device__ __forceinline__ void load_k(KVTile<T>& t, const T* kp) {
+  static constexpr int kSets = dim_sets(D);
+  static __device__ __forceinline__ bool owns(int col) { return D >= 128 || col < D / 8; }
+  static __device__ __forceinline__ void load_k(KVTile<T, D>& t, const T* kp) {
 #pragma unroll
     for (int j = 0; j < D / 32; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
   }
   template <bool STREAM>
-  static __device__ __forceinline__ void load_v(KVTile<T>& t, int i, const T* vp, bool own) {
-    t.v[i] = !own ? make_uint4(0u, 0u, 0u, 0u) : STREAM ? load16_stream(vp) : *reinterpret_cast<const uint4*>(vp);
+  static __device__ __forceinline__ void load_v(KVTile<T, D>& t, int i, const T* vp, bool own) {
+#pragma unroll
+    for (int s = 0; s < kSets; ++s)
+      t.v[4 * s + i] = !own ? make_uint4(0u, 0u, 0u, 0u)
+                            : STREAM ? load16_stream(vp + 128 * s) : *reinterpret_cast<const uint4*>(vp + 128 * s);
   }
-  static __device__ __forceinline__ void zero(KVTile<T>& t) {
+  static __device__ __forceinline__ void zero(KVTile<T, D>& t) {
 #pragma unroll
     for (int j = 0; j < D / 32; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
+    for (int i = 0; i < 4 * kSets; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
   }
 };
 template <int D>
@@ -226,12 +233,12 @@ struct TileIO<float, D> {
   static constexpr int kKLane = 4;
   static constexpr int kVLane = 4;
   static __device__ __forceinline__ bool owns(int) { return true; }     // 16 columns x 4 dims per 64-dim step
-  static __device__ __forceinline__ void load_k(KVTile<float>& t, const float* kp) {
+  static __device__ __forceinline__ void load_k(KVTile<float, D>& t, const float* kp) {
 #pragma unroll
     for (int j = 0; j < D / 16; ++j) t.k[j] = *reinterpret_cast<const float4*>(kp + 16 * j);
   }
   template <bool STREAM>
-  static __device__ __forceinline__ void load_v(KVTile<float>& t, int i, const float* vp, bool) {
+  static __device__ __forceinline__ void load_v(KVTile<float, D>& t, int i, const float* vp, bool) {
 #pragma unroll
     for (int jj = 0; jj < D / 64; ++jj) {
       if (STREAM) {
@@ -242,7 +249,7 @@ struct TileIO<float, D> {
       }
     }
   }
-  static __device__ __forceinline__ void zero(KVTile<float>& t) {
+  static __device__ __forceinline__ void zero(KVTile<float, D>& t) {
 #pragma unroll
     for (int j = 0; j < D / 16; ++j) t.k[j] = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
@@ -320,11 +327,13 @@ struct DecodeHead {
   using Elem = T;
   static constexpr int kDim = D;
   static constexpr int kSteps = D / 32;     // 32-dim steps of the first product
-  static constexpr int kCols = D / 8;       // lanes (l%16) that own 8 dims of the output
+  static constexpr int kSets = dim_sets(D); // sets of sixteen 8-dim output columns (2 for head_dim 256)
+  static constexpr int kCols = D >= 128 ? 16 : D / 8;   // lanes (l%16) that own 8 dims of the output per set
+  static constexpr int kAcc = 8 * kSets;
   uint4 qf[kSteps];           // Q fragments: B operand, column n = head n, k = 8*cls + 32 j
   float m;                    // running maximum of head `col` (log2 units), the same in its four lanes
   float l;                    // this lane's share of the head's denominator
-  v4f o[8];                   // o[e][j] = O[head 4*cls + j][dim 8*col + e]
+  v4f o[kAcc];                // o[8 s + e][j] = O[head 4*cls + j][dim 128 s + 8*col + e]
 
   // column lane%16 of the first product is the row of D elements at `row_ptr` (zero when not live)
   __device__ __forceinline__ void load_q(const T* row_ptr, bool live, int lane) {
@@ -337,7 +346,7 @@ struct DecodeHead {
     m = -INFINITY;
     l = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int e = 0; e < kAcc; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
   }
   __device__ __forceinline__ void start(const DecodeArgs& a, int b, int g, int group, int lane) {
     const int col = lane & 15;
@@ -347,25 +356,31 @@ struct DecodeHead {
   // this lane's dims of accumulator row j (head or query row 4*(lane/16) + j), scaled, into the row of D elements
   __device__ __forceinline__ void write_row(T* row_ptr, int j, float scale, int lane) const {
     const int col = lane & 15;
-    if (D == 128 || col < kCols) {
-      T r[8];
+    if (col < kCols) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) r[e] = from_float<T>(o[e][j] * scale);
-      *reinterpret_cast<uint4*>(row_ptr + col * 8) = *reinterpret_cast<const uint4*>(r);
+      for (int s = 0; s < kSets; ++s) {
+        T r[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r[e] = from_float<T>(o[8 * s + e][j] * scale);
+        *reinterpret_cast<uint4*>(row_ptr + 128 * s + col * 8) = *reinterpret_cast<const uint4*>(r);
+      }
     }
   }
   __device__ __forceinline__ void write_partial(float* row_ptr, int j, int lane) const {
     const int col = lane & 15;
-    if (D == 128 || col < kCols) {
-      float* dst = row_ptr + col * 8;
-      *reinterpret_cast<float4*>(dst) = make_float4(o[0][j], o[1][j], o[2][j], o[3][j]);
-      *reinterpret_cast<float4*>(dst + 4) = make_float4(o[4][j], o[5][j], o[6][j], o[7][j]);
+    if (col < kCols) {
+#pragma unroll
+      for (int s = 0; s < kSets; ++s) {
+        float* dst = row_ptr + 128 * s + col * 8;
+        *reinterpret_cast<float4*>(dst) = make_float4(o[8 * s + 0][j], o[8 * s + 1][j], o[8 * s + 2][j], o[8 * s + 3][j]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(o[8 * s + 4][j], o[8 * s + 5][j], o[8 * s + 6][j], o[8 * s + 7][j]);
+      }
     }
   }
 
   // one tile of 16 tokens starting at token t0 of the sequence; tokens at or past part_end do not count
   // (col_end: prefill only, where column n is a query row: tokens at or past it do not count for this lane's column)
-  __device__ __forceinline__ void consume(const KVTile<T>& t, int part_end, float scale_log2, int lane,
+  __device__ __forceinline__ void consume(const KVTile<T, D>& t, int part_end, float scale_log2, int lane,
                                           int col_end = 0x7fffffff) {
     const int cls = lane >> 4;
     const int tok_base = t.t0 + 4 * cls;
@@ -376,13 +391,16 @@ struct DecodeHead {
     float s2[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) s2[i] = s[i] * scale_log2;
-    uint4 v[4] = {t.v[0], t.v[1], t.v[2], t.v[3]};
+    uint4 v[4 * kSets];
+#pragma unroll
+    for (int i = 0; i < 4 * kSets; ++i) v[i] = t.v[i];
     if (partial) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         if (!t.ok || tok_base + i >= part_end) {
           s2[i] = -INFINITY;
-          v[i] = make_uint4(0u, 0u, 0u, 0u);       // whatever lies there must not meet p = 0 as NaN or Inf
+#pragma unroll
+          for (int s = 0; s < kSets; ++s) v[4 * s + i] = make_uint4(0u, 0u, 0u, 0u);   // whatever lies there must not meet p = 0 as NaN or Inf
         }
     }
     if (col_end != 0x7fffffff) {
@@ -406,7 +424,7 @@ struct DecodeHead {
       for (int j = 0; j < 4; ++j) {
         const float aj = __shfl(al, 4 * cls + j, 64);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e][j] *= aj;
+        for (int e = 0; e < kAcc; ++e) o[e][j] *= aj;
       }
     }
     const float m_eff = (m == -INFINITY) ? 0.f : m;
@@ -419,35 +437,39 @@ struct DecodeHead {
     const uint2 pa = make_uint2(pack_pair<T>(pr[0], pr[1]), pack_pair<T>(pr[2], pr[3]));
     // dim e of the lane's 8: the low or high half of component e/2 of each token's 16 bytes
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
-      const uint32_t c0 = e < 2 ? v[0].x : e < 4 ? v[0].y : e < 6 ? v[0].z : v[0].w;
-      const uint32_t c1 = e < 2 ? v[1].x : e < 4 ? v[1].y : e < 6 ? v[1].z : v[1].w;
-      const uint32_t c2 = e < 2 ? v[2].x : e < 4 ? v[2].y : e < 6 ? v[2].z : v[2].w;
-      const uint32_t c3 = e < 2 ? v[3].x : e < 4 ? v[3].y : e < 6 ? v[3].z : v[3].w;
-      const uint2 vb = make_uint2(__builtin_amdgcn_perm(c1, c0, sel), __builtin_amdgcn_perm(c3, c2, sel));
-      o[e] = mfma16x16x16<T>(pa, vb, o[e]);
-    }
+    for (int s = 0; s < kSets; ++s)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+        const uint4 &v0 = v[4 * s], &v1 = v[4 * s + 1], &v2 = v[4 * s + 2], &v3 = v[4 * s + 3];
+        const uint32_t c0 = e < 2 ? v0.x : e < 4 ? v0.y : e < 6 ? v0.z : v0.w;
+        const uint32_t c1 = e < 2 ? v1.x : e < 4 ? v1.y : e < 6 ? v1.z : v1.w;
+        const uint32_t c2 = e < 2 ? v2.x : e < 4 ? v2.y : e < 6 ? v2.z : v2.w;
+        const uint32_t c3 = e < 2 ? v3.x : e < 4 ? v3.y : e < 6 ? v3.z : v3.w;
+        const uint2 vb = make_uint2(__builtin_amdgcn_perm(c1, c0, sel), __builtin_amdgcn_perm(c3, c2, sel));
+        o[8 * s + e] = mfma16x16x16<T>(pa, vb, o[8 * s + e]);
+      }
   }
 
   // W waves hold partial results of the same heads over different tokens: waves 1 .. W-1 leave theirs in LDS
-  // (9 x 16 bytes per lane: m, l and the 8 x 4 accumulators), wave 0 folds them into its own with the usual
+  // (1 + kAcc float4 per lane: m, l and the accumulators), wave 0 folds them into its own with the usual
   // log-sum-exp weights and is the only one to return true.  Every wave of the workgroup must call this.
   template <int W>
   __device__ __forceinline__ bool merge(int w, int lane) {
-    __shared__ float4 part[(W - 1) * 9 * 64];
+    constexpr int kSlots = 1 + kAcc;
+    __shared__ float4 part[(W - 1) * kSlots * 64];
     const int cls = lane >> 4;
     if (w > 0) {
-      float4* dst = part + (w - 1) * 9 * 64 + lane;
+      float4* dst = part + (w - 1) * kSlots * 64 + lane;
       dst[0] = make_float4(m, l, 0.f, 0.f);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) dst[(1 + e) * 64] = make_float4(o[e][0], o[e][1], o[e][2], o[e][3]);
+      for (int e = 0; e < kAcc; ++e) dst[(1 + e) * 64] = make_float4(o[e][0], o[e][1], o[e][2], o[e][3]);
     }
     __syncthreads();
     if (w > 0) return false;
 #pragma unroll 1
     for (int x = 0; x < W - 1; ++x) {
-      const float4* src = part + x * 9 * 64 + lane;
+      const float4* src = part + x * kSlots * 64 + lane;
       const float4 ml = src[0];
       const float m_new = fmaxf(m, ml.x);
       const float f0 = safe_exp2_diff(m, m_new);          // both are 0 while neither wave has seen a token
@@ -461,7 +483,7 @@ struct DecodeHead {
         a1[j] = __shfl(f1, 4 * cls + j, 64);
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int e = 0; e < kAcc; ++e) {
         const float4 ow = src[(1 + e) * 64];
         o[e][0] = o[e][0] * a0[0] + ow.x * a1[0];
         o[e][1] = o[e][1] * a0[1] + ow.y * a1[1];
@@ -515,7 +537,7 @@ struct DecodeHead<float, D> {
     load_q(reinterpret_cast<const float*>(a.q) + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D, live, lane);
   }
 
-  __device__ __forceinline__ void consume(const KVTile<float>& t, int part_end, float scale_log2, int lane,
+  __device__ __forceinline__ void consume(const KVTile<float, D>& t, int part_end, float scale_log2, int lane,
                                           int col_end = 0x7fffffff) {
     const int cls = lane >> 4;
     const int tok_base = t.t0 + 4 * cls;
@@ -682,7 +704,7 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
   const int k_lane_off = col * (int)row + cls * IO::kKLane;        // token lane%16, first dim of class lane/16
   const int v_lane_off = 4 * cls * (int)row + col * IO::kVLane;    // token 4*(lane/16), first dim of column lane%16
 
-  auto load_tile = [&](KVTile<T>& t, int tile) {
+  auto load_tile = [&](KVTile<T, D>& t, int tile) {
     t.t0 = first + tile * (W * kTile);
     if (bi - win_base >= 64) {
       win_base = bi;
@@ -716,7 +738,7 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
   // Tiles in pairs (ta, tb: one consumed while the other is in flight), the odd one after the loop.  A single
   // loop exit keeps the accumulators in one set of registers (an exit between the two halves made the compiler
   // hold two: 184 VGPRs instead of 154, one wave per SIMD less).
-  KVTile<T> ta, tb;
+  KVTile<T, D> ta, tb;
   if (ntiles > 0) load_tile(ta, 0);
   int tile = 0;
   for (; tile + 1 < ntiles; tile += 2) {
@@ -797,7 +819,7 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
 
   // Tokens past kv_end are masked by consume(); in the packed tensors their loads are redirected to the last
   // visible row so that nothing past the end is touched (in a cache block they are rows of the same block).
-  auto load_tile = [&](KVTile<T>& t, int tile) __attribute__((always_inline)) {
+  auto load_tile = [&](KVTile<T, D>& t, int tile) __attribute__((always_inline)) {
     t.t0 = tile * kTile;
     t.ok = true;
     // An unmapped block reads as zero keys and values that still count (score 0), as in the other prefill
@@ -843,7 +865,7 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
       IO::zero(t);
     }
   };
-  KVTile<T> ta, tb;
+  KVTile<T, D> ta, tb;
   if (ntiles > 0) load_tile(ta, 0);
   int tile = 0;
   for (; tile + 1 < ntiles; tile += 2) {
@@ -1182,14 +1204,15 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
 // an upper bound, and a workgroup whose partition lies past its sequence's context returns at once.
 // ---------------------------------------------------------------------------
 template <typename T, int D>
-__global__ __launch_bounds__(512, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_kernel(const DecodeArgs a) {
+// head_dim 256 holds twice the accumulators and tiles: one wave per SIMD with up to 512 registers
+__global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_kernel(const DecodeArgs a) {
   int b, p, hg;
   if (!decode_item<false>(a, b, p, hg)) return;
   decode_mfma_item<T, 1, D>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
 }
 // Small batches: one workgroup of W waves per (partition, sequence, kv head), the waves splitting the tiles.
 template <typename T, int W, int D>
-__global__ __launch_bounds__(64 * W, MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_split_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(64 * W, D > 128 ? 1 : MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_split_kernel(const DecodeArgs a) {
   // kv head fastest: the workgroups of one (sequence, partition) start together and read the same token rows
   const int g = blockIdx.x, b = blockIdx.z;
   const int p = (int)((blockIdx.y + (unsigned)b) % (unsigned)a.num_parts);
@@ -1372,7 +1395,9 @@ static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int ma
 
 // shapes the MFMA kernels are built for (pointer alignment is checked by the caller)
 static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool int8) {
-  const bool dim_ok = head_dim == 128 || head_dim == 64;
+  // 16-bit caches: 32, 64, 128 or 256 dims per head; fp32 and INT8 caches: 64 or 128
+  const bool dim_ok = head_dim == 128 || head_dim == 64 ||
+                      (dtype != MVLLM_F32 && !int8 && (head_dim == 256 || head_dim == 32));
   return (dtype != MVLLM_F32 || !int8) && dim_ok && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
          (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
 }
@@ -1406,11 +1431,18 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
   const dim3 block(64 * wpb);
   if (fast_ok && !int8) {
     const dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, groups);
-    if (split && a.head_dim == 64) decode_mfma_split_kernel<T, kSplitWaves, 64><<<split_grid, split_block, 0, stream>>>(a);
-    else if (split) decode_mfma_split_kernel<T, kSplitWaves, 128><<<split_grid, split_block, 0, stream>>>(a);
-    else if (a.head_dim == 64) decode_mfma_kernel<T, 64><<<grid, block, 0, stream>>>(a);
-    else decode_mfma_kernel<T, 128><<<grid, block, 0, stream>>>(a);
-    launched = true;
+    auto go = [&](auto DIM) {
+      constexpr int D = decltype(DIM)::value;
+      if (split) decode_mfma_split_kernel<T, kSplitWaves, D><<<split_grid, split_block, 0, stream>>>(a);
+      else decode_mfma_kernel<T, D><<<grid, block, 0, stream>>>(a);
+      launched = true;
+    };
+    if (a.head_dim == 128) go(std::integral_constant<int, 128>{});
+    else if (a.head_dim == 64) go(std::integral_constant<int, 64>{});
+    if constexpr (IsSixteenBit<T>::value) {         // 16-bit caches also with 32 and 256 dims per head
+      if (a.head_dim == 256) go(std::integral_constant<int, 256>{});
+      else if (a.head_dim == 32) go(std::integral_constant<int, 32>{});
+    }
   }
   if constexpr (IsSixteenBit<T>::value) {           // the INT8 kernels take 16-bit queries
     if (fast_ok && int8) {
@@ -1497,7 +1529,7 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
 
 template <typename T, int D>
 static void launch_rows16(const PrefillRowsArgs& a, dim3 grid, int tiles, hipStream_t stream) {
-  if constexpr (sizeof(T) == 2) {
+  if constexpr (sizeof(T) == 2 && (D == 64 || D == 128)) {
     if (a.k_scale) {
       prefill_rows16_kernel<T, D, true, true><<<grid, dim3(256), 0, stream>>>(a, tiles);
       return;
@@ -1506,8 +1538,12 @@ static void launch_rows16(const PrefillRowsArgs& a, dim3 grid, int tiles, hipStr
   if (a.block_tables) prefill_rows16_kernel<T, D, true><<<grid, dim3(256), 0, stream>>>(a, tiles);
   else prefill_rows16_kernel<T, D, false><<<grid, dim3(256), 0, stream>>>(a, tiles);
 }
+bool prefill_rows16_takes(int head_dim, int dtype, bool int8_cache) {
+  if (head_dim == 64 || head_dim == 128) return true;
+  return (head_dim == 32 || head_dim == 256) && dtype != MVLLM_F32 && !int8_cache;
+}
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream) {
-  if (head_dim != 64 && head_dim != 128) return MVLLM_ERR_UNSUPPORTED;
+  if (!prefill_rows16_takes(head_dim, dtype, a.k_scale != nullptr)) return MVLLM_ERR_UNSUPPORTED;
   if (a.block_tables && a.block_size % kTile != 0) return MVLLM_ERR_UNSUPPORTED;
   if (a.k_scale && (!a.v_scale || !a.block_tables || dtype == MVLLM_F32)) return MVLLM_ERR_UNSUPPORTED;
   const int64_t tiles = a.total_tokens / kTile + a.num_seqs;      // upper bound on the 16-row tiles
@@ -1515,12 +1551,16 @@ int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hip
   if (dtype == MVLLM_F32) {
     if (head_dim == 64) launch_rows16<float, 64>(a, grid, (int)tiles, stream);
     else launch_rows16<float, 128>(a, grid, (int)tiles, stream);
-  } else if (dtype == MVLLM_BF16) {
-    if (head_dim == 64) launch_rows16<bf16_t, 64>(a, grid, (int)tiles, stream);
-    else launch_rows16<bf16_t, 128>(a, grid, (int)tiles, stream);
   } else {
-    if (head_dim == 64) launch_rows16<f16_t, 64>(a, grid, (int)tiles, stream);
-    else launch_rows16<f16_t, 128>(a, grid, (int)tiles, stream);
+    auto go = [&](auto DIM) {
+      constexpr int D = decltype(DIM)::value;
+      if (dtype == MVLLM_BF16) launch_rows16<bf16_t, D>(a, grid, (int)tiles, stream);
+      else launch_rows16<f16_t, D>(a, grid, (int)tiles, stream);
+    };
+    if (head_dim == 64) go(std::integral_constant<int, 64>{});
+    else if (head_dim == 128) go(std::integral_constant<int, 128>{});
+    else if (head_dim == 32) go(std::integral_constant<int, 32>{});
+    else go(std::integral_constant<int, 256>{});
   }
   return launch_status();
 }

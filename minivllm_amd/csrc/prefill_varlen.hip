@@ -772,6 +772,29 @@ static int prefill_dispatch(const PrefillArgs& a, int dtype, bool mfma_ok, hipSt
 
 using namespace mvllm;
 
+// Which kernel serves a prefill of these static sizes, pointers assumed 16-byte aligned: 2 = the LDS-tiled MFMA
+// kernel, 1 = the 16-row tile MFMA kernel, 0 = the generic kernel (one key per step: a correctness path), -1 = none.
+static int prefill_kernel_for(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool paged,
+                              bool int8_cache) {
+  const bool blocks_ok = !paged || block_size % 16 == 0;
+  if (int8_cache) return (dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64) && blocks_ok) ? 1 : -1;
+  if (dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64) && blocks_ok &&
+      (!paged || (int64_t)block_size * num_kv_heads * head_dim * 2 < ((int64_t)1 << 31)))
+    return 2;
+  if (prefill_rows16_takes(head_dim, dtype, false) && blocks_ok && (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31))
+    return 1;
+  return head_dim <= 64 * kGenMaxR ? 0 : -1;
+}
+
+extern "C" int mvllm_prefill_plan(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype,
+                                  int int8_cache, int* kernel) {
+  if (dtype_size(dtype) == 0) return MVLLM_ERR_BAD_DTYPE;
+  if (num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size < 0 || num_heads % num_kv_heads != 0)
+    return MVLLM_ERR_BAD_SHAPE;
+  if (kernel) *kernel = prefill_kernel_for(num_heads, num_kv_heads, head_dim, block_size, dtype, block_size > 0, int8_cache != 0);
+  return MVLLM_OK;
+}
+
 extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, const void* v,
                                     const int32_t* cu_seqlens, int num_seqs, int64_t total_tokens,
                                     int num_heads, int num_kv_heads, int head_dim, float scale, int dtype,
@@ -790,13 +813,11 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
   a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
   a.cu_seqlens_k = nullptr; a.block_tables = nullptr; a.max_num_blocks = 0; a.block_size = 0; a.num_blocks = 0;
-  const int group = num_heads / num_kv_heads;
-  const bool mfma_ok = dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64) &&
-                       aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
-                       num_kv_heads * group <= 65535;
-  // fp32 with head_dim 64 or 128: 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
-  if (!mfma_ok && (head_dim == 64 || head_dim == 128) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) &&
-      (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31)) {
+  const bool aligned = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out);
+  const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, 0, dtype, false, false) : 0;
+  const bool mfma_ok = kind == 2;
+  // fp32, and 16-bit head dims 32 and 256: 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
+  if (kind == 1) {
     PrefillRowsArgs r;
     r.out = out; r.q = q; r.k = k; r.v = v; r.cu_seqlens = cu_seqlens; r.total_tokens = total_tokens;
     r.num_seqs = num_seqs; r.num_heads = num_heads; r.num_kv_heads = num_kv_heads; r.scale_log2 = scale * kLog2e;
@@ -829,13 +850,10 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
   a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
   a.cu_seqlens_k = cu_seqlens_k; a.block_tables = block_tables; a.max_num_blocks = max_num_blocks;
   a.block_size = block_size; a.num_blocks = num_blocks;
-  const int group = num_heads / num_kv_heads;
-  const bool mfma_ok = dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64) &&
-                       block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) &&
-                       aligned16(out) && num_kv_heads * group <= 65535 &&
-                       (int64_t)block_size * num_kv_heads * head_dim * 2 < ((int64_t)1 << 31);
-  if (!mfma_ok && (head_dim == 64 || head_dim == 128) && block_size % 16 == 0 && aligned16(q) && aligned16(k_cache) &&
-      aligned16(v_cache) && aligned16(out) && (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31)) {
+  const bool aligned = aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out);
+  const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, block_size, dtype, true, false) : 0;
+  const bool mfma_ok = kind == 2;
+  if (kind == 1) {
     PrefillRowsArgs r;
     r.out = out; r.q = q; r.k = k_cache; r.v = v_cache; r.cu_seqlens = cu_seqlens_q; r.total_tokens = total_q_tokens;
     r.num_seqs = num_seqs; r.num_heads = num_heads; r.num_kv_heads = num_kv_heads; r.scale_log2 = scale * kLog2e;

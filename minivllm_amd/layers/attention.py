@@ -23,7 +23,8 @@ from minivllm_amd.utils.context import get_context
 __all__ = [
     "store_kvcache", "store_kvcache_int8", "flash_attention_prefill", "flash_attention_prefill_paged",
     "flash_attention_prefill_paged_int8",
-    "paged_attention_decode", "paged_attention_decode_int8", "decode_workspace_bytes", "Attention",
+    "paged_attention_decode", "paged_attention_decode_int8", "decode_workspace_bytes", "paged_decode_plan",
+    "prefill_plan", "Attention",
 ]
 
 _workspaces: dict = {}   # device index -> uint8 tensor reused by decode calls on that device that bring no workspace
@@ -55,6 +56,29 @@ def decode_workspace_bytes(batch: int, num_heads: int, head_dim: int, max_num_bl
 
 def _ptr(t):
     return 0 if t is None else t.data_ptr()
+
+
+_shapes_seen: set = set()    # (operation, heads, kv heads, head_dim, block_size, dtype, int8) already checked
+
+
+def _warn_if_generic(op: str, num_heads: int, num_kv_heads: int, head_dim: int, block_size: int, dtype, int8: bool):
+    """One warning per shape when a call runs on a generic kernel (a correctness path, about two orders of magnitude
+    slower than the MFMA kernels).  The reference's Triton kernels tile any power-of-two head_dim
+    (attention.py:249-257, 453); here the fast kernels cover head_dim 128 and 64 (bf16 / fp16 also 32 and 256),
+    blocks of a multiple of 16 tokens and up to 16 query heads per kv head."""
+    key = (op, num_heads, num_kv_heads, head_dim, block_size, dtype, int8)
+    if key in _shapes_seen:
+        return
+    _shapes_seen.add(key)
+    if op == "decode":
+        generic = paged_decode_plan(1, num_heads, num_kv_heads, head_dim, 1, block_size, dtype, int8)[2] == 0
+    else:
+        generic = prefill_plan(num_heads, num_kv_heads, head_dim, block_size, dtype, int8) == 0
+    if generic:
+        import warnings
+        warnings.warn(f"minivllm_amd {op}: no MFMA kernel for num_heads={num_heads}, num_kv_heads={num_kv_heads}, "
+                      f"head_dim={head_dim}, block_size={block_size}, {dtype}{', int8 cache' if int8 else ''}; "
+                      "running on the generic kernel (correct, but roughly 100x slower)", RuntimeWarning, stacklevel=3)
 
 
 def _check_cache(name, cache, num_kv_heads, head_dim):
@@ -157,6 +181,7 @@ def flash_attention_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, c
     cu_seqlens = cu_seqlens.contiguous()
     output = torch.empty_like(q)
     num_seqs = cu_seqlens.shape[0] - 1
+    _warn_if_generic("prefill", num_heads, num_kv_heads, head_dim, 0, q.dtype, False)
     lib = _C.load()
     st = lib.mvllm_prefill_varlen(_ptr(output), _ptr(q), _ptr(k), _ptr(v), _ptr(cu_seqlens), num_seqs, total,
                                   num_heads, num_kv_heads, head_dim, float(scale), _C.dtype_code(q.dtype),
@@ -198,6 +223,7 @@ def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cach
     cu_seqlens_q = cu_seqlens_q.to(torch.int32).contiguous()
     cu_seqlens_k = cu_seqlens_k.to(torch.int32).contiguous()
     output = torch.empty_like(q)
+    _warn_if_generic("prefill", num_heads, num_kv_heads, head_dim, block_size, q.dtype, False)
     lib = _C.load()
     st = lib.mvllm_prefill_paged(_ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                  block_tables.shape[1], _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), num_seqs,
@@ -284,6 +310,18 @@ def paged_decode_plan(batch: int, num_heads: int, num_kv_heads: int, head_dim: i
     return tuple(x.value for x in out)
 
 
+def prefill_plan(num_heads: int, num_kv_heads: int, head_dim: int, block_size: int = 0,
+                 dtype: torch.dtype = torch.bfloat16, int8_cache: bool = False) -> int:
+    """Kernel a prefill of these static sizes runs on (host arithmetic only): 2 = LDS-tiled MFMA kernel, 1 = 16-row
+    tile MFMA kernel, 0 = generic kernel, -1 = unsupported.  block_size 0 = packed prefill, > 0 = over a paged cache."""
+    import ctypes
+    out = ctypes.c_int(0)
+    st = _C.load().mvllm_prefill_plan(num_heads, num_kv_heads, head_dim, block_size, _C.dtype_code(dtype),
+                                      int(int8_cache), ctypes.byref(out))
+    _C.check(st, "prefill_plan")
+    return out.value
+
+
 def paged_attention_decode(query: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                            block_tables: torch.Tensor, context_lens: torch.Tensor, scale: float,
                            num_heads: int, num_kv_heads: int, head_dim: int, block_size: int, *,
@@ -305,6 +343,7 @@ def paged_attention_decode(query: torch.Tensor, k_cache: torch.Tensor, v_cache: 
     output = torch.empty_like(query)
     if batch == 0:
         return output
+    _warn_if_generic("decode", num_heads, num_kv_heads, head_dim, block_size, query.dtype, False)
     lib = _C.load()
     nbytes = lib.mvllm_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks, block_size)
     ws = _decode_workspace(query.device, nbytes, workspace)
@@ -336,6 +375,7 @@ def paged_attention_decode_int8(query: torch.Tensor, k_cache: torch.Tensor, v_ca
     output = torch.empty_like(query)
     if batch == 0:
         return output
+    _warn_if_generic("decode", num_heads, num_kv_heads, head_dim, block_size, query.dtype, True)
     lib = _C.load()
     nbytes = lib.mvllm_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks, block_size)
     ws = _decode_workspace(query.device, nbytes, workspace)

@@ -10,6 +10,8 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    # tests that exercise the generic kernels on purpose would each print the library's one-time warning
+    config.addinivalue_line("filterwarnings", "ignore:minivllm_amd .*generic kernel:RuntimeWarning")
 
 
 def pytest_collection_modifyitems(config, items):

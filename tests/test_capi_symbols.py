@@ -27,7 +27,7 @@ def _lib():
 def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
-              "mvllm_paged_decode_int8", "mvllm_paged_decode_noalloc", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_varlen",
+              "mvllm_paged_decode_int8", "mvllm_paged_decode_noalloc", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_plan", "mvllm_prefill_varlen",
               "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_workspace_bytes",
               "mvllm_add_rms_norm",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
@@ -74,6 +74,10 @@ def test_decode_plan_is_host_arithmetic():
     assert paged_decode_plan(64, 16, 16, 64, 256, 16, int8_cache=True)[2] == 1      # 1024 (sequence, head) pairs: first form
     assert paged_decode_plan(64, 16, 16, 96, 256, 16, int8_cache=True)[2] == 0
     assert paged_decode_plan(64, 16, 16, 96, 256, 16)[2] == 0                 # other head dims
+    assert paged_decode_plan(64, 16, 8, 256, 256, 16)[2] == 4                 # 16-bit caches: also 256 and 32 dims
+    assert paged_decode_plan(64, 16, 8, 32, 256, 16)[2] == 4
+    assert paged_decode_plan(64, 16, 8, 256, 256, 16, int8_cache=True)[2] == 0
+    assert paged_decode_plan(64, 16, 8, 256, 256, 16, dtype=__import__("torch").float32)[2] == 0
     import torch
     assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32)[2] == 4       # fp32 caches: fp32 MFMA
     assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32, int8_cache=True)[2] == 0
@@ -86,6 +90,36 @@ def test_decode_plan_is_host_arithmetic():
                 assert part % 16 == 0 and parts == -(-blocks * bs // part) and 1 <= parts <= 32
                 need = 0 if parts == 1 else batch * parts * 8 * hkv * 130 * 4
                 assert need <= lib.mvllm_paged_decode_workspace_bytes(batch, 8 * hkv, 128, blocks, bs)
+
+
+def test_prefill_plan_is_host_arithmetic():
+    """Which kernel a prefill takes: 2 LDS-tiled MFMA, 1 16-row tile MFMA, 0 generic."""
+    import torch
+    from minivllm_amd.layers.attention import prefill_plan
+    assert prefill_plan(32, 8, 128) == 2 and prefill_plan(16, 8, 64, dtype=torch.float16) == 2
+    assert prefill_plan(32, 8, 128, block_size=16) == 2 and prefill_plan(32, 8, 128, block_size=8) == 0
+    assert prefill_plan(32, 8, 128, dtype=torch.float32) == 1 and prefill_plan(16, 8, 64, 16, torch.float32) == 1
+    assert prefill_plan(8, 8, 256) == 1 and prefill_plan(8, 8, 32, block_size=32) == 1      # bf16 / fp16 only
+    assert prefill_plan(8, 8, 256, dtype=torch.float32) == 0
+    assert prefill_plan(6, 2, 80) == 0 and prefill_plan(6, 2, 96) == 0
+    assert prefill_plan(32, 8, 128, 16, int8_cache=True) == 1
+    assert prefill_plan(32, 8, 96, 16, int8_cache=True) == -1 and prefill_plan(32, 8, 128, 16, torch.float32, True) == -1
+    assert prefill_plan(8, 8, 1024) == -1
+
+
+def test_generic_kernel_warning_is_raised_once_per_shape():
+    import warnings
+    import torch
+    from minivllm_amd.layers import attention
+    attention._shapes_seen.clear()
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        attention._warn_if_generic("decode", 16, 16, 96, 16, torch.bfloat16, False)
+        attention._warn_if_generic("decode", 16, 16, 96, 16, torch.bfloat16, False)      # same shape: silent
+        attention._warn_if_generic("prefill", 6, 2, 80, 0, torch.bfloat16, False)
+        attention._warn_if_generic("decode", 32, 8, 128, 16, torch.bfloat16, False)      # MFMA kernel: silent
+        attention._warn_if_generic("prefill", 32, 8, 128, 0, torch.bfloat16, False)
+    assert len(seen) == 2 and all("generic kernel" in str(w.message) for w in seen)
 
 
 def test_argument_validation_without_gpu():

@@ -239,3 +239,29 @@ def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, d, form):
     else:
         assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
     assert torch.count_nonzero(got[3]) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,bs,d", [(16, 8, 16, 256), (8, 1, 32, 256), (5, 5, 48, 256), (16, 8, 16, 32), (12, 2, 256, 32)])
+@pytest.mark.parametrize("form", ["one wave per head", "waves share a head", "waves share a head, one partition"])
+def test_head_dim_256_and_32_on_the_mfma_kernels(dtype, hq, hkv, bs, d, form):
+    """The other power-of-two head dims the reference's kernels take (attention.py:249-257, 453): with 256 dims a
+    lane owns two sets of eight output dims and the first product has eight 32-dim steps; with 32 only four of the
+    sixteen output columns exist.  Both kernel forms, ragged contexts, one empty."""
+    batch = 7 if form == "waves share a head" else 64
+    width = {"one wave per head": 32768, "waves share a head": 8192}.get(form, 4096) // bs * bs
+    g = torch.Generator().manual_seed(177)
+    ctx_list = torch.randint(1, 901, (batch,), generator=g).tolist()
+    ctx_list[3] = 0
+    ctx_list[5] = 900
+    q, kc, vc, tables, ctx = make_paged_case(178, 0, 0, 0, hq, hkv, d, bs, dtype=dtype, ctx_list=ctx_list)
+    tables = _pad_tables(tables, width, bs)
+    part, parts, waves = paged_decode_plan(batch, hq, hkv, d, tables.shape[1], bs, dtype)
+    assert waves == (1 if form == "one wave per head" else 4), (part, parts, waves)
+    scale = 1 / math.sqrt(d)
+    got = _run(q, kc, vc, tables, ctx, scale, hq, hkv, d, bs)
+    live = ctx > 0
+    want = _oracle32(q[live], kc, vc, tables[live][:, :-(-900 // bs)], ctx[live], scale, hq, hkv, d, bs)
+    mx, mean = error_stats(got[live], want)
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+    assert torch.count_nonzero(got[3]) == 0

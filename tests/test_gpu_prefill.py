@@ -47,6 +47,18 @@ def test_prefill_vs_oracle(dtype, hq, hkv, d, lengths):
         assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,d,lengths", [(8, 2, 256, [70, 1, 33, 129]), (4, 4, 256, [200]), (8, 4, 32, [64, 17, 130])])
+def test_prefill_head_dim_256_and_32_on_the_16_row_tile_kernel(dtype, hq, hkv, d, lengths):
+    from minivllm_amd.layers.attention import prefill_plan
+    assert prefill_plan(hq, hkv, d, 0, dtype) == 1
+    case = make_varlen_case(55, lengths, hq, hkv, d, dtype=dtype)
+    scale = 1 / math.sqrt(d)
+    got = _run(*case, scale, hq, hkv, d)
+    mx, mean = error_stats(got, _oracle32(*case, scale, hq, hkv, d))
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
 def test_prefill_zero_length_sequences_and_independence():
     hq, hkv, d = 8, 2, 128
     lengths = [0, 70, 0, 0, 129, 0]

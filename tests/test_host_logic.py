@@ -51,7 +51,10 @@ def test_prefill_without_cu_seqlens_raises_value_error():
     a = Attention(4, 8, 1.0, 2, 4)
     with pytest.raises(ValueError):
         a(torch.zeros(3, 4, 8), torch.zeros(3, 2, 8), torch.zeros(3, 2, 8))
-    with pytest.raises(ValueError):
+    with pytest.raises(ValueError):                    # neither packed (3-D) nor batched (4-D)
+        a(torch.zeros(1, 1, 3, 4, 8), torch.zeros(1, 1, 3, 2, 8), torch.zeros(1, 1, 3, 2, 8))
+    from minivllm_amd._C import MinivllmAmdError
+    with pytest.raises(MinivllmAmdError):              # batched 4-D prefill is the packed kernel: no CPU path
         a(torch.zeros(1, 3, 4, 8), torch.zeros(1, 3, 2, 8), torch.zeros(1, 3, 2, 8))
     reset_context()
 
