@@ -178,8 +178,8 @@ int mvllm_prefill_varlen(void* out, const void* q, const void* k, const void* v,
 /*
  * Which kernel a prefill of these static sizes runs on (no counterpart in the reference, whose Triton kernels take any
  * power-of-two head_dim from a tile-size table, attention.py:249-257).  block_size 0 = the packed entry point,
- * > 0 = the paged ones.  *kernel: 2 the LDS-tiled MFMA kernel (bf16 / fp16, head_dim 128 or 64), 1 the 16-row tile
- * MFMA kernel (fp32 with head_dim 128 or 64, bf16 / fp16 with 32 or 256, INT8 caches), 0 the generic kernel (any
+ * > 0 = the paged ones.  *kernel: 2 the LDS-tiled MFMA kernel (bf16 / fp16, head_dim 128 or 64, also over an INT8
+ * cache), 1 the 16-row tile MFMA kernel (fp32 with head_dim 128 or 64, bf16 / fp16 with 32 or 256), 0 the generic kernel (any
  * head_dim <= 512; one key per step, a correctness path two orders of magnitude slower), -1 unsupported.
  * Pointers are assumed 16-byte aligned (unaligned ones take the generic kernel).  Pure host arithmetic.
  */

@@ -33,6 +33,10 @@ struct PrefillArgs {
   int max_num_blocks;
   int block_size;
   int64_t num_blocks;
+  // INT8 cache (paged mode; k, v are int8 codes [num_blocks, block_size, Hkv, D]): fp32 scales
+  // [num_blocks, block_size, Hkv], else null
+  const float* k_scale;
+  const float* v_scale;
 };
 
 // ---------------------------------------------------------------------------
@@ -154,6 +158,9 @@ constexpr unsigned kXcdChunk = MVLLM_PF_XCD_CHUNK;   // consecutive work items h
 #ifndef MVLLM_PF_PIN_KREADS
 #define MVLLM_PF_PIN_KREADS 1
 #endif
+#ifndef MVLLM_PF_INT8_TILED
+#define MVLLM_PF_INT8_TILED 1         // 0: INT8 caches always on the 16-row tile kernel
+#endif
 #ifndef MVLLM_PF_WAVES
 #define MVLLM_PF_WAVES 4
 #endif
@@ -211,6 +218,18 @@ template <> __device__ __forceinline__ float add_pair<bf16_t>(uint32_t w, float 
 template <> __device__ __forceinline__ float add_pair<f16_t>(uint32_t w, float acc) {
   const v2f16 ones = {(_Float16)1.0f, (_Float16)1.0f};
   return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2f16, w), ones, acc, false);
+}
+
+// Eight int8 codes (two dwords, biased by +128 so that the unsigned byte conversions apply) times one scale, rounded
+// once to the element type: fma(u, scale, -128 scale) is the exactly rounded (u - 128) * scale = code * scale.
+template <typename T> __device__ __forceinline__ uint4 dequant8_biased(uint32_t w0, uint32_t w1, float scale, float bias) {
+  const uint32_t u0 = w0 ^ 0x80808080u, u1 = w1 ^ 0x80808080u;
+  uint4 r;
+  r.x = pack2<T>(fmaf((float)(u0 & 0xffu), scale, bias), fmaf((float)((u0 >> 8) & 0xffu), scale, bias));
+  r.y = pack2<T>(fmaf((float)((u0 >> 16) & 0xffu), scale, bias), fmaf((float)(u0 >> 24), scale, bias));
+  r.z = pack2<T>(fmaf((float)(u1 & 0xffu), scale, bias), fmaf((float)((u1 >> 8) & 0xffu), scale, bias));
+  r.w = pack2<T>(fmaf((float)((u1 >> 16) & 0xffu), scale, bias), fmaf((float)(u1 >> 24), scale, bias));
+  return r;
 }
 
 // 16 bytes per lane from a buffer resource (wave-uniform descriptor + per-lane 32-bit byte offset) straight
@@ -304,8 +323,14 @@ __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, in
 // D = 128 or 64.  A row of a tile is D*2 bytes = kChunks 16-byte chunks; one copy instruction moves 1 KB = kCopyRows
 // rows.  The chunk swizzles (kswz for K, vswz for V) must not change when 8, 16 or 32 rows are added, because the
 // per-lane LDS offsets are computed once and the tile rows are reached through immediates.
-template <typename T, int HPW, bool PAGED, int D>
+// I8 (paged only): the cache holds int8 codes and fp32 scales per (token, kv head).  The codes of a tile are copied
+// into a staging area of LDS (the second K and V buffers, two tiles of codes each), and every wave dequantises its
+// 16 rows into the one 16-bit K and V tile (code * scale rounded once to the element type, exactly what the 16-row
+// tile kernel and decode see), after which the tile is an ordinary tile: two barriers per tile instead of one, the
+// conversion (about 180 vector instructions per lane and tile) in front of the products.
+template <typename T, int HPW, bool PAGED, int D, bool I8 = false>
 __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const PrefillArgs a) {
+  static_assert(!I8 || PAGED, "INT8 caches are paged");
   constexpr int kRowB = D * 2;                  // bytes per tile row
   constexpr int kChunks = kRowB / 16;           // 16-byte chunks per row: 16 or 8
   constexpr int kCopyRows = 1024 / kRowB;       // rows per copy instruction: 4 or 8
@@ -375,7 +400,8 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   const T* q = reinterpret_cast<const T*>(a.q);
   const char* kg = reinterpret_cast<const char*>(a.k);
   const char* vg = reinterpret_cast<const char*>(a.v);
-  const int64_t kv_row_bytes = (int64_t)a.num_kv_heads * D * 2;
+  constexpr int kElt = I8 ? 1 : 2;                    // bytes per cache element
+  const int64_t kv_row_bytes = (int64_t)a.num_kv_heads * D * kElt;
   const int64_t last_token = a.total_tokens - 1;
 
   // ---- K/V tile DMA: wave w moves ROWS_PER_WAVE rows (4 per instruction) of K and of V.
@@ -394,6 +420,13 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     k_src_off[i] = (uint32_t)(src_row * (int)kv_row_bytes + ((ld_chunk ^ kswz(row)) << 4));
     v_src_off[i] = (uint32_t)(src_row * (int)kv_row_bytes + ((ld_chunk ^ vswz(row)) << 4));
   }
+  // INT8: a row of codes is D bytes = D / 16 chunks, one copy instruction moves 1024 / D rows, unswizzled (the
+  // staging area is read back linearly); the same offset serves K and V
+  constexpr int kChunks8 = D / 16, kCopyRows8 = 1024 / D, kCopies8 = ROWS_PER_WAVE / kCopyRows8;
+  uint32_t c_src_off[kCopies8];
+#pragma unroll
+  for (int i = 0; i < kCopies8; ++i)
+    c_src_off[i] = (uint32_t)((kCopyRows8 * i + lane / kChunks8) * (int)kv_row_bytes + ((lane % kChunks8) << 4));
   // One tile's copy is 2 * kCopies instructions per wave (K copies first, then V).  Inside tile_step they are
   // issued one at a time, spread between the MFMAs of the tile before, because a wave that issues them back
   // to back sits in the memory pipeline's queue instead of feeding the matrix unit.  The descriptor of a tile
@@ -405,7 +438,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   // never written (and unmapped blocks) arrive as zeros.  Tiles are asked for in order, once each, so the
   // piece's block index and offset advance by 64 keys per call; block-table entries come from a 64-entry
   // window held one per lane, as in the decode kernel.
-  struct TileSrc { v4i k, v; };
+  struct TileSrc { v4i k, v; int64_t slot; int valid; };   // slot, valid: INT8 only (first token slot and live rows of the piece)
   const int row_bytes = (int)kv_row_bytes;
   const int total_rows = (int)a.total_tokens;
   const int rows_4g = (int)(0xffffffffu / (uint32_t)row_bytes);   // rows whose bytes no longer fit 32 bits
@@ -427,10 +460,12 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       const int phys = __builtin_amdgcn_readlane(win, pg_bi - win_base);
       const int valid = min(ROWS_PER_WAVE, kv_len - pg_pos);
       const bool ok = enable && valid > 0 && pg_bi < a.max_num_blocks && phys >= 0 && (int64_t)phys < a.num_blocks;
-      const uint32_t size = ok ? (uint32_t)((valid - 1) * row_bytes + D * 2) : 0u;
-      const int64_t start = ok ? ((int64_t)phys * bs + pg_off) * kv_row_bytes + (int64_t)g * (D * 2) : 0;
+      const uint32_t size = ok ? (uint32_t)((valid - 1) * row_bytes + D * kElt) : 0u;
+      const int64_t start = ok ? ((int64_t)phys * bs + pg_off) * kv_row_bytes + (int64_t)g * (D * kElt) : 0;
       t.k = make_rsrc(kg + start, size);
       t.v = make_rsrc(vg + start, size);
+      t.slot = ok ? (int64_t)phys * bs + pg_off : 0;
+      t.valid = ok ? valid : 0;
       pg_pos += kBN;
       pg_off += kBN;
       while (pg_off >= bs) {
@@ -446,6 +481,8 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       const int64_t start = (int64_t)row0 * kv_row_bytes + (int64_t)g * (D * 2);
       t.k = make_rsrc(kg + start, size);
       t.v = make_rsrc(vg + start, size);
+      t.slot = 0;
+      t.valid = 0;
     }
     return t;
   };
@@ -468,7 +505,48 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       dma16_to_lds<2 * kTileBytes + i * 1024>(t.v, v_src_off[i], base);
     });
   };
-  issue_tile(0, 0);
+  // ---- INT8: codes -> staging (k[1] / v[1], two tiles of codes each), scales -> registers, then conversion
+  const uint32_t lds_stage_base = lds_address(&lds.k[1][0]) + (uint32_t)(ROWS_PER_WAVE * wave * D);
+  const int cv_row = lane >> 2, cv_quarter = lane & 3;        // conversion: 4 lanes per row of the wave's 16
+  struct Scales { float k, v; };
+  auto issue_codes = [&](int j, bool enable) {                // codes of tile j -> staging[j & 1]; returns its scales
+    const TileSrc t = tile_src(j, enable);
+    const uint32_t base = lds_stage_base + (uint32_t)(j & 1) * (kTileBytes / 2);
+    static_for<kCopies8>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      dma16_to_lds<i * 1024>(t.k, c_src_off[i], base);
+      dma16_to_lds<2 * kTileBytes + i * 1024>(t.v, c_src_off[i], base);
+    });
+    Scales sc = {0.f, 0.f};
+    if (cv_row < t.valid) {
+      const int64_t at = (t.slot + cv_row) * a.num_kv_heads + g;
+      sc.k = a.k_scale[at];
+      sc.v = a.v_scale[at];
+    }
+    return sc;
+  };
+  auto convert_tile = [&](int j, const Scales& sc) {          // staging[j & 1] -> the 16-bit tile in k[0] / v[0]
+    constexpr int kReads = D / 64;                            // 16-byte reads per lane (D / 4 codes)
+    const int row = ROWS_PER_WAVE * wave + cv_row;            // row inside the tile
+    const char* ks8 = &lds.k[1][0] + (j & 1) * (kTileBytes / 2) + row * D + cv_quarter * (D / 4);
+    const char* vs8 = ks8 + 2 * kTileBytes;
+    char* kd = &lds.k[0][0] + row * kRowB;
+    char* vd = &lds.v[0][0] + row * kRowB;
+    const float kb = -128.f * sc.k, vb = -128.f * sc.v;
+#pragma unroll
+    for (int r = 0; r < kReads; ++r) {
+      const uint4 ck = *reinterpret_cast<const uint4*>(ks8 + 16 * r);
+      const uint4 cv = *reinterpret_cast<const uint4*>(vs8 + 16 * r);
+      const int c = cv_quarter * (2 * kReads) + 2 * r;        // first of the two 16-byte chunks these 16 codes fill
+      *reinterpret_cast<uint4*>(kd + (((c) ^ kswz(row)) << 4)) = dequant8_biased<T>(ck.x, ck.y, sc.k, kb);
+      *reinterpret_cast<uint4*>(kd + (((c + 1) ^ kswz(row)) << 4)) = dequant8_biased<T>(ck.z, ck.w, sc.k, kb);
+      *reinterpret_cast<uint4*>(vd + (((c) ^ vswz(row)) << 4)) = dequant8_biased<T>(cv.x, cv.y, sc.v, vb);
+      *reinterpret_cast<uint4*>(vd + (((c + 1) ^ vswz(row)) << 4)) = dequant8_biased<T>(cv.z, cv.w, sc.v, vb);
+    }
+  };
+  Scales sc_cur = {0.f, 0.f};
+  if constexpr (I8) sc_cur = issue_codes(0, true);
+  else issue_tile(0, 0);
 
   // Q fragments (B operand): column = query row l32, k = 16*ks + 8*hi ..
   uint4 qf[kKS];
@@ -534,7 +612,8 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     constexpr bool diag = decltype(DIAG)::value;
     constexpr int NH = decltype(NHALF)::value;
     using NEXT_BUF = std::integral_constant<int, buf ^ 1>;
-    const TileSrc next = tile_src(j + 1, prefetch);
+    TileSrc next;
+    if constexpr (!I8) next = tile_src(j + 1, prefetch);      // INT8: the codes of the next tile are already on their way
 
     // ---- S^T = K Q^T (on the diagonal tile rows past the causal limit are computed and then masked) ----
     // The two 32-row halves of the tile form two independent accumulator chains that are issued
@@ -558,7 +637,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
         }
 #pragma unroll
         for (int tk = 0; tk < NH; ++tk) s[tk] = mfma32x32x16<T>(kf[ks & 1][tk], qf[ks], ks == 0 ? neg_m : s[tk]);
-        if constexpr (ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);           // copies of the next tile, K first
+        if constexpr (!I8 && ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);    // copies of the next tile, K first
       });
     }
 
@@ -665,7 +744,30 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
     else tile_step(j, BUF, std::true_type{}, H2{}, j + 1 < ntiles);
   };
   int j = 0;
-  if (active) {
+  if constexpr (I8) {
+    // codes of tile j have landed and tile j - 1 is no longer read: send for tile j + 1, convert tile j
+    auto stage = [&](int jj) {
+      dma_wait_all();
+      __syncthreads();
+      const Scales sc_next = issue_codes(jj + 1, jj + 1 < ntiles);
+      convert_tile(jj, sc_cur);
+      sc_cur = sc_next;
+      __syncthreads();                  // the 16-bit tile is complete
+    };
+    if (active) {
+      for (; j < n_full; ++j) {
+        stage(j);
+        tile_step(j, B0{}, std::false_type{}, H2{}, false);
+      }
+      for (; j <= j_last; ++j) {
+        stage(j);
+        if (pos0 + kWaveRows - 1 < j * kBN + 32) tile_step(j, B0{}, std::true_type{}, H1{}, false);
+        else tile_step(j, B0{}, std::true_type{}, H2{}, false);
+      }
+    }
+    for (; j < ntiles; ++j) stage(j);
+  }
+  if (!I8 && active) {
     for (; j + 1 < n_full; j += 2) {
       full_step(j, B0{});
       full_step(j + 1, B1{});
@@ -682,7 +784,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   // Tiles that only other waves of the workgroup still compute on (their rows are further down): keep copying
   // this wave's share and meeting the barriers.  Kept out of the loop above so that the accumulators have one
   // straight-line life there.
-  for (; j < ntiles; ++j) {
+  for (; !I8 && j < ntiles; ++j) {
     dma_wait_all();
     __syncthreads();
     if (j + 1 < ntiles) issue_tile(j + 1, (j + 1) & 1);
@@ -720,7 +822,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   }
 }
 
-template <typename T, bool PAGED>
+template <typename T, bool PAGED, bool I8 = false>
 static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   const int group = a.num_heads / a.num_kv_heads;
   // query heads of a kv head per workgroup: 4 or 2 where they divide the group, else 1 (the workgroup is then four
@@ -740,13 +842,13 @@ static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
   dim3 grid((unsigned)((items + span - 1) / span * span));
   const dim3 block(64 * kPfWaves);
   if (a.head_dim == 64) {
-    if (hpw == 4) prefill_mfma_kernel<T, 4, PAGED, 64><<<grid, block, 0, stream>>>(b);
-    else if (hpw == 2) prefill_mfma_kernel<T, 2, PAGED, 64><<<grid, block, 0, stream>>>(b);
-    else prefill_mfma_kernel<T, 1, PAGED, 64><<<grid, block, 0, stream>>>(b);
+    if (hpw == 4) prefill_mfma_kernel<T, 4, PAGED, 64, I8><<<grid, block, 0, stream>>>(b);
+    else if (hpw == 2) prefill_mfma_kernel<T, 2, PAGED, 64, I8><<<grid, block, 0, stream>>>(b);
+    else prefill_mfma_kernel<T, 1, PAGED, 64, I8><<<grid, block, 0, stream>>>(b);
   } else {
-    if (hpw == 4) prefill_mfma_kernel<T, 4, PAGED, 128><<<grid, block, 0, stream>>>(b);
-    else if (hpw == 2) prefill_mfma_kernel<T, 2, PAGED, 128><<<grid, block, 0, stream>>>(b);
-    else prefill_mfma_kernel<T, 1, PAGED, 128><<<grid, block, 0, stream>>>(b);
+    if (hpw == 4) prefill_mfma_kernel<T, 4, PAGED, 128, I8><<<grid, block, 0, stream>>>(b);
+    else if (hpw == 2) prefill_mfma_kernel<T, 2, PAGED, 128, I8><<<grid, block, 0, stream>>>(b);
+    else prefill_mfma_kernel<T, 1, PAGED, 128, I8><<<grid, block, 0, stream>>>(b);
   }
   return launch_status();
 }
@@ -777,7 +879,10 @@ using namespace mvllm;
 static int prefill_kernel_for(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool paged,
                               bool int8_cache) {
   const bool blocks_ok = !paged || block_size % 16 == 0;
-  if (int8_cache) return (dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64) && blocks_ok) ? 1 : -1;
+  if (int8_cache) {
+    if (dtype == MVLLM_F32 || (head_dim != 128 && head_dim != 64) || !blocks_ok) return -1;
+    return (int64_t)block_size * num_kv_heads * head_dim < ((int64_t)1 << 31) ? 2 : 1;
+  }
   if (dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64) && blocks_ok &&
       (!paged || (int64_t)block_size * num_kv_heads * head_dim * 2 < ((int64_t)1 << 31)))
     return 2;
@@ -813,6 +918,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
   a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
   a.cu_seqlens_k = nullptr; a.block_tables = nullptr; a.max_num_blocks = 0; a.block_size = 0; a.num_blocks = 0;
+  a.k_scale = nullptr; a.v_scale = nullptr;
   const bool aligned = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out);
   const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, 0, dtype, false, false) : 0;
   const bool mfma_ok = kind == 2;
@@ -849,7 +955,7 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
   a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
   a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
   a.cu_seqlens_k = cu_seqlens_k; a.block_tables = block_tables; a.max_num_blocks = max_num_blocks;
-  a.block_size = block_size; a.num_blocks = num_blocks;
+  a.block_size = block_size; a.num_blocks = num_blocks; a.k_scale = nullptr; a.v_scale = nullptr;
   const bool aligned = aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out);
   const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, block_size, dtype, true, false) : 0;
   const bool mfma_ok = kind == 2;
@@ -882,6 +988,17 @@ extern "C" int mvllm_prefill_paged_int8(void* out, const void* q, const int8_t* 
       total_q_tokens > ((int64_t)1 << 30) || (int64_t)num_kv_heads * head_dim * 64 >= ((int64_t)1 << 31))
     return MVLLM_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(out) || !aligned16(k_cache) || !aligned16(v_cache)) return MVLLM_ERR_MISALIGNED;
+  if (prefill_kernel_for(num_heads, num_kv_heads, head_dim, block_size, dtype, true, true) == 2 && MVLLM_PF_INT8_TILED) {
+    PrefillArgs a;
+    a.out = out; a.q = q; a.k = k_cache; a.v = v_cache; a.cu_seqlens = cu_seqlens_q;
+    a.total_tokens = total_q_tokens; a.num_seqs = num_seqs; a.num_heads = num_heads;
+    a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
+    a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
+    a.cu_seqlens_k = cu_seqlens_k; a.block_tables = block_tables; a.max_num_blocks = max_num_blocks;
+    a.block_size = block_size; a.num_blocks = num_blocks; a.k_scale = k_scale; a.v_scale = v_scale;
+    return dtype == MVLLM_BF16 ? launch_prefill_mfma<bf16_t, true, true>(a, (hipStream_t)stream)
+                               : launch_prefill_mfma<f16_t, true, true>(a, (hipStream_t)stream);
+  }
   PrefillRowsArgs r;
   r.out = out; r.q = q; r.k = k_cache; r.v = v_cache; r.cu_seqlens = cu_seqlens_q; r.total_tokens = total_q_tokens;
   r.num_seqs = num_seqs; r.num_heads = num_heads; r.num_kv_heads = num_kv_heads; r.scale_log2 = scale * kLog2e;
