@@ -276,6 +276,25 @@ int mvllm_sample_tokens(int64_t* out_ids, const void* logits, int64_t row_stride
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * mvllm_sample_tokens with in-kernel noise whose call offset is read from device memory (*offset_dev), for a
+ * sampler inside a captured graph: a replay cannot change a launch argument, the graph increments the counter.
+ */
+int mvllm_sample_tokens_dev_offset(int64_t* out_ids, const void* logits, int64_t row_stride,
+                                   const float* temperatures, uint64_t seed, const uint64_t* offset_dev,
+                                   int batch, int vocab, int dtype,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The step metadata of a decode batch that continues the step before it (same sequences, each one token longer),
+ * advanced on the device in one launch instead of being rebuilt on the host as ModelRunner.prepare_decode does
+ * (src/myvllm/engine/model_runner.py:231-256): input_ids[i] = sampled[i]; context_lens[i] += 1;
+ * positions[i] = context_lens[i] - 1; slot_mapping[i] += 1.  All int64 [batch].  Rows that open a new block have
+ * their slot and table entry patched by the caller afterwards.
+ */
+int mvllm_decode_advance(int64_t* input_ids, int64_t* context_lens, int64_t* positions, int64_t* slot_mapping,
+                         const int64_t* sampled, int batch, void* stream);
+
+/*
  * LayerNorm.forward with and without residual -- src/myvllm/layers/layernorm.py:9-28, called from
  * Qwen3DecoderLayer.forward and the final norm (src/myvllm/models/qwen3.py:197-212, 306-312):
  *   x = x + residual (rounded to the element type);  out = x / sqrt(mean(x^2) + eps) * gamma;  residual_out = x
@@ -294,6 +313,17 @@ int mvllm_add_rms_norm(void* out, void* residual_out, const void* x, const void*
  */
 int mvllm_silu_and_mul(void* out, const void* in, int64_t rows, int width, int64_t in_row_stride,
                        int dtype, void* stream);
+
+/*
+ * The caller's projections around the attention path for the few rows of a decode step -- nn.Linear in
+ * src/myvllm/models/qwen3.py:90-94 (QKV), :118 (output projection) and the MLP (:121-160; layers/linear.py):
+ *   out[M, N] = x[M, K] W[N, K]^T + bias[N]
+ * M <= 64, bf16 / fp16 with fp32 accumulation, N % 16 == 0, K % 512 == 0; x rows x_row_stride elements apart
+ * (a multiple of 8), W dense, bias in the element type or NULL; x and W 16-byte aligned.  Larger M (prefill) stays
+ * a library GEMM: MVLLM_ERR_UNSUPPORTED.
+ */
+int mvllm_linear_small_m(void* out, const void* x, const void* w, const void* bias, int64_t x_row_stride,
+                         int M, int N, int K, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

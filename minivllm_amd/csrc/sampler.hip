@@ -65,7 +65,12 @@ template <typename T>
 __global__ __launch_bounds__(kSampleThreads) void sample_tokens_kernel(
     int64_t* __restrict__ out, float2* __restrict__ partial, const T* __restrict__ logits, int64_t row_stride,
     const float* __restrict__ temperatures, const float* __restrict__ noise, uint32_t seed_lo, uint32_t seed_hi,
-    uint32_t off_lo, uint32_t off_hi, int vocab, int slices) {
+    uint32_t off_lo, uint32_t off_hi, const uint64_t* __restrict__ offset_dev, int vocab, int slices) {
+  if (offset_dev) {      // the call offset lives on the device (a captured graph cannot change a launch argument)
+    const uint64_t off = *offset_dev + (((uint64_t)off_hi << 32) | off_lo);
+    off_lo = (uint32_t)off;
+    off_hi = (uint32_t)(off >> 32);
+  }
   __shared__ float best_s[kSampleThreads / 64];
   __shared__ int best_i[kSampleThreads / 64];
   const int b = blockIdx.x;
@@ -149,10 +154,9 @@ extern "C" size_t mvllm_sample_tokens_workspace_bytes(int batch, int vocab) {
   return slices <= 1 ? 0 : (size_t)batch * (size_t)slices * sizeof(float2);
 }
 
-extern "C" int mvllm_sample_tokens(int64_t* out_ids, const void* logits, int64_t row_stride,
-                                   const float* temperatures, const float* noise, uint64_t seed, uint64_t offset,
-                                   int batch, int vocab, int dtype, void* workspace, size_t workspace_bytes,
-                                   void* stream) {
+static int sample_entry(int64_t* out_ids, const void* logits, int64_t row_stride, const float* temperatures,
+                        const float* noise, uint64_t seed, uint64_t offset, const uint64_t* offset_dev, int batch,
+                        int vocab, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
   const int esize = dtype_size(dtype);
   if (esize == 0) return MVLLM_ERR_BAD_DTYPE;
   if (batch < 0 || vocab <= 0 || row_stride < vocab) return MVLLM_ERR_BAD_SHAPE;
@@ -173,17 +177,62 @@ extern "C" int mvllm_sample_tokens(int64_t* out_ids, const void* logits, int64_t
   switch (dtype) {
     case MVLLM_F32:
       sample_tokens_kernel<float><<<grid, block, 0, s>>>(out_ids, part, (const float*)logits, row_stride, temperatures,
-                                                        noise, sl, sh, ol, oh, vocab, slices);
+                                                        noise, sl, sh, ol, oh, offset_dev, vocab, slices);
       break;
     case MVLLM_BF16:
       sample_tokens_kernel<bf16_t><<<grid, block, 0, s>>>(out_ids, part, (const bf16_t*)logits, row_stride, temperatures,
-                                                         noise, sl, sh, ol, oh, vocab, slices);
+                                                         noise, sl, sh, ol, oh, offset_dev, vocab, slices);
       break;
     default:
       sample_tokens_kernel<f16_t><<<grid, block, 0, s>>>(out_ids, part, (const f16_t*)logits, row_stride, temperatures,
-                                                        noise, sl, sh, ol, oh, vocab, slices);
+                                                        noise, sl, sh, ol, oh, offset_dev, vocab, slices);
       break;
   }
   if (slices > 1) sample_combine_kernel<<<dim3((unsigned)batch), dim3(64), 0, s>>>(out_ids, part, slices);
+  return launch_status();
+}
+
+extern "C" int mvllm_sample_tokens(int64_t* out_ids, const void* logits, int64_t row_stride,
+                                   const float* temperatures, const float* noise, uint64_t seed, uint64_t offset,
+                                   int batch, int vocab, int dtype, void* workspace, size_t workspace_bytes,
+                                   void* stream) {
+  return sample_entry(out_ids, logits, row_stride, temperatures, noise, seed, offset, nullptr, batch, vocab, dtype,
+                      workspace, workspace_bytes, stream);
+}
+
+extern "C" int mvllm_sample_tokens_dev_offset(int64_t* out_ids, const void* logits, int64_t row_stride,
+                                              const float* temperatures, uint64_t seed, const uint64_t* offset_dev,
+                                              int batch, int vocab, int dtype, void* workspace,
+                                              size_t workspace_bytes, void* stream) {
+  if (!offset_dev) return MVLLM_ERR_NULL_POINTER;
+  return sample_entry(out_ids, logits, row_stride, temperatures, nullptr, seed, 0, offset_dev, batch, vocab, dtype,
+                      workspace, workspace_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------
+// The step metadata of a decode batch that continues the step before it (the same sequences, each one token longer),
+// moved forward on the device: next input = the id just sampled, context length, position and slot + 1.  One launch
+// in place of the host rebuilding and copying the four tensors (ModelRunner.prepare_decode,
+// src/myvllm/engine/model_runner.py:231-256).
+// ---------------------------------------------------------------------------
+__global__ void decode_advance_kernel(int64_t* __restrict__ input_ids, int64_t* __restrict__ context_lens,
+                                      int64_t* __restrict__ positions, int64_t* __restrict__ slot_mapping,
+                                      const int64_t* __restrict__ sampled, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  input_ids[i] = sampled[i];
+  const int64_t ctx = context_lens[i] + 1;
+  context_lens[i] = ctx;
+  positions[i] = ctx - 1;
+  slot_mapping[i] += 1;
+}
+
+extern "C" int mvllm_decode_advance(int64_t* input_ids, int64_t* context_lens, int64_t* positions,
+                                    int64_t* slot_mapping, const int64_t* sampled, int batch, void* stream) {
+  if (batch < 0) return MVLLM_ERR_BAD_SHAPE;
+  if (batch == 0) return MVLLM_OK;
+  if (!input_ids || !context_lens || !positions || !slot_mapping || !sampled) return MVLLM_ERR_NULL_POINTER;
+  decode_advance_kernel<<<dim3((unsigned)((batch + 63) / 64)), dim3(64), 0, (hipStream_t)stream>>>(
+      input_ids, context_lens, positions, slot_mapping, sampled, batch);
   return launch_status();
 }

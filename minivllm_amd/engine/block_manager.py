@@ -38,6 +38,7 @@ class BlockManager:
         self.blocks = [Block(i) for i in range(num_blocks)]
         self.hash_to_block_id: dict[int, int] = {}
         self.free_block_ids: deque[int] = deque(range(num_blocks))
+        self.deferred: list = []          # (sequence, block index) whose hash waits for a token id
         self.used_block_ids: set[int] = set()
 
     @staticmethod
@@ -118,10 +119,29 @@ class BlockManager:
             table.append(block.block_id)
         last = self.blocks[table[-1]]
         if len(seq) % self.block_size == 0:
-            token_ids = seq.block(seq.num_blocks - 1)
-            prefix = self.blocks[table[-2]].hash if len(table) > 1 else -1
-            h = self.compute_hash(token_ids, prefix)
-            last.update(h, token_ids)
-            self.hash_to_block_id[h] = last.block_id
+            if seq.token_ids[-1] < 0:
+                # the token that fills the block is still on its way from the device (engine steps launched ahead
+                # of their ids): the hash follows when it arrives
+                self.deferred.append((seq, seq.num_blocks - 1))
+            else:
+                self._hash_block(seq, seq.num_blocks - 1)
         else:
             assert last.hash == -1, "a partial block carries no hash"
+
+    def _hash_block(self, seq: Sequence, index: int) -> None:
+        table = seq.block_table
+        block = self.blocks[table[index]]
+        token_ids = seq.block(index)
+        prefix = self.blocks[table[index - 1]].hash if index > 0 else -1
+        h = self.compute_hash(token_ids, prefix)
+        block.update(h, token_ids)
+        self.hash_to_block_id[h] = block.block_id
+
+    def hash_deferred_blocks(self) -> None:
+        """Hashes postponed by ``append``; a sequence that was finished or preempted in between has given its
+        blocks back and is skipped (its blocks simply stay unshared)."""
+        for seq, index in self.deferred:
+            if index < len(seq.block_table) and self.blocks[seq.block_table[index]].hash == -1 \
+                    and all(t >= 0 for t in seq.block(index)):
+                self._hash_block(seq, index)
+        self.deferred = []

@@ -24,6 +24,8 @@ class LLMEngine:
         # longest sequence (prompt + new tokens) the rotary table and the graph's block-table buffer are sized for
         self.max_model_length = min(config.get("max_model_length", config.get("max_position", 4096)),
                                     config.get("max_position", 4096))
+        self.async_decode = config.get("async_decode", True)
+        self.pending = None          # (ids on their way, placeholders to fill, sequences that step finished)
         self.stats = {"prefill_tokens": 0, "decode_tokens": 0, "prefill_s": 0.0, "decode_s": 0.0, "steps": 0}
 
     def add_prompt(self, prompt_token_ids: list[int], sampling_params: SamplingParams) -> None:
@@ -39,28 +41,58 @@ class LLMEngine:
         self.scheduler.add_sequence(Sequence(prompt_token_ids, sampling_params, self.block_size))
 
     def step(self):
-        """One schedule -> run -> postprocess round.  Always a 3-tuple (finished, processed tokens, is_prefill)."""
+        """One schedule -> run -> postprocess round.  Always a 3-tuple (finished, processed tokens, is_prefill).
+
+        With ``async_decode`` (default) a decode step whose sequences all ignore EOS is launched without waiting
+        for its token ids: lengths, block tables and the finish-by-count do not depend on them, the next step's
+        input ids are taken from the device, and the host schedules and launches step t + 1 while the GPU runs
+        step t.  Such a step's ids are committed, and its finished sequences reported, one ``step`` later (or by
+        ``flush``); everything that needs real ids (a prefill, a sequence that stops at EOS, a batch that changed)
+        commits first."""
+        finished = []
+        if self.pending is not None and self.scheduler.waiting:
+            finished += self.flush()                   # admission hashes prompt blocks: ids must be real
         seqs, is_prefill = self.scheduler.schedule()
         if not seqs:
-            return [], 0, is_prefill
-        token_ids = self.model_runner.run(seqs, is_prefill)
+            return finished + self.flush(), 0, is_prefill
+        runner = self.model_runner
+        if (self.async_decode and not is_prefill and all(seq.ignore_eos for seq in seqs)
+                and hasattr(runner, "launch_decode") and runner.can_launch_decode(seqs)):
+            if not runner.continues_last_decode(seqs):
+                finished += self.flush()               # the buffers are refilled from the last tokens
+            handle = runner.launch_decode(seqs)
+            finished += self.flush()                   # the step before this one, while the GPU runs this one
+            slots = self.scheduler.postprocess_provisional(seqs)
+            self.pending = (handle, slots, [seq for seq in seqs if seq.is_finished])
+            return finished, len(seqs), False
+        finished += self.flush()
+        token_ids = runner.run(seqs, is_prefill)
         self.scheduler.postprocess(seqs, token_ids)
-        finished = [(seq.seq_id, seq.completion_token_ids) for seq in seqs if seq.is_finished]
+        finished += [(seq.seq_id, seq.completion_token_ids) for seq in seqs if seq.is_finished]
         processed = sum(len(seq) - 1 for seq in seqs) if is_prefill else len(seqs)
         return finished, processed, is_prefill
+
+    def flush(self):
+        """Commit the token ids of a decode step that was launched ahead; returns the sequences it finished."""
+        if self.pending is None:
+            return []
+        handle, slots, done = self.pending
+        self.pending = None
+        self.scheduler.commit(slots, handle.wait())
+        return [(seq.seq_id, seq.completion_token_ids) for seq in done]
 
     def generate(self, prompts: list[list[int]], sampling_params: SamplingParams, verbose: bool = False) -> dict:
         for prompt in prompts:
             self.add_prompt(prompt, sampling_params)
         done = {}
-        while not self.scheduler.is_finished():
+        while not self.scheduler.is_finished() or self.pending is not None:
             t0 = time.perf_counter()
             finished, processed, is_prefill = self.step()
             dt = time.perf_counter() - t0
             kind = "prefill" if is_prefill else "decode"
             self.stats[kind + "_tokens"] += processed
             self.stats[kind + "_s"] += dt
-            self.stats["steps"] += 1
+            self.stats["steps"] += 1 if processed else 0
             if verbose:
                 print(f"{processed} tokens, {processed / (dt + 1e-10):.1f} tokens/sec during {kind}")
             done.update(finished)

@@ -5,7 +5,9 @@ group, no SHM workers).
 Config keys (one set of names; the reference's runner and engine disagree on two of them): model keys
 ``vocab_size hidden_size num_layers num_heads num_kv_heads head_dim intermediate_size base
 rms_norm_epsilon qkv_bias ffn_bias scale tie_word_embeddings max_position``; engine keys ``block_size
-max_cached_blocks max_num_sequences max_num_batched_tokens dtype kv_cache_dtype seed``.
+max_cached_blocks max_num_sequences max_num_batched_tokens dtype kv_cache_dtype seed``; ``linear_small_rows`` (default
+32): projections of at most that many rows, a decode step, run as the single-launch ``linear_small_m`` (0: always the
+library GEMM; above 32 rows the library is faster).
 """
 from __future__ import annotations
 
@@ -14,12 +16,23 @@ import torch
 from minivllm_amd.engine.metadata import decode_metadata, prefill_metadata
 from minivllm_amd.layers.attention import decode_workspace_bytes
 from minivllm_amd.layers.basic import Sampler
-from minivllm_amd.layers.fused import sample_tokens
+from minivllm_amd.layers.fused import decode_advance, sample_tokens, sample_tokens_into, sample_workspace_bytes
 from minivllm_amd.models.qwen3 import Qwen3ForCausalLM
 from minivllm_amd.utils.context import reset_context, set_context
 
 _DTYPES = {"bf16": torch.bfloat16, "bfloat16": torch.bfloat16, "fp16": torch.float16, "float16": torch.float16,
            "fp32": torch.float32, "float32": torch.float32}
+
+
+class PendingTokens:
+    """Token ids of a launched decode step on their way to the host."""
+
+    def __init__(self, host: torch.Tensor, done: torch.cuda.Event):
+        self.host, self.done = host, done
+
+    def wait(self) -> list[int]:
+        self.done.synchronize()
+        return self.host.tolist()
 
 
 class ModelRunner:
@@ -39,13 +52,16 @@ class ModelRunner:
             intermediate_size=config["intermediate_size"], ffn_bias=config.get("ffn_bias", True),
             num_layers=config["num_layers"], tie_word_embeddings=config.get("tie_word_embeddings", True),
             block_size=self.block_size, kv_cache_dtype=self.kv_cache_dtype,
-            fused_qk=config.get("fused_qk", True), fused_elementwise=config.get("fused_elementwise", True))
+            fused_qk=config.get("fused_qk", True), fused_elementwise=config.get("fused_elementwise", True),
+            small_rows=config.get("linear_small_rows", 32))
         self.model.reset_parameters(seed=config.get("seed", 0))
         self.model.to(device=self.device, dtype=self.dtype).eval()
         self.sampler = Sampler()
         self.fused_sampler = config.get("fused_sampler", True)
         self.seed = config.get("seed", 0)
         self.sample_calls = 0
+        self._pinned = None          # pinned host buffers of launch_decode
+        self._dev_step = None        # host mirror of the graphs' device-side sampler call counter
         self._steady = None          # description of the batch in the static decode buffers (graph decode)
         self._last_sampled = None    # device tensor of the ids sampled by the last graph decode step
         self.generator = torch.Generator(device=self.device).manual_seed(config.get("seed", 0))
@@ -111,26 +127,35 @@ class ModelRunner:
 
     @torch.inference_mode()
     def capture_decode_graphs(self):
-        """Record one hipGraph of the decode forward pass per batch-size bucket (model_runner.py:316-369).
+        """Record one hipGraph of a whole decode step per batch-size bucket (model_runner.py:316-369): the forward
+        pass, the LM head and the sampler.
 
-        The step metadata lives in static device buffers that ``run`` refills before every replay; rows past
-        the real batch carry slot -1, context length 0 and whatever table entries were there, which the
-        kernels treat as "store nothing, output zeros".  Positions are derived from the context lengths inside
-        the graph.  The attention library allocates nothing and its grids depend only on the static shapes
-        (batch bucket, table width), so a replay is valid for any contents of the buffers."""
+        The step metadata lives in static device buffers that ``run`` refills or advances before every replay;
+        rows past the real batch carry slot -1, context length 0, temperature 1 and whatever table entries were
+        there, which the kernels treat as "store nothing, output zeros".  The attention library allocates nothing
+        and its grids depend only on the static shapes (batch bucket, table width), so a replay is valid for any
+        contents of the buffers.  The sampler's call offset is a device counter that the graph itself increments
+        (a replay cannot change a launch argument), kept equal to ``sample_calls``, so a run draws the same noise
+        whether its steps are replayed or launched one by one."""
         cfg = self.config
         max_bs = cfg.get("max_num_sequences", 16)
         max_len = cfg.get("max_model_length", cfg.get("max_position", 4096))
         max_blocks = -(-max_len // self.block_size)
         dev = self.device
+        buckets = sorted({b for b in [1, 2, 4, 8] + list(range(16, max_bs + 1, 16)) + [max_bs] if b <= max_bs})
+        ws_bytes = max(sample_workspace_bytes(b, cfg["vocab_size"]) for b in buckets) if self.fused_sampler else 0
         self.graph_vars = dict(
             input_ids=torch.zeros(max_bs, dtype=torch.int64, device=dev),
+            positions=torch.zeros(max_bs, dtype=torch.int64, device=dev),
             slot_mapping=torch.full((max_bs,), -1, dtype=torch.int64, device=dev),
             context_lens=torch.zeros(max_bs, dtype=torch.int64, device=dev),
             block_tables=torch.zeros(max_bs, max_blocks, dtype=torch.int32, device=dev),
+            temperatures=torch.ones(max_bs, dtype=torch.float32, device=dev),
+            sampled=torch.zeros(max_bs, dtype=torch.int64, device=dev),
+            step=torch.zeros(1, dtype=torch.int64, device=dev),
+            sample_ws=torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev),
             outputs=torch.zeros(max_bs, cfg["hidden_size"], dtype=self.dtype, device=dev))
         v = self.graph_vars
-        buckets = sorted({b for b in [1, 2, 4, 8] + list(range(16, max_bs + 1, 16)) + [max_bs] if b <= max_bs})
         self._own_decode_workspace(buckets, max_blocks)
         pool = None
         for bs in reversed(buckets):
@@ -138,8 +163,15 @@ class ModelRunner:
                         block_tables=v["block_tables"][:bs])
 
             def forward():
-                positions = (v["context_lens"][:bs] - 1).clamp_min(0)
-                v["outputs"][:bs] = self.model(v["input_ids"][:bs], positions)
+                hidden = self.model(v["input_ids"][:bs], v["positions"][:bs])
+                if not self.fused_sampler:                 # the module-chain sampler draws from a host-side generator
+                    v["outputs"][:bs] = hidden
+                    return
+                logits = torch.nn.functional.linear(hidden, self.model.lm_head_weight)
+                nbytes = sample_workspace_bytes(bs, cfg["vocab_size"])
+                sample_tokens_into(v["sampled"][:bs], logits, v["temperatures"][:bs], self.seed, v["step"],
+                                   v["sample_ws"][:nbytes] if nbytes else None)
+                v["step"] += 1
 
             forward()                                    # warm-up outside the capture (library handles, lazy loads)
             torch.cuda.synchronize()
@@ -150,6 +182,7 @@ class ModelRunner:
             self.graphs[bs] = graph
             torch.cuda.synchronize()
             reset_context()
+        self._dev_step = None                            # value of the device counter, unknown after the warm-ups
 
     def _own_decode_workspace(self, buckets, max_blocks):
         """One split-K scratch buffer for every decode call of this runner, allocated before any graph is
@@ -170,30 +203,36 @@ class ModelRunner:
         md = decode_metadata(seqs, self.block_size)
         v = self.graph_vars
         v["input_ids"][:bs].copy_(self._to_device(md["input_ids"], torch.int64))
+        v["positions"][:gbs].zero_()
+        v["positions"][:bs].copy_(self._to_device([n - 1 for n in md["context_lens"]], torch.int64))
+        v["temperatures"][:gbs].fill_(1.0)
+        v["temperatures"][:bs].copy_(self._to_device([seq.temperature for seq in seqs], torch.float32))
         v["slot_mapping"][:gbs].fill_(-1)
         v["slot_mapping"][:bs].copy_(self._to_device(md["slot_mapping"], torch.int64))
         v["context_lens"][:gbs].zero_()
         v["context_lens"][:bs].copy_(self._to_device(md["context_lens"], torch.int64))
         tables = self._to_device(md["block_tables"], torch.int32)
         v["block_tables"][:bs, :tables.size(1)].copy_(tables)
-        self._steady = dict(key=tuple(seq.seq_id for seq in seqs), lens=[len(seq) for seq in seqs],
-                            temperatures=self._to_device([seq.temperature for seq in seqs], torch.float32))
+        self._steady = dict(key=tuple(seq.seq_id for seq in seqs), lens=[len(seq) for seq in seqs])
+
+    def continues_last_decode(self, seqs) -> bool:
+        """The same sequences as in the last graph decode step, each one token longer."""
+        st = self._steady
+        if st is None or self._last_sampled is None or st["key"] != tuple(seq.seq_id for seq in seqs):
+            return False
+        return all(len(seq) == m + 1 for seq, m in zip(seqs, st["lens"]))
 
     def _advance_decode_buffers(self, seqs) -> bool:
         """The same sequences as in the last graph decode step, each one token longer: the buffers move on the
         device (input = the ids sampled last step, context length and slot + 1) and only sequences that started a
         new block are patched from the host.  Returns False when the batch is not such a continuation."""
+        if not self.continues_last_decode(seqs):
+            return False
         st = self._steady
-        if st is None or self._last_sampled is None or st["key"] != tuple(seq.seq_id for seq in seqs):
-            return False
         lens = [len(seq) for seq in seqs]
-        if any(n != m + 1 for n, m in zip(lens, st["lens"])):
-            return False
         bs = len(seqs)
         v = self.graph_vars
-        v["input_ids"][:bs].copy_(self._last_sampled)
-        v["context_lens"][:bs] += 1
-        v["slot_mapping"][:bs] += 1
+        decode_advance(v["input_ids"], v["context_lens"], v["positions"], v["slot_mapping"], self._last_sampled)
         fresh = [i for i, n in enumerate(lens) if (n - 1) % self.block_size == 0]     # token n-1 opens a block
         if fresh:
             rows = self._to_device(fresh, torch.int64)
@@ -205,34 +244,67 @@ class ModelRunner:
         return True
 
     def _replay_decode(self, seqs):
+        """One decode step from the captured graph; returns the sampled ids (a view of a static device buffer that
+        the next replay overwrites), or with the module-chain sampler the hidden states."""
         bs = len(seqs)
         gbs = next(b for b in sorted(self.graphs) if b >= bs)
         if not self._advance_decode_buffers(seqs):
             self._fill_decode_buffers(seqs, gbs)
+        v = self.graph_vars
+        if self.fused_sampler and self._dev_step != self.sample_calls:
+            v["step"].fill_(self.sample_calls)
         self.graphs[gbs].replay()
-        return self.graph_vars["outputs"][:bs], self._steady["temperatures"]
+        if not self.fused_sampler:
+            return v["outputs"][:bs]
+        self.sample_calls += 1
+        self._dev_step = self.sample_calls
+        return v["sampled"][:bs]
+
+    def can_launch_decode(self, seqs) -> bool:
+        """A decode step of these sequences can be launched without waiting for its token ids: the captured graph
+        covers the batch and the sampler is the single-launch one."""
+        return bool(self.graphs) and len(seqs) <= max(self.graphs) and self.fused_sampler
+
+    @torch.inference_mode()
+    def launch_decode(self, seqs) -> "PendingTokens":
+        """Enqueue one decode step and return at once; the sampled ids travel to a pinned host buffer behind the
+        step and are read with ``PendingTokens.wait()``.  The next step's input ids are taken from the device
+        copy, so the host can schedule and launch step t + 1 while the GPU still runs step t.  When the batch
+        does not continue the last step's, the buffers are refilled from the sequences' last tokens, which must be
+        real by then (the caller commits outstanding ids first)."""
+        sampled = self._replay_decode(seqs)
+        self._last_sampled = sampled
+        if self._pinned is None:
+            self._pinned = [torch.empty(max(self.graphs), dtype=torch.int64, pin_memory=True) for _ in range(2)]
+        host = self._pinned[self.sample_calls & 1][:len(seqs)]     # two buffers: step t's ids are read after step t + 1 is launched
+        host.copy_(sampled, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return PendingTokens(host, done)
 
     @torch.inference_mode()
     def run(self, seqs, is_prefill: bool) -> list[int]:
         if not is_prefill and self.graphs and len(seqs) <= max(self.graphs):
-            hidden, temperatures = self._replay_decode(seqs)
-            graphed = True
+            out = self._replay_decode(seqs)
+            if self.fused_sampler:
+                self._last_sampled = out                       # next step's input ids, if it continues this batch
+                token_ids = out.tolist()
+                reset_context()
+                return token_ids
+            logits = torch.nn.functional.linear(out, self.model.lm_head_weight)
+            temperatures = self._to_device([seq.temperature for seq in seqs], torch.float32)
         else:
             input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
             temperatures = self._to_device([seq.temperature for seq in seqs], torch.float32)
-            hidden = self.model(input_ids, positions)
-            graphed = False
-        logits = self.model.compute_logits(hidden) if not graphed else torch.nn.functional.linear(
-            hidden, self.model.lm_head_weight)
+            logits = self.model.compute_logits(self.model(input_ids, positions))
         if self.fused_sampler:
             # one launch over the LM-head output; draws are a function of (seed, step), so a run is reproducible
             sampled = sample_tokens(logits, temperatures, self.seed, self.sample_calls)
             self.sample_calls += 1
         else:
             sampled = self.sampler(logits, temperatures, self.generator)
-        self._last_sampled = sampled if graphed else None      # next step's input ids, if it continues this batch
-        if not graphed:
-            self._steady = None
+        self._last_sampled = None
+        self._steady = None
         token_ids = sampled.tolist()
         reset_context()
         return token_ids

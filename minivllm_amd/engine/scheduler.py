@@ -69,6 +69,31 @@ class Scheduler:
         seq.status = SequenceStatus.WAITING
         self.waiting.appendleft(seq)
 
+    PLACEHOLDER = -1        # stands for a sampled token whose id has not reached the host yet
+
+    def postprocess_provisional(self, seqs: list[Sequence]) -> list[tuple[Sequence, int]]:
+        """``postprocess`` for a decode step whose token ids are still on the device: every sequence grows by a
+        placeholder and finishes by count (callers use this only when every sequence ignores EOS, so nothing
+        else depends on the ids).  Returns (sequence, index of the placeholder) for ``commit``."""
+        slots = []
+        for seq in seqs:
+            seq.append_token(self.PLACEHOLDER)
+            slots.append((seq, seq.num_tokens - 1))
+            if seq.num_completion_tokens >= seq.max_tokens:
+                seq.status = SequenceStatus.FINISHED
+                self.block_manager.deallocate(seq)
+                self.running.remove(seq)
+        return slots
+
+    def commit(self, slots: list[tuple[Sequence, int]], token_ids: list[int]) -> None:
+        """The ids of a provisional step have arrived: replace the placeholders, then give the blocks that filled
+        up in the meantime their hashes."""
+        for (seq, index), token_id in zip(slots, token_ids):
+            seq.token_ids[index] = int(token_id)
+            if index == seq.num_tokens - 1:
+                seq.last_token = int(token_id)
+        self.block_manager.hash_deferred_blocks()
+
     def postprocess(self, seqs: list[Sequence], token_ids: list[int]) -> None:
         for seq, token_id in zip(seqs, token_ids):
             seq.append_token(int(token_id))

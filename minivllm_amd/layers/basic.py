@@ -8,7 +8,21 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from minivllm_amd.layers.fused import add_rms_norm, silu_and_mul
+from minivllm_amd.layers.fused import add_rms_norm, linear_small_m, linear_small_m_takes, silu_and_mul
+
+
+class Linear(nn.Linear):
+    """``nn.Linear`` (layers/linear.py) whose calls with at most ``small_rows`` rows (a decode step) run as one HIP
+    launch built for that size (``linear_small_m``); everything else, prefill included, is the library GEMM."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, small_rows: int = 0):
+        super().__init__(in_features, out_features, bias=bias)
+        self.small_rows = small_rows
+
+    def forward(self, x):
+        if self.small_rows and linear_small_m_takes(x, self.weight, self.small_rows):
+            return linear_small_m(x, self.weight, self.bias)
+        return F.linear(x, self.weight, self.bias)
 
 
 class RMSNorm(nn.Module):

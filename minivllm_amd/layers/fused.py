@@ -16,7 +16,7 @@ import torch
 
 from minivllm_amd import _C
 
-__all__ = ["qk_norm_rope_store", "sample_tokens", "add_rms_norm", "silu_and_mul"]
+__all__ = ["qk_norm_rope_store", "sample_tokens", "sample_tokens_into", "decode_advance", "add_rms_norm", "silu_and_mul", "linear_small_m", "linear_small_m_takes"]
 
 
 def _ptr(t):
@@ -152,6 +152,40 @@ def sample_tokens(logits: torch.Tensor, temperatures: torch.Tensor, seed: int = 
     return out
 
 
+def sample_tokens_into(out: torch.Tensor, logits: torch.Tensor, temperatures: torch.Tensor, seed: int,
+                       offset_dev: torch.Tensor, workspace: torch.Tensor | None) -> None:
+    """``sample_tokens`` for a captured graph: nothing is allocated (``out`` int64 (batch,), ``workspace`` uint8 from
+    ``sample_workspace_bytes`` or None) and the call offset is read from ``offset_dev`` (one uint64 / int64 on the
+    device, which the graph increments), so every replay draws fresh noise."""
+    _C.require_cuda(out, logits, temperatures, offset_dev, workspace)
+    batch, vocab = logits.shape
+    if logits.stride(1) != 1 or out.numel() != batch or out.dtype != torch.int64 or temperatures.dtype != torch.float32:
+        raise ValueError("logits rows must be dense, out int64 (batch,), temperatures float32 (batch,)")
+    st = _C.load().mvllm_sample_tokens_dev_offset(
+        _ptr(out), _ptr(logits), logits.stride(0) if batch > 1 else vocab, _ptr(temperatures),
+        int(seed) & (2 ** 64 - 1), _ptr(offset_dev), batch, vocab, _C.dtype_code(logits.dtype), _ptr(workspace),
+        0 if workspace is None else workspace.numel(), _C.current_stream_ptr(logits.device))
+    _C.check(st, "sample_tokens_into")
+
+
+def sample_workspace_bytes(batch: int, vocab: int) -> int:
+    return int(_C.load().mvllm_sample_tokens_workspace_bytes(batch, vocab))
+
+
+def decode_advance(input_ids: torch.Tensor, context_lens: torch.Tensor, positions: torch.Tensor,
+                   slot_mapping: torch.Tensor, sampled: torch.Tensor) -> None:
+    """Move a decode batch's step metadata one token forward on the device (all int64 (batch,), in place):
+    input = the id sampled last step, context length + 1, position = new length - 1, slot + 1."""
+    _C.require_cuda(input_ids, context_lens, positions, slot_mapping, sampled)
+    n = sampled.numel()
+    for t in (input_ids, context_lens, positions, slot_mapping, sampled):
+        if t.dtype != torch.int64 or t.numel() < n or not t.is_contiguous():
+            raise ValueError("decode_advance takes contiguous int64 tensors of at least the batch size")
+    st = _C.load().mvllm_decode_advance(_ptr(input_ids), _ptr(context_lens), _ptr(positions), _ptr(slot_mapping),
+                                        _ptr(sampled), n, _C.current_stream_ptr(sampled.device))
+    _C.check(st, "decode_advance")
+
+
 def _rows2d(name, t):
     if t.dim() != 2:
         raise ValueError(f"{name} must be (rows, features), got {tuple(t.shape)}")
@@ -201,4 +235,34 @@ def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
         st = lib.mvllm_silu_and_mul(_ptr(out), _ptr(x), rows, two_w // 2, stride, _C.dtype_code(x.dtype),
                                     _C.current_stream_ptr(x.device))
         _C.check(st, "silu_and_mul")
+    return out
+
+
+def linear_small_m_takes(x: torch.Tensor, weight: torch.Tensor, max_rows: int = 64) -> bool:
+    """Whether ``linear_small_m`` is built for this call: at most 64 rows, bf16 / fp16 on the GPU, N a multiple of 16,
+    K a multiple of 512, rows of x dense."""
+    return (x.is_cuda and x.dim() == 2 and 0 < x.shape[0] <= min(max_rows, 64) and x.dtype in (torch.bfloat16, torch.float16)
+            and weight.dtype == x.dtype and weight.is_contiguous() and weight.shape[0] % 16 == 0
+            and weight.shape[1] % 512 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0)
+
+
+def linear_small_m(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``F.linear(x, weight, bias)`` for the few rows of a decode step (the reference's projections,
+    models/qwen3.py:90-94, 118, 121-160, are library GEMMs): one HIP launch in which every wave asks for its whole
+    share of the weights at once, so the call costs about one memory round trip.  x (M <= 64, K), weight (N, K)
+    contiguous, bias (N,) or None, all in one 16-bit dtype; fp32 accumulation.  Returns (M, N)."""
+    _C.require_cuda(x, weight, bias)
+    if x.dim() != 2 or weight.dim() != 2 or weight.shape[1] != x.shape[1]:
+        raise ValueError(f"x (M, K) and weight (N, K) expected, got {tuple(x.shape)} and {tuple(weight.shape)}")
+    if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise ValueError("x, weight and bias must share one dtype")
+    if not weight.is_contiguous() or x.stride(1) != 1:
+        raise ValueError("weight must be contiguous and the rows of x dense")
+    m, k = x.shape
+    n = weight.shape[0]
+    out = torch.empty(m, n, dtype=x.dtype, device=x.device)
+    st = _C.load().mvllm_linear_small_m(_ptr(out), _ptr(x), _ptr(weight), _ptr(bias), x.stride(0) if m > 1 else k,
+                                        m, n, k, _C.dtype_code(x.dtype), _C.current_stream_ptr(x.device))
+    _C.check(st, "linear_small_m")
     return out

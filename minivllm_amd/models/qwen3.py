@@ -14,22 +14,22 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from minivllm_amd.layers.attention import Attention
-from minivllm_amd.layers.basic import RMSNorm, RotaryEmbedding, SiluAndMul
+from minivllm_amd.layers.basic import Linear, RMSNorm, RotaryEmbedding, SiluAndMul
 from minivllm_amd.utils.context import get_context
 
 
 class Qwen3Attention(nn.Module):
     def __init__(self, hidden_size, num_heads, head_dim, scale, num_kv_heads, rms_norm_epsilon, qkv_bias,
-                 rotary: RotaryEmbedding, block_size, kv_cache_dtype, fused_qk=True):
+                 rotary: RotaryEmbedding, block_size, kv_cache_dtype, fused_qk=True, small_rows=0):
         super().__init__()
         self.num_heads, self.num_kv_heads, self.head_dim = num_heads, num_kv_heads, head_dim
         self.q_size, self.kv_size = num_heads * head_dim, num_kv_heads * head_dim
-        self.qkv_projection = nn.Linear(hidden_size, self.q_size + 2 * self.kv_size, bias=qkv_bias)
+        self.qkv_projection = Linear(hidden_size, self.q_size + 2 * self.kv_size, bias=qkv_bias, small_rows=small_rows)
         self.qkv_bias = qkv_bias
         self.rms_norm = RMSNorm(head_dim, rms_norm_epsilon)      # one gamma shared by q and k (qwen3.py:50, 104-106)
         self.rotary_emb = rotary
         self.attention = Attention(num_heads, head_dim, scale, num_kv_heads, block_size, kv_cache_dtype)
-        self.output_projection = nn.Linear(self.q_size, hidden_size, bias=False)
+        self.output_projection = Linear(self.q_size, hidden_size, bias=False, small_rows=small_rows)
         self.fused_qk = fused_qk
 
     def forward(self, x, positions):
@@ -53,11 +53,11 @@ class Qwen3Attention(nn.Module):
 
 
 class Qwen3MLP(nn.Module):
-    def __init__(self, hidden_size, intermediate_size, bias, fused=True):
+    def __init__(self, hidden_size, intermediate_size, bias, fused=True, small_rows=0):
         super().__init__()
-        self.gate_up = nn.Linear(hidden_size, 2 * intermediate_size, bias=bias)
+        self.gate_up = Linear(hidden_size, 2 * intermediate_size, bias=bias, small_rows=small_rows)
         self.activation = SiluAndMul(fused)
-        self.gate_down = nn.Linear(intermediate_size, hidden_size, bias=bias)
+        self.gate_down = Linear(intermediate_size, hidden_size, bias=bias, small_rows=small_rows)
 
     def forward(self, x):
         return self.gate_down(self.activation(self.gate_up(x)))
@@ -65,12 +65,13 @@ class Qwen3MLP(nn.Module):
 
 class Qwen3DecoderLayer(nn.Module):
     def __init__(self, hidden_size, intermediate_size, ffn_bias, rms_norm_epsilon, fused_elementwise=True,
-                 **attn_kwargs):
+                 small_rows=0, **attn_kwargs):
         super().__init__()
         self.input_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
-        self.self_attn = Qwen3Attention(hidden_size=hidden_size, rms_norm_epsilon=rms_norm_epsilon, **attn_kwargs)
+        self.self_attn = Qwen3Attention(hidden_size=hidden_size, rms_norm_epsilon=rms_norm_epsilon,
+                                        small_rows=small_rows, **attn_kwargs)
         self.post_attention_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
-        self.mlp = Qwen3MLP(hidden_size, intermediate_size, ffn_bias, fused_elementwise)
+        self.mlp = Qwen3MLP(hidden_size, intermediate_size, ffn_bias, fused_elementwise, small_rows)
 
     def forward(self, x, residual, positions):
         if residual is None:
@@ -87,7 +88,7 @@ class Qwen3ForCausalLM(nn.Module):
     def __init__(self, vocab_size, hidden_size, num_heads, head_dim=None, scale=1.0, num_kv_heads=None,
                  rms_norm_epsilon=1e-6, qkv_bias=False, base=1_000_000, max_position=4096,
                  intermediate_size=3072, ffn_bias=True, num_layers=8, tie_word_embeddings=True,
-                 block_size=256, kv_cache_dtype="auto", fused_qk=True, fused_elementwise=True):
+                 block_size=256, kv_cache_dtype="auto", fused_qk=True, fused_elementwise=True, small_rows=0):
         super().__init__()
         head_dim = head_dim if head_dim is not None else hidden_size // num_heads
         num_kv_heads = num_kv_heads if num_kv_heads is not None else num_heads
@@ -97,7 +98,7 @@ class Qwen3ForCausalLM(nn.Module):
             Qwen3DecoderLayer(hidden_size, intermediate_size, ffn_bias, rms_norm_epsilon, num_heads=num_heads,
                               head_dim=head_dim, scale=scale, num_kv_heads=num_kv_heads, qkv_bias=qkv_bias,
                               rotary=rotary, block_size=block_size, kv_cache_dtype=kv_cache_dtype,
-                              fused_qk=fused_qk, fused_elementwise=fused_elementwise)
+                              fused_qk=fused_qk, fused_elementwise=fused_elementwise, small_rows=small_rows)
             for _ in range(num_layers)])
         self.final_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
         self.lm_head_weight = self.embedding_layer.weight if tie_word_embeddings else nn.Parameter(
@@ -116,7 +117,9 @@ class Qwen3ForCausalLM(nn.Module):
                     p.fill_(1.0)
 
     def forward(self, input_ids, positions):
-        x = self.embedding_layer(input_ids)
+        # a decode step's few rows by plain indexing: the embedding operator's small-batch kernel takes 11 us for 16
+        # rows, the gather 4
+        x = self.embedding_layer.weight[input_ids] if input_ids.numel() <= 256 else self.embedding_layer(input_ids)
         residual = None
         for layer in self.layer_stack:
             x, residual = layer(x, residual, positions)

@@ -28,8 +28,8 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_noalloc", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_plan", "mvllm_prefill_varlen",
-              "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_workspace_bytes",
-              "mvllm_add_rms_norm",
+              "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_dev_offset", "mvllm_decode_advance", "mvllm_sample_tokens_workspace_bytes",
+              "mvllm_add_rms_norm", "mvllm_linear_small_m",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
         assert n in names
 
@@ -160,6 +160,17 @@ def test_argument_validation_without_gpu():
     assert act(0, 0, 2, 3072, 6144, 1, 0) == -1
     assert act(0, 0, 2, 3072, 3072, 1, 0) == -3                            # stride < 2 * width
     assert act(0, 0, 2, 3001, 6002, 1, 0) == -4                            # width not a multiple of 16 bytes
+    lin = lib.mvllm_linear_small_m
+    assert lin(0, 0, 0, 0, 1024, 0, 4096, 1024, 1, 0) == 0                 # no rows
+    assert lin(0, 0, 0, 0, 1024, 4, 4096, 1024, 1, 0) == -1                # null pointers
+    assert lin(16, 16, 16, 0, 1024, 65, 4096, 1024, 1, 0) == -4            # more than 64 rows: the library GEMM's
+    assert lin(16, 16, 16, 0, 1024, 4, 4100, 1024, 1, 0) == -4             # N % 16
+    assert lin(16, 16, 16, 0, 1000, 4, 4096, 1000, 1, 0) == -4             # K % 512
+    assert lin(16, 16, 16, 0, 512, 4, 4096, 1024, 1, 0) == -3              # row stride < K
+    assert lin(16, 16, 16, 0, 1024, 4, 4096, 1024, 0, 0) == -4             # fp32
+    adv = lib.mvllm_decode_advance
+    assert adv(0, 0, 0, 0, 0, 0, 0) == 0 and adv(0, 0, 0, 0, 0, 4, 0) == -1 and adv(0, 0, 0, 0, 0, -1, 0) == -3
+    assert lib.mvllm_sample_tokens_dev_offset(8, 8, 100, 8, 1, 0, 4, 100, 1, 0, 0, 0) == -1       # no counter
     fused = lib.mvllm_qk_norm_rope_store
     #     q_out k_out v_out q k v | strides | gamma eps cos max_pos pos slots | caches scales int8 | T slots Hq Hkv D dt stream
     assert fused(0, 0, 0, 0, 0, 0, 512, 256, 256, 0, 1e-6, 0, 64, 0, 0, 0, 0, 0, 0, 0, 0, 0, 4, 2, 128, 1, 0) == 0   # no tokens

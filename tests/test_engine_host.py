@@ -217,3 +217,78 @@ def test_decode_workspace_need_is_not_monotonic_and_the_runner_sizes_for_the_max
         assert need[48] > need[64] > 0                 # 48 x 32 partitions against 64 x 16
         sized = max(need.values())
         assert all(n <= sized for n in need.values())
+
+
+class FakeAsyncRunner(FakeRunner):
+    """A runner that can launch decode steps ahead of their ids, as the model runner's hipGraph path does."""
+
+    class Handle:
+        def __init__(self, ids, log):
+            self.ids, self.log = ids, log
+
+        def wait(self):
+            self.log.append("wait")
+            return self.ids
+
+    def __init__(self):
+        super().__init__()
+        self.log = []
+        self.last = None
+
+    def can_launch_decode(self, seqs):
+        return True
+
+    def continues_last_decode(self, seqs):
+        return self.last is not None and self.last[0] == [s.seq_id for s in seqs] and \
+            all(len(s) == n + 1 for s, n in zip(seqs, self.last[1]))
+
+    def launch_decode(self, seqs):
+        if not self.continues_last_decode(seqs):
+            assert all(t >= 0 for s in seqs for t in s.token_ids), "a refill needs real last tokens"
+        self.log.append("launch")
+        ids = super().run(seqs, False)
+        self.last = ([s.seq_id for s in seqs], [len(s) for s in seqs])
+        return self.Handle(ids, self.log)
+
+    def run(self, seqs, is_prefill):
+        assert all(t >= 0 for s in seqs for t in s.token_ids), "a synchronous step needs real token ids"
+        self.last = None
+        self.log.append("run")
+        return super().run(seqs, is_prefill)
+
+
+def test_decode_steps_launched_ahead_of_their_ids_give_the_same_run():
+    """async_decode: decode steps of sequences that ignore EOS are launched before the previous step's ids reach
+    the host.  Tokens, finish order, freed blocks and the hashes of the blocks that filled up on the way must equal
+    the synchronous engine's; every launch but the first of a batch happens before the wait for the step before."""
+    cfg = dict(max_num_sequences=3, max_num_batched_tokens=64, max_cached_blocks=24, block_size=4, eos=-1,
+               max_position=64)
+    prompts = [[1, 2, 3], [4, 5, 6, 7, 8], [9], [10, 11, 12, 13, 14, 15, 16]]
+    sp = SamplingParams(temperature=0.6, max_tokens=9, ignore_eos=True)
+    engines = {}
+    for mode in (False, True):
+        runner = FakeAsyncRunner()
+        eng = LLMEngine(dict(cfg, async_decode=mode), model_runner=runner)
+        out = eng.generate(prompts, sp)["token_ids"]
+        engines[mode] = (out, eng, runner)
+        assert [len(t) for t in out] == [9] * 4 and all(t >= 0 for seq in out for t in seq)
+        assert eng.scheduler.is_finished() and eng.pending is None
+        assert len(eng.scheduler.block_manager.free_block_ids) == 24
+    assert engines[True][0] == engines[False][0]
+    hashes = [set(engines[mode][1].scheduler.block_manager.hash_to_block_id) for mode in (True, False)]
+    assert hashes[0] == hashes[1] and len(hashes[0]) >= 8
+    log = engines[True][2].log
+    assert "wait" in log and "launch" in log and "wait" not in engines[False][2].log
+    # steady state: launch(t + 1) comes before wait(t)
+    assert "launch launch launch" not in " ".join(log)             # one step outstanding besides the one just launched
+    assert sum(1 for a, b in zip(log, log[1:]) if a == "launch" and b == "wait") >= 6
+
+
+def test_a_sequence_that_stops_at_eos_keeps_the_synchronous_path():
+    cfg = dict(max_num_sequences=2, max_num_batched_tokens=64, max_cached_blocks=16, block_size=4, eos=1003,
+               max_position=64)
+    runner = FakeAsyncRunner()
+    eng = LLMEngine(cfg, model_runner=runner)
+    out = eng.generate([[1, 2, 3], [4, 5]], SamplingParams(temperature=0.6, max_tokens=8, ignore_eos=False))
+    assert "launch" not in runner.log                              # EOS decides the schedule: ids first
+    assert [t[-1] for t in out["token_ids"]].count(1003) == 1 and min(len(t) for t in out["token_ids"]) < 8

@@ -43,6 +43,7 @@ def test_decode_steps_agree_with_one_prefill_of_the_same_tokens():
         eng.add_prompt(p, sp)
     for _ in range(1 + 20):
         eng.step()
+    eng.flush()                                      # ids of a step launched ahead, if any
     seqs = list(eng.scheduler.running)
     assert len(seqs) == 5 and all(s.num_completion_tokens == 21 for s in seqs)
     runner = eng.model_runner
@@ -199,6 +200,7 @@ def test_config5_full_shape():
         eng.add_prompt(p, sp)
     for _ in range(1 + 60):
         eng.step()
+    eng.flush()
     seqs = list(eng.scheduler.running)
     assert len(seqs) == 12 and all(s.num_completion_tokens == 61 for s in seqs)
     assert any(len(s.block_table) == 2 for s in seqs)              # the block boundary was crossed in decode

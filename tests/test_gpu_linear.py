@@ -1,0 +1,71 @@
+"""linear_small_m (the decode step's projections as one HIP launch) against the fp32 product of the same 16-bit
+inputs.  Tolerance: the result is the fp32 sum rounded once to the element type, so |err| <= 2^-8 |want| (bf16; 2^-11
+for fp16) plus fp32 summation-order noise, allowed as 2e-3 absolute."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from minivllm_amd.layers.basic import Linear
+from minivllm_amd.layers.fused import decode_advance, linear_small_m, linear_small_m_takes
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _case(seed, m, n, k, dtype, bias, stride=None):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, stride or k, generator=g).to(dtype).to(DEV)[:, :k]
+    w = (torch.randn(n, k, generator=g) * 0.05).to(dtype).to(DEV)
+    b = (torch.randn(n, generator=g) * 0.5).to(dtype).to(DEV) if bias else None
+    return x, w, b
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 33, 48, 60, 64])
+@pytest.mark.parametrize("n,k,bias", [(4096, 1024, False), (1024, 2048, False), (6144, 1024, True), (1024, 3072, True),
+                                      (48, 512, True), (16, 8192, False)])
+def test_linear_small_m_vs_fp32_product(dtype, m, n, k, bias):
+    """The engine's four projection shapes (QKV, output, gate/up, down) and the extremes of the wave split: few
+    columns with a long K (16 waves share a column tile) and a short K."""
+    x, w, b = _case(70 + m, m, n, k, dtype, bias)
+    assert linear_small_m_takes(x, w)
+    got = linear_small_m(x, w, b).float().cpu()
+    want = (x.float() @ w.float().T + (b.float() if bias else 0)).cpu()
+    assert got.shape == (m, n)
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    slack = ((got - want).abs() - want.abs() * ulp).max().item()
+    assert slack <= 2e-3, slack
+
+
+def test_linear_small_m_strided_rows_and_module_dispatch():
+    """Rows of x may be slices of a wider tensor; the module takes the HIP launch up to its row limit and the
+    library GEMM beyond, with the same result up to the rounding of the output."""
+    x, w, b = _case(90, 24, 1024, 1024, torch.bfloat16, True, stride=1536)
+    assert x.stride(0) == 1536 and linear_small_m_takes(x, w)
+    want = F.linear(x, w, b).float()
+    got = linear_small_m(x, w, b).float()
+    assert (got - want).abs().max().item() <= 0.05 and (got - want).abs().mean().item() <= 2e-3
+    lin = Linear(1024, 1024, bias=True, small_rows=32).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        lin.bias.copy_(b)
+        small = lin(x.contiguous())
+        big = lin(x.contiguous().repeat(4, 1))                    # 96 rows: F.linear
+    assert big.shape == (96, 1024)
+    assert (small.float() - big[:24].float()).abs().max().item() <= 0.05
+    assert torch.equal(small, linear_small_m(x.contiguous(), w, b))
+    assert not linear_small_m_takes(x.float(), w.float())         # fp32 stays with the library
+    assert not linear_small_m_takes(torch.zeros(65, 1024, dtype=torch.bfloat16, device=DEV), w)
+    assert not linear_small_m_takes(torch.zeros(40, 1024, dtype=torch.bfloat16, device=DEV), w, max_rows=32)
+
+
+def test_decode_advance_moves_the_step_metadata_forward():
+    ids = torch.tensor([5, 6, 7, 8], device=DEV)
+    ctx = torch.tensor([10, 256, 3, 0], device=DEV)
+    pos = torch.zeros(4, dtype=torch.int64, device=DEV)
+    slots = torch.tensor([9, 511, 40, -1], device=DEV)
+    sampled = torch.tensor([100, 200, 300], device=DEV)           # a batch of three inside buffers of four
+    decode_advance(ids, ctx, pos, slots, sampled)
+    torch.cuda.synchronize()
+    assert ids.tolist() == [100, 200, 300, 8] and ctx.tolist() == [11, 257, 4, 0]
+    assert pos.tolist() == [10, 256, 3, 0] and slots.tolist() == [10, 512, 41, -1]
