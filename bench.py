@@ -619,6 +619,8 @@ def bench_mfma_probe(args):
                        "nv v_fma_f32 + ne v_exp_f32", "mixes": {}}
     for wps in (1, 2):
         res["mixes"][f"mfma_only_{wps}wave_per_simd"] = run(0, 0, 0, wps)
+    for chains, wps in ((1, 1), (2, 1), (1, 2), (2, 2)):      # fewer accumulator chains: an MFMA waits for the one before it
+        res["mixes"][f"mfma_only_{chains}chain_{wps}wave_per_simd"] = run(100, chains, 0, wps)
     for nv, ne in ((2, 0), (4, 0), (6, 0), (8, 0), (0, 1), (3, 1), (4, 1)):
         res["mixes"][f"same_wave_nv{nv}_ne{ne}_2waves_per_simd"] = run(nv, ne, 0, 2)
     res["mixes"]["same_wave_nv4_ne1_1wave_per_simd"] = run(4, 1, 0, 1)

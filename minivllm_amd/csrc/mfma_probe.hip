@@ -31,6 +31,9 @@ typedef __attribute__((ext_vector_type(8))) __bf16 v8bf16;
 // the whole iteration is ONE asm statement: the compiler puts nothing between the instructions
 #define MIXED(valu) asm volatile(MFMA(0, 0) valu MFMA(1, 1) valu MFMA(2, 0) valu MFMA(3, 1) valu : OPERANDS)
 #define VECTOR_ONLY(valu) asm volatile(valu valu valu valu : OPERANDS)
+// one accumulator chain (every MFMA waits for the one before it) and two chains
+#define CHAIN1 asm volatile(MFMA(0, 0) MFMA(0, 1) MFMA(0, 0) MFMA(0, 1) : OPERANDS)
+#define CHAIN2 asm volatile(MFMA(0, 0) MFMA(1, 1) MFMA(0, 0) MFMA(1, 1) : OPERANDS)
 
 // MIX = 10 * (fmas per slot) + (exps per slot)
 template <int MIX, bool DO_MFMA>
@@ -39,6 +42,8 @@ __device__ __forceinline__ void body(v16f& c0, v16f& c1, v16f& c2, v16f& c3, con
                                      float& x4, float& x5, float& x6, float& x7, float& x8, float k) {
   if constexpr (DO_MFMA) {
     if constexpr (MIX == 0) MIXED(V0);
+    if constexpr (MIX == 1001) CHAIN1;
+    if constexpr (MIX == 1002) CHAIN2;
     if constexpr (MIX == 20) MIXED(V2);
     if constexpr (MIX == 30) MIXED(V3);
     if constexpr (MIX == 40) MIXED(V4);
@@ -114,7 +119,7 @@ static int launch(int role, int waves_per_simd, int blocks, float* out, int iter
 // One launch of `blocks` workgroups of 4 * waves_per_simd waves; every wave runs `iters` iterations of 4 slots, a slot
 // being one MFMA + nv v_fma_f32 + ne v_exp_f32 (role 0), the two halves on different waves of a SIMD (role 1, needs
 // waves_per_simd == 2), or the vector half alone (role 2).  (nv, ne) in {(0,0) (2,0) (3,0) (4,0) (6,0) (8,0) (0,1)
-// (3,1) (4,1)}.  Returns 0, -1 for an unsupported mix, or a hipError_t.
+// (3,1) (4,1)}; (100,1) and (100,2): MFMAs only, on one and on two accumulator chains instead of four.  Returns 0, -1 for an unsupported mix, or a hipError_t.
 extern "C" int mvllm_probe_mfma_mix(int nv, int ne, int role, int waves_per_simd, int blocks, float* out, int iters,
                                     void* stream) {
   hipStream_t s = (hipStream_t)stream;
@@ -131,6 +136,8 @@ extern "C" int mvllm_probe_mfma_mix(int nv, int ne, int role, int waves_per_simd
     case 1: return launch<1>(role, waves_per_simd, blocks, out, iters, s);
     case 31: return launch<31>(role, waves_per_simd, blocks, out, iters, s);
     case 41: return launch<41>(role, waves_per_simd, blocks, out, iters, s);
+    case 1001: return launch<1001>(role, waves_per_simd, blocks, out, iters, s);   // nv = 100, ne = 1: one MFMA chain
+    case 1002: return launch<1002>(role, waves_per_simd, blocks, out, iters, s);   // nv = 100, ne = 2: two chains
   }
   return -1;
 }
