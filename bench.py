@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,engine,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,loads_probe,engine,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -83,6 +83,48 @@ def roofline(bound, achieved, kernel):
     return {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak, "kernel": kernel}
 
 
+_probe = None
+
+
+def probe_lib():
+    """libmvllm_probe.so with the decode entry points bound like the operator library's."""
+    global _probe
+    if _probe is None:
+        import ctypes
+        from minivllm_amd import _C
+        lib = ctypes.CDLL(os.path.join(ROOT, "minivllm_amd", "libmvllm_probe.so"))
+        for name in ("mvllm_paged_decode", "mvllm_paged_decode_int8", "mvllm_paged_decode_workspace_bytes"):
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = _C.SIGNATURES[name]
+        _probe = lib
+    return _probe
+
+
+def loads_only_decode_ms(args, q, kc, vc, td, cd, scale, hq, hkv, d, bs, scales=None):
+    """The same decode call on the probe library's build of the kernels, which issues every load of the real kernel
+    (same grid, partitions, block-table walk, instructions) and folds the registers with xor instead of computing:
+    what the access pattern alone reaches on this GPU.  Returns event ms per call."""
+    import torch
+    from minivllm_amd import _C
+    lib = probe_lib()
+    batch, mb = td.shape
+    out = torch.empty_like(q)
+    nbytes = lib.mvllm_paged_decode_workspace_bytes(batch, hq, d, mb, bs)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+    stream = torch.cuda.current_stream().cuda_stream
+    common = (td.data_ptr(), mb, cd.data_ptr(), int(cd.dtype == torch.int64), batch, hq, hkv, d, bs, kc.shape[0],
+              float(scale), _C.dtype_code(q.dtype), ws.data_ptr(), nbytes, stream)
+
+    def call():
+        if scales is None:
+            st = lib.mvllm_paged_decode(out.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), *common)
+        else:
+            st = lib.mvllm_paged_decode_int8(out.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                             scales[0].data_ptr(), scales[1].data_ptr(), *common)
+        assert st == 0, st
+    return time_steps(call, args.steps, args.warmup, EXTRA_WARM_MS)[1]
+
+
 def decode_bytes(ctx, block_size, num_heads, num_kv_heads, head_dim, kv_elem, q_elem, ctx_elem, int8_scales=False):
     """Algorithmic HBM bytes of one decode call: every live K/V element once, q read + out written once,
     one table entry per live block, one context length per sequence.  Split-K scratch is not counted."""
@@ -96,7 +138,7 @@ def decode_bytes(ctx, block_size, num_heads, num_kv_heads, head_dim, kv_elem, q_
     return total
 
 
-def bench_decode(args, block_size, want_cpu):
+def bench_decode(args, block_size, want_cpu, want_probe=False):
     import torch
     from helpers import extract_sequence, make_paged_case_on_device
     from minivllm_amd.layers.attention import paged_attention_decode
@@ -118,6 +160,11 @@ def bench_decode(args, block_size, want_cpu):
         "ms_per_step": wall_ms, "event_ms_per_step": event_ms,
         "gbs": nbytes / (wall_ms * 1e-3) / 1e9, "gbs_event": nbytes / (event_ms * 1e-3) / 1e9,
     }
+    if want_probe:
+        ms = loads_only_decode_ms(args, q, kc, vc, td, cd, scale, hq, hkv, d, block_size)
+        res["loads_only"] = {"event_ms_per_step": ms, "gbs": nbytes / (ms * 1e-3) / 1e9,
+                             "what": "the kernels' loads without the arithmetic (libmvllm_probe.so): the ceiling of this "
+                                     "access pattern; the real kernel reaches gbs_event / this"}
     cpu = None
     if want_cpu:
         import oracle
@@ -292,7 +339,7 @@ def bench_prefill_store(args, which, want_cpu=False):
     return out
 
 
-def bench_int8(args, want_cpu=True):
+def bench_int8(args, want_cpu=True, want_probe=False):
     """BASELINE.json config 4: B 128, ctx U[256,16384], Hq32/Hkv8/D128; K/V ~ N(0,1) with 1 % outliers at 8 sigma are
     quantised by store_kvcache_int8 into a block-16 int8 cache, then decoded with in-kernel dequantisation."""
     import torch
@@ -338,6 +385,10 @@ def bench_int8(args, want_cpu=True):
         args.steps, args.warmup, EXTRA_WARM_MS)
     nbytes = decode_bytes(ctx, bs, hq, hkv, d, 1, 2, 8, int8_scales=True)
     check = {}
+    if want_probe:
+        ms = loads_only_decode_ms(args, q, kc, vc, td, cd, scale, hq, hkv, d, bs, scales=(ks, vs))
+        check["loads_only"] = {"event_ms_per_step": ms, "gbs": nbytes / (ms * 1e-3) / 1e9,
+                               "what": "the INT8 kernels' loads without the arithmetic (libmvllm_probe.so)"}
     if want_cpu:
         # value check at full size on the launch plan of the full batch: the longest, the shortest and six more
         # sequences against the INT8 oracle (dequantise in fp32, naive decode)
@@ -689,7 +740,8 @@ def main():
     only = set(x for x in args.only.split(",") if x)
     want = lambda name: not only or name in only
     extra = {}
-    head, cpu = bench_decode(args, args.block_size, want_cpu=not args.no_cpu and want("cpu"))
+    head, cpu = bench_decode(args, args.block_size, want_cpu=not args.no_cpu and want("cpu"),
+                             want_probe=want("loads_probe"))
     if want("decode256") and args.block_size != 256:
         extra["decode_block256"], _ = bench_decode(args, 256, want_cpu=False)
     want_cpu = not args.no_cpu and want("cpu")
@@ -697,7 +749,7 @@ def main():
     if which:
         extra.update(bench_prefill_store(args, which, want_cpu))
     if want("int8"):
-        extra["int8"] = bench_int8(args, want_cpu)
+        extra["int8"] = bench_int8(args, want_cpu, want("loads_probe"))
     if want("reference_shapes"):
         extra["reference_benchmark_shapes"] = bench_reference_shapes(args, want_cpu)
     if want("decode_small"):
@@ -715,6 +767,8 @@ def main():
         extra["engine_16seq_graph"] = bench_engine(args, 16, True)
         extra["engine_64seq_graph"] = bench_engine(args, 64, True)
 
+    if "loads_only" in head:
+        extra["decode_loads_only"] = head["loads_only"]
     line = {
         "metric": "decode-attn HBM GB/s (% peak); prefill TFLOP/s (% MFMA); engine out tok/s",
         "value": head["gbs"],

@@ -43,9 +43,9 @@ def build_library(verbose: bool = True, jobs: int = 4) -> str:
     obj_dir = os.path.join(PKG_DIR, "build")
     os.makedirs(obj_dir, exist_ok=True)
 
-    def compile_one(src):
-        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    def compile_one(src, extra=(), suffix=""):
+        obj = os.path.join(obj_dir, src.replace(".hip", suffix + ".o"))
+        cmd = [hipcc, *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         res = subprocess.run(cmd, capture_output=True, text=True)
@@ -57,7 +57,10 @@ def build_library(verbose: bool = True, jobs: int = 4) -> str:
         return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
+        # the probe library also holds the decode kernels built as "loads only" (the access pattern's ceiling)
+        probe_decode = pool.submit(compile_one, "paged_decode.hip", ("-DMVLLM_DECODE_LOADS_ONLY=1",), "_loads_only")
         objs = list(pool.map(compile_one, SOURCES + PROBE_SOURCES))
+        objs.append(probe_decode.result())
     for lib, members in ((LIB_PATH, objs[:len(SOURCES)]), (PROBE_LIB_PATH, objs[len(SOURCES):])):
         cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *members]
         if verbose:

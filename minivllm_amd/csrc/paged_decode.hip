@@ -51,6 +51,9 @@ namespace mvllm {
 #ifndef MVLLM_DECODE_I8_WAVES_PER_EU
 #define MVLLM_DECODE_I8_WAVES_PER_EU 3
 #endif
+#ifndef MVLLM_DECODE_LOADS_ONLY
+#define MVLLM_DECODE_LOADS_ONLY 0   // 1: measurement build for libmvllm_probe.so: the MFMA decode kernels issue their loads and
+#endif                              // fold the loaded registers with xor instead of computing (results are meaningless)
 #ifndef MVLLM_DECODE_WPB
 #define MVLLM_DECODE_WPB 4          // waves (= kv heads) per workgroup, upper bound (8-wave workgroups: -1.5 %)
 #endif
@@ -387,6 +390,15 @@ struct DecodeHead {
   // (col_end: prefill only, where column n is a query row: tokens at or past it do not count for this lane's column)
   __device__ __forceinline__ void consume(const KVTile<T, D>& t, int part_end, float scale_log2, int lane,
                                           int col_end = 0x7fffffff) {
+    if constexpr (MVLLM_DECODE_LOADS_ONLY) {      // the loads of the tile and nothing else: the access pattern's ceiling
+      uint32_t x = 0;
+#pragma unroll
+      for (int j = 0; j < kSteps; ++j) x ^= t.k[j].x ^ t.k[j].y ^ t.k[j].z ^ t.k[j].w;
+#pragma unroll
+      for (int i = 0; i < 4 * kSets; ++i) x ^= t.v[i].x ^ t.v[i].y ^ t.v[i].z ^ t.v[i].w;
+      l += __uint_as_float(x & 1u);
+      return;
+    }
     const int cls = lane >> 4;
     const int tok_base = t.t0 + 4 * cls;
     const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
@@ -1048,6 +1060,15 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
   };
 
   auto consume = [&](const KVTileI8& t) {
+    if constexpr (MVLLM_DECODE_LOADS_ONLY) {
+      uint32_t x = __float_as_uint(t.ks) ^ __float_as_uint(t.vs);
+#pragma unroll
+      for (int j = 0; j < kSteps; ++j) x ^= t.k[j].x ^ t.k[j].y ^ t.k[j].z ^ t.k[j].w;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x ^= t.v[i].x ^ t.v[i].y;
+      l += __uint_as_float(x & 1u);
+      return;
+    }
     const int tok_base = t.t0 + 4 * q4;
     const bool partial = (!t.ok) || (t.t0 + kTile > part_end);
     const float ks4[4] = {quad_bcast<0>(t.ks), quad_bcast<1>(t.ks), quad_bcast<2>(t.ks), quad_bcast<3>(t.ks)};
