@@ -325,6 +325,32 @@ int mvllm_silu_and_mul(void* out, const void* in, int64_t rows, int width, int64
 int mvllm_linear_small_m(void* out, const void* x, const void* w, const void* bias, int64_t x_row_stride,
                          int M, int N, int K, int dtype, void* stream);
 
+/*
+ * The same product with the launches around it folded in, for the decoder layer's decode step
+ * (src/myvllm/models/qwen3.py:197-212: residual add + RMSNorm, projection; :151-160: gate/up, SiluAndMul):
+ *   gamma != NULL:  h = x + residual (rounded to the element type; residual NULL: h = x), residual_out = h (may be
+ *                   NULL), x' = h / sqrt(mean(h^2) + eps) * gamma rounded to the element type, exactly what
+ *                   mvllm_add_rms_norm writes (layers/layernorm.py:9-28) up to the order of the sum of squares;
+ *                   the product is taken of x'.  residual and residual_out are dense [M, K]; residual_out must not
+ *                   alias x or residual (every workgroup reads all of both while one of them writes a row).
+ *   glu != 0:       W is [2F, K] (gate rows, then up rows, as layers/activation.py:15-18 chunks the output), out is
+ *                   [M, F] = silu(x' Wg^T + bg) * (x' Wu^T + bu) with the roundings of mvllm_silu_and_mul on the
+ *                   rounded projection; N = 2F, N % 32 == 0.
+ * Shapes as mvllm_linear_small_m, and for gamma != NULL: M <= 32, N / 16 >= M, K / waves one burst of 128 or 256
+ * values (mvllm_linear_small_m_plan says whether a shape is taken); otherwise MVLLM_ERR_UNSUPPORTED and the caller
+ * runs the separate launches.
+ */
+int mvllm_norm_linear_small_m(void* out, void* residual_out, const void* x, const void* residual,
+                              const float* gamma, float eps, const void* w, const void* bias,
+                              int64_t x_row_stride, int M, int N, int K, int glu, int dtype, void* stream);
+
+/*
+ * Whether mvllm_linear_small_m (norm == 0 && glu == 0) or mvllm_norm_linear_small_m takes a shape, without a
+ * launch: MVLLM_OK and the waves per workgroup in *waves (may be NULL), or MVLLM_ERR_UNSUPPORTED.  No counterpart
+ * in the reference (its projections are library GEMMs of any shape).
+ */
+int mvllm_linear_small_m_plan(int M, int N, int K, int norm, int glu, int dtype, int* waves);
+
 #ifdef __cplusplus
 }
 #endif

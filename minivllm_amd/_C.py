@@ -50,6 +50,9 @@ SIGNATURES = {
     "mvllm_add_rms_norm": (c_int, [c_void_p] * 5 + [c_float, c_int64, c_int, c_int64, c_int64, c_int, c_void_p]),
     "mvllm_silu_and_mul": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int, c_void_p]),
     "mvllm_linear_small_m": (c_int, [c_void_p] * 4 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    "mvllm_norm_linear_small_m": (c_int, [c_void_p] * 5 + [c_float, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
+                                                            c_int, c_int, c_void_p]),
+    "mvllm_linear_small_m_plan": (c_int, [c_int] * 6 + [ctypes.POINTER(c_int)]),
     "mvllm_qk_norm_rope_store": (c_int, [c_void_p] * 6 + [c_int64] * 3 + [c_void_p, c_float, c_void_p, c_int64,
                                                            c_void_p, c_void_p] + [c_void_p] * 4 +
                                  [c_int, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p]),

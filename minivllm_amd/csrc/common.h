@@ -28,14 +28,10 @@ __device__ __forceinline__ float to_float(f16_t x) { return (float)x.v; }
 template <typename T> __device__ __forceinline__ T from_float(float x);
 template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float x) {
-  uint32_t u = __float_as_uint(x);
+  // the hardware conversion (v_cvt_pk_bf16_f32): nearest even, NaN stays NaN; as bit arithmetic with a NaN test it
+  // cost a dozen instructions and a branch per value
   bf16_t r;
-  if ((u & 0x7fffffffu) > 0x7f800000u) {  // NaN stays NaN
-    r.bits = (uint16_t)((u >> 16) | 0x0040u);
-  } else {
-    u += 0x7fffu + ((u >> 16) & 1u);
-    r.bits = (uint16_t)(u >> 16);
-  }
+  r.bits = __builtin_bit_cast(uint16_t, (__bf16)x);
   return r;
 }
 template <> __device__ __forceinline__ f16_t from_float<f16_t>(float x) {

@@ -16,7 +16,7 @@ import torch
 
 from minivllm_amd import _C
 
-__all__ = ["qk_norm_rope_store", "sample_tokens", "sample_tokens_into", "decode_advance", "add_rms_norm", "silu_and_mul", "linear_small_m", "linear_small_m_takes"]
+__all__ = ["qk_norm_rope_store", "sample_tokens", "sample_tokens_into", "decode_advance", "add_rms_norm", "silu_and_mul", "linear_small_m", "linear_small_m_takes", "norm_linear_small_m", "norm_linear_small_m_takes"]
 
 
 def _ptr(t):
@@ -266,3 +266,50 @@ def linear_small_m(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | N
                                         m, n, k, _C.dtype_code(x.dtype), _C.current_stream_ptr(x.device))
     _C.check(st, "linear_small_m")
     return out
+
+
+_PLAN_CACHE: dict = {}
+
+
+def norm_linear_small_m_takes(x: torch.Tensor, weight: torch.Tensor, max_rows: int = 32, norm: bool = True,
+                              glu: bool = False) -> bool:
+    """Whether ``norm_linear_small_m`` is built for this call (``mvllm_linear_small_m_plan``, remembered per shape)."""
+    if not linear_small_m_takes(x, weight, max_rows) or not x.is_contiguous():
+        return False
+    key = (x.shape[0], weight.shape[0], weight.shape[1], norm, glu, x.dtype)
+    if key not in _PLAN_CACHE:
+        st = _C.load().mvllm_linear_small_m_plan(key[0], key[1], key[2], int(norm), int(glu), _C.dtype_code(x.dtype), None)
+        _PLAN_CACHE[key] = st == 0
+    return _PLAN_CACHE[key]
+
+
+def norm_linear_small_m(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+                        gamma: torch.Tensor | None = None, eps: float = 1e-6, residual: torch.Tensor | None = None,
+                        want_residual: bool = False, glu: bool = False):
+    """A decode step's projection with the launches around it folded in (the reference runs them as separate
+    modules, models/qwen3.py:151-160, 197-212): with ``gamma`` (float32, (K,)) the rows are first replaced by
+    ``rms_norm(x + residual) * gamma`` as ``add_rms_norm`` computes it; with ``glu`` the weight is (2F, K) and the
+    result ``silu(gate) * up`` as ``silu_and_mul`` computes it.  Returns the (M, N) or (M, F) product, and with
+    ``want_residual`` also ``x + residual`` in x's dtype (a new tensor)."""
+    _C.require_cuda(x, weight, bias, gamma, residual)
+    if x.dim() != 2 or weight.dim() != 2 or weight.shape[1] != x.shape[1]:
+        raise ValueError(f"x (M, K) and weight (N, K) expected, got {tuple(x.shape)} and {tuple(weight.shape)}")
+    if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype) or (residual is not None and residual.dtype != x.dtype):
+        raise ValueError("x, weight, bias and residual must share one dtype")
+    if not weight.is_contiguous() or x.stride(1) != 1:
+        raise ValueError("weight must be contiguous and the rows of x dense")
+    m, k = x.shape
+    n = weight.shape[0]
+    if gamma is not None and (gamma.dtype != torch.float32 or tuple(gamma.shape) != (k,)):
+        raise ValueError("gamma must be float32 of shape (K,)")
+    if residual is not None and (tuple(residual.shape) != (m, k) or not residual.is_contiguous()):
+        raise ValueError("residual must be a contiguous (M, K) tensor")
+    if (residual is not None or want_residual) and gamma is None:
+        raise ValueError("a residual needs the norm (gamma)")
+    out = torch.empty(m, n // 2 if glu else n, dtype=x.dtype, device=x.device)
+    res_out = torch.empty(m, k, dtype=x.dtype, device=x.device) if want_residual else None
+    st = _C.load().mvllm_norm_linear_small_m(_ptr(out), _ptr(res_out), _ptr(x), _ptr(residual), _ptr(gamma), float(eps),
+                                             _ptr(weight), _ptr(bias), x.stride(0) if m > 1 else k, m, n, k, int(glu),
+                                             _C.dtype_code(x.dtype), _C.current_stream_ptr(x.device))
+    _C.check(st, "norm_linear_small_m")
+    return (out, res_out) if want_residual else out

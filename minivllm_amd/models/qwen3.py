@@ -15,6 +15,7 @@ import torch.nn.functional as F
 
 from minivllm_amd.layers.attention import Attention
 from minivllm_amd.layers.basic import Linear, RMSNorm, RotaryEmbedding, SiluAndMul
+from minivllm_amd.layers.fused import norm_linear_small_m, norm_linear_small_m_takes
 from minivllm_amd.utils.context import get_context
 
 
@@ -33,7 +34,11 @@ class Qwen3Attention(nn.Module):
         self.fused_qk = fused_qk
 
     def forward(self, x, positions):
-        q, k, v = self.qkv_projection(x).split([self.q_size, self.kv_size, self.kv_size], dim=-1)
+        return self.forward_qkv(self.qkv_projection(x), positions)
+
+    def forward_qkv(self, qkv, positions):
+        """Everything after the QKV projection (whose output a caller may have produced fused with the norm)."""
+        q, k, v = qkv.split([self.q_size, self.kv_size, self.kv_size], dim=-1)
         if self.fused_qk:
             # views of the projection output, no copies; norm + rotation + cache store in one launch
             q = q.unflatten(-1, (self.num_heads, self.head_dim))
@@ -72,8 +77,31 @@ class Qwen3DecoderLayer(nn.Module):
                                         small_rows=small_rows, **attn_kwargs)
         self.post_attention_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
         self.mlp = Qwen3MLP(hidden_size, intermediate_size, ffn_bias, fused_elementwise, small_rows)
+        self.small_rows, self.fused_elementwise = small_rows, fused_elementwise
+
+    def _forward_few_rows(self, x, residual, positions):
+        """A decode step's few rows: the two residual norms run as the prologues of the projections that follow them
+        and SiluAndMul as the epilogue of the gate/up projection (``norm_linear_small_m``): 6 launches per layer
+        instead of 9, same roundings."""
+        attn, mlp = self.self_attn, self.mlp
+        ln1, ln2 = self.input_layernorm, self.post_attention_layernorm
+        proj = attn.qkv_projection
+        if residual is None:
+            qkv = norm_linear_small_m(x, proj.weight, proj.bias, ln1.weight_fp32(), ln1.eps)
+            residual = x
+        else:
+            qkv, residual = norm_linear_small_m(x, proj.weight, proj.bias, ln1.weight_fp32(), ln1.eps, residual, True)
+        x = attn.forward_qkv(qkv, positions)
+        act, residual = norm_linear_small_m(x, mlp.gate_up.weight, mlp.gate_up.bias, ln2.weight_fp32(), ln2.eps,
+                                            residual, True, glu=True)
+        return mlp.gate_down(act), residual
 
     def forward(self, x, residual, positions):
+        rows = self.small_rows
+        if (rows and self.fused_elementwise and x.dim() == 2 and x.shape[0] <= rows and x.is_contiguous()
+                and norm_linear_small_m_takes(x, self.self_attn.qkv_projection.weight, rows)
+                and norm_linear_small_m_takes(x, self.mlp.gate_up.weight, rows, glu=True)):
+            return self._forward_few_rows(x, residual, positions)
         if residual is None:
             residual = x
             x = self.input_layernorm(x)

@@ -29,7 +29,7 @@ def test_header_declares_expected_entry_points():
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_noalloc", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_plan", "mvllm_prefill_varlen",
               "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_dev_offset", "mvllm_decode_advance", "mvllm_sample_tokens_workspace_bytes",
-              "mvllm_add_rms_norm", "mvllm_linear_small_m",
+              "mvllm_add_rms_norm", "mvllm_linear_small_m", "mvllm_norm_linear_small_m", "mvllm_linear_small_m_plan",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
         assert n in names
 
@@ -168,6 +168,23 @@ def test_argument_validation_without_gpu():
     assert lin(16, 16, 16, 0, 1000, 4, 4096, 1000, 1, 0) == -4             # K % 512
     assert lin(16, 16, 16, 0, 512, 4, 4096, 1024, 1, 0) == -3              # row stride < K
     assert lin(16, 16, 16, 0, 1024, 4, 4096, 1024, 0, 0) == -4             # fp32
+    nl = lib.mvllm_norm_linear_small_m
+    #    out res_out x res gamma eps w bias stride M N K glu dtype stream
+    assert nl(0, 0, 0, 0, 0, 1e-6, 0, 0, 1024, 0, 4096, 1024, 0, 1, 0) == 0          # no rows
+    assert nl(0, 0, 0, 0, 0, 1e-6, 0, 0, 1024, 4, 4096, 1024, 0, 1, 0) == -1         # null pointers
+    assert nl(16, 0, 16, 16, 0, 1e-6, 16, 0, 1024, 4, 4096, 1024, 0, 1, 0) == -1     # a residual without gamma
+    assert nl(16, 32, 32, 48, 64, 1e-6, 16, 0, 1024, 4, 4096, 1024, 0, 1, 0) == -3   # residual_out aliases x
+    assert nl(16, 0, 16, 0, 0, 1e-6, 16, 0, 1024, 4, 4112, 1024, 1, 1, 0) == -4      # glu: N % 32
+    plan = lib.mvllm_linear_small_m_plan
+    w = ctypes.c_int(0)
+    assert plan(16, 4096, 1024, 1, 0, 1, ctypes.byref(w)) == 0 and w.value == 4     # the engine's QKV projection
+    assert plan(32, 6144, 1024, 1, 1, 1, ctypes.byref(w)) == 0 and w.value == 4     # gate/up with norm and SiLU
+    assert plan(33, 4096, 1024, 1, 0, 1, None) == -4                                # norm: at most 32 rows
+    assert plan(33, 4096, 1024, 0, 0, 1, None) == 0                                 # plain: up to 64
+    assert plan(16, 1024, 3072, 1, 0, 1, None) == -4                                # K / waves is not one burst
+    assert plan(16, 1024, 2048, 1, 0, 1, ctypes.byref(w)) == 0 and w.value == 16    # 16 waves, 128 values each
+    assert plan(32, 1024, 2048, 1, 0, 1, None) == -4                                # ... with one row tile only
+    assert plan(16, 4096, 1024, 1, 0, 0, None) == -4 and plan(16, 4096, 1024, 1, 0, 9, None) == -2
     adv = lib.mvllm_decode_advance
     assert adv(0, 0, 0, 0, 0, 0, 0) == 0 and adv(0, 0, 0, 0, 0, 4, 0) == -1 and adv(0, 0, 0, 0, 0, -1, 0) == -3
     assert lib.mvllm_sample_tokens_dev_offset(8, 8, 100, 8, 1, 0, 4, 100, 1, 0, 0, 0) == -1       # no counter

@@ -6,7 +6,8 @@ import torch
 import torch.nn.functional as F
 
 from minivllm_amd.layers.basic import Linear
-from minivllm_amd.layers.fused import decode_advance, linear_small_m, linear_small_m_takes
+from minivllm_amd.layers.fused import (add_rms_norm, decode_advance, linear_small_m, linear_small_m_takes,
+                                       norm_linear_small_m, norm_linear_small_m_takes, silu_and_mul)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -57,6 +58,65 @@ def test_linear_small_m_strided_rows_and_module_dispatch():
     assert not linear_small_m_takes(x.float(), w.float())         # fp32 stays with the library
     assert not linear_small_m_takes(torch.zeros(65, 1024, dtype=torch.bfloat16, device=DEV), w)
     assert not linear_small_m_takes(torch.zeros(40, 1024, dtype=torch.bfloat16, device=DEV), w, max_rows=32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 32])
+@pytest.mark.parametrize("n,k,bias,glu", [(4096, 1024, False, False), (6144, 1024, True, True), (1024, 2048, True, False),
+                                          (2048, 512, True, True), (4096, 1024, True, True)])
+@pytest.mark.parametrize("with_residual", [True, False])
+def test_norm_linear_equals_the_separate_launches(dtype, m, n, k, bias, glu, with_residual):
+    """The fused projection against the launches it replaces (add_rms_norm -> linear_small_m -> silu_and_mul): the
+    next residual is bit-identical.  The product may differ only through the sum of squares, added in another order:
+    where its last bit differs, a normalised value can round the other way (about one in 2^13 fp16 values, 2^16 in
+    bf16), and that one input moves every output of its row by a fraction of a unit in the last place, so a row is
+    either bit-identical or has some outputs one unit off: every output within 2 units in the last place of the
+    largest output of its row, and at least 70 % of all outputs bit-identical."""
+    x, w, b = _case(300 + m, m, n, k, dtype, bias)
+    x = x.contiguous()
+    g = torch.Generator().manual_seed(m)
+    gamma = (1 + 0.2 * torch.randn(k, generator=g)).to(DEV)
+    res = torch.randn(m, k, generator=g).to(dtype).to(DEV) if with_residual else None
+    if not norm_linear_small_m_takes(x, w, 32, glu=glu):
+        assert m > 16 and k == 2048                      # 16 waves per column tile hold one row tile only
+        return
+    normed = add_rms_norm(x, gamma, 1e-6, res)
+    normed, want_res = normed if with_residual else (normed, x)
+    want = linear_small_m(normed, w, b)
+    if glu:
+        want = silu_and_mul(want)
+    got = norm_linear_small_m(x, w, b, gamma, 1e-6, res, want_residual=with_residual, glu=glu)
+    if with_residual:
+        got, got_res = got
+        assert torch.equal(got_res, want_res)
+    assert got.shape == want.shape == (m, n // 2 if glu else n)
+    same = (got == want).float().mean().item()
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    worst = ((got.float() - want.float()).abs() / want.float().abs().amax(dim=1, keepdim=True)).max().item()
+    assert same >= 0.7 and worst <= 2 * ulp, (same, worst)
+
+
+def test_norm_linear_without_norm_is_the_plain_product_and_glu_pairs_the_right_columns():
+    """gamma None: no norm, so the result equals linear_small_m bit for bit, and with glu equals silu_and_mul of it;
+    a weight whose gate rows are zero except one column pins the pairing of gate column j with up column j."""
+    x, w, b = _case(411, 9, 2048, 1024, torch.bfloat16, True)
+    x = x.contiguous()
+    assert torch.equal(norm_linear_small_m(x, w, b), linear_small_m(x, w, b))
+    assert torch.equal(norm_linear_small_m(x, w, b, glu=True), silu_and_mul(linear_small_m(x, w, b)))
+    w2 = torch.zeros_like(w)
+    b2 = torch.zeros_like(b)
+    j = 437                                              # silu(gate_j) * up_j: only column j can be non-zero
+    w2[j] = w[j]
+    w2[1024 + j] = w[1024 + j]
+    w2[1024 + j + 1] = w[1024 + j + 1]                   # an up column whose gate is zero: silu(0) * up = 0
+    out = norm_linear_small_m(x, w2, b2, glu=True).float()
+    full = x.float() @ w2.float().T
+    gate, up = full[:, j].bfloat16().float(), full[:, 1024 + j].bfloat16().float()
+    want = (torch.nn.functional.silu(gate).bfloat16().float() * up).bfloat16().float()
+    assert out[:, j].abs().max().item() > 0
+    assert (out[:, j] - want).abs().max().item() <= 2.0 ** -7 * want.abs().max().item()
+    out[:, j] = 0
+    assert out.abs().max().item() == 0
 
 
 def test_decode_advance_moves_the_step_metadata_forward():
