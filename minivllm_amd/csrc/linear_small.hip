@@ -25,6 +25,7 @@ struct LinearArgs {
   const void* bias;       // [N] in the element type, or null
   int64_t x_row_stride;   // elements between rows of x
   int M, N, K;
+  int cols;               // output columns per workgroup: 16, or 8 / 4 (plain product only) to spread few columns over more CUs
   // NORM: x is first replaced by rms_norm(x + residual) * gamma, as mvllm_add_rms_norm computes it
   const void* residual;   // [M, K] contiguous, or null (then the norm of x alone)
   void* residual_out;     // [M, K] contiguous: x + residual in the element type; must not alias x or residual
@@ -85,9 +86,10 @@ __global__ __launch_bounds__(64 * W) void linear_small_kernel(const LinearArgs a
     n0 = blockIdx.x * 8;
     wrow = col < 8 ? n0 + col : a.N / 2 + n0 + col - 8;
   } else {
-    n0 = blockIdx.x * 16;
-    wrow = n0 + col;
+    n0 = blockIdx.x * a.cols;
+    wrow = n0 + min(col, a.cols - 1);
   }
+  const bool wlive = GLU || col < a.cols;                // weight rows of a narrow tile: the other lanes load nothing
   const T* wp = reinterpret_cast<const T*>(a.w) + (int64_t)wrow * a.K + koff;
   int rowm[MT];
   const T* xp[MT];
@@ -102,7 +104,8 @@ __global__ __launch_bounds__(64 * W) void linear_small_kernel(const LinearArgs a
   for (int k = 0; k < ksl; k += 32 * U) {
     uint4 wf[U], xf[MT][U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) wf[u] = load16_stream(wp + k + 32 * u);      // weights are read once: stream them
+    for (int u = 0; u < U; ++u)                          // weights are read once: stream them
+      wf[u] = wlive ? load16_stream(wp + k + 32 * u) : make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -180,7 +183,7 @@ __global__ __launch_bounds__(64 * W) void linear_small_kernel(const LinearArgs a
   if (wave > 0) return;
   // lane l holds out[m = l % 16][weight row 4 (l / 16) + r of the workgroup], r < 4
   float b4[4] = {0.f, 0.f, 0.f, 0.f};
-  if (a.bias) {
+  if (a.bias && (GLU || 4 * cls < a.cols)) {
     const int brow = GLU ? (cls < 2 ? n0 + 4 * cls : a.N / 2 + n0 + 4 * (cls - 2)) : n0 + 4 * cls;
     const T* bp = reinterpret_cast<const T*>(a.bias) + brow;
 #pragma unroll
@@ -212,7 +215,7 @@ __global__ __launch_bounds__(64 * W) void linear_small_kernel(const LinearArgs a
         *reinterpret_cast<uint2*>(out + (int64_t)m * (a.N / 2) + n0 + 4 * cls) = *reinterpret_cast<const uint2*>(y4);
       }
     } else {
-      if (m < a.M)
+      if (m < a.M && 4 * cls < a.cols)
         *reinterpret_cast<uint2*>(out + (int64_t)m * a.N + n0 + 4 * cls) = *reinterpret_cast<const uint2*>(r4);
     }
   }
@@ -227,7 +230,7 @@ static bool norm_fits(int W, int mt, int steps) {
 
 template <typename T, int W, bool NORM, bool GLU>
 static int launch_linear_w(const LinearArgs& a, hipStream_t stream) {
-  const dim3 grid((unsigned)(a.N / 16)), block(64 * W);  // GLU: N / 2 / 8 workgroups, the same number
+  const dim3 grid((unsigned)(GLU ? a.N / 16 : a.N / a.cols)), block(64 * W);  // GLU: 8 gate + 8 up columns each
   const int mt = (a.M + 15) / 16;
   const int steps = a.K / W / 32;                        // 32-wide k steps per wave
   if constexpr (NORM) {
@@ -261,19 +264,33 @@ static int launch_linear_w(const LinearArgs& a, hipStream_t stream) {
   }
 }
 
-// waves per workgroup: more of them share a column tile's K when N alone gives too few workgroups to keep the
-// memory system busy (N = 1024: 64 column tiles)
-static int linear_waves(int N, int K) {
+#ifndef MVLLM_LINEAR_NARROW_COLS
+#define MVLLM_LINEAR_NARROW_COLS 8
+#endif
+// columns per workgroup of the plain product: narrower tiles when 16-column tiles would leave most CUs without
+// a workgroup (what a CU can keep in flight bounds its share of the weight stream)
+static int linear_cols(int N, bool plain) {
+  return plain && N / 16 < 128 ? MVLLM_LINEAR_NARROW_COLS : 16;
+}
+
+// waves per workgroup: more of them share a column tile's K when the column tiles alone give too few workgroups to
+// keep the memory system busy; 12 where 16 do not divide K but 12 do, each with one burst of 256 values (K = 3072:
+// the MLP's down projection)
+static int linear_waves(int tiles, int K, bool plain) {
   int w = 4;
-  while (w < 16 && (int64_t)(N / 16) * w < 1024 && K % (2 * w * 128) == 0) w *= 2;
+  while (w < 16 && (int64_t)tiles * w < 1024 && K % (2 * w * 128) == 0) w *= 2;
+  if (plain && w == 8 && (int64_t)tiles * w < 1024 && K == 12 * 256) w = 12;
   return w;
 }
 
 template <typename T, bool NORM, bool GLU>
 static int launch_linear_small(const LinearArgs& a, hipStream_t stream) {
-  switch (linear_waves(a.N, a.K)) {
+  switch (linear_waves(GLU ? a.N / 16 : a.N / a.cols, a.K, !NORM && !GLU)) {
     case 4: return launch_linear_w<T, 4, NORM, GLU>(a, stream);
     case 8: return launch_linear_w<T, 8, NORM, GLU>(a, stream);
+    case 12:
+      if constexpr (!NORM && !GLU) return launch_linear_w<T, 12, false, false>(a, stream);
+      else return MVLLM_ERR_UNSUPPORTED;
     default: return launch_linear_w<T, 16, NORM, GLU>(a, stream);
   }
 }
@@ -306,6 +323,7 @@ extern "C" int mvllm_linear_small_m(void* out, const void* x, const void* w, con
   if (bad || M == 0) return bad;
   LinearArgs a{};
   a.out = out; a.x = x; a.w = w; a.bias = bias; a.x_row_stride = x_row_stride; a.M = M; a.N = N; a.K = K;
+  a.cols = linear_cols(N, true);
   return dtype == MVLLM_BF16 ? launch_linear_fused<bf16_t>(a, false, (hipStream_t)stream)
                              : launch_linear_fused<f16_t>(a, false, (hipStream_t)stream);
 }
@@ -314,7 +332,7 @@ extern "C" int mvllm_linear_small_m_plan(int M, int N, int K, int norm, int glu,
   if (dtype != MVLLM_BF16 && dtype != MVLLM_F16) return dtype_size(dtype) == 0 ? MVLLM_ERR_BAD_DTYPE : MVLLM_ERR_UNSUPPORTED;
   if (M <= 0 || N <= 0 || K <= 0) return MVLLM_ERR_BAD_SHAPE;
   if (M > 64 || N % 16 != 0 || K % 512 != 0 || (glu && N % 32 != 0)) return MVLLM_ERR_UNSUPPORTED;
-  const int w = linear_waves(N, K), mt = (M + 15) / 16, steps = K / w / 32;
+  const int w = linear_waves(N / linear_cols(N, !norm && !glu), K, !norm && !glu), mt = (M + 15) / 16, steps = K / w / 32;
   if (norm ? (!norm_fits(w, mt, steps) || N / 16 < M) : (steps % 4 != 0)) return MVLLM_ERR_UNSUPPORTED;
   if (waves) *waves = w;
   return MVLLM_OK;
@@ -335,6 +353,7 @@ extern "C" int mvllm_norm_linear_small_m(void* out, void* residual_out, const vo
   LinearArgs a{};
   a.out = out; a.x = x; a.w = w; a.bias = bias; a.x_row_stride = x_row_stride; a.M = M; a.N = N; a.K = K;
   a.residual = residual; a.residual_out = residual_out; a.gamma = gamma; a.eps = eps;
+  a.cols = linear_cols(N, !gamma && !glu);
   return dtype == MVLLM_BF16 ? launch_linear_fused<bf16_t>(a, glu != 0, (hipStream_t)stream)
                              : launch_linear_fused<f16_t>(a, glu != 0, (hipStream_t)stream);
 }
