@@ -285,6 +285,27 @@ int mvllm_sample_tokens_dev_offset(int64_t* out_ids, const void* logits, int64_t
                                    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * LM head + sampler in one pass over the weights -- ParallelLMHead.forward (src/myvllm/layers/embedding_head.py:56-77:
+ * rows to sample from, hidden W^T) followed by SamplerLayer.forward (layers/sampler.py:14-19), without the
+ * (batch, vocab) logits reaching memory:
+ *   out_ids[b] = argmax_n( bf16(hidden[row_index[b]] . W[n]) / T[b] - log(max(E[b, n], 1e-10)) )
+ * with the logit rounded to the element type, as the materialised tensor would be, and E drawn as in
+ * mvllm_sample_tokens (Philox4x32-10, key = seed, counter = (n / 4, b, offset (+ *offset_dev when not NULL))): the
+ * same ids as mvllm_sample_tokens on the rounded product, up to the order of the fp32 sums inside a logit.
+ * hidden rows hidden_row_stride elements apart (a multiple of 8); row_index int64 [batch] or NULL (rows 0..batch-1:
+ * a decode step; the last token of every packed sequence in prefill, embedding_head.py:57-62); weight [vocab, K]
+ * dense.  batch <= 64, vocab % 16 == 0, K in {256, 512, 1024}, bf16 / fp16; otherwise MVLLM_ERR_UNSUPPORTED and the
+ * caller runs the library GEMM and mvllm_sample_tokens.  workspace: mvllm_lm_head_sample_workspace_bytes(batch, K)
+ * bytes, 8-byte aligned, caller-owned.  The first launch of a shape with more than 48 KB of hidden rows raises the
+ * kernel's dynamic LDS limit (a host-side attribute call: make it outside a graph capture).
+ */
+size_t mvllm_lm_head_sample_workspace_bytes(int batch, int K);
+int mvllm_lm_head_sample(int64_t* out_ids, const void* hidden, int64_t hidden_row_stride,
+                         const int64_t* row_index, const void* weight, const float* temperatures,
+                         uint64_t seed, uint64_t offset, const uint64_t* offset_dev, int batch, int vocab,
+                         int K, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * The step metadata of a decode batch that continues the step before it (same sequences, each one token longer),
  * advanced on the device in one launch instead of being rebuilt on the host as ModelRunner.prepare_decode does
  * (src/myvllm/engine/model_runner.py:231-256): input_ids[i] = sampled[i]; context_lens[i] += 1;

@@ -7,7 +7,8 @@ Config keys (one set of names; the reference's runner and engine disagree on two
 rms_norm_epsilon qkv_bias ffn_bias scale tie_word_embeddings max_position``; engine keys ``block_size
 max_cached_blocks max_num_sequences max_num_batched_tokens dtype kv_cache_dtype seed``; ``linear_small_rows`` (default
 32): projections of at most that many rows, a decode step, run as the single-launch ``linear_small_m`` (0: always the
-library GEMM; above 32 rows the library is faster).
+library GEMM; above 32 rows the library is faster); ``fused_lm_head`` (default true): LM head and sampler as one pass
+over the weights for at most 64 rows (``lm_head_sample``), otherwise the library GEMM and ``sample_tokens``.
 """
 from __future__ import annotations
 
@@ -16,9 +17,11 @@ import torch
 from minivllm_amd.engine.metadata import decode_metadata, prefill_metadata
 from minivllm_amd.layers.attention import decode_workspace_bytes
 from minivllm_amd.layers.basic import Sampler
-from minivllm_amd.layers.fused import decode_advance, sample_tokens, sample_tokens_into, sample_workspace_bytes
+from minivllm_amd.layers.fused import (decode_advance, lm_head_sample, lm_head_sample_takes,
+                                       lm_head_sample_workspace_bytes, sample_tokens, sample_tokens_into,
+                                       sample_workspace_bytes)
 from minivllm_amd.models.qwen3 import Qwen3ForCausalLM
-from minivllm_amd.utils.context import reset_context, set_context
+from minivllm_amd.utils.context import get_context, reset_context, set_context
 
 _DTYPES = {"bf16": torch.bfloat16, "bfloat16": torch.bfloat16, "fp16": torch.float16, "float16": torch.float16,
            "fp32": torch.float32, "float32": torch.float32}
@@ -58,6 +61,7 @@ class ModelRunner:
         self.model.to(device=self.device, dtype=self.dtype).eval()
         self.sampler = Sampler()
         self.fused_sampler = config.get("fused_sampler", True)
+        self.fused_lm_head = self.fused_sampler and config.get("fused_lm_head", True)
         self.seed = config.get("seed", 0)
         self.sample_calls = 0
         self._pinned = None          # pinned host buffers of launch_decode
@@ -144,6 +148,7 @@ class ModelRunner:
         dev = self.device
         buckets = sorted({b for b in [1, 2, 4, 8] + list(range(16, max_bs + 1, 16)) + [max_bs] if b <= max_bs})
         ws_bytes = max(sample_workspace_bytes(b, cfg["vocab_size"]) for b in buckets) if self.fused_sampler else 0
+        lm_bytes = max(lm_head_sample_workspace_bytes(b, cfg["hidden_size"]) for b in buckets) if self.fused_lm_head else 0
         self.graph_vars = dict(
             input_ids=torch.zeros(max_bs, dtype=torch.int64, device=dev),
             positions=torch.zeros(max_bs, dtype=torch.int64, device=dev),
@@ -154,6 +159,7 @@ class ModelRunner:
             sampled=torch.zeros(max_bs, dtype=torch.int64, device=dev),
             step=torch.zeros(1, dtype=torch.int64, device=dev),
             sample_ws=torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev),
+            lm_ws=torch.empty(max(lm_bytes, 16), dtype=torch.uint8, device=dev),
             outputs=torch.zeros(max_bs, cfg["hidden_size"], dtype=self.dtype, device=dev))
         v = self.graph_vars
         self._own_decode_workspace(buckets, max_blocks)
@@ -167,10 +173,15 @@ class ModelRunner:
                 if not self.fused_sampler:                 # the module-chain sampler draws from a host-side generator
                     v["outputs"][:bs] = hidden
                     return
-                logits = torch.nn.functional.linear(hidden, self.model.lm_head_weight)
-                nbytes = sample_workspace_bytes(bs, cfg["vocab_size"])
-                sample_tokens_into(v["sampled"][:bs], logits, v["temperatures"][:bs], self.seed, v["step"],
-                                   v["sample_ws"][:nbytes] if nbytes else None)
+                if self.fused_lm_head and lm_head_sample_takes(hidden, self.model.lm_head_weight):
+                    # LM head and sampler in one pass over the weights: no (bs, vocab) logits
+                    lm_head_sample(hidden, self.model.lm_head_weight, v["temperatures"][:bs], self.seed, 0,
+                                   out=v["sampled"][:bs], offset_dev=v["step"], workspace=v["lm_ws"])
+                else:
+                    logits = torch.nn.functional.linear(hidden, self.model.lm_head_weight)
+                    nbytes = sample_workspace_bytes(bs, cfg["vocab_size"])
+                    sample_tokens_into(v["sampled"][:bs], logits, v["temperatures"][:bs], self.seed, v["step"],
+                                       v["sample_ws"][:nbytes] if nbytes else None)
                 v["step"] += 1
 
             forward()                                    # warm-up outside the capture (library handles, lazy loads)
@@ -296,7 +307,21 @@ class ModelRunner:
         else:
             input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
             temperatures = self._to_device([seq.temperature for seq in seqs], torch.float32)
-            logits = self.model.compute_logits(self.model(input_ids, positions))
+            hidden = self.model(input_ids, positions)
+            if (self.fused_sampler and self.fused_lm_head
+                    and lm_head_sample_takes(hidden, self.model.lm_head_weight, len(seqs))):
+                # the rows to sample from are picked inside the kernel: the last token of every packed sequence in
+                # prefill (embedding_head.py:57-62), every row in decode
+                rows = (get_context().cu_seqlens_q[1:] - 1).long() if is_prefill else None
+                sampled = lm_head_sample(hidden, self.model.lm_head_weight, temperatures, self.seed,
+                                         self.sample_calls, row_index=rows)
+                self.sample_calls += 1
+                self._last_sampled = None
+                self._steady = None
+                token_ids = sampled.tolist()
+                reset_context()
+                return token_ids
+            logits = self.model.compute_logits(hidden)
         if self.fused_sampler:
             # one launch over the LM-head output; draws are a function of (seed, step), so a run is reproducible
             sampled = sample_tokens(logits, temperatures, self.seed, self.sample_calls)

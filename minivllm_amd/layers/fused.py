@@ -16,7 +16,8 @@ import torch
 
 from minivllm_amd import _C
 
-__all__ = ["qk_norm_rope_store", "sample_tokens", "sample_tokens_into", "decode_advance", "add_rms_norm", "silu_and_mul", "linear_small_m", "linear_small_m_takes", "norm_linear_small_m", "norm_linear_small_m_takes"]
+__all__ = ["qk_norm_rope_store", "sample_tokens", "sample_tokens_into", "decode_advance", "add_rms_norm", "silu_and_mul", "linear_small_m", "linear_small_m_takes", "norm_linear_small_m", "norm_linear_small_m_takes",
+           "lm_head_sample", "lm_head_sample_takes", "lm_head_sample_workspace_bytes"]
 
 
 def _ptr(t):
@@ -313,3 +314,52 @@ def norm_linear_small_m(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tenso
                                              _C.dtype_code(x.dtype), _C.current_stream_ptr(x.device))
     _C.check(st, "norm_linear_small_m")
     return (out, res_out) if want_residual else out
+
+
+def lm_head_sample_takes(hidden: torch.Tensor, weight: torch.Tensor, batch: int | None = None) -> bool:
+    """Whether ``lm_head_sample`` is built for this call: at most 64 rows to sample, bf16 / fp16 on the GPU, a
+    vocabulary that is a multiple of 16, hidden size 256, 512 or 1024."""
+    rows = hidden.shape[0] if batch is None else batch
+    return (hidden.is_cuda and hidden.dim() == 2 and 0 < rows <= 64 and hidden.dtype in (torch.bfloat16, torch.float16)
+            and weight.dtype == hidden.dtype and weight.dim() == 2 and weight.is_contiguous()
+            and weight.shape[0] % 16 == 0 and weight.shape[1] in (256, 512, 1024) and hidden.shape[1] == weight.shape[1]
+            and hidden.stride(1) == 1 and hidden.stride(0) % 8 == 0 and hidden.data_ptr() % 16 == 0)
+
+
+def lm_head_sample_workspace_bytes(batch: int, hidden_size: int) -> int:
+    return int(_C.load().mvllm_lm_head_sample_workspace_bytes(batch, hidden_size))
+
+
+def lm_head_sample(hidden: torch.Tensor, weight: torch.Tensor, temperatures: torch.Tensor, seed: int = 0,
+                   offset: int = 0, row_index: torch.Tensor | None = None, out: torch.Tensor | None = None,
+                   offset_dev: torch.Tensor | None = None, workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """The LM head and the sampler in one pass over ``weight`` (vocab, K): the reference's
+    ``ParallelLMHead.forward`` (layers/embedding_head.py:56-77) and ``SamplerLayer.forward`` (layers/sampler.py:14-19)
+    without the (batch, vocab) logits.  Row ``b`` samples from ``hidden[row_index[b]]`` (``row_index`` None: row b) at
+    ``temperatures[b]``; the noise is the in-kernel Philox stream of ``sample_tokens`` (same seed / offset: the same
+    ids as ``sample_tokens(F.linear(hidden, weight), ...)`` up to the summation order inside a logit).  ``out``,
+    ``offset_dev`` and ``workspace`` (uint8, ``lm_head_sample_workspace_bytes``) let a captured graph call it without
+    allocating and draw fresh noise on every replay."""
+    _C.require_cuda(hidden, weight, temperatures, row_index, out, offset_dev, workspace)
+    batch = hidden.shape[0] if row_index is None else row_index.numel()
+    if not lm_head_sample_takes(hidden, weight, batch):
+        raise ValueError("lm_head_sample: shape or dtype not taken (see lm_head_sample_takes)")
+    if temperatures.dtype != torch.float32 or temperatures.numel() != batch or not temperatures.is_contiguous():
+        raise ValueError("temperatures must be contiguous float32 (batch,)")
+    if row_index is not None and (row_index.dtype != torch.int64 or not row_index.is_contiguous()):
+        raise ValueError("row_index must be contiguous int64")
+    vocab, k = weight.shape
+    if out is None:
+        out = torch.empty(batch, dtype=torch.int64, device=hidden.device)
+    elif out.dtype != torch.int64 or out.numel() != batch or not out.is_contiguous():
+        raise ValueError("out must be contiguous int64 (batch,)")
+    need = lm_head_sample_workspace_bytes(batch, k)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=hidden.device)
+    st = _C.load().mvllm_lm_head_sample(_ptr(out), _ptr(hidden), hidden.stride(0) if hidden.shape[0] > 1 else k,
+                                        _ptr(row_index), _ptr(weight), _ptr(temperatures), int(seed) & (2 ** 64 - 1),
+                                        int(offset) & (2 ** 64 - 1), _ptr(offset_dev), batch, vocab, k,
+                                        _C.dtype_code(hidden.dtype), _ptr(workspace), workspace.numel(),
+                                        _C.current_stream_ptr(hidden.device))
+    _C.check(st, "lm_head_sample")
+    return out

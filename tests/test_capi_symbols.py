@@ -30,6 +30,7 @@ def test_header_declares_expected_entry_points():
               "mvllm_paged_decode_int8", "mvllm_paged_decode_noalloc", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_plan", "mvllm_prefill_varlen",
               "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_dev_offset", "mvllm_decode_advance", "mvllm_sample_tokens_workspace_bytes",
               "mvllm_add_rms_norm", "mvllm_linear_small_m", "mvllm_norm_linear_small_m", "mvllm_linear_small_m_plan",
+              "mvllm_lm_head_sample", "mvllm_lm_head_sample_workspace_bytes",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
         assert n in names
 
@@ -185,6 +186,17 @@ def test_argument_validation_without_gpu():
     assert plan(16, 1024, 2048, 1, 0, 1, ctypes.byref(w)) == 0 and w.value == 16    # 16 waves, 128 values each
     assert plan(32, 1024, 2048, 1, 0, 1, None) == -4                                # ... with one row tile only
     assert plan(16, 4096, 1024, 1, 0, 0, None) == -4 and plan(16, 4096, 1024, 1, 0, 9, None) == -2
+    lm = lib.mvllm_lm_head_sample
+    #   out hidden stride row_index weight temps seed offset offset_dev batch vocab K dtype ws ws_bytes stream
+    assert lm(0, 0, 1024, 0, 0, 0, 0, 0, 0, 0, 151936, 1024, 1, 0, 0, 0) == 0                  # no rows
+    assert lm(0, 0, 1024, 0, 0, 0, 0, 0, 0, 4, 151936, 1024, 1, 0, 0, 0) == -1                 # null pointers
+    assert lm(8, 16, 1024, 0, 16, 8, 0, 0, 0, 65, 151936, 1024, 1, 0, 0, 0) == -4              # more than 64 rows
+    assert lm(8, 16, 1024, 0, 16, 8, 0, 0, 0, 4, 151930, 1024, 1, 0, 0, 0) == -4               # vocab % 16
+    assert lm(8, 16, 768, 0, 16, 8, 0, 0, 0, 4, 151936, 768, 1, 0, 0, 0) == -4                 # hidden size
+    assert lm(8, 16, 1024, 0, 16, 8, 0, 0, 0, 4, 151936, 1024, 0, 0, 0, 0) == -4               # fp32
+    assert lm(8, 16, 1024, 0, 16, 8, 0, 0, 0, 4, 151936, 1024, 1, 0, 0, 0) == -5               # no workspace
+    wsb = lib.mvllm_lm_head_sample_workspace_bytes
+    assert wsb(16, 1024) == 16 * 512 * 8 and wsb(64, 1024) == 64 * 256 * 8 and wsb(65, 1024) == 0
     adv = lib.mvllm_decode_advance
     assert adv(0, 0, 0, 0, 0, 0, 0) == 0 and adv(0, 0, 0, 0, 0, 4, 0) == -1 and adv(0, 0, 0, 0, 0, -1, 0) == -3
     assert lib.mvllm_sample_tokens_dev_offset(8, 8, 100, 8, 1, 0, 4, 100, 1, 0, 0, 0) == -1       # no counter
