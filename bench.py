@@ -478,8 +478,32 @@ def bench_sampler(args):
     _, fused_ms = time_steps(lambda: sample_tokens(logits, temps, 0, 0), args.steps, args.warmup, EXTRA_WARM_MS)
     _, modules_ms = time_steps(lambda: sampler(logits, temps, dg), args.steps, args.warmup, EXTRA_WARM_MS)
     nbytes = batch * vocab * 2 + batch * 12
-    return {"workload": "sampler: 64 x 151936 bf16 logits, T 0.6", "algorithmic_bytes": nbytes,
-            "event_ms_per_step": fused_ms, "gbs": nbytes / (fused_ms * 1e-3) / 1e9, "unfused_modules_event_ms": modules_ms}
+    out = {"workload": "sampler: 64 x 151936 bf16 logits, T 0.6", "algorithmic_bytes": nbytes,
+           "event_ms_per_step": fused_ms, "gbs": nbytes / (fused_ms * 1e-3) / 1e9, "unfused_modules_event_ms": modules_ms}
+    # the LM head in front of it, config 5's: (rows, 1024) x (151936, 1024)^T, as the library GEMM + the sampler
+    # launch and as one pass over the weights that never writes the logits
+    import torch.nn.functional as F
+    from minivllm_amd.layers.fused import lm_head_sample, lm_head_sample_workspace_bytes
+    hidden_size = 1024
+    w = (torch.randn(vocab, hidden_size, generator=dg, device=dev) * 0.02).to(torch.bfloat16)
+    legs = {}
+    for rows in (16, 64):
+        x = torch.randn(rows, hidden_size, generator=dg, device=dev).to(torch.bfloat16)
+        t = temps[:rows].contiguous()
+        ws = torch.empty(lm_head_sample_workspace_bytes(rows, hidden_size), dtype=torch.uint8, device=dev)
+        ids = torch.empty(rows, dtype=torch.int64, device=dev)
+        _, one_ms = time_steps(lambda: lm_head_sample(x, w, t, 0, 0, out=ids, workspace=ws), args.steps, args.warmup,
+                               EXTRA_WARM_MS)
+        _, two_ms = time_steps(lambda: sample_tokens(F.linear(x, w), t, 0, 0), args.steps, args.warmup, EXTRA_WARM_MS)
+        wbytes = vocab * hidden_size * 2 + rows * hidden_size * 2 + rows * 12
+        same = float((lm_head_sample(x, w, t, 0, 0) == sample_tokens(F.linear(x, w), t, 0, 0)).float().mean())
+        legs[f"rows{rows}"] = {"event_ms_per_step": one_ms, "gemm_then_sampler_event_ms": two_ms,
+                               "ids_equal_to_gemm_then_sampler": same,
+                               "roofline": roofline("hbm", wbytes / (one_ms * 1e-3) / 1e9,
+                                                    "lm_head_sample_kernel + sample_combine_kernel")}
+    out["lm_head_sample"] = dict(workload="LM head + sampler in one pass: rows x 1024 hidden, 151936 x 1024 bf16 weights",
+                                 algorithmic_bytes=vocab * hidden_size * 2, **legs)
+    return out
 
 
 def bench_decode_small(args):
