@@ -86,3 +86,22 @@ def test_lm_head_sample_follows_the_tempered_distribution():
     freq = counts / (calls * m)
     # 25 600 draws: the standard error of a frequency p is sqrt(p (1 - p) / n) <= 0.0031; five of them
     assert float((freq - probs).abs().max()) <= 5 * float((probs * (1 - probs) / (calls * m)).sqrt().max()) + 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_lm_head_sample_against_the_cpu_oracle(dtype):
+    """Against the oracle end to end: fp32 product of the 16-bit operands on the CPU rounded to the element type
+    (the LM head's logits), the oracle's restatement of the Philox noise stream, and the oracle's sampler.  The fp32
+    sums may differ in their last bits, so a row may differ where its two best scores nearly tie: at least 95 % of the
+    rows equal (all of them when this was written)."""
+    import oracle
+    agree = total = 0
+    for seed, m, vocab, k, offset in [(1, 5, 2048, 256, 0), (2, 33, 4096, 512, 7), (3, 64, 1024, 1024, (1 << 32) + 5)]:
+        x, w, t = _case(900 + seed, m, vocab, k, dtype)
+        logits = (x.float().cpu() @ w.float().cpu().T).to(dtype)
+        noise = oracle.exponential_noise_oracle(40 + seed, offset, m, vocab)
+        want = oracle.sampler_oracle(logits, t.cpu(), noise)
+        got = lm_head_sample(x, w, t, seed=40 + seed, offset=offset).cpu()
+        agree += int((got == want).sum())
+        total += m
+    assert agree >= 0.95 * total, (agree, total)
