@@ -26,8 +26,8 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # HBM bytes one decode_mfma_kernel launch moves on the default workload (seed 0, block_size 16), from the
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/bench_hbm_traffic_pmc.txt:
-# 2708917 KiB x 2.0 (copy-kernel calibration) fetched + 22855 KiB written.
-DECODE_TRAFFIC_BYTES_DEFAULT = int(2708917 * 2.0 * 1024 + 22855 * 1024)
+# 2708778 KiB x 2.0 (copy-kernel calibration) fetched + 22855 KiB written.
+DECODE_TRAFFIC_BYTES_DEFAULT = int(2708778 * 2.0 * 1024 + 22855 * 1024)
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,loads_probe,engine,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,loads_probe,engine,engine16,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -790,6 +790,8 @@ def main():
         extra["engine_16seq_eager"] = bench_engine(args, 16, False)
         extra["engine_16seq_graph"] = bench_engine(args, 16, True)
         extra["engine_64seq_graph"] = bench_engine(args, 64, True)
+    elif "engine16" in only:                           # the one configuration a kernel trace of a decode step wants
+        extra["engine_16seq_graph"] = bench_engine(args, 16, True)
 
     if "loads_only" in head:
         extra["decode_loads_only"] = head["loads_only"]

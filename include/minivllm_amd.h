@@ -309,11 +309,14 @@ int mvllm_lm_head_sample(int64_t* out_ids, const void* hidden, int64_t hidden_ro
  * The step metadata of a decode batch that continues the step before it (same sequences, each one token longer),
  * advanced on the device in one launch instead of being rebuilt on the host as ModelRunner.prepare_decode does
  * (src/myvllm/engine/model_runner.py:231-256): input_ids[i] = sampled[i]; context_lens[i] += 1;
- * positions[i] = context_lens[i] - 1; slot_mapping[i] += 1.  All int64 [batch].  Rows that open a new block have
- * their slot and table entry patched by the caller afterwards.
+ * positions[i] = context_lens[i] - 1; slot_mapping[i] += 1.  All int64 [batch].  Rows whose context length is
+ * not positive (the padding of a captured batch size) are left alone.  Rows that open a new block have their slot
+ * and table entry patched by the caller afterwards.  step_counter (may be NULL): one uint64 on the device, the
+ * call counter of mvllm_sample_tokens_dev_offset / mvllm_lm_head_sample, incremented by one, so that a captured
+ * decode step can end with this launch and be replayed without any host-side update.
  */
 int mvllm_decode_advance(int64_t* input_ids, int64_t* context_lens, int64_t* positions, int64_t* slot_mapping,
-                         const int64_t* sampled, int batch, void* stream);
+                         const int64_t* sampled, uint64_t* step_counter, int batch, void* stream);
 
 /*
  * LayerNorm.forward with and without residual -- src/myvllm/layers/layernorm.py:9-28, called from

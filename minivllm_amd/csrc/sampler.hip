@@ -387,27 +387,32 @@ extern "C" int mvllm_sample_tokens_dev_offset(int64_t* out_ids, const void* logi
 // The step metadata of a decode batch that continues the step before it (the same sequences, each one token longer),
 // moved forward on the device: next input = the id just sampled, context length, position and slot + 1.  One launch
 // in place of the host rebuilding and copying the four tensors (ModelRunner.prepare_decode,
-// src/myvllm/engine/model_runner.py:231-256).
+// src/myvllm/engine/model_runner.py:231-256).  Rows whose context length is not positive are padding of a captured
+// batch size and stay as they are; `step` (optional) is the sampler's call counter, incremented once per launch, so
+// that a captured decode step ends with everything the next replay needs.
 // ---------------------------------------------------------------------------
 __global__ void decode_advance_kernel(int64_t* __restrict__ input_ids, int64_t* __restrict__ context_lens,
                                       int64_t* __restrict__ positions, int64_t* __restrict__ slot_mapping,
-                                      const int64_t* __restrict__ sampled, int n) {
+                                      const int64_t* __restrict__ sampled, uint64_t* __restrict__ step, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i == 0 && step) *step += 1;
   if (i >= n) return;
+  const int64_t ctx = context_lens[i];
+  if (ctx <= 0) return;
   input_ids[i] = sampled[i];
-  const int64_t ctx = context_lens[i] + 1;
-  context_lens[i] = ctx;
-  positions[i] = ctx - 1;
+  context_lens[i] = ctx + 1;
+  positions[i] = ctx;
   slot_mapping[i] += 1;
 }
 
 extern "C" int mvllm_decode_advance(int64_t* input_ids, int64_t* context_lens, int64_t* positions,
-                                    int64_t* slot_mapping, const int64_t* sampled, int batch, void* stream) {
+                                    int64_t* slot_mapping, const int64_t* sampled, uint64_t* step_counter, int batch,
+                                    void* stream) {
   if (batch < 0) return MVLLM_ERR_BAD_SHAPE;
-  if (batch == 0) return MVLLM_OK;
-  if (!input_ids || !context_lens || !positions || !slot_mapping || !sampled) return MVLLM_ERR_NULL_POINTER;
-  decode_advance_kernel<<<dim3((unsigned)((batch + 63) / 64)), dim3(64), 0, (hipStream_t)stream>>>(
-      input_ids, context_lens, positions, slot_mapping, sampled, batch);
+  if (batch == 0 && !step_counter) return MVLLM_OK;
+  if (batch > 0 && (!input_ids || !context_lens || !positions || !slot_mapping || !sampled)) return MVLLM_ERR_NULL_POINTER;
+  decode_advance_kernel<<<dim3((unsigned)((batch + 63) / 64 > 0 ? (batch + 63) / 64 : 1)), dim3(64), 0, (hipStream_t)stream>>>(
+      input_ids, context_lens, positions, slot_mapping, sampled, step_counter, batch);
   return launch_status();
 }
 

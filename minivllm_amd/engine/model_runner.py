@@ -182,7 +182,10 @@ class ModelRunner:
                     nbytes = sample_workspace_bytes(bs, cfg["vocab_size"])
                     sample_tokens_into(v["sampled"][:bs], logits, v["temperatures"][:bs], self.seed, v["step"],
                                        v["sample_ws"][:nbytes] if nbytes else None)
-                v["step"] += 1
+                # the step ends with the next step's inputs (rows of padding stay) and the sampler's counter + 1:
+                # a batch that goes on as it is needs nothing from the host but the rows that open a new block
+                decode_advance(v["input_ids"][:bs], v["context_lens"][:bs], v["positions"][:bs],
+                               v["slot_mapping"][:bs], v["sampled"][:bs], step=v["step"])
 
             forward()                                    # warm-up outside the capture (library handles, lazy loads)
             torch.cuda.synchronize()
@@ -234,16 +237,17 @@ class ModelRunner:
         return all(len(seq) == m + 1 for seq, m in zip(seqs, st["lens"]))
 
     def _advance_decode_buffers(self, seqs) -> bool:
-        """The same sequences as in the last graph decode step, each one token longer: the buffers move on the
-        device (input = the ids sampled last step, context length and slot + 1) and only sequences that started a
-        new block are patched from the host.  Returns False when the batch is not such a continuation."""
+        """The same sequences as in the last graph decode step, each one token longer: the buffers were moved on by
+        that step itself, on the device (input = the ids it sampled, context length and slot + 1), and only
+        sequences that started a new block are patched from the host.  Returns False when the batch is not such a
+        continuation."""
         if not self.continues_last_decode(seqs):
             return False
         st = self._steady
         lens = [len(seq) for seq in seqs]
         bs = len(seqs)
         v = self.graph_vars
-        decode_advance(v["input_ids"], v["context_lens"], v["positions"], v["slot_mapping"], self._last_sampled)
+        # the captured step has already moved its buffers on (decode_advance is its last launch)
         fresh = [i for i, n in enumerate(lens) if (n - 1) % self.block_size == 0]     # token n-1 opens a block
         if fresh:
             rows = self._to_device(fresh, torch.int64)

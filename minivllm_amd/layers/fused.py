@@ -174,16 +174,20 @@ def sample_workspace_bytes(batch: int, vocab: int) -> int:
 
 
 def decode_advance(input_ids: torch.Tensor, context_lens: torch.Tensor, positions: torch.Tensor,
-                   slot_mapping: torch.Tensor, sampled: torch.Tensor) -> None:
+                   slot_mapping: torch.Tensor, sampled: torch.Tensor, step: torch.Tensor | None = None) -> None:
     """Move a decode batch's step metadata one token forward on the device (all int64 (batch,), in place):
-    input = the id sampled last step, context length + 1, position = new length - 1, slot + 1."""
-    _C.require_cuda(input_ids, context_lens, positions, slot_mapping, sampled)
+    input = the id sampled last step, context length + 1, position = new length - 1, slot + 1; rows whose context
+    length is not positive (padding of a captured batch size) stay as they are.  ``step`` (one int64 / uint64 on the
+    device): the sampler's call counter, incremented by one in the same launch."""
+    _C.require_cuda(input_ids, context_lens, positions, slot_mapping, sampled, step)
     n = sampled.numel()
     for t in (input_ids, context_lens, positions, slot_mapping, sampled):
         if t.dtype != torch.int64 or t.numel() < n or not t.is_contiguous():
             raise ValueError("decode_advance takes contiguous int64 tensors of at least the batch size")
+    if step is not None and (step.numel() != 1 or step.element_size() != 8):
+        raise ValueError("step must be one 64-bit integer on the device")
     st = _C.load().mvllm_decode_advance(_ptr(input_ids), _ptr(context_lens), _ptr(positions), _ptr(slot_mapping),
-                                        _ptr(sampled), n, _C.current_stream_ptr(sampled.device))
+                                        _ptr(sampled), _ptr(step), n, _C.current_stream_ptr(sampled.device))
     _C.check(st, "decode_advance")
 
 

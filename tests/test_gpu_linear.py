@@ -129,3 +129,9 @@ def test_decode_advance_moves_the_step_metadata_forward():
     torch.cuda.synchronize()
     assert ids.tolist() == [100, 200, 300, 8] and ctx.tolist() == [11, 257, 4, 0]
     assert pos.tolist() == [10, 256, 3, 0] and slots.tolist() == [10, 512, 41, -1]
+    # all four rows of a captured batch size: the padding row (context 0, slot -1) stays, and the call counter moves
+    step = torch.tensor([41], device=DEV)
+    decode_advance(ids, ctx, pos, slots, torch.tensor([1, 2, 3, 4], device=DEV), step=step)
+    torch.cuda.synchronize()
+    assert ids.tolist() == [1, 2, 3, 8] and ctx.tolist() == [12, 258, 5, 0] and slots.tolist() == [11, 513, 42, -1]
+    assert pos.tolist() == [11, 257, 4, 0] and step.item() == 42
