@@ -313,10 +313,15 @@ int mvllm_lm_head_sample(int64_t* out_ids, const void* hidden, int64_t hidden_ro
  * not positive (the padding of a captured batch size) are left alone.  Rows that open a new block have their slot
  * and table entry patched by the caller afterwards.  step_counter (may be NULL): one uint64 on the device, the
  * call counter of mvllm_sample_tokens_dev_offset / mvllm_lm_head_sample, incremented by one, so that a captured
- * decode step can end with this launch and be replayed without any host-side update.
+ * decode step can end with this launch and be replayed without any host-side update.  host_ids (may be NULL; needs
+ * step_counter): two rows of host_row_stride >= batch + 1 int64 in pinned, device-visible host memory; row
+ * (counter before the increment) & 1 receives sampled[0 .. batch) and then, behind a system-scope fence, the new
+ * counter value in its last entry: the host reads a step's ids once it sees that value, with no copy operation and
+ * no event queued between two replays (two rows: step t is read while step t + 1 runs).
  */
 int mvllm_decode_advance(int64_t* input_ids, int64_t* context_lens, int64_t* positions, int64_t* slot_mapping,
-                         const int64_t* sampled, uint64_t* step_counter, int batch, void* stream);
+                         const int64_t* sampled, uint64_t* step_counter, int64_t* host_ids,
+                         int64_t host_row_stride, int batch, void* stream);
 
 /*
  * LayerNorm.forward with and without residual -- src/myvllm/layers/layernorm.py:9-28, called from

@@ -46,7 +46,7 @@ SIGNATURES = {
                                     c_int, c_void_p, c_size_t, c_void_p]),
     "mvllm_sample_tokens_dev_offset": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_uint64, c_void_p, c_int, c_int,
                                                c_int, c_void_p, c_size_t, c_void_p]),
-    "mvllm_decode_advance": (c_int, [c_void_p] * 6 + [c_int, c_void_p]),
+    "mvllm_decode_advance": (c_int, [c_void_p] * 7 + [c_int64, c_int, c_void_p]),
     "mvllm_add_rms_norm": (c_int, [c_void_p] * 5 + [c_float, c_int64, c_int, c_int64, c_int64, c_int, c_void_p]),
     "mvllm_silu_and_mul": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int, c_void_p]),
     "mvllm_lm_head_sample_workspace_bytes": (c_size_t, [c_int, c_int]),

@@ -12,6 +12,8 @@ over the weights for at most 64 rows (``lm_head_sample``), otherwise the library
 """
 from __future__ import annotations
 
+import time
+
 import torch
 
 from minivllm_amd.engine.metadata import decode_metadata, prefill_metadata
@@ -28,14 +30,23 @@ _DTYPES = {"bf16": torch.bfloat16, "bfloat16": torch.bfloat16, "fp16": torch.flo
 
 
 class PendingTokens:
-    """Token ids of a launched decode step on their way to the host."""
+    """Token ids of a launched decode step on their way to the host: the step's last kernel writes them into a
+    row of pinned memory and then the step's sequence number into the row's last entry."""
 
-    def __init__(self, host: torch.Tensor, done: torch.cuda.Event):
-        self.host, self.done = host, done
+    def __init__(self, row, count: int, sequence: int):
+        self.row, self.count, self.sequence = row, count, sequence     # row: numpy view of the pinned row
 
     def wait(self) -> list[int]:
-        self.done.synchronize()
-        return self.host.tolist()
+        row, want = self.row, self.sequence
+        deadline = None
+        while int(row[-1]) != want:
+            if deadline is None:
+                deadline = time.monotonic() + 60.0
+            elif time.monotonic() > deadline:
+                torch.cuda.synchronize()               # surfaces a device error instead of spinning for ever
+                if int(row[-1]) != want:
+                    raise RuntimeError("decode step finished without delivering its token ids")
+        return row[:self.count].tolist()
 
 
 class ModelRunner:
@@ -64,7 +75,7 @@ class ModelRunner:
         self.fused_lm_head = self.fused_sampler and config.get("fused_lm_head", True)
         self.seed = config.get("seed", 0)
         self.sample_calls = 0
-        self._pinned = None          # pinned host buffers of launch_decode
+        self._pinned = None          # (2, max batch) pinned ids, written by the captured step itself
         self._dev_step = None        # host mirror of the graphs' device-side sampler call counter
         self._steady = None          # description of the batch in the static decode buffers (graph decode)
         self._last_sampled = None    # device tensor of the ids sampled by the last graph decode step
@@ -162,6 +173,9 @@ class ModelRunner:
             lm_ws=torch.empty(max(lm_bytes, 16), dtype=torch.uint8, device=dev),
             outputs=torch.zeros(max_bs, cfg["hidden_size"], dtype=self.dtype, device=dev))
         v = self.graph_vars
+        # the ids of a step, written by the step's last kernel into pinned host memory: row (sampler counter & 1)
+        self._pinned = torch.zeros(2, max_bs + 1, dtype=torch.int64, pin_memory=True)
+        self._pinned_rows = self._pinned.numpy()       # the same memory, for polling without tensor overhead
         self._own_decode_workspace(buckets, max_blocks)
         pool = None
         for bs in reversed(buckets):
@@ -185,7 +199,7 @@ class ModelRunner:
                 # the step ends with the next step's inputs (rows of padding stay) and the sampler's counter + 1:
                 # a batch that goes on as it is needs nothing from the host but the rows that open a new block
                 decode_advance(v["input_ids"][:bs], v["context_lens"][:bs], v["positions"][:bs],
-                               v["slot_mapping"][:bs], v["sampled"][:bs], step=v["step"])
+                               v["slot_mapping"][:bs], v["sampled"][:bs], step=v["step"], host_ids=self._pinned)
 
             forward()                                    # warm-up outside the capture (library handles, lazy loads)
             torch.cuda.synchronize()
@@ -197,6 +211,8 @@ class ModelRunner:
             torch.cuda.synchronize()
             reset_context()
         self._dev_step = None                            # value of the device counter, unknown after the warm-ups
+        torch.cuda.synchronize()
+        self._pinned.zero_()                             # the warm-ups left their sequence numbers: steps count from 1
 
     def _own_decode_workspace(self, buckets, max_blocks):
         """One split-K scratch buffer for every decode call of this runner, allocated before any graph is
@@ -282,20 +298,17 @@ class ModelRunner:
 
     @torch.inference_mode()
     def launch_decode(self, seqs) -> "PendingTokens":
-        """Enqueue one decode step and return at once; the sampled ids travel to a pinned host buffer behind the
-        step and are read with ``PendingTokens.wait()``.  The next step's input ids are taken from the device
+        """Enqueue one decode step and return at once; the step's last kernel writes the sampled ids into pinned host
+        memory, followed by the step's sequence number (no copy operation and no event between two replays), and
+        they are read with ``PendingTokens.wait()``.  The next step's input ids are taken from the device
         copy, so the host can schedule and launch step t + 1 while the GPU still runs step t.  When the batch
         does not continue the last step's, the buffers are refilled from the sequences' last tokens, which must be
         real by then (the caller commits outstanding ids first)."""
+        calls = self.sample_calls                     # the counter's value when the step starts picks the pinned row
         sampled = self._replay_decode(seqs)
         self._last_sampled = sampled
-        if self._pinned is None:
-            self._pinned = [torch.empty(max(self.graphs), dtype=torch.int64, pin_memory=True) for _ in range(2)]
-        host = self._pinned[self.sample_calls & 1][:len(seqs)]     # two buffers: step t's ids are read after step t + 1 is launched
-        host.copy_(sampled, non_blocking=True)
-        done = torch.cuda.Event()
-        done.record()
-        return PendingTokens(host, done)
+        # step t's row is read after step t + 1 has been launched (into the other row)
+        return PendingTokens(self._pinned_rows[calls & 1], len(seqs), calls + 1)
 
     @torch.inference_mode()
     def run(self, seqs, is_prefill: bool) -> list[int]:

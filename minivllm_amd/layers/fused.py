@@ -174,11 +174,15 @@ def sample_workspace_bytes(batch: int, vocab: int) -> int:
 
 
 def decode_advance(input_ids: torch.Tensor, context_lens: torch.Tensor, positions: torch.Tensor,
-                   slot_mapping: torch.Tensor, sampled: torch.Tensor, step: torch.Tensor | None = None) -> None:
+                   slot_mapping: torch.Tensor, sampled: torch.Tensor, step: torch.Tensor | None = None,
+                   host_ids: torch.Tensor | None = None) -> None:
     """Move a decode batch's step metadata one token forward on the device (all int64 (batch,), in place):
     input = the id sampled last step, context length + 1, position = new length - 1, slot + 1; rows whose context
     length is not positive (padding of a captured batch size) stay as they are.  ``step`` (one int64 / uint64 on the
-    device): the sampler's call counter, incremented by one in the same launch."""
+    device): the sampler's call counter, incremented by one in the same launch.  ``host_ids`` (with ``step``): a
+    pinned int64 CPU tensor (2, n >= batch + 1); row ``step & 1`` (before the increment) receives the sampled ids and
+    then, in its last entry, the new counter value, written by the kernel itself: the host may read the ids as soon as
+    it sees that value."""
     _C.require_cuda(input_ids, context_lens, positions, slot_mapping, sampled, step)
     n = sampled.numel()
     for t in (input_ids, context_lens, positions, slot_mapping, sampled):
@@ -186,8 +190,15 @@ def decode_advance(input_ids: torch.Tensor, context_lens: torch.Tensor, position
             raise ValueError("decode_advance takes contiguous int64 tensors of at least the batch size")
     if step is not None and (step.numel() != 1 or step.element_size() != 8):
         raise ValueError("step must be one 64-bit integer on the device")
+    host_ptr, host_stride = 0, 0
+    if host_ids is not None:
+        if step is None or host_ids.is_cuda or not host_ids.is_pinned() or host_ids.dtype != torch.int64 \
+                or host_ids.dim() != 2 or host_ids.shape[0] != 2 or host_ids.shape[1] < n + 1 or not host_ids.is_contiguous():
+            raise ValueError("host_ids must be a pinned contiguous int64 CPU tensor (2, >= batch + 1), given with step")
+        host_ptr, host_stride = host_ids.data_ptr(), host_ids.shape[1]
     st = _C.load().mvllm_decode_advance(_ptr(input_ids), _ptr(context_lens), _ptr(positions), _ptr(slot_mapping),
-                                        _ptr(sampled), _ptr(step), n, _C.current_stream_ptr(sampled.device))
+                                        _ptr(sampled), _ptr(step), host_ptr, host_stride, n,
+                                        _C.current_stream_ptr(sampled.device))
     _C.check(st, "decode_advance")
 
 

@@ -198,7 +198,9 @@ def test_argument_validation_without_gpu():
     wsb = lib.mvllm_lm_head_sample_workspace_bytes
     assert wsb(16, 1024) == 16 * 512 * 8 and wsb(64, 1024) == 64 * 256 * 8 and wsb(65, 1024) == 0
     adv = lib.mvllm_decode_advance
-    assert adv(0, 0, 0, 0, 0, 0, 0, 0) == 0 and adv(0, 0, 0, 0, 0, 0, 4, 0) == -1 and adv(0, 0, 0, 0, 0, 0, -1, 0) == -3
+    assert adv(0, 0, 0, 0, 0, 0, 0, 0, 0, 0) == 0 and adv(0, 0, 0, 0, 0, 0, 0, 0, 4, 0) == -1
+    assert adv(0, 0, 0, 0, 0, 0, 0, 0, -1, 0) == -3 and adv(8, 8, 8, 8, 8, 0, 8, 8, 4, 0) == -1     # host ids without the counter
+    assert adv(8, 8, 8, 8, 8, 8, 8, 4, 4, 0) == -3                                                # host rows shorter than the batch + 1
     assert lib.mvllm_sample_tokens_dev_offset(8, 8, 100, 8, 1, 0, 4, 100, 1, 0, 0, 0) == -1       # no counter
     fused = lib.mvllm_qk_norm_rope_store
     #     q_out k_out v_out q k v | strides | gamma eps cos max_pos pos slots | caches scales int8 | T slots Hq Hkv D dt stream

@@ -135,3 +135,14 @@ def test_decode_advance_moves_the_step_metadata_forward():
     torch.cuda.synchronize()
     assert ids.tolist() == [1, 2, 3, 8] and ctx.tolist() == [12, 258, 5, 0] and slots.tolist() == [11, 513, 42, -1]
     assert pos.tolist() == [11, 257, 4, 0] and step.item() == 42
+    # the ids also go to pinned host memory: the row is the counter's parity before the increment, its last entry the
+    # new counter value, written after the ids (the host may read the ids once it sees it)
+    host = torch.zeros(2, 6, dtype=torch.int64, pin_memory=True)
+    decode_advance(ids, ctx, pos, slots, torch.tensor([9, 8, 7, 6], device=DEV), step=step, host_ids=host)   # 42: row 0
+    decode_advance(ids, ctx, pos, slots, torch.tensor([5, 4, 3, 2], device=DEV), step=step, host_ids=host)   # 43: row 1
+    torch.cuda.synchronize()
+    assert host[0].tolist() == [9, 8, 7, 6, 0, 43] and host[1].tolist() == [5, 4, 3, 2, 0, 44] and step.item() == 44
+    with pytest.raises(ValueError):
+        decode_advance(ids, ctx, pos, slots, sampled, step=step, host_ids=torch.zeros(2, 6, dtype=torch.int64))   # not pinned
+    with pytest.raises(ValueError):
+        decode_advance(ids, ctx, pos, slots, sampled, host_ids=host)                                             # no counter
