@@ -71,7 +71,7 @@ def test_norm_linear_equals_the_separate_launches(dtype, m, n, k, bias, glu, wit
     where its last bit differs, a normalised value can round the other way (about one in 2^13 fp16 values, 2^16 in
     bf16), and that one input moves every output of its row by a fraction of a unit in the last place, so a row is
     either bit-identical or has some outputs one unit off: every output within 2 units in the last place of the
-    largest output of its row, and at least 70 % of all outputs bit-identical."""
+    largest output of its row (4 behind the activation), and at least 70 % of all outputs bit-identical."""
     x, w, b = _case(300 + m, m, n, k, dtype, bias)
     x = x.contiguous()
     g = torch.Generator().manual_seed(m)
@@ -93,7 +93,8 @@ def test_norm_linear_equals_the_separate_launches(dtype, m, n, k, bias, glu, wit
     same = (got == want).float().mean().item()
     ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     worst = ((got.float() - want.float()).abs() / want.float().abs().amax(dim=1, keepdim=True)).max().item()
-    assert same >= 0.7 and worst <= 2 * ulp, (same, worst)
+    # with the activation behind it, one unit in the gate and one in the up projection meet in a product: 4 units
+    assert same >= 0.7 and worst <= (4 if glu else 2) * ulp, (same, worst)
 
 
 def test_norm_linear_without_norm_is_the_plain_product_and_glu_pairs_the_right_columns():
