@@ -43,12 +43,13 @@ class LLMEngine:
     def step(self):
         """One schedule -> run -> postprocess round.  Always a 3-tuple (finished, processed tokens, is_prefill).
 
-        With ``async_decode`` (default) a decode step whose sequences all ignore EOS is launched without waiting
-        for its token ids: lengths, block tables and the finish-by-count do not depend on them, the next step's
-        input ids are taken from the device, and the host schedules and launches step t + 1 while the GPU runs
-        step t.  Such a step's ids are committed, and its finished sequences reported, one ``step`` later (or by
-        ``flush``); everything that needs real ids (a prefill, a sequence that stops at EOS, a batch that changed)
-        commits first."""
+        With ``async_decode`` (default) a decode step is launched without waiting for the token ids of the step
+        before: lengths, block tables and the finish-by-count do not depend on them, the next step's input ids are
+        taken from the device, and the host schedules and launches step t + 1 while the GPU runs step t.  Such a
+        step's ids are committed, and its finished sequences reported, one ``step`` later (or by ``flush``).  A
+        sequence whose id turns out to be its EOS ends at that commit; the row the step launched in the meantime
+        computed for it is dropped (its cache slot belongs to blocks that are freed with the sequence).  Everything
+        that needs real ids (a prefill, a batch that changed) commits first."""
         finished = []
         if self.pending is not None and self.scheduler.waiting:
             finished += self.flush()                   # admission hashes prompt blocks: ids must be real
@@ -56,15 +57,15 @@ class LLMEngine:
         if not seqs:
             return finished + self.flush(), 0, is_prefill
         runner = self.model_runner
-        if (self.async_decode and not is_prefill and all(seq.ignore_eos for seq in seqs)
-                and hasattr(runner, "launch_decode") and runner.can_launch_decode(seqs)):
+        if (self.async_decode and not is_prefill and hasattr(runner, "launch_decode")
+                and runner.can_launch_decode(seqs)):
             if not runner.continues_last_decode(seqs):
                 finished += self.flush()               # the buffers are refilled from the last tokens
             handle = runner.launch_decode(seqs)
             finished += self.flush()                   # the step before this one, while the GPU runs this one
-            slots = self.scheduler.postprocess_provisional(seqs)
-            self.pending = (handle, slots, [seq for seq in seqs if seq.is_finished])
-            return finished, len(seqs), False
+            slots, done = self.scheduler.postprocess_provisional(seqs)
+            self.pending = (handle, slots, done)
+            return finished, sum(slot is not None for slot in slots), False
         finished += self.flush()
         token_ids = runner.run(seqs, is_prefill)
         self.scheduler.postprocess(seqs, token_ids)
@@ -78,8 +79,8 @@ class LLMEngine:
             return []
         handle, slots, done = self.pending
         self.pending = None
-        self.scheduler.commit(slots, handle.wait())
-        return [(seq.seq_id, seq.completion_token_ids) for seq in done]
+        ended = self.scheduler.commit(slots, handle.wait())
+        return [(seq.seq_id, seq.completion_token_ids) for seq in done + ended]
 
     def generate(self, prompts: list[list[int]], sampling_params: SamplingParams, verbose: bool = False) -> dict:
         for prompt in prompts:

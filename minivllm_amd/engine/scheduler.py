@@ -71,28 +71,46 @@ class Scheduler:
 
     PLACEHOLDER = -1        # stands for a sampled token whose id has not reached the host yet
 
-    def postprocess_provisional(self, seqs: list[Sequence]) -> list[tuple[Sequence, int]]:
+    def postprocess_provisional(self, seqs: list[Sequence]):
         """``postprocess`` for a decode step whose token ids are still on the device: every sequence grows by a
-        placeholder and finishes by count (callers use this only when every sequence ignores EOS, so nothing
-        else depends on the ids).  Returns (sequence, index of the placeholder) for ``commit``."""
-        slots = []
+        placeholder and finishes by count.  A sequence that has ended in the meantime (the ids of the step before
+        arrived after this step was launched and held its EOS) is skipped: its row of this step is computed for
+        nothing.  Returns the slots for ``commit``, one per row ((sequence, index of the placeholder) or None), and
+        the sequences this step finished by count."""
+        slots, done = [], []
         for seq in seqs:
+            if seq.is_finished:
+                slots.append(None)
+                continue
             seq.append_token(self.PLACEHOLDER)
             slots.append((seq, seq.num_tokens - 1))
             if seq.num_completion_tokens >= seq.max_tokens:
                 seq.status = SequenceStatus.FINISHED
                 self.block_manager.deallocate(seq)
                 self.running.remove(seq)
-        return slots
+                done.append(seq)
+        return slots, done
 
-    def commit(self, slots: list[tuple[Sequence, int]], token_ids: list[int]) -> None:
-        """The ids of a provisional step have arrived: replace the placeholders, then give the blocks that filled
-        up in the meantime their hashes."""
-        for (seq, index), token_id in zip(slots, token_ids):
-            seq.token_ids[index] = int(token_id)
+    def commit(self, slots: list, token_ids: list[int]) -> list[Sequence]:
+        """The ids of a provisional step have arrived: replace the placeholders, end the sequences whose id is their
+        EOS (one step late: the step launched in the meantime has computed a row for them that is dropped), then give
+        the blocks that filled up in the meantime their hashes.  Returns the sequences ended here."""
+        ended = []
+        for slot, token_id in zip(slots, token_ids):
+            if slot is None:
+                continue
+            seq, index = slot
+            token_id = int(token_id)
+            seq.token_ids[index] = token_id
             if index == seq.num_tokens - 1:
-                seq.last_token = int(token_id)
+                seq.last_token = token_id
+            if not seq.ignore_eos and token_id == self.eos and not seq.is_finished:
+                seq.status = SequenceStatus.FINISHED
+                self.block_manager.deallocate(seq)
+                self.running.remove(seq)
+                ended.append(seq)
         self.block_manager.hash_deferred_blocks()
+        return ended
 
     def postprocess(self, seqs: list[Sequence], token_ids: list[int]) -> None:
         for seq, token_id in zip(seqs, token_ids):

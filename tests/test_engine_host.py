@@ -284,11 +284,71 @@ def test_decode_steps_launched_ahead_of_their_ids_give_the_same_run():
     assert sum(1 for a, b in zip(log, log[1:]) if a == "launch" and b == "wait") >= 6
 
 
-def test_a_sequence_that_stops_at_eos_keeps_the_synchronous_path():
-    cfg = dict(max_num_sequences=2, max_num_batched_tokens=64, max_cached_blocks=16, block_size=4, eos=1003,
+class FakeFunctionRunner(FakeAsyncRunner):
+    """Ids that depend only on (sequence, position), so a run does not depend on which rows were computed for
+    nothing; ``eos_at`` maps a sequence's position in the batch order to the length at which it emits EOS."""
+
+    def __init__(self, eos, eos_at):
+        super().__init__()
+        self.eos, self.eos_at, self.order = eos, eos_at, {}
+
+    def _ids(self, seqs):
+        out = []
+        for s in seqs:
+            k = self.order.setdefault(s.seq_id, len(self.order))
+            out.append(self.eos if self.eos_at.get(k) == len(s) else 2000 + 37 * k + len(s))
+        return out
+
+    def launch_decode(self, seqs):
+        if not self.continues_last_decode(seqs):
+            assert all(t >= 0 for s in seqs for t in s.token_ids), "a refill needs real last tokens"
+        self.log.append("launch")
+        self.calls.append((False, [s.seq_id for s in seqs], [len(s) for s in seqs]))
+        self.last = ([s.seq_id for s in seqs], [len(s) for s in seqs])
+        return self.Handle(self._ids(seqs), self.log)
+
+    def run(self, seqs, is_prefill):
+        assert all(t >= 0 for s in seqs for t in s.token_ids), "a synchronous step needs real token ids"
+        self.last = None
+        self.log.append("run")
+        self.calls.append((is_prefill, [s.seq_id for s in seqs], [len(s) for s in seqs]))
+        return self._ids(seqs)
+
+
+def test_sequences_that_stop_at_eos_also_run_ahead_and_end_one_commit_late():
+    """Decode steps are launched ahead of their ids also when a sequence may stop at EOS: the EOS is seen when the
+    ids arrive, one step late, the sequence ends there, and the row the next step computed for it is dropped.  Tokens,
+    finish order and freed blocks equal the synchronous engine's; sequences that end by EOS, by count, at a block
+    boundary and in the step right after their prefill are all in the batch."""
+    eos = 7
+    cfg = dict(max_num_sequences=3, max_num_batched_tokens=64, max_cached_blocks=24, block_size=4, eos=eos,
                max_position=64)
-    runner = FakeAsyncRunner()
-    eng = LLMEngine(cfg, model_runner=runner)
-    out = eng.generate([[1, 2, 3], [4, 5]], SamplingParams(temperature=0.6, max_tokens=8, ignore_eos=False))
-    assert "launch" not in runner.log                              # EOS decides the schedule: ids first
-    assert [t[-1] for t in out["token_ids"]].count(1003) == 1 and min(len(t) for t in out["token_ids"]) < 8
+    prompts = [[1, 2, 3], [4, 5, 6, 8, 9], [10], [11, 12, 13, 14, 15, 16, 17], [18, 19]]
+    # sequence k emits EOS when it is eos_at[k] tokens long: 0 in its second decode step, 1 as the token that opens a
+    # new block (length 8), 2 never (ends by count), 3 with its first sampled token (the prefill's), 4 at length 9
+    eos_at = {0: 5, 1: 8, 3: 7, 4: 9}
+    sp = SamplingParams(temperature=0.6, max_tokens=10, ignore_eos=False)
+    runs = {}
+    for mode in (False, True):
+        runner = FakeFunctionRunner(eos, eos_at)
+        eng = LLMEngine(dict(cfg, async_decode=mode), model_runner=runner)
+        order = []
+        for p in prompts:
+            eng.add_prompt(p, sp)
+        while not eng.scheduler.is_finished() or eng.pending is not None:
+            finished, _, _ = eng.step()
+            order += [sid for sid, _ in finished]
+        runs[mode] = (order, eng, runner)
+        assert eng.pending is None and len(eng.scheduler.block_manager.free_block_ids) == 24
+    tokens = {}
+    for mode in (False, True):
+        runner = FakeFunctionRunner(eos, eos_at)
+        eng = LLMEngine(dict(cfg, async_decode=mode), model_runner=runner)
+        tokens[mode] = eng.generate(prompts, sp)["token_ids"]
+    assert tokens[True] == tokens[False]
+    lengths = [len(t) for t in tokens[True]]
+    assert lengths == [3, 4, 10, 1, 8] and [t[-1] for t in tokens[True]].count(eos) == 4
+    assert all(eos not in t[:-1] for t in tokens[True])                # nothing is generated past an EOS
+    assert all(len(runs[m][0]) == 5 and len(set(runs[m][0])) == 5 for m in (True, False))   # each reported once
+    log = runs[True][2].log
+    assert sum(1 for a, b in zip(log, log[1:]) if a == "launch" and b == "wait") >= 4  # steps did run ahead

@@ -245,3 +245,32 @@ def test_graph_decode_with_split_partitions_in_every_bucket():
     assert [len(t) for t in graphed] == [20] * 64
     same = sum(a == b for a, b in zip(eager, graphed))
     assert same >= 58, (same,)                        # a 1-ulp GEMM difference between buckets may flip a tie, rarely
+
+
+def test_steps_run_ahead_for_sequences_that_stop_at_eos():
+    """The hipGraph engine launches decode steps ahead of their ids also for sequences that can stop at EOS; the
+    EOS is noticed one step late and the extra row is dropped.  With an EOS id taken from the middle of a run that
+    ignores EOS: several sequences end early, each exactly at its first EOS, nothing is generated past one, every
+    block returns to the pool, and the first tokens of the first batch equal the run of an engine that waits for every
+    step's ids.  (Later tokens need not: the sampler's noise is keyed by step and row, and the engine that runs ahead
+    admits the next waiting sequence one step later than the one that waits.)"""
+    cfg = dict(SMALL, enforce_eager=False, max_num_sequences=4, max_cached_blocks=96, max_model_length=160)
+    prompts = _prompts(9, 3, 40, seed=61)
+    free = LLMEngine(cfg).generate(prompts, SamplingParams(temperature=0.9, max_tokens=48, ignore_eos=True))["token_ids"]
+    # the id that occurs in the most sequences somewhere after their 3rd and before their last token
+    counts = {}
+    for toks in free:
+        for t in set(toks[3:-1]):
+            counts[t] = counts.get(t, 0) + 1
+    eos = max(counts, key=counts.get)
+    assert counts[eos] >= 2
+    sp = SamplingParams(temperature=0.9, max_tokens=48, ignore_eos=False)
+    outs = {}
+    for ahead in (True, False):
+        eng = LLMEngine(dict(cfg, eos=eos, async_decode=ahead))
+        outs[ahead] = out = eng.generate(prompts, sp)["token_ids"]
+        assert len(eng.scheduler.block_manager.free_block_ids) == cfg["max_cached_blocks"] and eng.pending is None
+        assert all(1 <= len(t) <= 48 and (t[-1] == eos or len(t) == 48) and eos not in t[:-1] for t in out)
+        assert sum(len(t) < 48 for t in out) >= 2
+    first_eos = min(len(t) for t in outs[False][:4])            # the first batch runs in step until its first EOS
+    assert all(a[:first_eos] == b[:first_eos] for a, b in zip(outs[True][:4], outs[False][:4]))
