@@ -352,3 +352,47 @@ def test_sequences_that_stop_at_eos_also_run_ahead_and_end_one_commit_late():
     assert all(len(runs[m][0]) == 5 and len(set(runs[m][0])) == 5 for m in (True, False))   # each reported once
     log = runs[True][2].log
     assert sum(1 for a, b in zip(log, log[1:]) if a == "launch" and b == "wait") >= 4  # steps did run ahead
+
+
+def test_run_ahead_equals_waiting_engine_on_random_schedules():
+    """Property: for random prompts, EOS positions, token limits, batch limits and block sizes (preemption when the
+    pool is small included) the engine that launches decode steps ahead of their ids returns the same tokens per
+    sequence as the one that waits, reports every sequence once, and returns every block."""
+    from hypothesis import given, settings, strategies as st
+
+    @settings(max_examples=120, deadline=None)
+    @given(st.data())
+    def check(data):
+        n = data.draw(st.integers(1, 7))
+        prompts = [list(range(100 * i + 1, 100 * i + 1 + data.draw(st.integers(1, 14)))) for i in range(n)]
+        max_tokens = data.draw(st.integers(1, 12))
+        block_size = data.draw(st.sampled_from([2, 4, 8]))
+        longest = max(map(len, prompts)) + max_tokens
+        blocks = data.draw(st.integers(-(-longest // block_size) + 1, 40))      # at least one sequence always fits
+        cfg = dict(max_num_sequences=data.draw(st.integers(1, 4)), max_num_batched_tokens=64, max_cached_blocks=blocks,
+                   block_size=block_size, eos=7, max_position=64)
+        eos_at = {k: data.draw(st.integers(len(p), len(p) + max_tokens + 2)) for k, p in enumerate(prompts)
+                  if data.draw(st.booleans())}
+        sp = SamplingParams(temperature=0.6, max_tokens=max_tokens, ignore_eos=data.draw(st.booleans()))
+        outs = []
+        for ahead in (True, False):
+            eng = LLMEngine(dict(cfg, async_decode=ahead), model_runner=FakeFunctionRunner(7, eos_at))
+            for p in prompts:
+                eng.add_prompt(p, sp)
+            reported = []
+            steps = 0
+            while not eng.scheduler.is_finished() or eng.pending is not None:
+                finished, _, _ = eng.step()
+                reported += finished
+                steps += 1
+                assert steps < 2000
+            assert len(reported) == n and len({sid for sid, _ in reported}) == n
+            assert len(eng.scheduler.block_manager.free_block_ids) == blocks and eng.pending is None
+            outs.append([toks for _, toks in sorted(reported)])
+        assert outs[0] == outs[1]
+        for toks in outs[0]:
+            assert 1 <= len(toks) <= max_tokens and all(t >= 0 for t in toks)
+            if not sp.ignore_eos:
+                assert 7 not in toks[:-1]
+
+    check()
