@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,loads_probe,engine,engine16,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,loads_probe,engine,engine16,engine64,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -790,8 +790,11 @@ def main():
         extra["engine_16seq_eager"] = bench_engine(args, 16, False)
         extra["engine_16seq_graph"] = bench_engine(args, 16, True)
         extra["engine_64seq_graph"] = bench_engine(args, 64, True)
-    elif "engine16" in only:                           # the one configuration a kernel trace of a decode step wants
-        extra["engine_16seq_graph"] = bench_engine(args, 16, True)
+    else:                                              # one configuration alone, as a kernel trace of a decode step wants
+        if "engine16" in only:
+            extra["engine_16seq_graph"] = bench_engine(args, 16, True)
+        if "engine64" in only:
+            extra["engine_64seq_graph"] = bench_engine(args, 64, True)
 
     if "loads_only" in head:
         extra["decode_loads_only"] = head["loads_only"]
