@@ -8,6 +8,8 @@
 //   per wave and 32-wide k step: A = W (row n0 + lane%16, 16 B = 8 k values of class lane/16), B = x^T (column m =
 //   lane%16, the same k values), v_mfma_f32_16x16x32: lane l ends with out[m = l%16][n0 + 4 (l/16) + r], r < 4.
 //   The partial sums meet in LDS; wave 0 adds them, adds the bias and stores 8 bytes per lane.
+// From 17 rows on every 16 rows get workgroups of their own (the same code; the workgroups of one column tile run on
+// one XCD and share the weights in its L2) rather than one workgroup holding up to four row tiles in registers.
 // mvllm_norm_linear_small_m is the same product with the launches around it folded in: the residual add + RMSNorm in
 // front of the layer's first projections (src/myvllm/models/qwen3.py:197-212 through layers/layernorm.py:9-28) as
 // the kernel's prologue, and SiluAndMul behind the gate/up projection (layers/activation.py:15-18) as its epilogue,
@@ -26,6 +28,7 @@ struct LinearArgs {
   int64_t x_row_stride;   // elements between rows of x
   int M, N, K;
   int cols;               // output columns per workgroup: 16, or 8 / 4 (plain product only) to spread few columns over more CUs
+  int row_tiles;          // > 1: the grid holds this many workgroups per column tile, one per 16 rows of x (MT == 1)
   // NORM: x is first replaced by rms_norm(x + residual) * gamma, as mvllm_add_rms_norm computes it
   const void* residual;   // [M, K] contiguous, or null (then the norm of x alone)
   void* residual_out;     // [M, K] contiguous: x + residual in the element type; must not alias x or residual
@@ -81,12 +84,28 @@ __global__ __launch_bounds__(64 * W) void linear_small_kernel(const LinearArgs a
   const int col = lane & 15, cls = lane >> 4;
   const int ksl = a.K / W;                               // this wave's share of K
   const int koff = wave * ksl + cls * 8;                 // first k of this lane in every 32-wide step
+  // column tile and first row of this workgroup.  With row tiles the workgroups of one column tile read the same
+  // weights: consecutive workgroups go to the eight XCDs in turn, so the row tiles of a column tile are dealt 8
+  // apart and meet in one L2.
+  int ct = blockIdx.x, m0 = 0;
+  if (MT == 1 && a.row_tiles > 1) {
+    const int tiles = gridDim.x / a.row_tiles;
+    if ((tiles & 7) == 0) {
+      const int g = ct >> 3;
+      m0 = 16 * (g % a.row_tiles);
+      ct = (g / a.row_tiles) * 8 + (ct & 7);
+    } else {
+      m0 = 16 * (ct % a.row_tiles);
+      ct = ct / a.row_tiles;
+    }
+  }
+  const int mrows = min(a.M - m0, 16 * MT);              // rows of this workgroup
   int wrow, n0;                                          // weight row of this lane; first output column of the workgroup
   if constexpr (GLU) {
-    n0 = blockIdx.x * 8;
+    n0 = ct * 8;
     wrow = col < 8 ? n0 + col : a.N / 2 + n0 + col - 8;
   } else {
-    n0 = blockIdx.x * a.cols;
+    n0 = ct * a.cols;
     wrow = n0 + min(col, a.cols - 1);
   }
   const bool wlive = GLU || col < a.cols;                // weight rows of a narrow tile: the other lanes load nothing
@@ -95,7 +114,7 @@ __global__ __launch_bounds__(64 * W) void linear_small_kernel(const LinearArgs a
   const T* xp[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    rowm[mt] = min(16 * mt + col, a.M - 1);              // rows past M repeat the last one; they are not stored
+    rowm[mt] = m0 + min(16 * mt + col, mrows - 1);       // rows past the last repeat it; they are not stored
     xp[mt] = reinterpret_cast<const T*>(a.x) + (int64_t)rowm[mt] * a.x_row_stride + koff;
   }
   v4f acc[MT];
@@ -103,9 +122,15 @@ __global__ __launch_bounds__(64 * W) void linear_small_kernel(const LinearArgs a
   for (int mt = 0; mt < MT; ++mt) acc[mt] = (v4f){0.f, 0.f, 0.f, 0.f};
   for (int k = 0; k < ksl; k += 32 * U) {
     uint4 wf[U], xf[MT][U];
+    if (MT == 1 && a.row_tiles > 1) {                    // the other row tiles' workgroups read the same weights: keep them in L2
 #pragma unroll
-    for (int u = 0; u < U; ++u)                          // weights are read once: stream them
-      wf[u] = wlive ? load16_stream(wp + k + 32 * u) : make_uint4(0u, 0u, 0u, 0u);
+      for (int u = 0; u < U; ++u)
+        wf[u] = wlive ? *reinterpret_cast<const uint4*>(wp + k + 32 * u) : make_uint4(0u, 0u, 0u, 0u);
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u)                        // weights are read once: stream them
+        wf[u] = wlive ? load16_stream(wp + k + 32 * u) : make_uint4(0u, 0u, 0u, 0u);
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -139,9 +164,10 @@ __global__ __launch_bounds__(64 * W) void linear_small_kernel(const LinearArgs a
 #pragma unroll
           for (int e = 0; e < 8; ++e) ss[mt] = ss[mt] + h[e] * h[e];
         }
-        // the next residual: row b of h is written by workgroup b (every workgroup holds every row)
-        if (a.residual_out && 16 * mt + col == (int)blockIdx.x && (int)blockIdx.x < a.M) {
-          T* hp = reinterpret_cast<T*>(a.residual_out) + (int64_t)blockIdx.x * a.K + koff;
+        // the next residual: row b of the workgroup's rows is written by the workgroup of column tile b (all of
+        // them hold these rows)
+        if (a.residual_out && 16 * mt + col == ct && ct < mrows) {
+          T* hp = reinterpret_cast<T*>(a.residual_out) + (int64_t)(m0 + ct) * a.K + koff;
 #pragma unroll
           for (int u = 0; u < U; ++u) *reinterpret_cast<uint4*>(hp + 32 * u) = xf[mt][u];
         }
@@ -197,7 +223,7 @@ __global__ __launch_bounds__(64 * W) void linear_small_kernel(const LinearArgs a
       const float4 p = part[(w * MT + mt) * 64 + lane];
       s[0] += p.x; s[1] += p.y; s[2] += p.z; s[3] += p.w;
     }
-    const int m = 16 * mt + col;
+    const int m = m0 + 16 * mt + col;
     T r4[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) r4[r] = from_float<T>(s[r] + b4[r]);
@@ -230,13 +256,14 @@ static bool norm_fits(int W, int mt, int steps) {
 
 template <typename T, int W, bool NORM, bool GLU>
 static int launch_linear_w(const LinearArgs& a, hipStream_t stream) {
-  const dim3 grid((unsigned)(GLU ? a.N / 16 : a.N / a.cols)), block(64 * W);  // GLU: 8 gate + 8 up columns each
-  const int mt = (a.M + 15) / 16;
+  const int tiles = GLU ? a.N / 16 : a.N / a.cols;       // GLU: 8 gate + 8 up columns each
+  const dim3 grid((unsigned)(tiles * a.row_tiles)), block(64 * W);
+  const int mt = a.row_tiles > 1 ? 1 : (a.M + 15) / 16;  // row tiles per workgroup
   const int steps = a.K / W / 32;                        // 32-wide k steps per wave
   if constexpr (NORM) {
     // the wave's whole share of K in one burst, at most two row tiles; the combinations left out would not fit the
     // registers of their workgroup size
-    if (!norm_fits(W, mt, steps) || (int)grid.x < a.M) return MVLLM_ERR_UNSUPPORTED;
+    if (!norm_fits(W, mt, steps) || tiles < (a.M < 16 * mt ? a.M : 16 * mt)) return MVLLM_ERR_UNSUPPORTED;
     if (steps == 8) {
       if constexpr (W <= 8) {
         if (mt == 1) linear_small_kernel<T, 1, 8, W, true, GLU><<<grid, block, 0, stream>>>(a);
@@ -273,10 +300,34 @@ static int linear_cols(int N, bool plain) {
   return plain && N / 16 < 128 ? MVLLM_LINEAR_NARROW_COLS : 16;
 }
 
+#ifndef MVLLM_LINEAR_ROW_TILE_FROM
+#define MVLLM_LINEAR_ROW_TILE_FROM 17
+#endif
+// workgroups per column tile: from this many rows on, every 16 rows of x get a workgroup of their own (the code of
+// the 16-row case, which holds few registers and asks for everything at once) instead of one workgroup that walks
+// all rows; the weights are then read once from HBM and again from L2
+static int linear_row_tiles(int M) {
+#ifdef MVLLM_EXPERIMENT
+  if (const char* e = getenv("MVLLM_LINEAR_ROW_TILE_FROM")) return M >= atoi(e) ? (M + 15) / 16 : 1;
+#endif
+  return M >= MVLLM_LINEAR_ROW_TILE_FROM ? (M + 15) / 16 : 1;
+}
+
 // waves per workgroup: more of them share a column tile's K when the column tiles alone give too few workgroups to
 // keep the memory system busy; 12 where 16 do not divide K but 12 do, each with one burst of 256 values (K = 3072:
 // the MLP's down projection)
-static int linear_waves(int tiles, int K, bool plain) {
+static int linear_waves(int tiles, int K, bool plain, bool norm, int mt) {
+  if (norm) {
+    // a wave's share of K must be one burst of 4 or 8 steps: the fewest waves that give 1024 of them in all, else the
+    // most that fit; 0 when no split does
+    int best = 0;
+    for (int w = 4; w <= 16; w *= 2) {
+      if (K % (32 * w) != 0 || !norm_fits(w, mt, K / w / 32)) continue;
+      best = w;
+      if ((int64_t)tiles * w >= 1024) break;
+    }
+    return best;
+  }
   int w = 4;
   while (w < 16 && (int64_t)tiles * w < 1024 && K % (2 * w * 128) == 0) w *= 2;
   if (plain && w == 8 && (int64_t)tiles * w < 1024 && K == 12 * 256) w = 12;
@@ -285,7 +336,9 @@ static int linear_waves(int tiles, int K, bool plain) {
 
 template <typename T, bool NORM, bool GLU>
 static int launch_linear_small(const LinearArgs& a, hipStream_t stream) {
-  switch (linear_waves(GLU ? a.N / 16 : a.N / a.cols, a.K, !NORM && !GLU)) {
+  switch (linear_waves((GLU ? a.N / 16 : a.N / a.cols) * a.row_tiles, a.K, !NORM && !GLU, NORM,
+                       a.row_tiles > 1 ? 1 : (a.M + 15) / 16)) {
+    case 0: return MVLLM_ERR_UNSUPPORTED;
     case 4: return launch_linear_w<T, 4, NORM, GLU>(a, stream);
     case 8: return launch_linear_w<T, 8, NORM, GLU>(a, stream);
     case 12:
@@ -324,6 +377,7 @@ extern "C" int mvllm_linear_small_m(void* out, const void* x, const void* w, con
   LinearArgs a{};
   a.out = out; a.x = x; a.w = w; a.bias = bias; a.x_row_stride = x_row_stride; a.M = M; a.N = N; a.K = K;
   a.cols = linear_cols(N, true);
+  a.row_tiles = linear_row_tiles(M);
   return dtype == MVLLM_BF16 ? launch_linear_fused<bf16_t>(a, false, (hipStream_t)stream)
                              : launch_linear_fused<f16_t>(a, false, (hipStream_t)stream);
 }
@@ -332,8 +386,11 @@ extern "C" int mvllm_linear_small_m_plan(int M, int N, int K, int norm, int glu,
   if (dtype != MVLLM_BF16 && dtype != MVLLM_F16) return dtype_size(dtype) == 0 ? MVLLM_ERR_BAD_DTYPE : MVLLM_ERR_UNSUPPORTED;
   if (M <= 0 || N <= 0 || K <= 0) return MVLLM_ERR_BAD_SHAPE;
   if (M > 64 || N % 16 != 0 || K % 512 != 0 || (glu && N % 32 != 0)) return MVLLM_ERR_UNSUPPORTED;
-  const int w = linear_waves(N / linear_cols(N, !norm && !glu), K, !norm && !glu), mt = (M + 15) / 16, steps = K / w / 32;
-  if (norm ? (!norm_fits(w, mt, steps) || N / 16 < M) : (steps % 4 != 0)) return MVLLM_ERR_UNSUPPORTED;
+  const int rt = linear_row_tiles(M), mt = rt > 1 ? 1 : (M + 15) / 16;
+  const int w = linear_waves(N / linear_cols(N, !norm && !glu) * rt, K, !norm && !glu, norm != 0, mt);
+  if (w == 0) return MVLLM_ERR_UNSUPPORTED;
+  const int steps = K / w / 32;
+  if (norm ? (!norm_fits(w, mt, steps) || N / 16 < (M < 16 * mt ? M : 16 * mt)) : (steps % 4 != 0)) return MVLLM_ERR_UNSUPPORTED;
   if (waves) *waves = w;
   return MVLLM_OK;
 }
@@ -354,6 +411,7 @@ extern "C" int mvllm_norm_linear_small_m(void* out, void* residual_out, const vo
   a.out = out; a.x = x; a.w = w; a.bias = bias; a.x_row_stride = x_row_stride; a.M = M; a.N = N; a.K = K;
   a.residual = residual; a.residual_out = residual_out; a.gamma = gamma; a.eps = eps;
   a.cols = linear_cols(N, !gamma && !glu);
+  a.row_tiles = linear_row_tiles(M);
   return dtype == MVLLM_BF16 ? launch_linear_fused<bf16_t>(a, glu != 0, (hipStream_t)stream)
                              : launch_linear_fused<f16_t>(a, glu != 0, (hipStream_t)stream);
 }

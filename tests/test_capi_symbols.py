@@ -180,11 +180,12 @@ def test_argument_validation_without_gpu():
     w = ctypes.c_int(0)
     assert plan(16, 4096, 1024, 1, 0, 1, ctypes.byref(w)) == 0 and w.value == 4     # the engine's QKV projection
     assert plan(32, 6144, 1024, 1, 1, 1, ctypes.byref(w)) == 0 and w.value == 4     # gate/up with norm and SiLU
-    assert plan(33, 4096, 1024, 1, 0, 1, None) == -4                                # norm: at most 32 rows
+    assert plan(33, 4096, 1024, 1, 0, 1, ctypes.byref(w)) == 0 and w.value == 4     # 17 rows and more: a workgroup per 16 rows
+    assert plan(64, 6144, 1024, 1, 1, 1, ctypes.byref(w)) == 0 and w.value == 4
     assert plan(33, 4096, 1024, 0, 0, 1, None) == 0                                 # plain: up to 64
     assert plan(16, 1024, 3072, 1, 0, 1, None) == -4                                # K / waves is not one burst
     assert plan(16, 1024, 2048, 1, 0, 1, ctypes.byref(w)) == 0 and w.value == 16    # 16 waves, 128 values each
-    assert plan(32, 1024, 2048, 1, 0, 1, None) == -4                                # ... with one row tile only
+    assert plan(32, 1024, 2048, 1, 0, 1, ctypes.byref(w)) == 0 and w.value == 8     # two row tiles: twice the workgroups, half the waves
     assert plan(16, 4096, 1024, 1, 0, 0, None) == -4 and plan(16, 4096, 1024, 1, 0, 9, None) == -2
     lm = lib.mvllm_lm_head_sample
     #   out hidden stride row_index weight temps seed offset offset_dev batch vocab K dtype ws ws_bytes stream

@@ -61,7 +61,7 @@ def test_linear_small_m_strided_rows_and_module_dispatch():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("m", [1, 5, 16, 17, 32])
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 32, 48, 64])
 @pytest.mark.parametrize("n,k,bias,glu", [(4096, 1024, False, False), (6144, 1024, True, True), (1024, 2048, True, False),
                                           (2048, 512, True, True), (4096, 1024, True, True)])
 @pytest.mark.parametrize("with_residual", [True, False])
@@ -77,9 +77,7 @@ def test_norm_linear_equals_the_separate_launches(dtype, m, n, k, bias, glu, wit
     g = torch.Generator().manual_seed(m)
     gamma = (1 + 0.2 * torch.randn(k, generator=g)).to(DEV)
     res = torch.randn(m, k, generator=g).to(dtype).to(DEV) if with_residual else None
-    if not norm_linear_small_m_takes(x, w, 32, glu=glu):
-        assert m > 16 and k == 2048                      # 16 waves per column tile hold one row tile only
-        return
+    assert norm_linear_small_m_takes(x, w, 64, glu=glu)   # 17 rows and more: one workgroup per 16 rows and column tile
     normed = add_rms_norm(x, gamma, 1e-6, res)
     normed, want_res = normed if with_residual else (normed, x)
     want = linear_small_m(normed, w, b)
