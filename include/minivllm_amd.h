@@ -365,8 +365,8 @@ int mvllm_linear_small_m(void* out, const void* x, const void* w, const void* bi
  *   glu != 0:       W is [2F, K] (gate rows, then up rows, as layers/activation.py:15-18 chunks the output), out is
  *                   [M, F] = silu(x' Wg^T + bg) * (x' Wu^T + bu) with the roundings of mvllm_silu_and_mul on the
  *                   rounded projection; N = 2F, N % 32 == 0.
- * Shapes as mvllm_linear_small_m, and for gamma != NULL: M <= 32, N / 16 >= M, K / waves one burst of 128 or 256
- * values (mvllm_linear_small_m_plan says whether a shape is taken); otherwise MVLLM_ERR_UNSUPPORTED and the caller
+ * Shapes as mvllm_linear_small_m, and for gamma != NULL: N / 16 >= min(M, 16), K / waves one burst of 128 or 256
+ * values with 4, 8 or 16 waves (mvllm_linear_small_m_plan says whether a shape is taken); otherwise MVLLM_ERR_UNSUPPORTED and the caller
  * runs the separate launches.
  */
 int mvllm_norm_linear_small_m(void* out, void* residual_out, const void* x, const void* residual,
