@@ -279,6 +279,22 @@ def bench_prefill_store(args, which, want_cpu=False):
             out["prefill"]["cpu_baseline"] = cpu_prefill_baseline(q, k, v, cu, lengths, scale, hq, hkv, d, flops,
                                                                   flash_attention_prefill)
     if "prefill" in which:
+        # the same kernel away from config 2's short prompts: 4 prompts of 8192 tokens (the start and end of a
+        # workgroup's life are a small share of its 128 key tiles)
+        long_lengths = [8192] * 4
+        ql, kl, vl = (torch.randn(sum(long_lengths), h, d, generator=dg, device=dev).to(torch.bfloat16) for h in (hq, hkv, hkv))
+        cul = torch.tensor([0] + long_lengths, dtype=torch.int32).cumsum(0).to(torch.int32).to(dev)
+        _, event_ms_l = time_steps(lambda: flash_attention_prefill(ql, kl, vl, cul, scale, hq, hkv, d),
+                                   max(3, args.steps // 4), 2, EXTRA_WARM_MS)
+        flops_l = 4 * hq * d * sum(n * (n + 1) // 2 for n in long_lengths)
+        out["prefill_long_prompts"] = {
+            "workload": "varlen causal prefill, 4 prompts of 8192 tokens, Hq32 Hkv8 D128 bf16",
+            "tokens": sum(long_lengths), "algorithmic_flops": flops_l, "event_ms_per_step": event_ms_l,
+            "tflops": flops_l / (event_ms_l * 1e-3) / 1e12,
+            "roofline": roofline("mfma", flops_l / (event_ms_l * 1e-3) / 1e12, "prefill_mfma_kernel"),
+        }
+        del ql, kl, vl
+    if "prefill" in which:
         # the same prompts with the first half (whole 16-token blocks) already cached: only the second half is
         # computed, every key comes from a block-16 paged cache
         from minivllm_amd.layers.attention import flash_attention_prefill_paged
