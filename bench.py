@@ -418,7 +418,7 @@ def bench_int8(args, want_cpu=True, want_probe=False):
                                              vs[ids].cpu(), torch.arange(need[b], dtype=torch.int32).unsqueeze(0),
                                              ctx[b:b + 1], scale, hq, hkv, d, bs)
             worst = max(worst, (got[b:b + 1] - want).abs().max().item())
-        check = {"gpu_vs_oracle_max_abs": worst, "oracle_sequences": 8}
+        check.update({"gpu_vs_oracle_max_abs": worst, "oracle_sequences": 8})
     return {
         **check,
         "roofline": roofline("hbm", nbytes / (event_ms * 1e-3) / 1e9, "decode_mfma_int8_kernel + decode_reduce_kernel"),
