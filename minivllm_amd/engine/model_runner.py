@@ -6,8 +6,9 @@ Config keys (one set of names; the reference's runner and engine disagree on two
 ``vocab_size hidden_size num_layers num_heads num_kv_heads head_dim intermediate_size base
 rms_norm_epsilon qkv_bias ffn_bias scale tie_word_embeddings max_position``; engine keys ``block_size
 max_cached_blocks max_num_sequences max_num_batched_tokens dtype kv_cache_dtype seed``; ``linear_small_rows`` (default
-32): projections of at most that many rows, a decode step, run as the single-launch ``linear_small_m`` (0: always the
-library GEMM; above 32 rows the library is faster); ``fused_lm_head`` (default true): LM head and sampler as one pass
+64): projections of at most that many rows, a decode step, run as the single-launch ``linear_small_m``, the gate/up
+projection with SiluAndMul as its epilogue (0: always the library GEMM); ``linear_norm_rows`` (default 32): up to that
+many rows the residual norms run as prologues of the projections behind them; ``fused_lm_head`` (default true): LM head and sampler as one pass
 over the weights for at most 64 rows (``lm_head_sample``), otherwise the library GEMM and ``sample_tokens``.
 """
 from __future__ import annotations
@@ -67,7 +68,7 @@ class ModelRunner:
             num_layers=config["num_layers"], tie_word_embeddings=config.get("tie_word_embeddings", True),
             block_size=self.block_size, kv_cache_dtype=self.kv_cache_dtype,
             fused_qk=config.get("fused_qk", True), fused_elementwise=config.get("fused_elementwise", True),
-            small_rows=config.get("linear_small_rows", 32))
+            small_rows=config.get("linear_small_rows", 64), norm_rows=config.get("linear_norm_rows", 32))
         self.model.reset_parameters(seed=config.get("seed", 0))
         self.model.to(device=self.device, dtype=self.dtype).eval()
         self.sampler = Sampler()

@@ -63,21 +63,27 @@ class Qwen3MLP(nn.Module):
         self.gate_up = Linear(hidden_size, 2 * intermediate_size, bias=bias, small_rows=small_rows)
         self.activation = SiluAndMul(fused)
         self.gate_down = Linear(intermediate_size, hidden_size, bias=bias, small_rows=small_rows)
+        self.small_rows, self.fused = small_rows, fused
 
     def forward(self, x):
+        # a decode step's rows: SiluAndMul as the epilogue of the gate/up projection (one launch instead of two)
+        if (self.small_rows and self.fused and x.dim() == 2 and x.shape[0] <= self.small_rows and x.is_contiguous()
+                and norm_linear_small_m_takes(x, self.gate_up.weight, self.small_rows, norm=False, glu=True)):
+            return self.gate_down(norm_linear_small_m(x, self.gate_up.weight, self.gate_up.bias, glu=True))
         return self.gate_down(self.activation(self.gate_up(x)))
 
 
 class Qwen3DecoderLayer(nn.Module):
     def __init__(self, hidden_size, intermediate_size, ffn_bias, rms_norm_epsilon, fused_elementwise=True,
-                 small_rows=0, **attn_kwargs):
+                 small_rows=0, norm_rows=32, **attn_kwargs):
         super().__init__()
         self.input_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
         self.self_attn = Qwen3Attention(hidden_size=hidden_size, rms_norm_epsilon=rms_norm_epsilon,
                                         small_rows=small_rows, **attn_kwargs)
         self.post_attention_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
         self.mlp = Qwen3MLP(hidden_size, intermediate_size, ffn_bias, fused_elementwise, small_rows)
-        self.small_rows, self.fused_elementwise = small_rows, fused_elementwise
+        # the norm prologue normalises a workgroup's rows once per column tile: it pays up to about 32 rows
+        self.norm_rows, self.fused_elementwise = min(small_rows, norm_rows), fused_elementwise
 
     def _forward_few_rows(self, x, residual, positions):
         """A decode step's few rows: the two residual norms run as the prologues of the projections that follow them
@@ -97,7 +103,7 @@ class Qwen3DecoderLayer(nn.Module):
         return mlp.gate_down(act), residual
 
     def forward(self, x, residual, positions):
-        rows = self.small_rows
+        rows = self.norm_rows
         if (rows and self.fused_elementwise and x.dim() == 2 and x.shape[0] <= rows and x.is_contiguous()
                 and norm_linear_small_m_takes(x, self.self_attn.qkv_projection.weight, rows)
                 and norm_linear_small_m_takes(x, self.mlp.gate_up.weight, rows, glu=True)):
@@ -116,7 +122,8 @@ class Qwen3ForCausalLM(nn.Module):
     def __init__(self, vocab_size, hidden_size, num_heads, head_dim=None, scale=1.0, num_kv_heads=None,
                  rms_norm_epsilon=1e-6, qkv_bias=False, base=1_000_000, max_position=4096,
                  intermediate_size=3072, ffn_bias=True, num_layers=8, tie_word_embeddings=True,
-                 block_size=256, kv_cache_dtype="auto", fused_qk=True, fused_elementwise=True, small_rows=0):
+                 block_size=256, kv_cache_dtype="auto", fused_qk=True, fused_elementwise=True, small_rows=0,
+                 norm_rows=32):
         super().__init__()
         head_dim = head_dim if head_dim is not None else hidden_size // num_heads
         num_kv_heads = num_kv_heads if num_kv_heads is not None else num_heads
@@ -126,7 +133,8 @@ class Qwen3ForCausalLM(nn.Module):
             Qwen3DecoderLayer(hidden_size, intermediate_size, ffn_bias, rms_norm_epsilon, num_heads=num_heads,
                               head_dim=head_dim, scale=scale, num_kv_heads=num_kv_heads, qkv_bias=qkv_bias,
                               rotary=rotary, block_size=block_size, kv_cache_dtype=kv_cache_dtype,
-                              fused_qk=fused_qk, fused_elementwise=fused_elementwise, small_rows=small_rows)
+                              fused_qk=fused_qk, fused_elementwise=fused_elementwise, small_rows=small_rows,
+                              norm_rows=norm_rows)
             for _ in range(num_layers)])
         self.final_layernorm = RMSNorm(hidden_size, rms_norm_epsilon, fused_elementwise)
         self.lm_head_weight = self.embedding_layer.weight if tie_word_embeddings else nn.Parameter(
