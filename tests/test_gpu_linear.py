@@ -102,6 +102,11 @@ def test_norm_linear_without_norm_is_the_plain_product_and_glu_pairs_the_right_c
     x = x.contiguous()
     assert torch.equal(norm_linear_small_m(x, w, b), linear_small_m(x, w, b))
     assert torch.equal(norm_linear_small_m(x, w, b, glu=True), silu_and_mul(linear_small_m(x, w, b)))
+    for m, n, k in ((60, 6144, 1024), (33, 2048, 1024), (64, 96, 512)):     # a workgroup per 16 rows (the engine's MLP at 33-64 rows)
+        xm, wm, bm = _case(412 + m, m, n, k, torch.bfloat16, True)
+        xm = xm.contiguous()
+        assert torch.equal(norm_linear_small_m(xm, wm, bm), linear_small_m(xm, wm, bm))
+        assert torch.equal(norm_linear_small_m(xm, wm, bm, glu=True), silu_and_mul(linear_small_m(xm, wm, bm)))
     w2 = torch.zeros_like(w)
     b2 = torch.zeros_like(b)
     j = 437                                              # silu(gate_j) * up_j: only column j can be non-zero
