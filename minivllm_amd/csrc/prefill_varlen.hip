@@ -340,8 +340,11 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   // K rows are read 16 at a time with the same logical chunk: the swizzle spreads them over the banks.  With 128-byte
   // rows two rows share a 256-byte bank line, so the row index is halved first.
   auto kswz = [](int row) __attribute__((always_inline)) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
-  // V is read by the transposing loads as 4 rows x 64 bytes per 16 lanes
-  auto vswz = [](int row) __attribute__((always_inline)) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
+  // V is read by the transposing loads as 4 rows x 64 bytes per 16 lanes: bits 2-3 of the chunk index take the row's
+  // low bits so that the four rows land in four 64-byte groups.  Bit 0 (D = 128) swaps the chunks of a pair in odd
+  // rows; the reads do not care (the pair stays in its group), and the INT8 conversion's LDS writes, which go two rows
+  // x four quarters at a time over 128 bytes of banks, meet 2-way instead of 4-way (32 -> 16 clocks per write).
+  auto vswz = [](int row) __attribute__((always_inline)) { return D == 128 ? (((row & 3) << 2) | (row & 1)) : (((row >> 1) & 1) << 2); };
   constexpr int ROW_TILES = kPfWaves / HPW;     // 32-row query tiles per workgroup
   constexpr int ROWS_PER_WAVE = kBN / kPfWaves; // K/V tile rows one wave copies (4 per instruction)
   constexpr int BM = kWaveRows * ROW_TILES;     // query rows per workgroup
@@ -590,7 +593,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   // Per-lane LDS byte offsets, computed once: the xor swizzle keeps the compiler from folding them into
   // instruction offsets, so they live in registers and every LDS read below is base + immediate.
   //   K: row l32 (+32 rows per tk = +8192 B), 16-byte chunk (2*ks + hi) ^ (l32 & 15)
-  //   V: row 4*hi + (lane&15)/4 (+8, +16*st, +32*tk rows), chunk (4*td + 2*half + ...) ^ 4*(row & 3)
+  //   V: row 4*hi + (lane&15)/4 (+8, +16*st, +32*tk rows), chunk (4*td + 2*half + ...) ^ (4*(row & 3) | (row & 1))
   const int i16 = lane & 15;
   const int half = (lane >> 4) & 1;
   int k_off[kKS];
