@@ -121,3 +121,44 @@ def test_store_int8_full_size_invariants():
     assert torch.equal(kc.view(-1, hkv, d)[slots.to(DEV)].cpu(), codes)
     assert torch.equal(ks.view(-1, hkv)[slots.to(DEV)].cpu(), scales)
     assert int(kc.abs().amax(-1).min()) == 127 and int(vc.abs().amax(-1).min()) == 127
+
+
+def test_store_int8_codes_at_rounding_boundaries():
+    """Values whose quotient x / scale lies on or within a few units in the last place of k + 1/2, where a reciprocal
+    multiply and the IEEE division can round to different codes, and the divisors at the ends of the range (denormal,
+    tiny, huge): the codes and scales equal the oracle's (torch's fp32 division and round-half-even) bit for bit."""
+    d, hkv, bs = 128, 2, 16
+    g = torch.Generator().manual_seed(77)
+    rows = []
+    for amax in (127.0, 100.0, 3.3, 1e-3, 7e4, 1.0 / 3.0, 2e-38, 1e-41, 3e38, 6.02e23):
+        scale = torch.tensor(amax, dtype=torch.float32) / 127.0
+        for _ in range(6):
+            kk = torch.randint(-126, 126, (d,), generator=g).float()
+            x = (kk + 0.5) * scale                                  # the quotient is k + 1/2 up to rounding
+            steps = torch.randint(-3, 4, (d,), generator=g)
+            for _ in range(3):                                      # ... and up to 3 units in the last place around it
+                x = torch.where(steps > 0, torch.nextafter(x, torch.tensor(float("inf"))), x)
+                x = torch.where(steps < 0, torch.nextafter(x, torch.tensor(float("-inf"))), x)
+                steps = steps - steps.sign()
+            x[int(torch.randint(0, d, (1,), generator=g))] = amax   # the vector's maximum fixes the scale
+            rows.append(x)
+    t = len(rows) // hkv
+    k = torch.stack(rows[:t * hkv]).view(t, hkv, d)
+    v = -k.flip(0)
+    nb = -(-t // bs)
+    slots = torch.randperm(nb * bs, generator=g)[:t]
+    want = [torch.zeros(nb, bs, hkv, d, dtype=torch.int8), torch.zeros(nb, bs, hkv, d, dtype=torch.int8),
+            torch.zeros(nb, bs, hkv), torch.zeros(nb, bs, hkv)]
+    got = [w.clone().to(DEV) for w in want]
+    oracle.store_kvcache_int8_oracle(k, v, *want, slots, bs)
+    store_kvcache_int8(k.to(DEV), v.to(DEV), *got, slots.to(DEV), bs)
+    for name, a, b in zip(["k codes", "v codes", "k scales", "v scales"], got, want):
+        a = a.cpu()
+        if a.dtype == torch.float32:
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32)), name
+        else:
+            assert torch.equal(a, b), f"{name}: {(a != b).sum().item()} codes differ"
+    # the case is what it claims: a good part of the quotients round differently under a reciprocal multiply
+    q = k / (k.abs().amax(-1, keepdim=True) / 127.0)
+    near = ((q - q.round()).abs() > 0.4999).float().mean().item()
+    assert near > 0.3, near
