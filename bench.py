@@ -26,8 +26,8 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # HBM bytes one decode_mfma_kernel launch moves on the default workload (seed 0, block_size 16), from the
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/bench_hbm_traffic_pmc.txt:
-# 2708782 KiB x 2.0 (copy-kernel calibration) fetched + 22855 KiB written.
-DECODE_TRAFFIC_BYTES_DEFAULT = int(2708782 * 2.0 * 1024 + 22855 * 1024)
+# 2708783 KiB x 2.0 (copy-kernel calibration) fetched + 22856 KiB written.
+DECODE_TRAFFIC_BYTES_DEFAULT = int(2708783 * 2.0 * 1024 + 22856 * 1024)
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,loads_probe,engine,engine16,engine64,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,prefill_long,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,loads_probe,engine,engine16,engine64,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -278,10 +278,11 @@ def bench_prefill_store(args, which, want_cpu=False):
         if want_cpu:
             out["prefill"]["cpu_baseline"] = cpu_prefill_baseline(q, k, v, cu, lengths, scale, hq, hkv, d, flops,
                                                                   flash_attention_prefill)
-    if "prefill" in which:
+    if "prefill_long" in which:
         # the same kernel away from config 2's short prompts: 4 prompts of 8192 tokens (the start and end of a
         # workgroup's life are a small share of its 128 key tiles)
         long_lengths = [8192] * 4
+        scale = 1.0 / math.sqrt(d)
         ql, kl, vl = (torch.randn(sum(long_lengths), h, d, generator=dg, device=dev).to(torch.bfloat16) for h in (hq, hkv, hkv))
         cul = torch.tensor([0] + long_lengths, dtype=torch.int32).cumsum(0).to(torch.int32).to(dev)
         _, event_ms_l = time_steps(lambda: flash_attention_prefill(ql, kl, vl, cul, scale, hq, hkv, d),
@@ -785,7 +786,7 @@ def main():
     if want("decode256") and args.block_size != 256:
         extra["decode_block256"], _ = bench_decode(args, 256, want_cpu=False)
     want_cpu = not args.no_cpu and want("cpu")
-    which = [n for n in ("prefill", "store") if want(n)]
+    which = [n for n in ("prefill", "prefill_long", "store") if want(n)]
     if which:
         extra.update(bench_prefill_store(args, which, want_cpu))
     if want("int8"):
