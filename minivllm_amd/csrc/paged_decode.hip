@@ -1407,6 +1407,71 @@ __global__ __launch_bounds__(256) void decode_reduce_kernel(const DecodeArgs a) 
   }
 }
 
+// The same merge for head dims 32, 64, 128 and 256: D / 4 lanes per head with 16-byte loads, and the partials of
+// eight partitions requested before the first is merged (the loop above waits for every partition in turn: a
+// sequence of config 3 has 4 to 16 of them, and the launch was 12 us of the 0.92 ms call).  Same arithmetic in
+// the same order, so the result is the same bit for bit.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void decode_reduce_vec_kernel(const DecodeArgs a) {
+  constexpr int kLanes = D / 4;                      // lanes per head
+  const int h = blockIdx.x * (256 / kLanes) + (int)threadIdx.x / kLanes;
+  const int li = (int)threadIdx.x % kLanes;
+  const int b = blockIdx.y;
+  if (h >= a.num_heads) return;
+  const int ctx = (int)load_ctx(a, b);
+  int np = (ctx + a.part_tokens - 1) / a.part_tokens;
+  if (np > a.num_parts) np = a.num_parts;
+  if (np <= 1) return;                               // written directly by the partition-0 workgroup
+  const int64_t slot0 = ((int64_t)b * a.num_parts) * a.num_heads + h;
+  const int64_t stride = a.num_heads;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  float mx = -INFINITY, lsum = 0.f;
+  for (int p0 = 0; p0 < np; p0 += 8) {
+    float2 ml[8];
+    float4 part[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int64_t s = slot0 + (int64_t)min(p0 + i, np - 1) * stride;     // past the last: the last again, unused
+      ml[i] = *reinterpret_cast<const float2*>(a.ws_ml + s * 2);
+      part[i] = *reinterpret_cast<const float4*>(a.ws_acc + s * D + 4 * li);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (p0 + i < np) {
+        const float mn = fmaxf(mx, ml[i].x);
+        const float keep = safe_exp2_diff(mx, mn);
+        const float wgt = safe_exp2_diff(ml[i].x, mn);
+        lsum = lsum * keep + ml[i].y * wgt;
+        acc[0] = acc[0] * keep + part[i].x * wgt;
+        acc[1] = acc[1] * keep + part[i].y * wgt;
+        acc[2] = acc[2] * keep + part[i].z * wgt;
+        acc[3] = acc[3] * keep + part[i].w * wgt;
+        mx = mn;
+      }
+    }
+  }
+  const float linv = lsum > 0.f ? 1.f / lsum : 0.f;
+  T o4[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) o4[r] = from_float<T>(acc[r] * linv);
+  T* out = reinterpret_cast<T*>(a.out) + ((int64_t)b * a.num_heads + h) * D + 4 * li;
+  if constexpr (sizeof(T) == 4) *reinterpret_cast<float4*>(out) = *reinterpret_cast<const float4*>(o4);
+  else *reinterpret_cast<uint2*>(out) = *reinterpret_cast<const uint2*>(o4);
+}
+
+template <typename T>
+static void launch_decode_reduce(const DecodeArgs& a, hipStream_t stream) {
+  const dim3 block(256);
+  const auto grid = [&](int lanes) { return dim3((unsigned)((a.num_heads + 256 / lanes - 1) / (256 / lanes)), (unsigned)a.batch); };
+  // the 16-byte loads and 8- or 16-byte stores need the output rows aligned (the workspace is checked to be)
+  const bool vec = (reinterpret_cast<uintptr_t>(a.out) & 15u) == 0;
+  if (vec && a.head_dim == 128) decode_reduce_vec_kernel<T, 128><<<grid(32), block, 0, stream>>>(a);
+  else if (vec && a.head_dim == 64) decode_reduce_vec_kernel<T, 64><<<grid(16), block, 0, stream>>>(a);
+  else if (vec && a.head_dim == 256) decode_reduce_vec_kernel<T, 256><<<grid(64), block, 0, stream>>>(a);
+  else if (vec && a.head_dim == 32) decode_reduce_vec_kernel<T, 32><<<grid(8), block, 0, stream>>>(a);
+  else decode_reduce_kernel<T><<<dim3((unsigned)((a.num_heads + 3) / 4), (unsigned)a.batch), block, 0, stream>>>(a);
+}
+
 // ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
@@ -1488,7 +1553,7 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
   int st = launch_status();
   if (st != 0) return st;
   if (a.num_parts > 1) {
-    decode_reduce_kernel<T><<<dim3((unsigned)((a.num_heads + 3) / 4), (unsigned)a.batch), dim3(256), 0, stream>>>(a);
+    launch_decode_reduce<T>(a, stream);
     st = launch_status();
   }
   return st;
