@@ -422,7 +422,7 @@ def bench_int8(args, want_cpu=True, want_probe=False):
         check.update({"gpu_vs_oracle_max_abs": worst, "oracle_sequences": 8})
     return {
         **check,
-        "roofline": roofline("hbm", nbytes / (event_ms * 1e-3) / 1e9, "decode_mfma_int8_kernel + decode_reduce_kernel"),
+        "roofline": roofline("hbm", nbytes / (event_ms * 1e-3) / 1e9, "decode_mfma_int8_kernel + decode_reduce_vec_kernel"),
         "store_roofline": roofline("hbm", store_bytes / (store_ms[0] * 1e-3) / 1e9, "store_int8_kernel"),
         "workload": "INT8 KV cache: decode B128 ctx~U[256,16384] Hq32 Hkv8 D128 block_size 16, bf16 q",
         "tokens": int(ctx.sum()), "algorithmic_bytes": nbytes, "ms_per_step": wall_ms,
@@ -838,7 +838,7 @@ def main():
             "traffic": DECODE_TRAFFIC_BYTES_DEFAULT if (args.seed == 0 and args.block_size == 16) else None,
             "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload summarised in "
                               "profiles/bench_hbm_traffic_pmc.txt (a counter run cannot time; not re-measured in this run)",
-            "kernel": "decode_mfma_kernel + decode_reduce_kernel (one decode call, HIP events on the launch stream)",
+            "kernel": "decode_mfma_kernel + decode_reduce_vec_kernel (one decode call, HIP events on the launch stream)",
         },
         "cpu_baseline": cpu,
         "extra": extra,
