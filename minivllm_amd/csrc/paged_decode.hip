@@ -1408,12 +1408,13 @@ __global__ __launch_bounds__(256) void decode_reduce_kernel(const DecodeArgs a) 
 }
 
 // The same merge for head dims 32, 64, 128 and 256: D / 4 lanes per head with 16-byte loads, and the partials of
-// eight partitions requested before the first is merged (the loop above waits for every partition in turn: a
-// sequence of config 3 has 4 to 16 of them, and the launch was 12 us of the 0.92 ms call).  Same arithmetic in
+// eight partitions requested before the first is merged (the loop above waits for every partition in turn; a
+// sequence of config 3 has up to 16 of them).  Same arithmetic in
 // the same order, so the result is the same bit for bit.
 template <typename T, int D>
 __global__ __launch_bounds__(256) void decode_reduce_vec_kernel(const DecodeArgs a) {
   constexpr int kLanes = D / 4;                      // lanes per head
+  constexpr int kBatch = 8;                          // partitions in flight (16: no faster, the short sequences' loads double)
   const int h = blockIdx.x * (256 / kLanes) + (int)threadIdx.x / kLanes;
   const int li = (int)threadIdx.x % kLanes;
   const int b = blockIdx.y;
@@ -1426,17 +1427,17 @@ __global__ __launch_bounds__(256) void decode_reduce_vec_kernel(const DecodeArgs
   const int64_t stride = a.num_heads;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   float mx = -INFINITY, lsum = 0.f;
-  for (int p0 = 0; p0 < np; p0 += 8) {
-    float2 ml[8];
-    float4 part[8];
+  for (int p0 = 0; p0 < np; p0 += kBatch) {
+    float2 ml[kBatch];
+    float4 part[kBatch];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kBatch; ++i) {
       const int64_t s = slot0 + (int64_t)min(p0 + i, np - 1) * stride;     // past the last: the last again, unused
       ml[i] = *reinterpret_cast<const float2*>(a.ws_ml + s * 2);
       part[i] = *reinterpret_cast<const float4*>(a.ws_acc + s * D + 4 * li);
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kBatch; ++i) {
       if (p0 + i < np) {
         const float mn = fmaxf(mx, ml[i].x);
         const float keep = safe_exp2_diff(mx, mn);
