@@ -26,8 +26,8 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # HBM bytes one decode_mfma_kernel launch moves on the default workload (seed 0, block_size 16), from the
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/bench_hbm_traffic_pmc.txt:
-# 2708783 KiB x 2.0 (copy-kernel calibration) fetched + 22856 KiB written.
-DECODE_TRAFFIC_BYTES_DEFAULT = int(2708783 * 2.0 * 1024 + 22856 * 1024)
+# 2708744 KiB x 2.0 (copy-kernel calibration) fetched + 22855 KiB written.
+DECODE_TRAFFIC_BYTES_DEFAULT = int(2708744 * 2.0 * 1024 + 22855 * 1024)
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
