@@ -193,7 +193,7 @@ __device__ __forceinline__ bool decode_item(const DecodeArgs& a, int& b, int& p,
 // ---------------------------------------------------------------------------
 // Fast path
 // ---------------------------------------------------------------------------
-// head dims of the 16-bit kernels: 32, 64, 128 (one set of up to sixteen 8-dim output columns) and 256 (two sets)
+// head dims of the 16-bit kernels: 32, 64, 96, 128 (one set of up to sixteen 8-dim output columns) and 256 (two sets)
 constexpr int dim_sets(int d) { return d > 128 ? d / 128 : 1; }
 template <typename T, int D = 128>
 struct KVTile {          // 16-bit elements: lane l holds 8 dims (16 B) of token l%16 per 32-dim step, and of its four V tokens
@@ -1487,9 +1487,9 @@ static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int ma
 
 // shapes the MFMA kernels are built for (pointer alignment is checked by the caller)
 static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool int8) {
-  // 16-bit caches: 32, 64, 128 or 256 dims per head; fp32 and INT8 caches: 64 or 128
+  // 16-bit caches: 32, 64, 96, 128 or 256 dims per head; fp32 and INT8 caches: 64 or 128
   const bool dim_ok = head_dim == 128 || head_dim == 64 ||
-                      (dtype != MVLLM_F32 && !int8 && (head_dim == 256 || head_dim == 32));
+                      (dtype != MVLLM_F32 && !int8 && (head_dim == 256 || head_dim == 96 || head_dim == 32));
   return (dtype != MVLLM_F32 || !int8) && dim_ok && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
          (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
 }
@@ -1531,8 +1531,9 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
     };
     if (a.head_dim == 128) go(std::integral_constant<int, 128>{});
     else if (a.head_dim == 64) go(std::integral_constant<int, 64>{});
-    if constexpr (IsSixteenBit<T>::value) {         // 16-bit caches also with 32 and 256 dims per head
+    if constexpr (IsSixteenBit<T>::value) {         // 16-bit caches also with 32, 96 and 256 dims per head
       if (a.head_dim == 256) go(std::integral_constant<int, 256>{});
+      else if (a.head_dim == 96) go(std::integral_constant<int, 96>{});
       else if (a.head_dim == 32) go(std::integral_constant<int, 32>{});
     }
   }
@@ -1632,7 +1633,7 @@ static void launch_rows16(const PrefillRowsArgs& a, dim3 grid, int tiles, hipStr
 }
 bool prefill_rows16_takes(int head_dim, int dtype, bool int8_cache) {
   if (head_dim == 64 || head_dim == 128) return true;
-  return (head_dim == 32 || head_dim == 256) && dtype != MVLLM_F32 && !int8_cache;
+  return (head_dim == 32 || head_dim == 96 || head_dim == 256) && dtype != MVLLM_F32 && !int8_cache;
 }
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream) {
   if (!prefill_rows16_takes(head_dim, dtype, a.k_scale != nullptr)) return MVLLM_ERR_UNSUPPORTED;
@@ -1652,6 +1653,7 @@ int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hip
     if (head_dim == 64) go(std::integral_constant<int, 64>{});
     else if (head_dim == 128) go(std::integral_constant<int, 128>{});
     else if (head_dim == 32) go(std::integral_constant<int, 32>{});
+    else if (head_dim == 96) go(std::integral_constant<int, 96>{});
     else go(std::integral_constant<int, 256>{});
   }
   return launch_status();

@@ -48,8 +48,9 @@ def test_prefill_vs_oracle(dtype, hq, hkv, d, lengths):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("hq,hkv,d,lengths", [(8, 2, 256, [70, 1, 33, 129]), (4, 4, 256, [200]), (8, 4, 32, [64, 17, 130])])
-def test_prefill_head_dim_256_and_32_on_the_16_row_tile_kernel(dtype, hq, hkv, d, lengths):
+@pytest.mark.parametrize("hq,hkv,d,lengths", [(8, 2, 256, [70, 1, 33, 129]), (4, 4, 256, [200]), (8, 4, 32, [64, 17, 130]),
+                                              (8, 2, 96, [70, 1, 33, 129]), (6, 6, 96, [200])])
+def test_prefill_head_dim_256_96_and_32_on_the_16_row_tile_kernel(dtype, hq, hkv, d, lengths):
     from minivllm_amd.layers.attention import prefill_plan
     assert prefill_plan(hq, hkv, d, 0, dtype) == 1
     case = make_varlen_case(55, lengths, hq, hkv, d, dtype=dtype)
