@@ -98,7 +98,7 @@ size_t mvllm_paged_decode_workspace_bytes(int batch, int num_heads, int head_dim
  *   *waves_per_head   1: a workgroup holds up to 4 kv heads, one wave each, and every wave walks its partition;
  *                     >1: small-batch form, a workgroup is that many waves on one kv head that share the
  *                     partition's 16-token tiles and merge in LDS; 0: the generic kernel (head_dim other than
- *                     128 or 64 (bf16 / fp16 caches: also 32, 96 and 256), block_size % 16 != 0, more than 16 query
+ *                     128 or 64 (bf16 / fp16 caches: also 32, 80, 96, 112 and 256), block_size % 16 != 0, more than 16 query
  *                     heads per kv head, or fp32 queries over an INT8 cache)
  * Returns MVLLM_OK or MVLLM_ERR_BAD_SHAPE / MVLLM_ERR_BAD_DTYPE.
  */
@@ -179,7 +179,7 @@ int mvllm_prefill_varlen(void* out, const void* q, const void* k, const void* v,
  * Which kernel a prefill of these static sizes runs on (no counterpart in the reference, whose Triton kernels take any
  * power-of-two head_dim from a tile-size table, attention.py:249-257).  block_size 0 = the packed entry point,
  * > 0 = the paged ones.  *kernel: 2 the LDS-tiled MFMA kernel (bf16 / fp16, head_dim 128 or 64, also over an INT8
- * cache), 1 the 16-row tile MFMA kernel (fp32 with head_dim 128 or 64, bf16 / fp16 with 32, 96 or 256), 0 the generic kernel (any
+ * cache), 1 the 16-row tile MFMA kernel (fp32 with head_dim 128 or 64, bf16 / fp16 with 32, 80, 96, 112 or 256), 0 the generic kernel (any
  * head_dim <= 512; one key per step, a correctness path two orders of magnitude slower), -1 unsupported.
  * Pointers are assumed 16-byte aligned (unaligned ones take the generic kernel).  Pure host arithmetic.
  */

@@ -206,7 +206,7 @@ struct PrefillRowsArgs {
   const float* v_scale;
 };
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream);
-// shapes that kernel is built for: fp32 and INT8 caches with 64 or 128 dims per head, 16-bit also with 32, 96 and 256
+// shapes that kernel is built for: fp32 and INT8 caches with 64 or 128 dims per head, 16-bit also with 32, 80, 96, 112 and 256
 bool prefill_rows16_takes(int head_dim, int dtype, bool int8_cache);
 
 }  // namespace mvllm

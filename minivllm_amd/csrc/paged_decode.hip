@@ -218,9 +218,14 @@ struct TileIO {
   static constexpr int kVLane = 8;     // dims per column (lane%16) of the second product
   static constexpr int kSets = dim_sets(D);
   static __device__ __forceinline__ bool owns(int col) { return D >= 128 || col < D / 8; }
-  static __device__ __forceinline__ void load_k(KVTile<T, D>& t, const T* kp) {
+  static constexpr int kSteps = (D + 31) / 32;   // 32-dim steps of the first product; the last one may be partial
+  // cls = lane / 16: the lane's 8 dims inside a step.  Head dims that are not a multiple of 32 (80, 112): the classes
+  // of the last step that lie past the row's end load nothing (the next head's values are not this head's zeros).
+  static __device__ __forceinline__ bool has_dims(int j, int cls) { return D % 32 == 0 || 32 * j + 8 * cls < D; }
+  static __device__ __forceinline__ void load_k(KVTile<T, D>& t, const T* kp, int cls) {
 #pragma unroll
-    for (int j = 0; j < D / 32; ++j) t.k[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
+    for (int j = 0; j < kSteps; ++j)
+      t.k[j] = has_dims(j, cls) ? *reinterpret_cast<const uint4*>(kp + 32 * j) : make_uint4(0u, 0u, 0u, 0u);
   }
   template <bool STREAM>
   static __device__ __forceinline__ void load_v(KVTile<T, D>& t, int i, const T* vp, bool own) {
@@ -231,7 +236,7 @@ struct TileIO {
   }
   static __device__ __forceinline__ void zero(KVTile<T, D>& t) {
 #pragma unroll
-    for (int j = 0; j < D / 32; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
+    for (int j = 0; j < kSteps; ++j) t.k[j] = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
     for (int i = 0; i < 4 * kSets; ++i) t.v[i] = make_uint4(0u, 0u, 0u, 0u);
   }
@@ -241,7 +246,7 @@ struct TileIO<float, D> {
   static constexpr int kKLane = 4;
   static constexpr int kVLane = 4;
   static __device__ __forceinline__ bool owns(int) { return true; }     // 16 columns x 4 dims per 64-dim step
-  static __device__ __forceinline__ void load_k(KVTile<float, D>& t, const float* kp) {
+  static __device__ __forceinline__ void load_k(KVTile<float, D>& t, const float* kp, int /*cls*/) {
 #pragma unroll
     for (int j = 0; j < D / 16; ++j) t.k[j] = *reinterpret_cast<const float4*>(kp + 16 * j);
   }
@@ -334,7 +339,7 @@ template <typename T, int D>
 struct DecodeHead {
   using Elem = T;
   static constexpr int kDim = D;
-  static constexpr int kSteps = D / 32;     // 32-dim steps of the first product
+  static constexpr int kSteps = (D + 31) / 32;   // 32-dim steps of the first product; the last one may be partial
   static constexpr int kSets = dim_sets(D); // sets of sixteen 8-dim output columns (2 for head_dim 256)
   static constexpr int kCols = D >= 128 ? 16 : D / 8;   // lanes (l%16) that own 8 dims of the output per set
   static constexpr int kAcc = 8 * kSets;
@@ -348,8 +353,8 @@ struct DecodeHead {
     const T* src = row_ptr + (lane >> 4) * 8;
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
-      const uint4 x = *reinterpret_cast<const uint4*>(src + 32 * j);
-      qf[j] = live ? x : make_uint4(0u, 0u, 0u, 0u);
+      const bool has = live && TileIO<T, D>::has_dims(j, lane >> 4);
+      qf[j] = has ? *reinterpret_cast<const uint4*>(src + 32 * j) : make_uint4(0u, 0u, 0u, 0u);
     }
     m = -INFINITY;
     l = 0.f;
@@ -737,7 +742,7 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
       // K is read in the MFMA operand layout, 64 bytes of a row per instruction, so the second half of each
       // 128-byte line has to survive in cache until the next instruction: ordinary loads (the hint costs 7 %
       // there).
-      IO::load_k(t, kp);
+      IO::load_k(t, kp, lane >> 4);
 #pragma unroll
       for (int i = 0; i < 4; ++i) IO::template load_v<true>(t, i, vp + (int64_t)i * row, IO::owns(col));
     } else {
@@ -875,7 +880,7 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
         IO::zero(t);
       }
     } else if (mapped) {
-      IO::load_k(t, kc + k_tok * row);
+      IO::load_k(t, kc + k_tok * row, lane >> 4);
 #pragma unroll
       for (int i = 0; i < 4; ++i) IO::template load_v<false>(t, i, vc + v_tok[i] * row, IO::owns(col));
     } else {
@@ -1487,9 +1492,9 @@ static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int ma
 
 // shapes the MFMA kernels are built for (pointer alignment is checked by the caller)
 static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool int8) {
-  // 16-bit caches: 32, 64, 96, 128 or 256 dims per head; fp32 and INT8 caches: 64 or 128
+  // 16-bit caches: 32, 64, 80, 96, 112, 128 or 256 dims per head; fp32 and INT8 caches: 64 or 128
   const bool dim_ok = head_dim == 128 || head_dim == 64 ||
-                      (dtype != MVLLM_F32 && !int8 && (head_dim == 256 || head_dim == 96 || head_dim == 32));
+                      (dtype != MVLLM_F32 && !int8 && (head_dim == 256 || head_dim == 112 || head_dim == 96 || head_dim == 80 || head_dim == 32));
   return (dtype != MVLLM_F32 || !int8) && dim_ok && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
          (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
 }
@@ -1534,6 +1539,8 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
     if constexpr (IsSixteenBit<T>::value) {         // 16-bit caches also with 32, 96 and 256 dims per head
       if (a.head_dim == 256) go(std::integral_constant<int, 256>{});
       else if (a.head_dim == 96) go(std::integral_constant<int, 96>{});
+      else if (a.head_dim == 80) go(std::integral_constant<int, 80>{});
+      else if (a.head_dim == 112) go(std::integral_constant<int, 112>{});
       else if (a.head_dim == 32) go(std::integral_constant<int, 32>{});
     }
   }
@@ -1633,7 +1640,7 @@ static void launch_rows16(const PrefillRowsArgs& a, dim3 grid, int tiles, hipStr
 }
 bool prefill_rows16_takes(int head_dim, int dtype, bool int8_cache) {
   if (head_dim == 64 || head_dim == 128) return true;
-  return (head_dim == 32 || head_dim == 96 || head_dim == 256) && dtype != MVLLM_F32 && !int8_cache;
+  return (head_dim == 32 || head_dim == 80 || head_dim == 96 || head_dim == 112 || head_dim == 256) && dtype != MVLLM_F32 && !int8_cache;
 }
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream) {
   if (!prefill_rows16_takes(head_dim, dtype, a.k_scale != nullptr)) return MVLLM_ERR_UNSUPPORTED;
@@ -1654,6 +1661,8 @@ int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hip
     else if (head_dim == 128) go(std::integral_constant<int, 128>{});
     else if (head_dim == 32) go(std::integral_constant<int, 32>{});
     else if (head_dim == 96) go(std::integral_constant<int, 96>{});
+    else if (head_dim == 80) go(std::integral_constant<int, 80>{});
+    else if (head_dim == 112) go(std::integral_constant<int, 112>{});
     else go(std::integral_constant<int, 256>{});
   }
   return launch_status();

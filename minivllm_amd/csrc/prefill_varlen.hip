@@ -925,7 +925,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   const bool aligned = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out);
   const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, 0, dtype, false, false) : 0;
   const bool mfma_ok = kind == 2;
-  // fp32, and 16-bit head dims 32, 96 and 256: 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
+  // fp32, and 16-bit head dims 32, 80, 96, 112 and 256: 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
   if (kind == 1) {
     PrefillRowsArgs r;
     r.out = out; r.q = q; r.k = k; r.v = v; r.cu_seqlens = cu_seqlens; r.total_tokens = total_tokens;

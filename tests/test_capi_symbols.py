@@ -75,7 +75,8 @@ def test_decode_plan_is_host_arithmetic():
     assert paged_decode_plan(64, 16, 16, 64, 256, 16, int8_cache=True)[2] == 1      # 1024 (sequence, head) pairs: first form
     assert paged_decode_plan(64, 16, 16, 96, 256, 16, int8_cache=True)[2] == 0
     assert paged_decode_plan(64, 16, 16, 96, 256, 16)[2] == 4                 # 16-bit caches: also 96 dims (three 32-dim steps)
-    assert paged_decode_plan(64, 16, 16, 80, 256, 16)[2] == 0                 # other head dims
+    assert paged_decode_plan(64, 16, 16, 80, 256, 16)[2] == 4 and paged_decode_plan(64, 16, 16, 112, 256, 16)[2] == 4   # ... and a partial last step
+    assert paged_decode_plan(64, 16, 16, 72, 256, 16)[2] == 0                 # other head dims
     assert paged_decode_plan(64, 16, 8, 256, 256, 16)[2] == 4                 # 16-bit caches: also 256 and 32 dims
     assert paged_decode_plan(64, 16, 8, 32, 256, 16)[2] == 4
     assert paged_decode_plan(64, 16, 8, 256, 256, 16, int8_cache=True)[2] == 0
@@ -103,7 +104,8 @@ def test_prefill_plan_is_host_arithmetic():
     assert prefill_plan(32, 8, 128, dtype=torch.float32) == 1 and prefill_plan(16, 8, 64, 16, torch.float32) == 1
     assert prefill_plan(8, 8, 256) == 1 and prefill_plan(8, 8, 32, block_size=32) == 1      # bf16 / fp16 only
     assert prefill_plan(8, 8, 256, dtype=torch.float32) == 0
-    assert prefill_plan(6, 2, 80) == 0 and prefill_plan(6, 2, 96) == 1 and prefill_plan(6, 2, 96, dtype=torch.float32) == 0
+    assert prefill_plan(6, 2, 80) == 1 and prefill_plan(6, 2, 96) == 1 and prefill_plan(6, 2, 96, dtype=torch.float32) == 0
+    assert prefill_plan(6, 2, 72) == 0
     assert prefill_plan(32, 8, 128, 16, int8_cache=True) == 2
     assert prefill_plan(32, 8, 96, 16, int8_cache=True) == -1 and prefill_plan(32, 8, 128, 16, torch.float32, True) == -1
     assert prefill_plan(8, 8, 1024) == -1
@@ -116,9 +118,9 @@ def test_generic_kernel_warning_is_raised_once_per_shape():
     attention._shapes_seen.clear()
     with warnings.catch_warnings(record=True) as seen:
         warnings.simplefilter("always")
-        attention._warn_if_generic("decode", 16, 16, 80, 16, torch.bfloat16, False)
-        attention._warn_if_generic("decode", 16, 16, 80, 16, torch.bfloat16, False)      # same shape: silent
-        attention._warn_if_generic("prefill", 6, 2, 80, 0, torch.bfloat16, False)
+        attention._warn_if_generic("decode", 16, 16, 72, 16, torch.bfloat16, False)
+        attention._warn_if_generic("decode", 16, 16, 72, 16, torch.bfloat16, False)      # same shape: silent
+        attention._warn_if_generic("prefill", 6, 2, 72, 0, torch.bfloat16, False)
         attention._warn_if_generic("decode", 32, 8, 128, 16, torch.bfloat16, False)      # MFMA kernel: silent
         attention._warn_if_generic("prefill", 32, 8, 128, 0, torch.bfloat16, False)
     assert len(seen) == 2 and all("generic kernel" in str(w.message) for w in seen)

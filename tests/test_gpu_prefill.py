@@ -30,7 +30,8 @@ def _oracle32(q, k, v, cu, scale, hq, hkv, d):
     (16, 8, 128, [96, 33, 32, 128]),
     (8, 8, 128, [200]),
     (16, 16, 64, [60, 60]),             # the reference demo's head_dim
-    (6, 2, 80, [17, 5]),
+    (6, 2, 80, [17, 5]),                # 16-bit: the 16-row tile kernel with a partial last step; fp32: generic
+    (6, 2, 72, [17, 5]),                # a head_dim no matrix-unit kernel takes
     (6, 2, 128, [300, 17, 64]),         # three query heads per kv head: one head per workgroup
     (10, 2, 128, [33, 129]),            # five
 ])
@@ -49,7 +50,8 @@ def test_prefill_vs_oracle(dtype, hq, hkv, d, lengths):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("hq,hkv,d,lengths", [(8, 2, 256, [70, 1, 33, 129]), (4, 4, 256, [200]), (8, 4, 32, [64, 17, 130]),
-                                              (8, 2, 96, [70, 1, 33, 129]), (6, 6, 96, [200])])
+                                              (8, 2, 96, [70, 1, 33, 129]), (6, 6, 96, [200]), (8, 2, 80, [70, 1, 33, 129]),
+                                              (6, 3, 112, [200, 17])])
 def test_prefill_head_dim_256_96_and_32_on_the_16_row_tile_kernel(dtype, hq, hkv, d, lengths):
     from minivllm_amd.layers.attention import prefill_plan
     assert prefill_plan(hq, hkv, d, 0, dtype) == 1
