@@ -105,9 +105,13 @@ class Scheduler:
             if index == seq.num_tokens - 1:
                 seq.last_token = token_id
             if not seq.ignore_eos and token_id == self.eos and not seq.is_finished:
+                if seq.status == SequenceStatus.WAITING:
+                    # preempted by the scheduling of the step launched in the meantime: its blocks are back already
+                    self.waiting.remove(seq)
+                else:
+                    self.block_manager.deallocate(seq)
+                    self.running.remove(seq)
                 seq.status = SequenceStatus.FINISHED
-                self.block_manager.deallocate(seq)
-                self.running.remove(seq)
                 ended.append(seq)
         self.block_manager.hash_deferred_blocks()
         return ended

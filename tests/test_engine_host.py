@@ -360,7 +360,7 @@ def test_run_ahead_equals_waiting_engine_on_random_schedules():
     sequence as the one that waits, reports every sequence once, and returns every block."""
     from hypothesis import given, settings, strategies as st
 
-    @settings(max_examples=120, deadline=None)
+    @settings(max_examples=300, deadline=None, derandomize=True)
     @given(st.data())
     def check(data):
         n = data.draw(st.integers(1, 7))
@@ -396,3 +396,28 @@ def test_run_ahead_equals_waiting_engine_on_random_schedules():
                 assert 7 not in toks[:-1]
 
     check()
+
+
+def test_eos_of_a_sequence_preempted_while_its_id_was_on_the_way():
+    """A sequence whose step was launched, that is then preempted by the scheduling of the next step (the pool is
+    full) and whose id turns out to be its EOS: the commit ends it from the waiting queue, its blocks having been
+    returned by the preemption.  (Found by the random-schedule property above: three one-token prompts, blocks of
+    two tokens, a pool of six.)"""
+    cfg = dict(max_num_sequences=3, max_num_batched_tokens=64, max_cached_blocks=6, block_size=2, eos=7,
+               max_position=64)
+    prompts = [[1], [101], [201]]
+    sp = SamplingParams(temperature=0.6, max_tokens=5, ignore_eos=False)
+    outs = []
+    for ahead in (True, False):
+        eng = LLMEngine(dict(cfg, async_decode=ahead), model_runner=FakeFunctionRunner(7, {2: 4}))
+        for p in prompts:
+            eng.add_prompt(p, sp)
+        reported = []
+        for _ in range(200):
+            if eng.scheduler.is_finished() and eng.pending is None:
+                break
+            finished, _, _ = eng.step()
+            reported += finished
+        assert len(reported) == 3 and len(eng.scheduler.block_manager.free_block_ids) == 6
+        outs.append([toks for _, toks in sorted(reported)])
+    assert outs[0] == outs[1]
