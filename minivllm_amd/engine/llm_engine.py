@@ -61,12 +61,21 @@ class LLMEngine:
                 and runner.can_launch_decode(seqs)):
             if not runner.continues_last_decode(seqs):
                 finished += self.flush()               # the buffers are refilled from the last tokens
+                # an id that just arrived may have been a scheduled sequence's EOS: it has ended and given its
+                # blocks (the one this step's scheduling appended included) back
+                seqs = [seq for seq in seqs if not seq.is_finished]
+                if not seqs:
+                    return finished, 0, False
             handle = runner.launch_decode(seqs)
             finished += self.flush()                   # the step before this one, while the GPU runs this one
             slots, done = self.scheduler.postprocess_provisional(seqs)
             self.pending = (handle, slots, done)
             return finished, sum(slot is not None for slot in slots), False
         finished += self.flush()
+        if not is_prefill:                             # as above: a scheduled sequence may just have ended
+            seqs = [seq for seq in seqs if not seq.is_finished]
+            if not seqs:
+                return finished, 0, False
         token_ids = runner.run(seqs, is_prefill)
         self.scheduler.postprocess(seqs, token_ids)
         finished += [(seq.seq_id, seq.completion_token_ids) for seq in seqs if seq.is_finished]

@@ -243,6 +243,8 @@ class FakeAsyncRunner(FakeRunner):
             all(len(s) == n + 1 for s, n in zip(seqs, self.last[1]))
 
     def launch_decode(self, seqs):
+        assert not any(s.is_finished for s in seqs), "a finished sequence has no blocks to build metadata from"
+        assert all(len(s.block_table) == s.num_blocks for s in seqs), "every token of the step needs a cache slot"
         if not self.continues_last_decode(seqs):
             assert all(t >= 0 for s in seqs for t in s.token_ids), "a refill needs real last tokens"
         self.log.append("launch")
@@ -252,6 +254,7 @@ class FakeAsyncRunner(FakeRunner):
 
     def run(self, seqs, is_prefill):
         assert all(t >= 0 for s in seqs for t in s.token_ids), "a synchronous step needs real token ids"
+        assert not any(s.is_finished for s in seqs) and all(len(s.block_table) == s.num_blocks for s in seqs)
         self.last = None
         self.log.append("run")
         return super().run(seqs, is_prefill)
@@ -300,6 +303,8 @@ class FakeFunctionRunner(FakeAsyncRunner):
         return out
 
     def launch_decode(self, seqs):
+        assert not any(s.is_finished for s in seqs), "a finished sequence has no blocks to build metadata from"
+        assert all(len(s.block_table) == s.num_blocks for s in seqs), "every token of the step needs a cache slot"
         if not self.continues_last_decode(seqs):
             assert all(t >= 0 for s in seqs for t in s.token_ids), "a refill needs real last tokens"
         self.log.append("launch")
@@ -309,6 +314,7 @@ class FakeFunctionRunner(FakeAsyncRunner):
 
     def run(self, seqs, is_prefill):
         assert all(t >= 0 for s in seqs for t in s.token_ids), "a synchronous step needs real token ids"
+        assert not any(s.is_finished for s in seqs) and all(len(s.block_table) == s.num_blocks for s in seqs)
         self.last = None
         self.log.append("run")
         self.calls.append((is_prefill, [s.seq_id for s in seqs], [len(s) for s in seqs]))
