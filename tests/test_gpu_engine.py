@@ -274,3 +274,32 @@ def test_steps_run_ahead_for_sequences_that_stop_at_eos():
         assert sum(len(t) < 48 for t in out) >= 2
     first_eos = min(len(t) for t in outs[False][:4])            # the first batch runs in step until its first EOS
     assert all(a[:first_eos] == b[:first_eos] for a, b in zip(outs[True][:4], outs[False][:4]))
+
+
+def test_two_sequences_reach_eos_in_consecutive_steps_while_running_ahead():
+    """Sequence A's EOS arrives one step late and changes the batch; the flush that precedes the changed batch's
+    launch then delivers sequence B's EOS, of the step after, while B is already scheduled for that launch: B is
+    dropped from it (its blocks are back in the pool), and both end exactly at their EOS.  The EOS id is picked from a
+    run that ignores EOS (a vocabulary of 64 makes such a pair certain), so until A ends the runs are identical."""
+    cfg = dict(SMALL, vocab_size=64, enforce_eager=False, max_num_sequences=4, max_cached_blocks=96,
+               max_model_length=160)
+    found = None
+    for seed in range(62, 70):
+        prompts = _prompts(4, 3, 20, seed=seed, vocab=64)
+        free = LLMEngine(cfg).generate(prompts, SamplingParams(temperature=0.9, max_tokens=40, ignore_eos=True))["token_ids"]
+        first = lambda toks, e: toks.index(e) if e in toks else 10 ** 6
+        for e in range(64):
+            at = sorted((first(toks, e), k) for k, toks in enumerate(free))
+            (s, a), (s2, b) = at[0], at[1]
+            if 2 <= s and s2 == s + 1 and at[2][0] > s + 3:
+                found = (prompts, free, e, a, b, s)
+                break
+        if found:
+            break
+    assert found, "no id that two sequences emit for the first time in consecutive steps"
+    prompts, free, eos, a, b, s = found
+    eng = LLMEngine(dict(cfg, eos=eos, async_decode=True))
+    out = eng.generate(prompts, SamplingParams(temperature=0.9, max_tokens=40, ignore_eos=False))["token_ids"]
+    assert out[a] == free[a][:s + 1] and out[b] == free[b][:s + 2]
+    assert all(t[-1] == eos or len(t) == 40 for t in out) and all(eos not in t[:-1] for t in out)
+    assert len(eng.scheduler.block_manager.free_block_ids) == cfg["max_cached_blocks"] and eng.pending is None
