@@ -360,17 +360,27 @@ def test_sequences_that_stop_at_eos_also_run_ahead_and_end_one_commit_late():
     assert sum(1 for a, b in zip(log, log[1:]) if a == "launch" and b == "wait") >= 4  # steps did run ahead
 
 
-def test_run_ahead_equals_waiting_engine_on_random_schedules():
-    """Property: for random prompts, EOS positions, token limits, batch limits and block sizes (preemption when the
-    pool is small included) the engine that launches decode steps ahead of their ids returns the same tokens per
-    sequence as the one that waits, reports every sequence once, and returns every block."""
+@pytest.mark.parametrize("shared_prefixes", [False, True])
+def test_run_ahead_equals_waiting_engine_on_random_schedules(shared_prefixes):
+    """Property: for random prompts (distinct, or cut from one stem so that prefix blocks are shared), EOS positions,
+    token limits, batch limits and block sizes (preemption when the pool is small included) the engine that launches
+    decode steps ahead of their ids returns the same tokens per sequence as the one that waits, reports every sequence
+    once, and leaves the block manager empty: every block free, no reference, no hash waiting for an id."""
     from hypothesis import given, settings, strategies as st
 
     @settings(max_examples=300, deadline=None, derandomize=True)
     @given(st.data())
     def check(data):
         n = data.draw(st.integers(1, 7))
-        prompts = [list(range(100 * i + 1, 100 * i + 1 + data.draw(st.integers(1, 14)))) for i in range(n)]
+        if shared_prefixes:
+            stem = [data.draw(st.integers(1, 3)) for _ in range(20)]
+            prompts = []
+            for _ in range(n):
+                keep = data.draw(st.integers(0, 16))
+                tail = [50 + data.draw(st.integers(0, 2)) for _ in range(data.draw(st.integers(0 if keep else 1, 6)))]
+                prompts.append(stem[:keep] + tail)
+        else:
+            prompts = [list(range(100 * i + 1, 100 * i + 1 + data.draw(st.integers(1, 14)))) for i in range(n)]
         max_tokens = data.draw(st.integers(1, 12))
         block_size = data.draw(st.sampled_from([2, 4, 8]))
         longest = max(map(len, prompts)) + max_tokens
@@ -391,9 +401,12 @@ def test_run_ahead_equals_waiting_engine_on_random_schedules():
                 finished, _, _ = eng.step()
                 reported += finished
                 steps += 1
-                assert steps < 2000
+                assert steps < 3000
+            bm = eng.scheduler.block_manager
             assert len(reported) == n and len({sid for sid, _ in reported}) == n
-            assert len(eng.scheduler.block_manager.free_block_ids) == blocks and eng.pending is None
+            assert len(bm.free_block_ids) == blocks and not bm.used_block_ids and eng.pending is None
+            assert all(b.ref_count == 0 for b in bm.blocks) and not bm.deferred
+            assert all(t >= 0 for b in bm.blocks if b.hash != -1 for t in b.token_ids)    # no hash over a placeholder
             outs.append([toks for _, toks in sorted(reported)])
         assert outs[0] == outs[1]
         for toks in outs[0]:
