@@ -53,6 +53,10 @@ class BlockManager:
     def _allocate_block(self, block_id: int) -> Block:
         block = self.blocks[block_id]
         assert block.ref_count == 0, "Block is already allocated"
+        # the block is about to hold something else: its old hash must not lead here any more (a later prompt whose
+        # block has the same tokens behind ANOTHER prefix would pass the token comparison and share the wrong K/V)
+        if block.hash != -1 and self.hash_to_block_id.get(block.hash) == block_id:
+            del self.hash_to_block_id[block.hash]
         block.reset()
         self.free_block_ids.remove(block_id)
         self.used_block_ids.add(block_id)
@@ -75,7 +79,7 @@ class BlockManager:
             token_ids = seq.block(i)
             h = self.compute_hash(token_ids, h) if len(token_ids) == self.block_size else -1
             block_id = self.hash_to_block_id.get(h, -1)
-            if block_id == -1 or self.blocks[block_id].token_ids != token_ids:
+            if block_id == -1 or self.blocks[block_id].hash != h or self.blocks[block_id].token_ids != token_ids:
                 cache_miss = True        # a prefix is only reusable up to the first miss
             if cache_miss:
                 block = self._allocate_block(self.free_block_ids[0])

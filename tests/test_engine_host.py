@@ -440,3 +440,88 @@ def test_eos_of_a_sequence_preempted_while_its_id_was_on_the_way():
         assert len(reported) == 3 and len(eng.scheduler.block_manager.free_block_ids) == 6
         outs.append([toks for _, toks in sorted(reported)])
     assert outs[0] == outs[1]
+
+
+def test_a_reused_block_is_not_shared_through_its_old_hash():
+    """A freed block keeps its hash so that a later prompt can share it.  Once the block is taken for something else,
+    that hash must stop leading to it: here block 2 first ends the prefix [2, 1, 1], is freed, then holds the third
+    token of [3, 1, 1], the same token 1, and a new [2, 1, 1] must not share it (its K/V were computed behind another
+    prefix; the reference's check compares the block's own tokens only, block_manager.py:72-86).  Found by the random
+    operation sequences below."""
+    bm = BlockManager(7, 1)
+    a = Sequence([2, 1, 1], SamplingParams(), 1)
+    bm.allocate(a)
+    first = list(a.block_table)
+    bm.deallocate(a)
+    b, c = Sequence([3], SamplingParams(), 1), Sequence([1, 1], SamplingParams(), 1)
+    bm.allocate(b)
+    bm.allocate(c)
+    for _ in range(2):
+        b.append_token(1)
+        bm.append(b)
+    assert b.block_table[2] == first[2]                      # the old third block of [2, 1, 1] now belongs to [3, 1, 1]
+    bm.deallocate(c)
+    d = Sequence([2, 1, 1], SamplingParams(), 1)
+    bm.allocate(d)
+    assert d.block_table[:2] == first[:2] and d.num_cached_tokens == 2      # the first two blocks are still shareable
+    assert d.block_table[2] != b.block_table[2] and len(set(d.block_table)) == 3
+
+
+def test_block_manager_invariants_under_random_operations():
+    """Random allocate / append / free sequences over prompts cut from one stem (so that prefixes are shared and freed
+    blocks are found again): reference counts equal the number of tables a block is in, free and used blocks partition
+    the pool, no table holds a block twice, cached prefixes hold the sequence's own tokens, and two sequences share a
+    block only behind equal prefixes."""
+    from hypothesis import given, settings, strategies as st
+
+    def invariants(bm, live, bs):
+        counts = {}
+        for s in live:
+            assert len(s.block_table) == s.num_blocks and len(set(s.block_table)) == len(s.block_table)
+            for b in s.block_table:
+                counts[b] = counts.get(b, 0) + 1
+            assert s.num_cached_tokens % bs == 0 and 0 <= s.num_cached_tokens <= max(len(s) - 1, 0)
+            for i in range(s.num_cached_tokens // bs):
+                assert bm.blocks[s.block_table[i]].token_ids == s.block(i)
+        assert all(b.ref_count == counts.get(b.block_id, 0) for b in bm.blocks)
+        assert set(bm.free_block_ids).isdisjoint(bm.used_block_ids) and bm.used_block_ids == set(counts)
+        assert len(bm.free_block_ids) + len(bm.used_block_ids) == len(bm.blocks)
+        for a in live:
+            for c in live:
+                for i, (x, y) in enumerate(zip(a.block_table, c.block_table)):
+                    assert x != y or a.token_ids[:(i + 1) * bs] == c.token_ids[:(i + 1) * bs]
+
+    @settings(max_examples=400, deadline=None, derandomize=True)
+    @given(st.data())
+    def check(data):
+        bs = data.draw(st.sampled_from([1, 2, 4]))
+        nblocks = data.draw(st.integers(4, 24))
+        bm = BlockManager(nblocks, bs)
+        stem = [data.draw(st.integers(1, 2)) for _ in range(16)]
+        live = []
+        for _ in range(data.draw(st.integers(1, 40))):
+            op = data.draw(st.sampled_from(["alloc", "alloc", "append", "append", "append", "free"]))
+            if op == "alloc":
+                keep = data.draw(st.integers(0, 12))
+                tail = [data.draw(st.integers(1, 3)) for _ in range(data.draw(st.integers(0 if keep else 1, 5)))]
+                s = Sequence(stem[:keep] + tail, SamplingParams(), bs)
+                if bm.can_allocate(s):
+                    bm.allocate(s)
+                    live.append(s)
+            elif op == "append" and live:
+                s = live[data.draw(st.integers(0, len(live) - 1))]
+                if len(bm.free_block_ids) >= 1:                 # the token may open a block
+                    s.append_token(data.draw(st.sampled_from([1, 2, 3, -1])))      # -1: an id still on its way
+                    bm.append(s)
+                    if s.token_ids[-1] < 0:
+                        s.token_ids[-1] = s.last_token = data.draw(st.integers(1, 3))
+                        bm.hash_deferred_blocks()
+            elif op == "free" and live:
+                bm.deallocate(live.pop(data.draw(st.integers(0, len(live) - 1))))
+            invariants(bm, live, bs)
+        for s in live:
+            bm.deallocate(s)
+        invariants(bm, [], bs)
+        assert len(bm.free_block_ids) == nblocks
+
+    check()
