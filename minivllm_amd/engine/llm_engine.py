@@ -31,13 +31,23 @@ class LLMEngine:
     def add_prompt(self, prompt_token_ids: list[int], sampling_params: SamplingParams) -> None:
         """Queue a prompt.  A request that could outgrow ``max_model_length`` / ``max_position`` is refused here:
         the reference's demo exceeds its own limit silently (main.py:35,38,49) and would index the rotary table
-        out of range (rotary_embedding.py:78)."""
+        out of range (rotary_embedding.py:78).  So is one that no step's token budget or the block pool can hold."""
         if not prompt_token_ids:
             raise ValueError("empty prompt")
         longest = len(prompt_token_ids) + sampling_params.max_tokens
         if longest > self.max_model_length:
             raise ValueError(f"prompt of {len(prompt_token_ids)} tokens + max_tokens {sampling_params.max_tokens} "
                              f"exceeds max_model_length / max_position {self.max_model_length}")
+        # what the scheduler could never place would wait for ever (the reference's generate loop spins on it,
+        # llm_engine.py:62-75): a sequence is re-admitted as a whole after a preemption, so its full length must fit
+        # the token budget of a step, and its blocks the pool
+        slots = longest - 1                                     # the last sampled token is never fed back
+        if slots > self.scheduler.max_num_batched_tokens:
+            raise ValueError(f"prompt + max_tokens - 1 = {slots} tokens exceed max_num_batched_tokens "
+                             f"{self.scheduler.max_num_batched_tokens}")
+        pool = len(self.scheduler.block_manager.blocks)
+        if -(-slots // self.block_size) > pool:
+            raise ValueError(f"{slots} tokens need {-(-slots // self.block_size)} blocks of {self.block_size}, the pool has {pool}")
         self.scheduler.add_sequence(Sequence(prompt_token_ids, sampling_params, self.block_size))
 
     def step(self):

@@ -525,3 +525,18 @@ def test_block_manager_invariants_under_random_operations():
         assert len(bm.free_block_ids) == nblocks
 
     check()
+
+
+def test_requests_the_scheduler_could_never_place_are_refused():
+    """A prompt that no step's token budget can take, or whose tokens need more blocks than the pool has, would wait for
+    ever (also after a preemption, when it is prefilled again at its full length): ``add_prompt`` raises instead."""
+    cfg = dict(max_num_sequences=2, max_num_batched_tokens=16, max_cached_blocks=3, block_size=4, eos=-1, max_position=64)
+    eng = LLMEngine(cfg, model_runner=FakeRunner())
+    sp = SamplingParams(temperature=0.6, max_tokens=4, ignore_eos=True)
+    with pytest.raises(ValueError, match="max_num_batched_tokens"):
+        eng.add_prompt(list(range(1, 15)), sp)                 # 14 + 4 - 1 = 17 tokens in a step of 16
+    with pytest.raises(ValueError, match="blocks"):
+        eng.add_prompt(list(range(1, 11)), sp)                 # 13 tokens = 4 blocks of 4, the pool has 3
+    eng.add_prompt(list(range(1, 10)), sp)                     # 12 tokens = 3 blocks: fits exactly
+    out = eng.generate([], sp)
+    assert [len(t) for t in out["token_ids"]] == [4] and len(eng.scheduler.block_manager.free_block_ids) == 3
