@@ -483,6 +483,11 @@ def test_block_manager_invariants_under_random_operations():
             assert s.num_cached_tokens % bs == 0 and 0 <= s.num_cached_tokens <= max(len(s) - 1, 0)
             for i in range(s.num_cached_tokens // bs):
                 assert bm.blocks[s.block_table[i]].token_ids == s.block(i)
+            h = -1
+            for i in range(len(s) // bs):                       # a full block's hash, if it has one, is its prefix chain's
+                h = BlockManager.compute_hash(s.block(i), h)
+                if all(t >= 0 for t in s.token_ids[:(i + 1) * bs]):
+                    assert bm.blocks[s.block_table[i]].hash in (-1, h)
         assert all(b.ref_count == counts.get(b.block_id, 0) for b in bm.blocks)
         assert set(bm.free_block_ids).isdisjoint(bm.used_block_ids) and bm.used_block_ids == set(counts)
         assert len(bm.free_block_ids) + len(bm.used_block_ids) == len(bm.blocks)
