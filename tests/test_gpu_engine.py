@@ -303,3 +303,51 @@ def test_two_sequences_reach_eos_in_consecutive_steps_while_running_ahead():
     assert out[a] == free[a][:s + 1] and out[b] == free[b][:s + 2]
     assert all(t[-1] == eos or len(t) == 40 for t in out) and all(eos not in t[:-1] for t in out)
     assert len(eng.scheduler.block_manager.free_block_ids) == cfg["max_cached_blocks"] and eng.pending is None
+
+
+@pytest.mark.parametrize("ignore_eos", [True, False])
+def test_static_decode_buffers_equal_the_host_metadata_before_every_replay(ignore_eos):
+    """The captured step advances its own inputs on the device (ids, positions, context lengths, slots) and the host
+    only patches rows that open a block; a changed batch is refilled.  Before every replay the static buffers must hold
+    exactly what ``decode_metadata`` computes from the sequences on the host: checked here in front of each replay of
+    a run whose sequences cross block boundaries, finish at different times and are replaced by waiting ones (and,
+    with EOS honoured, end one commit late)."""
+    from minivllm_amd.engine.metadata import decode_metadata
+    cfg = dict(SMALL, vocab_size=64, enforce_eager=False, max_num_sequences=4, max_cached_blocks=96,
+               max_model_length=160, eos=5 if not ignore_eos else -1)
+    eng = LLMEngine(cfg)
+    runner = eng.model_runner
+    current, checked = {}, [0]
+
+    class Checked:
+        def __init__(self, graph):
+            self.graph = graph
+
+        def replay(self):
+            seqs, v, bs = current["seqs"], runner.graph_vars, len(current["seqs"])
+            md = decode_metadata(seqs, runner.block_size)
+            torch.cuda.synchronize()
+            assert v["context_lens"][:bs].tolist() == md["context_lens"]
+            assert v["positions"][:bs].tolist() == [n - 1 for n in md["context_lens"]]
+            assert v["slot_mapping"][:bs].tolist() == md["slot_mapping"]
+            for i, seq in enumerate(seqs):
+                assert v["block_tables"][i, :len(seq.block_table)].tolist() == seq.block_table
+                if seq.last_token >= 0:                      # else the id is still on its way: the device has it
+                    assert int(v["input_ids"][i]) == seq.last_token
+            checked[0] += 1
+            self.graph.replay()
+
+    runner.graphs = {bs: Checked(g) for bs, g in runner.graphs.items()}
+    launch = runner.launch_decode
+
+    def launch_decode(seqs):
+        current["seqs"] = list(seqs)
+        return launch(seqs)
+
+    runner.launch_decode = launch_decode
+    prompts = _prompts(7, 10, 18, seed=71, vocab=64)
+    out = eng.generate(prompts, SamplingParams(temperature=0.9, max_tokens=40, ignore_eos=ignore_eos))["token_ids"]
+    assert checked[0] > 40 and len(out) == 7
+    assert len(eng.scheduler.block_manager.free_block_ids) == cfg["max_cached_blocks"]
+    if not ignore_eos:
+        assert any(len(t) < 40 for t in out) and all(5 not in t[:-1] for t in out)
