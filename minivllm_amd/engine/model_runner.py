@@ -141,10 +141,13 @@ class ModelRunner:
                     block_tables=self._to_device(md["block_tables"], torch.int32))
         return self._to_device(md["input_ids"], torch.int64), context_lens - 1
 
-    @torch.inference_mode()
+    @torch.no_grad()
     def capture_decode_graphs(self):
         """Record one hipGraph of a whole decode step per batch-size bucket (model_runner.py:316-369): the forward
-        pass, the LM head and the sampler.
+        pass, the LM head and the sampler.  Captured under ``no_grad``, not ``inference_mode`` (which the reference's
+        capture runs under): torch creates the default generator's graph-side seed and offset tensors at the first
+        capture and updates them in place at every later one, so captured in inference mode they would make every
+        capture elsewhere in the process fail ("inplace update to inference tensor") for as long as these graphs live.
 
         The step metadata lives in static device buffers that ``run`` refills or advances before every replay;
         rows past the real batch carry slot -1, context length 0, temperature 1 and whatever table entries were

@@ -351,3 +351,22 @@ def test_static_decode_buffers_equal_the_host_metadata_before_every_replay(ignor
     assert len(eng.scheduler.block_manager.free_block_ids) == cfg["max_cached_blocks"]
     if not ignore_eos:
         assert any(len(t) < 40 for t in out) and all(5 not in t[:-1] for t in out)
+    runner.launch_decode = launch                      # undo the wrapper: it closes a reference cycle through the runner
+
+
+def test_another_graph_can_be_captured_while_an_engine_is_alive():
+    """torch keeps the default generator's graph-side seed and offset tensors from the first capture in the process and
+    updates them in place at every later one; had the engine captured its steps in inference mode, a capture anywhere
+    else (outside inference mode) would fail for as long as the engine's graphs live.  The engine then still runs."""
+    eng = LLMEngine(dict(SMALL, enforce_eager=False))
+    sp = SamplingParams(temperature=0.9, max_tokens=6, ignore_eos=True)
+    first = eng.generate(_prompts(3, 3, 9, seed=81), sp)["token_ids"]
+    x = torch.zeros(16, device=DEV)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = x + 1
+    graph.replay()
+    torch.cuda.synchronize()
+    assert float(y.sum()) == 16.0
+    again = eng.generate(_prompts(3, 3, 9, seed=81), sp)["token_ids"]
+    assert [len(t) for t in again] == [len(t) for t in first] == [6, 6, 6]
