@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,prefill_long,store,int8,reference_shapes,decode_small,demo_shape,fused_qk,sampler,mfma_probe,loads_probe,engine,engine16,engine64,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,prefill_long,store,int8,reference_shapes,decode_small,demo_shape,head_dims,fused_qk,sampler,mfma_probe,loads_probe,engine,engine16,engine64,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -596,6 +596,40 @@ def bench_demo_shape(args):
     return out
 
 
+def bench_other_head_dims(args):
+    """bf16 head dims beside 64 and 128 that run on matrix-unit kernels (32, 80, 96, 112, 256: the decode kernels and
+    the 16-row tile prefill) and one that does not (72: the generic kernels), on the demo leg's batch: decode of 64
+    sequences of 1000-3000 tokens, prefill of 16 prompts of 64-2048 tokens, 16 query / 8 kv heads."""
+    import torch
+    from helpers import make_paged_case_on_device, make_varlen_case
+    from minivllm_amd.layers.attention import flash_attention_prefill, paged_attention_decode, paged_decode_plan, prefill_plan
+
+    dev = "cuda:0"
+    hq, hkv, bs = 16, 8, 16
+    g = torch.Generator().manual_seed(args.seed)
+    lengths = torch.randint(64, 2049, (16,), generator=g).tolist()
+    out = {"workload": "bf16, Hq16 Hkv8: decode B64 ctx~U[1000,3000] block_size 16; prefill 16 prompts L~U[64,2048]"}
+    for d in (32, 80, 96, 112, 256, 72):
+        q, kc, vc, tables, ctx = make_paged_case_on_device(args.seed, dev, 64, 1000, 3000, hq, hkv, d, bs,
+                                                           dtype=torch.bfloat16, log_uniform=False)
+        td, cd = tables.to(dev), ctx.to(dev)
+        steps = args.steps if d != 72 else 3                       # the generic kernels are slow
+        _, ms = time_steps(lambda: paged_attention_decode(q, kc, vc, td, cd, 1 / math.sqrt(d), hq, hkv, d, bs),
+                           steps, min(args.warmup, steps), 0.0)
+        nbytes = int(ctx.sum()) * hkv * d * 2 * kc.element_size()
+        qq, kk, vv, cu = (t.to(dev) for t in make_varlen_case(args.seed + 1, lengths, hq, hkv, d, dtype=torch.bfloat16))
+        _, pms = time_steps(lambda: flash_attention_prefill(qq, kk, vv, cu, 1 / math.sqrt(d), hq, hkv, d),
+                            steps, min(args.warmup, steps), 0.0)
+        flops = 4 * hq * d * sum(n * (n + 1) // 2 for n in lengths)
+        out[f"head_dim_{d}"] = {
+            "decode_kernel": "generic" if paged_decode_plan(64, hq, hkv, d, tables.shape[1], bs, torch.bfloat16)[2] == 0 else "mfma",
+            "decode_us": ms * 1e3, "decode_gbs": nbytes / (ms * 1e-3) / 1e9,
+            "prefill_kernel": {0: "generic", 1: "16-row tiles", 2: "lds-tiled"}[prefill_plan(hq, hkv, d, dtype=torch.bfloat16)],
+            "prefill_ms": pms, "prefill_tflops": flops / (pms * 1e-3) / 1e12,
+        }
+    return out
+
+
 def bench_reference_shapes(args, want_cpu):
     """The shapes the reference's own benchmark scripts run (fp16, 32 query / 8 kv heads of 128 dims, block 16,
     identity block tables, every context the same length): decode (B, L) = (2,60) (1,512) (16,256) (4,2048)
@@ -797,6 +831,8 @@ def main():
         extra["decode_small_batch"] = bench_decode_small(args)
     if want("demo_shape"):
         extra["reference_demo_shape"] = bench_demo_shape(args)
+    if want("head_dims"):
+        extra["other_head_dims"] = bench_other_head_dims(args)
     if want("fused_qk"):
         extra["fused_qk"] = bench_fused_qk(args)
     if want("sampler"):
