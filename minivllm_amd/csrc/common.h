@@ -209,4 +209,27 @@ int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hip
 // shapes that kernel is built for: fp32 and INT8 caches with 64 or 128 dims per head, 16-bit also with 32, 80, 96, 112 and 256
 bool prefill_rows16_takes(int head_dim, int dtype, bool int8_cache);
 
+// Varlen causal prefill in the two-group form (prefill_pingpong.hip): one persistent 8-wave workgroup per CU whose two
+// wave groups alternate between the matrix unit and the softmax.  Launched from the prefill entry point for the batches
+// it takes; everything else stays on prefill_mfma_kernel.
+struct PrefillPpArgs {
+  void* out;
+  const void* q;
+  const void* k;
+  const void* v;
+  const int32_t* cu_seqlens;
+  int64_t total_tokens;
+  int num_seqs;
+  int num_heads;
+  int num_kv_heads;
+  float scale_log2;
+  // filled in by the launcher
+  int slices;       // head slices: kv heads x (query heads per kv head / 4)
+  int n_teams;      // gcd(8, slices): workgroup teams, each with its own item list
+  int team_size;    // workgroups per team
+  int level_bits;   // bits that hold the block count of the longest possible sequence
+};
+bool prefill_pp_takes(int num_seqs, int num_heads, int num_kv_heads, int head_dim, int dtype);
+int launch_prefill_pp(const PrefillPpArgs& a, int dtype, hipStream_t stream);
+
 }  // namespace mvllm

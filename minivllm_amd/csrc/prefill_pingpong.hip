@@ -1,0 +1,675 @@
+// Varlen causal flash-attention prefill for gfx950, two-group ("ping-pong") form.
+// Replaces the Triton kernel of src/myvllm/layers/attention.py:111-209 for batches this kernel is built for
+// (16-bit q/k/v, head_dim 128, query heads per kv head a multiple of 4, at most 64 sequences); the launcher in
+// prefill_varlen.hip falls back to prefill_mfma_kernel for everything else.
+//
+// One persistent workgroup of 8 waves per CU (two waves per SIMD, 160 KB of LDS).  A work item is one kv head, four
+// of its query heads and a block of 64 consecutive query rows of one sequence; wave w owns query head w % 4 and the
+// 32-row half w / 4 of the block.  Waves 0-3 (group 0) and waves 4-7 (group 1) run the same tile loop one barrier
+// interval apart: while one group feeds the matrix unit (O += V^T P^T of tile n, then S^T = K Q^T of tile n + 1: 32
+// MFMAs, no other vector work) the other does the softmax of its tile on the vector unit, and they swap at every
+// barrier.  The two waves that share a SIMD are then never both in their softmax nor both waiting for the matrix
+// unit, which is what a workgroup per group (no ordering between them) left to chance.
+//
+// Everything a workgroup needs arrives in LDS by buffer_load ... lds: 64-row K and V tiles in rings of three,
+// issued three barrier intervals before their first use, and each wave's 32 query rows, into a private 8 KB slot
+// that is also the transposing buffer of the wave's output rows.  The tile stream runs on across item boundaries
+// (the ring does not care which item a tile belongs to), the next item's Q rows are on their way while the current
+// item is computed, and an item's output is normalised, transposed and stored during the softmax interval of the
+// next item's first tile, so a workgroup pays the start-up latency once, not once per item.
+//
+// Items are dealt statically, heaviest first: level = index of the 64-row block inside its sequence (a block at
+// level b walks b + 1 key tiles), levels descending, inside a level head slice then sequence.  The workgroups that
+// share a list ("team": the workgroups of the XCDs that serve the same head slices, so that a kv head's keys stay in
+// one L2) take ranks in serpentine order (r T + t in even rounds, r T + T - 1 - t in odd ones), which evens out the
+// cost per workgroup.  Every wave finds its items from cu_seqlens with ballots; nothing is prepared by the host.
+#include "prefill_tiles.h"
+
+namespace mvllm {
+
+namespace {
+
+constexpr int kPpBN = 64;          // keys per tile
+constexpr int kPpRing = 3;         // K and V tiles in flight
+constexpr int kPpWaves = 8;
+#ifndef MVLLM_PP_PRIO
+#define MVLLM_PP_PRIO 3
+#endif
+#ifndef MVLLM_PP_LB
+#define MVLLM_PP_LB 512
+#endif
+
+template <int D>
+struct PpLds {
+  static constexpr int kRowB = D * 2;
+  static constexpr int kTileBytes = kPpBN * kRowB;
+  static constexpr int kSlotBytes = 32 * kRowB;
+  char k[kPpRing][kTileBytes];
+  char v[kPpRing][kTileBytes];
+  char qo[kPpWaves][kSlotBytes];    // per wave: Q rows of the next item on their way in, then the output rows on their way out
+};
+
+template <int N> __device__ __forceinline__ void vm_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// all waves of the workgroup; orders nothing but the compiler's own memory accesses (no LDS or memory counter is
+// drained: data other waves read arrives by DMA, whose completion the issuing wave awaits explicitly)
+__device__ __forceinline__ void pp_barrier() {
+  __builtin_amdgcn_sched_barrier(0);            // no instruction of the softmax interval drifts into the matrix interval, nor back
+  asm volatile("s_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// 16 bytes per lane into LDS at m0_base + 16 * lane, from rsrc + lane_off.
+__device__ __forceinline__ void dma16(v4i rsrc, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(lane_off), "s"(rsrc) : "m0", "memory");
+}
+
+}  // namespace
+
+// One team's item list, walked in rank order.  Wave-uniform.
+struct PpItems {
+  int level;          // level the walk has reached (-1: past the last item)
+  unsigned base;      // rank of that level's first item
+  unsigned taken;     // items this workgroup has asked for
+};
+struct PpItem {
+  int seq_start, seq_len, rb, y;
+  bool valid;
+};
+
+template <typename T, int D, int GRP>
+__device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, const int wave) {
+  constexpr int kRowB = D * 2;
+  constexpr int kTileBytes = kPpBN * kRowB;
+  constexpr int kKS = D / 16;
+  constexpr int kTD = D / 32;
+  static_assert(D == 128, "swizzles and copy shapes are written for 256-byte rows");
+  auto kswz = [](int row) __attribute__((always_inline)) { return row & 15; };
+  auto vswz = [](int row) __attribute__((always_inline)) { return ((row & 3) << 2) | (row & 1); };
+
+  const int lane = threadIdx.x & 63;
+  const int l32 = lane & 31;
+  const int hi = lane >> 5;
+  const int wq = wave & 3;                     // query head inside the slice
+
+  // ---- the batch, one sequence per lane ----
+  int lo = 0, len = 0;
+  if (lane < a.num_seqs) {
+    lo = a.cu_seqlens[lane];
+    len = a.cu_seqlens[lane + 1] - lo;
+  }
+  const int nb = (len + 63) >> 6;              // 64-row blocks of the lane's sequence
+  int top = 0;                                 // highest block count in the batch
+  for (int bit = a.level_bits - 1; bit >= 0; --bit) {
+    const int trial = top | (1 << bit);
+    if (__ballot(nb >= trial) != 0ull) top = trial;
+  }
+
+  // ---- which items are this workgroup's ----
+  const unsigned wg = blockIdx.x;
+  const unsigned xcd = wg & 7u;
+  const int team = (int)(xcd % (unsigned)a.n_teams);
+  const unsigned TS = (unsigned)a.team_size;
+  const unsigned t = (wg >> 3) * (8u / (unsigned)a.n_teams) + xcd / (unsigned)a.n_teams;   // index inside the team
+  const unsigned spt = (unsigned)(a.slices / a.n_teams);                                  // slices per team
+  auto next_item = [&](PpItems& w) {
+    PpItem it;
+    it.seq_start = 0; it.seq_len = 0; it.rb = 0; it.y = 0; it.valid = false;
+    const unsigned round = w.taken++;
+    const unsigned R = round * TS + ((round & 1u) ? TS - 1u - t : t);
+    unsigned long long mask = 0ull;
+    unsigned cnt = 0;
+    while (w.level >= 0) {
+      mask = __ballot(nb > w.level);
+      cnt = (unsigned)__popcll(mask);
+      const unsigned items = cnt * spt;
+      if (R - w.base < items) break;
+      w.base += items;
+      --w.level;
+    }
+    if (w.level < 0) return it;
+    const unsigned idx = R - w.base;
+    const unsigned sl = idx / cnt;
+    const int qth = (int)(idx - sl * cnt);
+    const int below = __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+    const unsigned long long pick = __ballot(((mask >> lane) & 1ull) != 0ull && below == qth);
+    const int owner = __ffsll((long long)pick) - 1;
+    it.seq_start = __builtin_amdgcn_readfirstlane(__shfl(lo, owner, 64));
+    it.seq_len = __builtin_amdgcn_readfirstlane(__shfl(len, owner, 64));
+    it.rb = __builtin_amdgcn_readfirstlane(w.level);
+    it.y = __builtin_amdgcn_readfirstlane(team + a.n_teams * (int)sl);
+    it.valid = true;
+    return it;
+  };
+
+  PpItems walk_c = {top - 1, 0u, 0u};          // the walk that feeds the compute cursor (runs one item ahead)
+  PpItems walk_d = walk_c;                     // ... and the one of the K/V copy cursor
+  PpItem cur = next_item(walk_c);
+  if (!cur.valid) return;                      // no item for this workgroup (all waves agree)
+  PpItem nxt = next_item(walk_c);
+  PpItem dit = next_item(walk_d);              // item the copy cursor is in
+  int dj = 0;                                  // ... and its tile there
+
+  const int group = a.num_heads / a.num_kv_heads;
+  const int chunks = group / 4;
+  const T* qg = reinterpret_cast<const T*>(a.q);
+  const char* kg = reinterpret_cast<const char*>(a.k);
+  const char* vg = reinterpret_cast<const char*>(a.v);
+  const int kv_row_bytes = a.num_kv_heads * kRowB;
+  const int q_row_bytes = a.num_heads * kRowB;
+  const int total_rows = (int)a.total_tokens;
+
+  // ---- copies ----
+  // Group 0 copies the K tiles, group 1 the V tiles, each at the start of its softmax interval: wave w of a group
+  // moves rows 16 w .. 16 w + 15 of the tile, 4 rows (1 KB) per instruction.  A copy is issued three barrier
+  // intervals before the barrier that publishes it and overwrites the tile three places back in its ring, whose
+  // last readers finished an interval before.
+  const int ld_row = lane >> 4, ld_chunk = lane & 15;
+  uint32_t src_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 16 * wq + 4 * i + ld_row;
+    src_off[i] = (uint32_t)(row * kv_row_bytes + ((ld_chunk ^ (GRP == 0 ? kswz(row) : vswz(row))) << 4));
+  }
+  const char* copy_src = GRP == 0 ? kg : vg;
+  const uint32_t lds_copy0 = (GRP == 0 ? lds_address(&lds.k[0][0]) : lds_address(&lds.v[0][0])) + (uint32_t)(16 * wq * kRowB);
+  // A tile's descriptor starts at its first row (for the item's kv head) and ends with the tensor, so rows past the
+  // last token arrive as zeros; size 0 (nothing read, zeros written) when the stream has ended.  The cursor keeps
+  // the tile's byte offset and the rows that follow it.
+  const int rows_4g = (int)(0xffffffffu / (uint32_t)kv_row_bytes);
+  int64_t d_off = 0;                           // byte offset of the cursor's tile in k (and v)
+  int d_rows_left = 0;                         // rows from the tile's first to the tensor's last; <= 0: no tile
+  int d_head_off = 0;                          // byte offset of the kv head inside a row
+  auto enter_item = [&]() {                    // the cursor's tile = first tile of `dit`
+    d_head_off = (dit.y / chunks) * kRowB;
+    d_off = (int64_t)dit.seq_start * kv_row_bytes + d_head_off;
+    d_rows_left = dit.valid ? total_rows - dit.seq_start : 0;
+  };
+  enter_item();
+  int d_slot = 0;                              // ring slot of the cursor's tile ( = its stream index % 3)
+  auto copy_step = [&]() {
+    const uint32_t size = d_rows_left <= 0        ? 0u
+                          : d_rows_left > rows_4g ? 0xffffffffu
+                                                  : (uint32_t)d_rows_left * (uint32_t)kv_row_bytes - (uint32_t)d_head_off;
+    const v4i r = make_rsrc(copy_src + d_off, size);
+    const uint32_t dst = lds_copy0 + (uint32_t)(d_slot * kTileBytes);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16(r, src_off[i], dst + 1024u * i);
+    d_slot = d_slot == kPpRing - 1 ? 0 : d_slot + 1;
+    if (dit.valid) {
+      if (++dj > dit.rb) {
+        dit = next_item(walk_d);
+        dj = 0;
+        enter_item();
+      } else {
+        d_off += (int64_t)kPpBN * kv_row_bytes;      // the next 64 rows of the same sequence and head
+        d_rows_left -= kPpBN;
+      }
+    }
+  };
+  // Q rows of an item -> this wave's slot, 4 rows per instruction, chunks swizzled like a K tile's
+  const uint32_t lds_q = lds_address(&lds.qo[wave][0]);
+  auto copy_q = [&](const PpItem& it) {
+    const int h = (it.y / chunks) * group + (it.y % chunks) * 4 + wq;
+    const int row = it.seq_start + it.rb * 64 + 32 * GRP;
+    const int rows_left = total_rows - row;
+    const int rows_4g = (int)(0xffffffffu / (uint32_t)q_row_bytes);
+    const uint32_t size = rows_left <= 0 ? 0u
+                          : rows_left > rows_4g ? 0xffffffffu
+                                                : (uint32_t)rows_left * (uint32_t)q_row_bytes - (uint32_t)(h * kRowB);
+    const v4i r = make_rsrc(reinterpret_cast<const char*>(qg) + (int64_t)row * q_row_bytes + (int64_t)h * kRowB, size);
+    int lane_q = lane;
+    asm volatile("" : "+v"(lane_q));              // the eight source offsets are computed per item, not kept in registers
+    const int qrow = lane_q >> 4, qchunk = lane_q & 15;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int rowi = 4 * i + qrow;
+      const uint32_t off = (uint32_t)(rowi * q_row_bytes + ((qchunk ^ kswz(rowi)) << 4));
+      dma16(r, off, lds_q + (uint32_t)(i * 1024));
+    }
+  };
+
+  // ---- per-lane LDS offsets of the operand fragments (as in prefill_mfma_kernel) ----
+  const int i16 = lane & 15;
+  const int half = (lane >> 4) & 1;
+  int k_off[kKS];
+#pragma unroll
+  for (int ks = 0; ks < kKS; ++ks) k_off[ks] = l32 * kRowB + (((2 * ks + hi) ^ kswz(l32)) << 4);
+  const int v_row = 4 * hi + (i16 >> 2);
+  int v_off[kTD];
+#pragma unroll
+  for (int td = 0; td < kTD; ++td)
+    v_off[td] = v_row * kRowB + (((4 * td + 2 * half + ((i16 & 3) >> 1)) ^ vswz(v_row)) << 4) + ((i16 & 1) << 3);
+
+  // ---- state ----
+  uint4 qf[kKS];
+  v16f o[kTD];
+  v16f s[2];
+  uint4 pf[4];                                  // P of the tile whose softmax was last, packed: [2 tk + st]
+  float l = 0.f;
+  // Running maximum of the lane's row, negated, in all 16 registers of an accumulator tuple: the score products
+  // start from it (C operand of their first MFMA), so a tile's scores arrive as  score * scale * log2 e - m, ready
+  // for exp2.  (An item's first tile starts from zero instead: its maximum is not known yet.)
+  v16f neg_m;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) neg_m[r] = 0.f;
+#pragma unroll
+  for (int td = 0; td < kTD; ++td)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[td][r] = 0.f;
+
+  // slot -> registers, times scale * log2 e (rounded to the element type once), so that the scores leave the matrix
+  // unit as exp2 arguments.  The multiplications run in a matrix interval, whose wave has vector slots to spare.
+  auto load_q = [&]() {
+    const char* qs = &lds.qo[wave][0];
+#pragma unroll
+    for (int ks = 0; ks < kKS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(qs + k_off[ks]);
+#pragma unroll
+    for (int ks = 0; ks < kKS; ++ks) {
+      qf[ks].x = scale_pair<T>(qf[ks].x, a.scale_log2);
+      qf[ks].y = scale_pair<T>(qf[ks].y, a.scale_log2);
+      qf[ks].z = scale_pair<T>(qf[ks].z, a.scale_log2);
+      qf[ks].w = scale_pair<T>(qf[ks].w, a.scale_log2);
+    }
+  };
+  // Operand fragments from LDS.  K: rows l32 and l32 + 32 of the tile in K ring slot `slot`, dims 16 ks + 8 hi ..;
+  // V^T: the transposing reads of the 16 keys of `step` ( = 2 tk + st) of the tile in V ring slot `slot`.
+  auto k_frags = [&](int slot, auto KS, uint4 (&kf)[2]) {
+    constexpr int ks = decltype(KS)::value;
+#ifdef PP_EXP_NOLDS
+    kf[0] = qf[ks]; kf[1] = qf[(ks + 1) & 7]; (void)slot;
+    return;
+#endif
+    const char* kb = &lds.k[0][0] + slot * kTileBytes + k_off[ks];
+    kf[0] = *reinterpret_cast<const uint4*>(kb);
+    kf[1] = *reinterpret_cast<const uint4*>(kb + 32 * kRowB);
+  };
+  auto v_frags = [&](int slot, auto STEP, uint4 (&af)[kTD]) {
+    constexpr int step = decltype(STEP)::value;
+#ifdef PP_EXP_NOLDS
+    for (int td = 0; td < kTD; ++td) af[td] = qf[(td + step) & 7];
+    (void)slot;
+    return;
+#endif
+    const char* vb = &lds.v[0][0] + slot * kTileBytes + 16 * step * kRowB;
+#pragma unroll
+    for (int td = 0; td < kTD; ++td) {
+      const char* p0 = vb + v_off[td];
+      const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
+      const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * kRowB));
+      af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;
+      af[td].z = __builtin_bit_cast(uint2, a1).x; af[td].w = __builtin_bit_cast(uint2, a1).y;
+    }
+  };
+  // the scores of the stream's first tile (the later ones are computed at the end of each matrix interval)
+  auto first_scores = [&](int slot) {
+    static_for<kKS>([&](auto KS) {
+      constexpr int ks = decltype(KS)::value;
+      uint4 kf[2];
+      k_frags(slot, KS, kf);
+      if constexpr (ks == 0) {
+        v16f z;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) z[r] = 0.f;
+#pragma unroll
+        for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf[tk], qf[0], z);
+      } else {
+#pragma unroll
+        for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf[tk], qf[ks], s[tk]);
+      }
+    });
+  };
+  // normalise, transpose through the wave's slot, store whole rows (rows past the sequence's end are not stored)
+  T* out = reinterpret_cast<T*>(a.out);
+  auto store_item = [&](int seq_start, int seq_len, int rb, int y, float lsum) {
+    char* ot = &lds.qo[wave][0];
+    const float lt = lsum + __shfl_xor(lsum, 32, 64);
+    const float inv = 1.f / lt;
+    int lane_o = lane;
+    asm volatile("" : "+v"(lane_o));              // addresses below are computed per item, not kept in registers between items
+    const int ol32 = lane_o & 31, ohi = lane_o >> 5;
+#pragma unroll
+    for (int td = 0; td < kTD; ++td)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        uint2 w;
+        w.x = pack2<T>(o[td][4 * r4 + 0] * inv, o[td][4 * r4 + 1] * inv);
+        w.y = pack2<T>(o[td][4 * r4 + 2] * inv, o[td][4 * r4 + 3] * inv);
+        *reinterpret_cast<uint2*>(ot + ol32 * kRowB + (((4 * td + r4) ^ kswz(ol32)) << 4) + 8 * ohi) = w;
+      }
+    const int h = (y / chunks) * group + (y % chunks) * 4 + wq;
+    const int r0 = rb * 64 + 32 * GRP;
+    const int orow = lane_o >> 4, ochunk = lane_o & 15;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = 4 * i + orow;
+      const uint4 w = *reinterpret_cast<const uint4*>(ot + row * kRowB + ((ochunk ^ kswz(row)) << 4));
+      if (r0 + row < seq_len)
+        store16_stream(out + ((int64_t)(seq_start + r0 + row) * a.num_heads + h) * D + 8 * ochunk, w);
+    }
+  };
+  auto wait_copies = [&](int later) {            // everything but the `later` newest VMEM instructions has completed
+    if (later == 4) vm_wait<4>();
+    else if (later == 12) vm_wait<12>();
+    else if (later == 20) vm_wait<20>();
+    else vm_wait<0>();
+  };
+
+  // ---- start: the first item's Q rows and the first three copy steps ----
+  copy_q(cur);
+  copy_step();
+  copy_step();
+  vm_wait<0>();
+  pp_barrier();
+  load_q();
+  int c_slot = 0;                               // ring slot of the tile whose softmax comes next
+  int p_seq_start = 0, p_seq_len = 0, p_rb = 0, p_y = 0;   // item whose output is still in the accumulators
+  bool have_prev = false;
+  float l_prev = 0.f;
+
+#ifdef PP_TIMING
+  unsigned long long* tlog = reinterpret_cast<unsigned long long*>(reinterpret_cast<T*>(a.out) + a.total_tokens * a.num_heads * D) + (GRP ? 2048 : 0) + 512 * (wave & 3);
+  int tn = 0;
+  const bool tlogging = blockIdx.x == PP_TIMING;
+#define TSTAMP() do { if (tlogging && tn < 500) { const unsigned long long t_ = __builtin_amdgcn_s_memtime(); if (lane == 0) tlog[tn] = t_; ++tn; } } while (0)
+#else
+#define TSTAMP() do {} while (0)
+#endif
+  if (GRP == 1) pp_barrier();                   // group 1 runs one interval behind
+  first_scores(c_slot);
+  asm volatile("" : "+v"(s[0]), "+v"(s[1]));
+  pp_barrier();
+
+  // The causal diagonal runs through half GRP of an item's last tile: key offset 8 (r / 4) + r % 4 + 4 hi inside
+  // that half against query row l32.  Group 0's rows see nothing of the second half, group 1's all of the first.
+  auto mask_diagonal = [&]() {
+    int lim = l32 - 4 * hi;
+    asm volatile("" : "+v"(lim));                 // computed here, not kept as sixteen lane masks across the loop
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if (8 * (r >> 2) + (r & 3) > lim) s[GRP][r] = -INFINITY;
+      if (GRP == 0) s[1][r] = -INFINITY;
+    }
+  };
+  auto tile_max = [&]() {                        // maximum of the lane's row over the tile, relative to the running one
+    const float mx0 = fmaxf(s[0][15], s[1][15]);
+    float mx = mx0, mx1 = mx0;
+#pragma unroll
+    for (int r = 0; r < 14; r += 2) {
+      mx = max3(mx, s[0][r], s[0][r + 1]);
+      mx1 = max3(mx1, s[1][r], s[1][r + 1]);
+    }
+    mx = max3(mx, s[0][14], s[1][14]);
+    mx = fmaxf(mx, mx1);
+    return max_with_lane_xor32(mx);
+  };
+  // P = exp2(s - d) packed into pf (s itself is kept: a tile whose weights turn out too large is redone from it);
+  // returns the lane's share of the row sum (of the weights before they are rounded to 16 bits: the roundings are
+  // unbiased and average out over a row).  SHIFT: d != 0.
+  auto weights = [&](auto SHIFT, float d) {
+    float sum = 0.f;
+#ifdef PP_EXP_NOSM
+    for (int i = 0; i < 4; ++i) { pf[i].x = __float_as_uint(s[i >> 1][8 * (i & 1)]); pf[i].y = __float_as_uint(s[i >> 1][8 * (i & 1) + 1]); pf[i].z = pf[i].x; pf[i].w = pf[i].y; }
+    return 1.f + d;
+#endif
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        float e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float x = s[tk][8 * st + i];
+#ifdef PP_EXP_NOEXP
+          e[i] = decltype(SHIFT)::value ? x - d : x;
+#else
+          e[i] = fast_exp2(decltype(SHIFT)::value ? x - d : x);
+#endif
+        }
+        uint4 p;
+        p.x = pack2<T>(e[0], e[1]);
+        p.y = pack2<T>(e[2], e[3]);
+        p.z = pack2<T>(e[4], e[5]);
+        p.w = pack2<T>(e[6], e[7]);
+        // Row sum with ordinary additions, four short chains.  (v_dot2_f32_bf16 on the packed pairs would halve the
+        // instruction count, but the dot instructions queue behind the other group's MFMAs: sixteen of them took as
+        // long as a whole matrix interval.)
+        sum += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+        pf[2 * tk + st] = p;
+      }
+    return sum;
+  };
+  auto set_neg_m = [&](float v) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) neg_m[r] = v;
+  };
+  // The matrix interval after the softmax of tile j of `cur`: O^T (+)= V^T P^T of that tile (FRESH: from zero, the
+  // item's first tile), then S^T = K Q^T of the stream's next tile, which belongs to the next item when j is the
+  // item's last (its Q rows were copied during this item's first softmax interval).  32 MFMAs in eight stages of
+  // four; every operand fragment is requested two stages (8 MFMAs, 256 matrix-unit clocks) before the stage that
+  // uses it, because nothing else runs on this SIMD's matrix unit meanwhile that could cover an LDS round trip.
+  // vf0, vf1: the V^T fragments of the tile's first two steps, requested before the barrier.  Group 0 also issues
+  // its share of the next copy step here, one instruction per stage.  Returns false when the stream ends here.
+  auto stage_end = [&]() { __builtin_amdgcn_sched_barrier(0); };
+  // The compiler computes a value where it is first used, and moves pure arithmetic across a barrier freely.  These
+  // empty statements make the softmax's results exist before the barrier that ends its interval, and the matrix
+  // interval's before the one that ends it, so that each interval holds the work it is named for.
+  auto pin_weights = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(pf[i].x), "+v"(pf[i].y), "+v"(pf[i].z), "+v"(pf[i].w));
+    asm volatile("" : "+v"(l), "+v"(neg_m));
+  };
+  auto pin_products = [&]() {
+    asm volatile("" : "+v"(s[0]), "+v"(s[1]));
+    asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
+  };
+  auto matrix_interval = [&](auto FRESH, bool last, uint4 (&vf0)[kTD], uint4 (&vf1)[kTD]) {
+    using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>; using I3 = std::integral_constant<int, 3>;
+    using I4 = std::integral_constant<int, 4>; using I5 = std::integral_constant<int, 5>;
+    using I6 = std::integral_constant<int, 6>; using I7 = std::integral_constant<int, 7>;
+    const int n_slot = c_slot == kPpRing - 1 ? 0 : c_slot + 1;
+    const bool more = !last || nxt.valid;
+    // this wave's MFMAs go in front of the other group's vector instructions on the shared SIMD
+    __builtin_amdgcn_s_setprio(MVLLM_PP_PRIO);
+    uint4 vf2[kTD], vf3[kTD];
+    uint4 kf0[2], kf1[2], kf2[2], kf3[2], kf4[2], kf5[2], kf6[2], kf7[2];
+    // stage A
+    v_frags(c_slot, I2{}, vf2);
+    if (last && nxt.valid) {
+      // the next item's Q rows, copied since this item's first softmax interval; one copy step was issued behind
+      // them unless the item has a single tile
+      if (cur.rb > 0) vm_wait<4>();
+      else vm_wait<0>();
+      load_q();
+    }
+    if constexpr (decltype(FRESH)::value) {
+      v16f z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+#pragma unroll
+      for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf0[td], pf[0], z);
+    } else {
+#pragma unroll
+      for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf0[td], pf[0], o[td]);
+    }
+    stage_end();
+    // stage B
+    v_frags(c_slot, I3{}, vf3);
+#pragma unroll
+    for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf1[td], pf[1], o[td]);
+    stage_end();
+    // stage C
+    if (more) { k_frags(n_slot, I0{}, kf0); k_frags(n_slot, I1{}, kf1); }
+#pragma unroll
+    for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf2[td], pf[2], o[td]);
+    stage_end();
+    // stage D
+    if (more) { k_frags(n_slot, I2{}, kf2); k_frags(n_slot, I3{}, kf3); }
+#pragma unroll
+    for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf3[td], pf[3], o[td]);
+    stage_end();
+    if (more) {
+      // stage E
+      k_frags(n_slot, I4{}, kf4); k_frags(n_slot, I5{}, kf5);
+      if (last) {
+        // another item's first tile: its maximum is not known yet, the scores arrive as they are
+        v16f z;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) z[r] = 0.f;
+#pragma unroll
+        for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf0[tk], qf[0], z);
+      } else {
+#pragma unroll
+        for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf0[tk], qf[0], neg_m);
+      }
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf1[tk], qf[1], s[tk]);
+      stage_end();
+      // stage F
+      k_frags(n_slot, I6{}, kf6); k_frags(n_slot, I7{}, kf7);
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf2[tk], qf[2], s[tk]);
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf3[tk], qf[3], s[tk]);
+      stage_end();
+      // stage G
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf4[tk], qf[4], s[tk]);
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf5[tk], qf[5], s[tk]);
+      stage_end();
+      // stage H
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf6[tk], qf[6], s[tk]);
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf7[tk], qf[7], s[tk]);
+      stage_end();
+    }
+    pin_products();
+    __builtin_amdgcn_s_setprio(0);
+    TSTAMP();
+    pp_barrier();
+    c_slot = n_slot;
+    return more;
+  };
+
+  while (true) {
+    // ======== first tile of an item ========
+    bool last = cur.rb == 0;
+    int later = 4;
+    TSTAMP();
+    copy_step();
+    if (last) mask_diagonal();
+    const float mx_first = tile_max();           // neg_m is zero here: the tile's maximum itself
+    // the item before this one leaves (its last P V ran in the interval before) ...
+    if (have_prev) {
+      store_item(p_seq_start, p_seq_len, p_rb, p_y, l_prev);
+      later += 8;
+    }
+    // ... and the next one's Q rows set out
+    if (nxt.valid) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slot's last readers are done
+      copy_q(nxt);
+      later += 8;
+    }
+    TSTAMP();
+    l = weights(std::true_type{}, mx_first);
+    TSTAMP();
+    set_neg_m(-mx_first);
+    uint4 vf0[kTD], vf1[kTD];
+    pin_weights();
+    TSTAMP();
+    v_frags(c_slot, std::integral_constant<int, 0>{}, vf0);   // the tile's first V^T fragments: on their way across the barrier
+    v_frags(c_slot, std::integral_constant<int, 1>{}, vf1);
+    wait_copies(later);
+    pp_barrier();
+    TSTAMP();
+    bool more = matrix_interval(std::true_type{}, last, vf0, vf1);
+    // ======== the item's other tiles ========
+    for (int j = 1; j <= cur.rb; ++j) {
+      last = j == cur.rb;
+      TSTAMP();
+      copy_step();
+      if (last) mask_diagonal();
+      // The scores are relative to the running maximum, which is not looked at again unless it is badly out of
+      // date: the weights are computed first, and only when a lane's share of the tile's row sum passes 2^12 (a
+      // weight above 2^7 at least; 16-bit weights and fp32 sums are far from their limits there) is the tile redone
+      // the long way: true maximum, accumulators and row sum scaled down, weights again from the kept scores.
+      TSTAMP();
+      float sum = weights(std::false_type{}, 0.f);
+      asm volatile("" : "+v"(sum));
+      TSTAMP();
+      if (__any(!(sum <= 4096.f))) {
+        const float mx = tile_max();
+        const float d = mx > 8.f ? mx : 0.f;       // per row (both lanes of a row see the same maximum)
+        if (d != 0.f) {
+          const float alpha = fast_exp2(-d);
+          l *= alpha;
+#pragma unroll
+          for (int td = 0; td < kTD; ++td)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[td][r] *= alpha;
+        }
+        set_neg_m(neg_m[0] - d);
+        sum = weights(std::true_type{}, d);
+      }
+      l += sum;
+      pin_weights();
+      TSTAMP();
+      v_frags(c_slot, std::integral_constant<int, 0>{}, vf0);
+      v_frags(c_slot, std::integral_constant<int, 1>{}, vf1);
+      wait_copies(4);
+      pp_barrier();
+      TSTAMP();
+      more = matrix_interval(std::false_type{}, last, vf0, vf1);
+    }
+    l_prev = l;
+    p_seq_start = cur.seq_start; p_seq_len = cur.seq_len; p_rb = cur.rb; p_y = cur.y;
+    have_prev = true;
+    if (!more) break;
+    cur = nxt;
+    nxt = next_item(walk_c);
+  }
+  if (GRP == 0) pp_barrier();                   // group 1's last interval
+  vm_wait<0>();
+  store_item(p_seq_start, p_seq_len, p_rb, p_y, l_prev);
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(MVLLM_PP_LB) void prefill_pp_kernel(const PrefillPpArgs a) {
+  __shared__ __attribute__((aligned(1024))) PpLds<D> lds;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (wave < 4) pp_run<T, D, 0>(a, lds, wave);
+  else pp_run<T, D, 1>(a, lds, wave);
+}
+
+bool prefill_pp_takes(int num_seqs, int num_heads, int num_kv_heads, int head_dim, int dtype) {
+  if (dtype == MVLLM_F32 || head_dim != 128 || num_seqs > 64 || num_seqs <= 0) return false;
+  const int group = num_heads / num_kv_heads;
+  return group % 4 == 0 && (int64_t)num_heads * head_dim * 2 * 64 < ((int64_t)1 << 31);
+}
+
+int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) {
+  PrefillPpArgs a = args;
+  const int group = a.num_heads / a.num_kv_heads;
+  a.slices = a.num_kv_heads * (group / 4);
+  int n_teams = 8;
+  while (a.slices % n_teams != 0) n_teams >>= 1;      // gcd(8, slices)
+  a.n_teams = n_teams;
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  const int grid = cus / 8 * 8 > 0 ? cus / 8 * 8 : 8;
+  a.team_size = grid / n_teams;
+  a.level_bits = 1;
+  while (((int64_t)1 << a.level_bits) <= a.total_tokens / 64 + 1) ++a.level_bits;
+  if (dtype == MVLLM_BF16) prefill_pp_kernel<bf16_t, 128><<<dim3(grid), dim3(64 * kPpWaves), 0, stream>>>(a);
+  else prefill_pp_kernel<f16_t, 128><<<dim3(grid), dim3(64 * kPpWaves), 0, stream>>>(a);
+  return launch_status();
+}
+
+}  // namespace mvllm

@@ -6,8 +6,7 @@
 // and a workgroup finds its (sequence, local tile) by walking cu_seqlens, so
 // the grid needs only total_tokens and num_seqs (upper bound
 // total_tokens/BM + num_seqs tiles) and no host-side maximum length.
-#include <type_traits>
-#include "common.h"
+#include "prefill_tiles.h"
 
 namespace mvllm {
 
@@ -143,11 +142,6 @@ __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs 
 // 4*(row%4)) so both access patterns spread over all banks.  Causal tiles past
 // the diagonal are never visited; only the diagonal tile is masked.
 // ---------------------------------------------------------------------------
-typedef __attribute__((ext_vector_type(4))) short v4s;
-typedef __attribute__((ext_vector_type(2))) float v2f;
-typedef __attribute__((ext_vector_type(2))) __bf16 v2bf16;
-typedef __attribute__((ext_vector_type(2))) _Float16 v2f16;
-
 #ifndef MVLLM_PF_XCD_CHUNK
 #define MVLLM_PF_XCD_CHUNK 32
 #endif
@@ -161,64 +155,15 @@ constexpr unsigned kXcdChunk = MVLLM_PF_XCD_CHUNK;   // consecutive work items h
 #ifndef MVLLM_PF_INT8_TILED
 #define MVLLM_PF_INT8_TILED 1         // 0: INT8 caches always on the 16-row tile kernel
 #endif
+#ifndef MVLLM_PF_PINGPONG
+#define MVLLM_PF_PINGPONG 1             // 0: every batch on prefill_mfma_kernel
+#endif
 #ifndef MVLLM_PF_WAVES
 #define MVLLM_PF_WAVES 4
 #endif
 constexpr int kPfWaves = MVLLM_PF_WAVES;             // waves per workgroup: 4, so that two workgroups share a CU
 constexpr int kBN = 64;                 // K/V rows per LDS tile
 constexpr int kWaveRows = 32;           // query rows per wave
-
-// v_max3_f32 without the canonicalising self-max the compiler puts in front of every fmaxf operand that
-// comes out of an MFMA (scores are finite or -inf here, never NaN).  The compiler does not know what the asm
-// reads, so it does not space it from an MFMA that writes an operand: the caller has to order it after an
-// ordinary instruction that reads the newest MFMA result.
-__device__ __forceinline__ float max3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
-
-// max(x[l], x[l ^ 32]) in every lane l, by v_permlane32_swap.
-__device__ __forceinline__ float max_with_lane_xor32(float x) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  // r[0] = (x[0..31], x[0..31]), r[1] = (x[32..63], x[32..63]): their maximum is max(x[l], x[l ^ 32]) in every lane
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-
-// Compile-time loop: f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{}).
-template <typename F, int... Is>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
-  (f(std::integral_constant<int, Is>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
-template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
-template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
-  v2f x = {a, b};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, v2bf16));
-}
-template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
-  v2f x = {a, b};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, v2f16));
-}
-
-// (lo, hi) of a packed 16-bit pair, each multiplied by c and rounded back to the element type.
-template <typename T> __device__ __forceinline__ uint32_t scale_pair(uint32_t w, float c) {
-  return pack2<T>(lo_to_float<T>(w) * c, hi_to_float<T>(w) * c);
-}
-// acc + lo + hi of a packed 16-bit pair in one instruction (v_dot2_f32_bf16 / v_dot2_f32_f16 against (1, 1)).
-template <typename T> __device__ __forceinline__ float add_pair(uint32_t w, float acc);
-template <> __device__ __forceinline__ float add_pair<bf16_t>(uint32_t w, float acc) {
-  const v2bf16 ones = {(__bf16)1.0f, (__bf16)1.0f};
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf16, w), ones, acc, false);
-}
-template <> __device__ __forceinline__ float add_pair<f16_t>(uint32_t w, float acc) {
-  const v2f16 ones = {(_Float16)1.0f, (_Float16)1.0f};
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2f16, w), ones, acc, false);
-}
 
 // Eight int8 codes (two dwords, biased by +128 so that the unsigned byte conversions apply) times one scale, rounded
 // once to the element type: fma(u, scale, -128 scale) is the exactly rounded (u - 128) * scale = code * scale.
@@ -230,34 +175,6 @@ template <typename T> __device__ __forceinline__ uint4 dequant8_biased(uint32_t 
   r.z = pack2<T>(fmaf((float)(u1 & 0xffu), scale, bias), fmaf((float)((u1 >> 8) & 0xffu), scale, bias));
   r.w = pack2<T>(fmaf((float)((u1 >> 16) & 0xffu), scale, bias), fmaf((float)(u1 >> 24), scale, bias));
   return r;
-}
-
-// 16 bytes per lane from a buffer resource (wave-uniform descriptor + per-lane 32-bit byte offset) straight
-// into LDS at lds_base + 16 * lane (buffer_load_dwordx4 ... lds).  Lanes whose offset is at or past the
-// descriptor's size read nothing and get zeros written, so tiles that run past the end of the tensor need no
-// clamping.  Written as inline asm on purpose: the compiler then neither tracks the transfer in vmcnt nor
-// inserts a full vmcnt(0) wait before the next LDS read, so the copy of tile j+1 really overlaps the math on
-// tile j; completion is awaited explicitly with dma_wait_all() before the barrier.  No "memory" clobber: the
-// destination buffer is not touched by ordinary code until after that wait and barrier (which do clobber), and
-// a clobber here would pin every LDS read of the tile in flight to its side of the copy.
-typedef __attribute__((ext_vector_type(4))) int v4i;
-template <int LDS_IMM>   // LDS destination = lds_base + LDS_IMM: one scalar register serves all copies of a wave
-__device__ __forceinline__ void dma16_to_lds(v4i rsrc, uint32_t lane_off, uint32_t lds_base) {
-  asm volatile("s_add_u32 m0, %0, %3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(lane_off), "s"(rsrc), "n"(LDS_IMM) : "scc", "m0");
-}
-// Raw buffer descriptor: 48-bit base, stride 0, size in bytes, 32-bit untyped data.
-__device__ __forceinline__ v4i make_rsrc(const char* base, uint32_t bytes) {
-  const uint64_t b = (uint64_t)base;
-  v4i r;
-  r[0] = (int)(uint32_t)b;
-  r[1] = (int)((uint32_t)(b >> 32) & 0xffffu);
-  r[2] = (int)bytes;
-  r[3] = 0x00020000;
-  return r;
-}
-__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ uint32_t lds_address(const void* p) {
-  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
 
 // Work item -> (head slice, sequence, first row) for batches of at most 64 sequences, heaviest items first.
@@ -925,6 +842,13 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   const bool aligned = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out);
   const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, 0, dtype, false, false) : 0;
   const bool mfma_ok = kind == 2;
+  if (MVLLM_PF_PINGPONG && mfma_ok && scale > 0.f && prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype)) {
+    PrefillPpArgs p;
+    p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
+    p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
+    p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0;
+    return launch_prefill_pp(p, dtype, (hipStream_t)stream);
+  }
   // fp32, and 16-bit head dims 32, 80, 96, 112 and 256: 16-row tiles on the decode kernel's tile arithmetic (paged_decode.hip)
   if (kind == 1) {
     PrefillRowsArgs r;

@@ -65,8 +65,9 @@ def test_paged_prefill_vs_oracle(dtype, hq, hkv, d, bs, lengths, cached):
 
 
 def test_paged_prefill_without_prefix_matches_plain_prefill_bitwise():
-    """No cached prefix: same tiles, same arithmetic as the packed kernel, only the copies' source differs."""
-    hq, hkv, d, bs = 32, 8, 128, 16
+    """No cached prefix: same tiles, same arithmetic as the packed kernel, only the copies' source differs.  (Two query
+    heads per kv head: both calls run on prefill_mfma_kernel.)"""
+    hq, hkv, d, bs = 16, 8, 128, 16
     lengths = [257, 64, 31, 400]
     c = make_paged_prefill_case(62, lengths, [0] * 4, hq, hkv, d, bs, dtype=torch.bfloat16)
     scale = 1 / math.sqrt(d)
@@ -74,6 +75,21 @@ def test_paged_prefill_without_prefix_matches_plain_prefill_bitwise():
     plain = flash_attention_prefill(c["q"].to(DEV), c["k"].to(DEV), c["v"].to(DEV), c["cu_k"].to(DEV), scale,
                                     hq, hkv, d).cpu()
     assert torch.equal(got, plain)
+
+
+def test_paged_prefill_without_prefix_close_to_two_group_prefill():
+    """Four query heads per kv head: the packed call runs on the two-group kernel, which sums a row's weights before
+    they are rounded to 16 bits; the two results agree to the last bits of the 16-bit outputs."""
+    hq, hkv, d, bs = 32, 8, 128, 16
+    lengths = [257, 64, 31, 400]
+    c = make_paged_prefill_case(62, lengths, [0] * 4, hq, hkv, d, bs, dtype=torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    got = _run(c, scale, hq, hkv, d, bs).float()
+    plain = flash_attention_prefill(c["q"].to(DEV), c["k"].to(DEV), c["v"].to(DEV), c["cu_k"].to(DEV), scale,
+                                    hq, hkv, d).cpu().float()
+    err = (got - plain).abs()
+    assert (err <= plain.abs() * 2.0 ** -6 + 1e-3).all()      # two bf16 steps of the value
+    assert err.mean() <= 2e-4
 
 
 def test_paged_prefill_single_new_token_matches_decode():
