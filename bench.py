@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--block-size", type=int, default=16, help="block size of the headline decode workload")
-    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,prefill_long,store,int8,reference_shapes,decode_small,demo_shape,head_dims,fused_qk,sampler,mfma_probe,loads_probe,engine,engine16,engine64,cpu to restrict the extras (the headline decode always runs)")
+    ap.add_argument("--only", default="", help="comma list out of decode256,prefill,prefill_long,store,int8,reference_shapes,decode_small,demo_shape,head_dims,fused_qk,sampler,mfma_probe,prefill_timeline,loads_probe,engine,engine16,engine64,cpu to restrict the extras (the headline decode always runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three 1 GiB device copies (reads 1 GiB, writes 1 GiB each) so a rocprofv3 "
@@ -273,7 +273,7 @@ def bench_prefill_store(args, which, want_cpu=False):
             "steps": args.steps, "warmup": f"{args.warmup} launches, then at least {EXTRA_WARM_MS:.0f} ms of launches",
             "tflops": flops / (event_ms * 1e-3) / 1e12,
             "frac_of_bf16_mfma_peak": flops / (event_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-            "roofline": roofline("mfma", flops / (event_ms * 1e-3) / 1e12, "prefill_mfma_kernel (one launch = the whole ragged batch)"),
+            "roofline": roofline("mfma", flops / (event_ms * 1e-3) / 1e12, "prefill_pp_kernel (one launch = the whole ragged batch)"),
         }
         if want_cpu:
             out["prefill"]["cpu_baseline"] = cpu_prefill_baseline(q, k, v, cu, lengths, scale, hq, hkv, d, flops,
@@ -292,7 +292,7 @@ def bench_prefill_store(args, which, want_cpu=False):
             "workload": "varlen causal prefill, 4 prompts of 8192 tokens, Hq32 Hkv8 D128 bf16",
             "tokens": sum(long_lengths), "algorithmic_flops": flops_l, "event_ms_per_step": event_ms_l,
             "tflops": flops_l / (event_ms_l * 1e-3) / 1e12,
-            "roofline": roofline("mfma", flops_l / (event_ms_l * 1e-3) / 1e12, "prefill_mfma_kernel"),
+            "roofline": roofline("mfma", flops_l / (event_ms_l * 1e-3) / 1e12, "prefill_pp_kernel"),
         }
         del ql, kl, vl
     if "prefill" in which:
@@ -756,6 +756,56 @@ def bench_mfma_probe(args):
     return res
 
 
+def bench_prefill_timeline(args):
+    """Where a workgroup of the two-group prefill kernel spends a tile: the probe library's timing build logs the
+    shader clock at the four corners of every tile (softmax begins / done, matrix part begins / done) for the waves of
+    one workgroup.  A stamp costs about 100 clocks, so every logged interval is that much longer than in the product
+    build; the shares are what the figures are for."""
+    import ctypes
+    import statistics
+    import torch
+    lib = ctypes.CDLL(os.path.join(ROOT, "minivllm_amd", "libmvllm_probe.so"))
+    fn = lib.mvllm_probe_prefill_timeline
+    c = ctypes
+    fn.restype = c.c_int
+    fn.argtypes = [c.c_void_p] * 5 + [c.c_int, c.c_int64, c.c_int, c.c_int, c.c_int, c.c_float, c.c_int, c.c_void_p, c.c_int,
+                   c.c_int, c.c_void_p]
+    from minivllm_amd import _C
+    dev = "cuda:0"
+    hq, hkv, d = 32, 8, 128
+    g = torch.Generator().manual_seed(args.seed)
+    cfg2 = torch.randint(64, 2049, (16,), generator=g).tolist()
+    out = {}
+    for name, lengths in (("config2", cfg2), ("4x8192", [8192] * 4)):
+        dg = torch.Generator(device=dev).manual_seed(args.seed + 1)
+        total = sum(lengths)
+        q, k, v = (torch.randn(total, h, d, generator=dg, device=dev).to(torch.bfloat16) for h in (hq, hkv, hkv))
+        cu = torch.tensor([0] + lengths, dtype=torch.int32).cumsum(0).to(torch.int32).to(dev)
+        o = torch.empty_like(q)
+        entries = 2048
+        log = torch.zeros(8, entries, dtype=torch.int64, device=dev)
+        for _ in range(3):                                   # the last launch's stamps are read (clock settled)
+            log.zero_()
+            st = fn(o.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), cu.data_ptr(), len(lengths), total, hq, hkv, d,
+                    1.0 / math.sqrt(d), _C.dtype_code(q.dtype), log.data_ptr(), entries, 9,
+                    torch.cuda.current_stream().cuda_stream)
+            assert st == 0, st
+        torch.cuda.synchronize()
+        rows = log.cpu().tolist()
+        res = {"workgroup": 9, "note": "clocks; stamps at softmax begin, softmax done, matrix part begin, matrix part done"}
+        for grp, wave in (("group0_wave0", 0), ("group1_wave4", 4)):
+            t = [x for x in rows[wave] if x > 0]
+            tiles = (len(t) - 1) // 4
+            seg = [[t[4 * i + j + 1] - t[4 * i + j] for i in range(tiles)] for j in range(4)]
+            per_tile = [t[4 * i + 4] - t[4 * i] for i in range(tiles)]
+            med = lambda xs: int(statistics.median(xs)) if xs else None
+            res[grp] = {"tiles_logged": tiles, "softmax": med(seg[0]), "wait_for_matrix_part": med(seg[1]),
+                        "matrix_part": med(seg[2]), "wait_for_softmax": med(seg[3]), "tile": med(per_tile),
+                        "life": t[-1] - t[0] if t else None}
+        out[name] = res
+    return out
+
+
 def bench_engine(args, max_num_sequences, graph):
     """BASELINE.json config 5: random-init Qwen3-style decoder (hidden 1024, 8 layers, Hq16/Hkv8/D128, FFN 3072,
     vocab 151936, bf16), 60 prompts of random ids with lengths U[32,96], 256 new tokens each, T 0.6."""
@@ -790,6 +840,43 @@ def bench_engine(args, max_num_sequences, graph):
         "output_tokens": new_tokens, "wall_s": wall, "tok_per_s": new_tokens / wall,
         "steps": engine.stats["steps"], "decode_s": engine.stats["decode_s"], "prefill_s": engine.stats["prefill_s"],
     }
+
+
+def summary_of(line):
+    """The figures of every quantity the metric names, in a few hundred characters, for the end of the JSON line."""
+    ex = line["extra"]
+    r3 = lambda x: None if x is None else round(x, 3)
+    out = {"decode_frac_hbm": r3(line["roofline"]["frac"]), "decode_gbs": round(line["roofline"]["achieved"])}
+    def put(key, leg, *path):
+        node = ex.get(leg)
+        for p_ in path:
+            node = node.get(p_) if isinstance(node, dict) else None
+        if node is not None:
+            out[key] = r3(node) if isinstance(node, float) else node
+    b256 = ex.get("decode_block256")
+    if isinstance(b256, dict) and "gbs_event" in b256:
+        out["decode_bs256_frac_hbm"] = r3(b256["gbs_event"] / HBM_PEAK_GBS)
+    put("prefill_frac_mfma", "prefill", "roofline", "frac")
+    put("prefill_tflops", "prefill", "tflops")
+    put("prefill_us", "prefill", "event_ms_per_step")
+    put("prefill_vs_oracle_max_abs", "prefill", "cpu_baseline", "gpu_vs_oracle_max_abs")
+    put("prefill_4x8192_frac", "prefill_long_prompts", "roofline", "frac")
+    put("prefill_paged_frac", "prefill_cached_prefix", "roofline", "frac")
+    put("prefill_paged_int8_frac", "prefill_cached_prefix_int8", "roofline", "frac")
+    put("store_frac_hbm", "store", "roofline", "frac")
+    put("int8_decode_frac_hbm", "int8", "roofline", "frac")
+    put("int8_store_frac_hbm", "int8", "store_roofline", "frac")
+    put("int8_decode_vs_oracle_max_abs", "int8", "gpu_vs_oracle_max_abs")
+    for key, leg in (("engine16_eager_tok_s", "engine_16seq_eager"), ("engine16_tok_s", "engine_16seq_graph"), ("engine64_tok_s", "engine_64seq_graph")):
+        node = ex.get(leg)
+        if isinstance(node, dict):
+            for name in ("out_tok_per_s", "tok_per_s", "output_tokens_per_s"):
+                if name in node:
+                    out[key] = round(node[name])
+                    break
+    if "prefill_us" in out:
+        out["prefill_us"] = round(out["prefill_us"] * 1e3, 1)
+    return out
 
 
 def main():
@@ -839,6 +926,8 @@ def main():
         extra["sampler"] = bench_sampler(args)
     if want("mfma_probe"):
         extra["mfma_probe"] = bench_mfma_probe(args)
+    if want("prefill_timeline"):
+        extra["prefill_timeline"] = bench_prefill_timeline(args)
     if want("engine"):
         extra["engine_16seq_eager"] = bench_engine(args, 16, False)
         extra["engine_16seq_graph"] = bench_engine(args, 16, True)
@@ -879,6 +968,7 @@ def main():
         "cpu_baseline": cpu,
         "extra": extra,
     }
+    line["summary"] = summary_of(line)     # last on purpose: a record that keeps only the end of the line keeps this
     print(json.dumps(line))
 
 

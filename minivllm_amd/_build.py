@@ -59,8 +59,11 @@ def build_library(verbose: bool = True, jobs: int = 4) -> str:
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         # the probe library also holds the decode kernels built as "loads only" (the access pattern's ceiling)
         probe_decode = pool.submit(compile_one, "paged_decode.hip", ("-DMVLLM_DECODE_LOADS_ONLY=1",), "_loads_only")
+        # ... and the two-group prefill kernel with its per-tile clock stamps
+        probe_prefill = pool.submit(compile_one, "prefill_pingpong.hip", ("-DMVLLM_PP_TIMELINE=1",), "_timeline")
         objs = list(pool.map(compile_one, SOURCES + PROBE_SOURCES))
         objs.append(probe_decode.result())
+        objs.append(probe_prefill.result())
     for lib, members in ((LIB_PATH, objs[:len(SOURCES)]), (PROBE_LIB_PATH, objs[len(SOURCES):])):
         cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *members]
         if verbose:

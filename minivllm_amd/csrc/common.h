@@ -228,6 +228,10 @@ struct PrefillPpArgs {
   int n_teams;      // gcd(8, slices): workgroup teams, each with its own item list
   int team_size;    // workgroups per team
   int level_bits;   // bits that hold the block count of the longest possible sequence
+  // timing build only (the probe library): where workgroup `timeline_block` logs its clock stamps; null otherwise
+  unsigned long long* timeline;
+  int timeline_entries;
+  int timeline_block;
 };
 bool prefill_pp_takes(int num_seqs, int num_heads, int num_kv_heads, int head_dim, int dtype);
 int launch_prefill_pp(const PrefillPpArgs& a, int dtype, hipStream_t stream);

@@ -32,6 +32,9 @@ namespace {
 constexpr int kPpBN = 64;          // keys per tile
 constexpr int kPpRing = 3;         // K and V tiles in flight
 constexpr int kPpWaves = 8;
+#ifndef MVLLM_PP_TIMELINE
+#define MVLLM_PP_TIMELINE 0            // 1: the timing build of the probe library (per-tile clock stamps)
+#endif
 #ifndef MVLLM_PP_PRIO
 #define MVLLM_PP_PRIO 3
 #endif
@@ -91,6 +94,17 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   const int hi = lane >> 5;
   const int wq = wave & 3;                     // query head inside the slice
 
+#if MVLLM_PP_TIMELINE
+  // Timing build (the probe library): the waves of one workgroup log the shader clock at the four corners of every
+  // tile (softmax begins, softmax done, matrix part begins, matrix part done), `timeline_entries` stamps per wave.
+  // A stamp costs about a hundred clocks, so the logged intervals are each that much longer than in the product build.
+  unsigned long long* tlog = a.timeline + (size_t)wave * a.timeline_entries;
+  int tn = 0;
+  const bool tlogging = a.timeline != nullptr && (int)blockIdx.x == a.timeline_block;
+#define TSTAMP() do { if (tlogging && tn < a.timeline_entries) { const unsigned long long t_ = __builtin_amdgcn_s_memtime(); if (lane == 0) tlog[tn] = t_; ++tn; } } while (0)
+#else
+#define TSTAMP() do {} while (0)
+#endif
   // ---- the batch, one sequence per lane ----
   int lo = 0, len = 0;
   if (lane < a.num_seqs) {
@@ -275,21 +289,12 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // V^T: the transposing reads of the 16 keys of `step` ( = 2 tk + st) of the tile in V ring slot `slot`.
   auto k_frags = [&](int slot, auto KS, uint4 (&kf)[2]) {
     constexpr int ks = decltype(KS)::value;
-#ifdef PP_EXP_NOLDS
-    kf[0] = qf[ks]; kf[1] = qf[(ks + 1) & 7]; (void)slot;
-    return;
-#endif
     const char* kb = &lds.k[0][0] + slot * kTileBytes + k_off[ks];
     kf[0] = *reinterpret_cast<const uint4*>(kb);
     kf[1] = *reinterpret_cast<const uint4*>(kb + 32 * kRowB);
   };
   auto v_frags = [&](int slot, auto STEP, uint4 (&af)[kTD]) {
     constexpr int step = decltype(STEP)::value;
-#ifdef PP_EXP_NOLDS
-    for (int td = 0; td < kTD; ++td) af[td] = qf[(td + step) & 7];
-    (void)slot;
-    return;
-#endif
     const char* vb = &lds.v[0][0] + slot * kTileBytes + 16 * step * kRowB;
 #pragma unroll
     for (int td = 0; td < kTD; ++td) {
@@ -366,14 +371,6 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   bool have_prev = false;
   float l_prev = 0.f;
 
-#ifdef PP_TIMING
-  unsigned long long* tlog = reinterpret_cast<unsigned long long*>(reinterpret_cast<T*>(a.out) + a.total_tokens * a.num_heads * D) + (GRP ? 2048 : 0) + 512 * (wave & 3);
-  int tn = 0;
-  const bool tlogging = blockIdx.x == PP_TIMING;
-#define TSTAMP() do { if (tlogging && tn < 500) { const unsigned long long t_ = __builtin_amdgcn_s_memtime(); if (lane == 0) tlog[tn] = t_; ++tn; } } while (0)
-#else
-#define TSTAMP() do {} while (0)
-#endif
   if (GRP == 1) pp_barrier();                   // group 1 runs one interval behind
   first_scores(c_slot);
   asm volatile("" : "+v"(s[0]), "+v"(s[1]));
@@ -407,10 +404,6 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // unbiased and average out over a row).  SHIFT: d != 0.
   auto weights = [&](auto SHIFT, float d) {
     float sum = 0.f;
-#ifdef PP_EXP_NOSM
-    for (int i = 0; i < 4; ++i) { pf[i].x = __float_as_uint(s[i >> 1][8 * (i & 1)]); pf[i].y = __float_as_uint(s[i >> 1][8 * (i & 1) + 1]); pf[i].z = pf[i].x; pf[i].w = pf[i].y; }
-    return 1.f + d;
-#endif
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk)
 #pragma unroll
@@ -419,11 +412,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const float x = s[tk][8 * st + i];
-#ifdef PP_EXP_NOEXP
-          e[i] = decltype(SHIFT)::value ? x - d : x;
-#else
           e[i] = fast_exp2(decltype(SHIFT)::value ? x - d : x);
-#endif
         }
         uint4 p;
         p.x = pack2<T>(e[0], e[1]);
@@ -449,7 +438,19 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // uses it, because nothing else runs on this SIMD's matrix unit meanwhile that could cover an LDS round trip.
   // vf0, vf1: the V^T fragments of the tile's first two steps, requested before the barrier.  Group 0 also issues
   // its share of the next copy step here, one instruction per stage.  Returns false when the stream ends here.
-  auto stage_end = [&]() { __builtin_amdgcn_sched_barrier(0); };
+  // A wave issues about one instruction in five clocks, an MFMA keeps the matrix unit for 32: at most five other
+  // instructions fit between two MFMAs without a bubble, so each stage's fragment reads and their address
+  // arithmetic are dealt out between its four MFMAs instead of standing in front of them.
+  auto stage_end = [&](int reads_per_mfma) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // one MFMA
+      if (reads_per_mfma == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // LDS reads
+      else if (reads_per_mfma == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (reads_per_mfma > 0) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);    // one vector instruction (an address)
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
   // The compiler computes a value where it is first used, and moves pure arithmetic across a barrier freely.  These
   // empty statements make the softmax's results exist before the barrier that ends its interval, and the matrix
   // interval's before the one that ends it, so that each interval holds the work it is named for.
@@ -475,13 +476,6 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     uint4 kf0[2], kf1[2], kf2[2], kf3[2], kf4[2], kf5[2], kf6[2], kf7[2];
     // stage A
     v_frags(c_slot, I2{}, vf2);
-    if (last && nxt.valid) {
-      // the next item's Q rows, copied since this item's first softmax interval; one copy step was issued behind
-      // them unless the item has a single tile
-      if (cur.rb > 0) vm_wait<4>();
-      else vm_wait<0>();
-      load_q();
-    }
     if constexpr (decltype(FRESH)::value) {
       v16f z;
 #pragma unroll
@@ -492,22 +486,29 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 #pragma unroll
       for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf0[td], pf[0], o[td]);
     }
-    stage_end();
+    stage_end(2);
     // stage B
     v_frags(c_slot, I3{}, vf3);
 #pragma unroll
     for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf1[td], pf[1], o[td]);
-    stage_end();
+    stage_end(2);
     // stage C
-    if (more) { k_frags(n_slot, I0{}, kf0); k_frags(n_slot, I1{}, kf1); }
+    k_frags(n_slot, I0{}, kf0); k_frags(n_slot, I1{}, kf1);      // (read and not used when the stream ends here)
 #pragma unroll
     for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf2[td], pf[2], o[td]);
-    stage_end();
+    stage_end(1);
     // stage D
-    if (more) { k_frags(n_slot, I2{}, kf2); k_frags(n_slot, I3{}, kf3); }
+    k_frags(n_slot, I2{}, kf2); k_frags(n_slot, I3{}, kf3);
 #pragma unroll
     for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf3[td], pf[3], o[td]);
-    stage_end();
+    stage_end(1);
+    if (last && nxt.valid) {
+      // the next item's Q rows, copied since this item's first softmax interval; one copy step was issued behind
+      // them unless the item has a single tile
+      if (cur.rb > 0) vm_wait<4>();
+      else vm_wait<0>();
+      load_q();
+    }
     if (more) {
       // stage E
       k_frags(n_slot, I4{}, kf4); k_frags(n_slot, I5{}, kf5);
@@ -524,26 +525,26 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       }
 #pragma unroll
       for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf1[tk], qf[1], s[tk]);
-      stage_end();
+      stage_end(1);
       // stage F
       k_frags(n_slot, I6{}, kf6); k_frags(n_slot, I7{}, kf7);
 #pragma unroll
       for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf2[tk], qf[2], s[tk]);
 #pragma unroll
       for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf3[tk], qf[3], s[tk]);
-      stage_end();
+      stage_end(1);
       // stage G
 #pragma unroll
       for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf4[tk], qf[4], s[tk]);
 #pragma unroll
       for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf5[tk], qf[5], s[tk]);
-      stage_end();
+      stage_end(0);
       // stage H
 #pragma unroll
       for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf6[tk], qf[6], s[tk]);
 #pragma unroll
       for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf7[tk], qf[7], s[tk]);
-      stage_end();
+      stage_end(0);
     }
     pin_products();
     __builtin_amdgcn_s_setprio(0);
@@ -572,9 +573,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       copy_q(nxt);
       later += 8;
     }
-    TSTAMP();
     l = weights(std::true_type{}, mx_first);
-    TSTAMP();
     set_neg_m(-mx_first);
     uint4 vf0[kTD], vf1[kTD];
     pin_weights();
@@ -595,10 +594,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       // date: the weights are computed first, and only when a lane's share of the tile's row sum passes 2^12 (a
       // weight above 2^7 at least; 16-bit weights and fp32 sums are far from their limits there) is the tile redone
       // the long way: true maximum, accumulators and row sum scaled down, weights again from the kept scores.
-      TSTAMP();
       float sum = weights(std::false_type{}, 0.f);
-      asm volatile("" : "+v"(sum));
-      TSTAMP();
       if (__any(!(sum <= 4096.f))) {
         const float mx = tile_max();
         const float d = mx > 8.f ? mx : 0.f;       // per row (both lanes of a row see the same maximum)
@@ -673,3 +669,24 @@ int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) 
 }
 
 }  // namespace mvllm
+
+#if MVLLM_PP_TIMELINE
+// Probe library only: the two-group prefill with the clock stamps of workgroup `block` written to `log`
+// ([8 waves][entries_per_wave] 64-bit shader clocks; entries past a wave's last stamp stay as the caller filled them).
+extern "C" int mvllm_probe_prefill_timeline(void* out, const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
+                                            int num_seqs, int64_t total_tokens, int num_heads, int num_kv_heads, int head_dim,
+                                            float scale, int dtype, unsigned long long* log, int entries_per_wave, int block,
+                                            void* stream) {
+  using namespace mvllm;
+  if (!out || !q || !k || !v || !cu_seqlens || !log || entries_per_wave <= 0) return MVLLM_ERR_NULL_POINTER;
+  if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || !(scale > 0.f) ||
+      !prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype))
+    return MVLLM_ERR_UNSUPPORTED;
+  PrefillPpArgs p;
+  p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
+  p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
+  p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0;
+  p.timeline = log; p.timeline_entries = entries_per_wave; p.timeline_block = block;
+  return launch_prefill_pp(p, dtype, (hipStream_t)stream);
+}
+#endif
