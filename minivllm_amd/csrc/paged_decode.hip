@@ -1712,15 +1712,28 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 constexpr int kMaxDevices = 64;
 static std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
-// Device address of `scratch` on the current device; null (and *status set) when the lookup fails.
-static void* static_scratch(int* status) {
-  int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
+// Device address of `scratch` on the device that owns `stream` (the current device for the null stream): every GPU
+// holds its own copy of the array at its own address, and the kernels run where the stream lives, which need not be
+// the caller's current device.  Looked up once per device, with that device current for the lookup; null (and
+// *status set) when it fails.
+static void* static_scratch(hipStream_t stream, int* status) {
+  int cur = -1;
+  hipError_t e = hipGetDevice(&cur);
   if (e != hipSuccess) { *status = (int)e; return nullptr; }
+  int dev = cur;
+  if (stream != nullptr) {
+    e = hipStreamGetDevice(stream, &dev);
+    if (e != hipSuccess) { *status = (int)e; return nullptr; }
+  }
   if (dev < 0 || dev >= kMaxDevices) { *status = MVLLM_ERR_UNSUPPORTED; return nullptr; }
   void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
   if (p) return p;
+  if (dev != cur && (e = hipSetDevice(dev)) != hipSuccess) { *status = (int)e; return nullptr; }
   e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (dev != cur) {
+    const hipError_t back = hipSetDevice(cur);
+    if (e == hipSuccess) e = back;
+  }
   if (e != hipSuccess || !p) { *status = e != hipSuccess ? (int)e : MVLLM_ERR_WORKSPACE; return nullptr; }
   g_scratch_ptr[dev].store(p, std::memory_order_release);   // two threads racing here store the same address
   return p;
@@ -1736,7 +1749,7 @@ extern "C" int mvllm_paged_decode_noalloc(void* out, const void* q, const void* 
   if (status != MVLLM_OK || batch == 0) return status;
   const size_t need = workspace_bytes_for(batch, num_heads, head_dim, max_num_blocks, block_size);
   if (need > kStaticScratchBytes) return MVLLM_ERR_WORKSPACE;
-  void* ws = static_scratch(&status);
+  void* ws = static_scratch((hipStream_t)stream, &status);
   if (!ws) return status;
   // Every partial a merge reads has been written by a workgroup of the same call (a sequence's live partitions
   // all run), so nothing in the array has to start at zero.

@@ -136,16 +136,27 @@ class BlockManager:
         table = seq.block_table
         block = self.blocks[table[index]]
         token_ids = seq.block(index)
-        prefix = self.blocks[table[index - 1]].hash if index > 0 else -1
+        prefix = -1
+        if index > 0:
+            prefix = self.blocks[table[index - 1]].hash
+            if prefix == -1:
+                # the block before it was never hashed: chaining from -1 would give this block the hash of a first
+                # block and let it be shared behind another prefix; it stays unshared instead
+                return
         h = self.compute_hash(token_ids, prefix)
         block.update(h, token_ids)
         self.hash_to_block_id[h] = block.block_id
 
     def hash_deferred_blocks(self) -> None:
         """Hashes postponed by ``append``; a sequence that was finished or preempted in between has given its
-        blocks back and is skipped (its blocks simply stay unshared)."""
+        blocks back and is skipped (its blocks simply stay unshared).  An entry whose block still holds a
+        placeholder id stays on the list for the next call."""
+        keep = []
         for seq, index in self.deferred:
-            if index < len(seq.block_table) and self.blocks[seq.block_table[index]].hash == -1 \
-                    and all(t >= 0 for t in seq.block(index)):
+            if index >= len(seq.block_table) or self.blocks[seq.block_table[index]].hash != -1:
+                continue
+            if all(t >= 0 for t in seq.block(index)):
                 self._hash_block(seq, index)
-        self.deferred = []
+            else:
+                keep.append((seq, index))
+        self.deferred = keep

@@ -32,19 +32,33 @@ _DTYPES = {"bf16": torch.bfloat16, "bfloat16": torch.bfloat16, "fp16": torch.flo
 
 class PendingTokens:
     """Token ids of a launched decode step on their way to the host: the step's last kernel writes them into a
-    row of pinned memory and then the step's sequence number into the row's last entry."""
+    row of pinned memory and then the step's sequence number into the row's last entry.
 
-    def __init__(self, row, count: int, sequence: int):
+    The row is polled while the kernel may still be running, which is only meaningful for coherent (fine-grained)
+    pinned host memory, what torch's pinned allocations are on ROCm unless the process runs with
+    HIP_HOST_COHERENT=0.  With non-coherent pinned memory a write becomes visible at a synchronisation point only,
+    so the poll gives up after a few milliseconds and synchronises the launch stream: slower, never wrong."""
+
+    SPIN_SECONDS = 2e-3          # a decode step takes tens of microseconds; past this the host stops burning a core
+
+    def __init__(self, row, count: int, sequence: int, stream=None):
         self.row, self.count, self.sequence = row, count, sequence     # row: numpy view of the pinned row
+        self.stream = stream
 
     def wait(self) -> list[int]:
         row, want = self.row, self.sequence
-        deadline = None
-        while int(row[-1]) != want:
-            if deadline is None:
-                deadline = time.monotonic() + 60.0
-            elif time.monotonic() > deadline:
-                torch.cuda.synchronize()               # surfaces a device error instead of spinning for ever
+        if int(row[-1]) != want:
+            give_up = time.monotonic() + self.SPIN_SECONDS
+            polls = 0
+            while int(row[-1]) != want:
+                polls += 1
+                if polls & 0x3ff == 0:
+                    if time.monotonic() > give_up:
+                        break
+                    time.sleep(0)                          # let another thread of the process run
+            if int(row[-1]) != want:
+                # blocks without spinning, makes non-coherent pinned memory visible, surfaces a device error
+                (self.stream.synchronize() if self.stream is not None else torch.cuda.synchronize())
                 if int(row[-1]) != want:
                     raise RuntimeError("decode step finished without delivering its token ids")
         return row[:self.count].tolist()
@@ -132,14 +146,33 @@ class ModelRunner:
                     block_tables=None if tables is None else self._to_device(tables, torch.int32))
         return self._to_device(md["input_ids"], torch.int64), self._to_device(positions, torch.int64)
 
+    def decode_buckets(self):
+        """Batch sizes a decode step is captured at (model_runner.py:316-369 uses the same ladder)."""
+        max_bs = self.config.get("max_num_sequences", 16)
+        return sorted({b for b in [1, 2, 4, 8] + list(range(16, max_bs + 1, 16)) + [max_bs] if b <= max_bs})
+
     def prepare_decode(self, seqs):
         md = decode_metadata(seqs, self.block_size)
-        context_lens = self._to_device(md["context_lens"], torch.int64)
+        context_lens, slots, tables, ids = md["context_lens"], md["slot_mapping"], md["block_tables"], md["input_ids"]
+        if self.config.get("eager_decode_as_captured", False) and len(seqs) <= self.config.get("max_num_sequences", 16):
+            # The shapes a captured step has: the batch padded to its bucket with rows that store nothing and attend
+            # to nothing, the block tables as wide as the longest sequence the model allows.  Every kernel then runs
+            # on the plan (tiles, partitions) of the graph path, so an eager run reproduces a graph run bit for bit.
+            cfg = self.config
+            bucket = next(b for b in self.decode_buckets() if b >= len(seqs))
+            max_len = cfg.get("max_model_length", cfg.get("max_position", 4096))
+            width = -(-max_len // self.block_size)
+            pad = bucket - len(seqs)
+            tables = [list(t) + [0] * (width - len(t)) for t in tables] + [[0] * width] * pad
+            context_lens = list(context_lens) + [0] * pad
+            slots = list(slots) + [-1] * pad
+            ids = list(ids) + [0] * pad
+        context_lens = self._to_device(context_lens, torch.int64)
         set_context(False,
-                    slot_mapping=self._to_device(md["slot_mapping"], torch.int64),
+                    slot_mapping=self._to_device(slots, torch.int64),
                     context_lens=context_lens,
-                    block_tables=self._to_device(md["block_tables"], torch.int32))
-        return self._to_device(md["input_ids"], torch.int64), context_lens - 1
+                    block_tables=self._to_device(tables, torch.int32))
+        return self._to_device(ids, torch.int64), (context_lens - 1).clamp_(min=0)
 
     @torch.no_grad()
     def capture_decode_graphs(self):
@@ -161,7 +194,7 @@ class ModelRunner:
         max_len = cfg.get("max_model_length", cfg.get("max_position", 4096))
         max_blocks = -(-max_len // self.block_size)
         dev = self.device
-        buckets = sorted({b for b in [1, 2, 4, 8] + list(range(16, max_bs + 1, 16)) + [max_bs] if b <= max_bs})
+        buckets = self.decode_buckets()
         ws_bytes = max(sample_workspace_bytes(b, cfg["vocab_size"]) for b in buckets) if self.fused_sampler else 0
         lm_bytes = max(lm_head_sample_workspace_bytes(b, cfg["hidden_size"]) for b in buckets) if self.fused_lm_head else 0
         self.graph_vars = dict(
@@ -312,7 +345,7 @@ class ModelRunner:
         sampled = self._replay_decode(seqs)
         self._last_sampled = sampled
         # step t's row is read after step t + 1 has been launched (into the other row)
-        return PendingTokens(self._pinned_rows[calls & 1], len(seqs), calls + 1)
+        return PendingTokens(self._pinned_rows[calls & 1], len(seqs), calls + 1, torch.cuda.current_stream(self.device))
 
     @torch.inference_mode()
     def run(self, seqs, is_prefill: bool) -> list[int]:
@@ -327,10 +360,11 @@ class ModelRunner:
             temperatures = self._to_device([seq.temperature for seq in seqs], torch.float32)
         else:
             input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
-            temperatures = self._to_device([seq.temperature for seq in seqs], torch.float32)
+            rows_out = len(seqs) if is_prefill else input_ids.shape[0]     # decode: the padded batch, if padded
+            temperatures = self._to_device([seq.temperature for seq in seqs] + [1.0] * (rows_out - len(seqs)), torch.float32)
             hidden = self.model(input_ids, positions)
             if (self.fused_sampler and self.fused_lm_head
-                    and lm_head_sample_takes(hidden, self.model.lm_head_weight, len(seqs))):
+                    and lm_head_sample_takes(hidden, self.model.lm_head_weight, rows_out)):
                 # the rows to sample from are picked inside the kernel: the last token of every packed sequence in
                 # prefill (embedding_head.py:57-62), every row in decode
                 rows = (get_context().cu_seqlens_q[1:] - 1).long() if is_prefill else None
@@ -339,7 +373,7 @@ class ModelRunner:
                 self.sample_calls += 1
                 self._last_sampled = None
                 self._steady = None
-                token_ids = sampled.tolist()
+                token_ids = sampled.tolist()[:len(seqs)]
                 reset_context()
                 return token_ids
             logits = self.model.compute_logits(hidden)
@@ -351,6 +385,6 @@ class ModelRunner:
             sampled = self.sampler(logits, temperatures, self.generator)
         self._last_sampled = None
         self._steady = None
-        token_ids = sampled.tolist()
+        token_ids = sampled.tolist()[:len(seqs)]
         reset_context()
         return token_ids

@@ -461,10 +461,24 @@ class Attention(nn.Module):
             if q.dim() == 4:
                 # Batched mode (B, N, Hq, D): B sequences of N tokens each.  The reference dispatches to a function
                 # it never defines (attention.py:526-533); here the batch is the packed case with equal lengths.
-                if context.block_tables is not None:
-                    raise ValueError("batched 4-D prefill over a cached prefix is not provided; pack the new tokens")
                 bsz, n = q.shape[:2]
                 cu = torch.arange(bsz + 1, dtype=torch.int32, device=q.device) * n
+                if context.block_tables is not None:
+                    # ... over cached prefixes: every sequence brings N new tokens, its keys (prefix + new) are
+                    # counted by cu_seqlens_k and read from the paged cache, which the store above has completed
+                    if context.cu_seqlens_k is None or k_cache.numel() == 0:
+                        raise ValueError("cu_seqlens_k and the KV cache must be provided for prefill over a cached prefix")
+                    q_rows = q.reshape(bsz * n, self.num_heads, self.head_dim)
+                    if int8:
+                        o = flash_attention_prefill_paged_int8(q_rows, k_cache, v_cache, self.k_scale, self.v_scale,
+                                                               context.block_tables, cu, context.cu_seqlens_k, scale,
+                                                               self.num_heads, self.num_kv_heads, self.head_dim,
+                                                               self.block_size)
+                    else:
+                        o = flash_attention_prefill_paged(q_rows, k_cache, v_cache, context.block_tables, cu,
+                                                          context.cu_seqlens_k, scale, self.num_heads,
+                                                          self.num_kv_heads, self.head_dim, self.block_size)
+                    return o.reshape(bsz, n, self.num_heads * self.head_dim)
                 o = flash_attention_prefill(q.reshape(bsz * n, self.num_heads, self.head_dim),
                                             k.reshape(bsz * n, self.num_kv_heads, self.head_dim),
                                             v.reshape(bsz * n, self.num_kv_heads, self.head_dim), cu, scale,

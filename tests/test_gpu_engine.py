@@ -170,17 +170,16 @@ def test_config5_full_shape():
     """BASELINE.json config 5 at its own shape (llm_engine.py:71-88 driven as main.py:15-41 does): Qwen3-style
     decoder 8 x 1024, 16 query / 8 kv heads of 128 dims, vocabulary 151 936, blocks of 256 tokens, 60 prompts of
     32-96 random ids, 256 new tokens each at temperature 0.6.  Checked: the run completes with every id in range;
-    the hipGraph decode run and the eager run (same seed, so the same sampler noise) agree on at least 90 % of the
-    sequences' first 32 new tokens and on at least 20 % of the whole 256-token sequences (the eager run decodes 60
-    rows, the graph run its 64-row bucket: a 1-ulp GEMM difference flips a near-tie of the almost flat
-    distribution of a random-init model now and then, and one flip changes everything after it); and the paged cache that 60 decode steps leave behind equals the K/V of one varlen
-    prefill over the same tokens."""
+    the hipGraph decode run and an eager run on the captured shapes (the batch padded to its bucket, the block
+    tables at their static width: ``eager_decode_as_captured``; same seed, so the same sampler noise) produce the
+    same 60 x 256 ids, token for token; and the paged cache that 60 decode steps leave behind equals the K/V of one
+    varlen prefill over the same tokens."""
     vocab = CONFIG5["vocab_size"]
     prompts = _prompts(60, 32, 96, seed=50, vocab=vocab)
     sp = SamplingParams(temperature=0.6, max_tokens=256, ignore_eos=True)
     runs = {}
     for graph in (True, False):
-        eng = LLMEngine(dict(CONFIG5, max_num_sequences=64, enforce_eager=not graph))
+        eng = LLMEngine(dict(CONFIG5, max_num_sequences=64, enforce_eager=not graph, eager_decode_as_captured=True))
         out = eng.generate(prompts, sp)["token_ids"]
         assert [len(t) for t in out] == [256] * 60
         assert all(0 <= t < vocab for seq in out for t in seq)
@@ -188,9 +187,9 @@ def test_config5_full_shape():
         runs[graph] = out
         del eng
         torch.cuda.empty_cache()
-    head = sum(a[:32] == b[:32] for a, b in zip(runs[True], runs[False]))
     whole = sum(a == b for a, b in zip(runs[True], runs[False]))
-    assert head >= 54 and whole >= 12, (head, whole)          # measured: 60 and 20 of 60
+    first_diff = [next((i for i, (x, y) in enumerate(zip(a, b)) if x != y), None) for a, b in zip(runs[True], runs[False])]
+    assert whole == 60, (whole, first_diff)
 
     # the cache after 60 decode steps == one prefill of the same tokens, at this shape; prompts of 200-250 tokens,
     # so that sequences open their second 256-token block while decoding
@@ -221,8 +220,11 @@ def test_config5_full_shape():
     for s, old in zip(seqs, paged):
         new = flat()[:, :, rows_of(s)]
         assert (old[:, 0].float() - new[:, 0].float()).abs().max() <= 3.2e-2
+        # every layer: within the attention bound plus one bf16 step of the value (keys and values of magnitude 8
+        # to 16 are stored in steps of 0.0625; the decode steps ran other GEMM and attention kernels than the prefill)
         diff = (old.float() - new.float()).abs()
-        assert diff.max() <= 0.25 and diff.mean() <= 4e-3, (diff.max().item(), diff.mean().item())
+        assert (diff <= 2e-2 + new.float().abs() * 2.0 ** -7).all() and diff.mean() <= 2e-3, \
+            (diff.max().item(), diff.mean().item())
 
 
 def test_graph_decode_with_split_partitions_in_every_bucket():

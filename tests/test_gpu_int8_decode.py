@@ -34,6 +34,11 @@ def _quantised_case(seed, batch, ctx_lo, ctx_hi, hq, hkv, d, bs, dtype=torch.bfl
 
 
 def _check(case, hq, hkv, d, bs, scale, ctx_dtype=torch.int64):
+    """Max-abs 2e-2 / mean-abs 2e-3 against the fp32 oracle on the dequantised cache, with one allowance: the kernel's
+    output is 16 bits wide, and these small cases (a handful of keys, 1 % of them 8-sigma outliers) have outputs of
+    magnitude 4 to 10, where half a bf16 step alone (|want| * 2^-9) is 0.008 to 0.02.  One bf16 step of the value is
+    therefore taken off the difference before it is held against 2e-2.  The full-size configuration-4 test, whose
+    outputs average thousands of keys, uses the bound as stated."""
     q, ck, cv, sk, sv, tables, ctx = case
     got = paged_attention_decode_int8(q.to(DEV), ck, cv, sk, sv, tables.to(DEV), ctx.to(ctx_dtype).to(DEV), scale,
                                       hq, hkv, d, bs).cpu()
@@ -164,8 +169,7 @@ def test_config4_full_size_on_its_own_plan():
         want = oracle.decode_int8_oracle(q[b:b + 1].cpu().float(), ck[ids].cpu(), cv[ids].cpu(), sk[ids].cpu(),
                                          sv[ids].cpu(), table, ctx[b:b + 1], scale, hq, hkv, d, bs)
         mx, mean = error_stats(got[b:b + 1], want)
-        excess = ((got[b:b + 1].float() - want).abs() - want.abs() * 2.0 ** -8).max().item()
-        assert excess <= 2e-2 and mean <= 2e-3, (b, int(ctx[b]), mx, excess, mean)
+        assert mx <= 2e-2 and mean <= 2e-3, (b, int(ctx[b]), mx, mean)    # the stated bound, no allowance
     # size-independent property over the whole batch: the output is linear in the V scales
     sv *= 2
     got2 = paged_attention_decode_int8(q, ck, cv, sk, sv, td, cd, scale, hq, hkv, d, bs).cpu()

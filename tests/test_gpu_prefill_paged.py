@@ -193,3 +193,25 @@ def test_paged_prefill_over_an_int8_cache(dtype, hq, hkv, d, bs, lengths, cached
                                       torch.tensor(lengths, device=DEV), scale, hq, hkv, d, bs).cpu()
     mx, mean = error_stats(got[last], dec.float())
     assert mx <= 3e-2 and mean <= 3e-3, (mx, mean)
+
+
+def test_attention_module_batched_4d_prefill_over_cached_prefix():
+    """Batched mode of Attention.forward (attention.py:526-533: q (B, N, Hq, D)) with block tables in the context:
+    every sequence brings N new tokens after its own cached prefix; the rows are packed with equal cu_seqlens_q and
+    run on the paged prefill.  Output (B, N, Hq * D), against the paged-prefill oracle."""
+    from minivllm_amd.layers.attention import Attention
+    from minivllm_amd.utils import reset_context, set_context
+    hq, hkv, d, bs, n = 8, 2, 128, 16, 40
+    cached = [32, 0, 96]
+    kv_lengths = [c + n for c in cached]
+    c = make_paged_prefill_case(71, kv_lengths, cached, hq, hkv, d, bs, dtype=torch.bfloat16)
+    layer = Attention(hq, d, 1.0, hkv, bs)
+    layer.k_cache, layer.v_cache = c["k_cache"].to(DEV), c["v_cache"].to(DEV)
+    k_new, v_new = c["k"][c["new_rows"]].contiguous(), c["v"][c["new_rows"]].contiguous()
+    # slot_mapping None: the cache already holds the new tokens' keys (the helper stored every key)
+    set_context(True, None, c["cu_k"].to(DEV), n, max(kv_lengths), None, None, c["block_tables"].to(DEV))
+    out = layer(c["q_new"].view(3, n, hq, d).to(DEV), k_new.view(3, n, hkv, d).to(DEV), v_new.view(3, n, hkv, d).to(DEV))
+    reset_context()
+    assert out.shape == (3, n, hq * d)
+    want = _oracle32(c, 1 / math.sqrt(d), hq, hkv, d, bs)
+    _check(out.cpu().view(3 * n, hq, d), want, torch.bfloat16)

@@ -63,3 +63,43 @@ def test_noalloc_rejects_shapes_beyond_the_static_array():
     assert st == -5                                                # MVLLM_ERR_WORKSPACE, nothing launched
     with pytest.raises(ValueError):
         _C.check(st, "paged_decode_noalloc")
+
+
+def test_noalloc_allocates_nothing():
+    """Device memory in use is the same before and after a call (the partials live in the library's static array, not
+    in an allocation), and the call can be recorded into a graph, where an allocation would fail the capture; every
+    replay equals the eager result."""
+    hq, hkv, d, bs = 32, 8, 128, 16
+    scale = 1 / math.sqrt(d)
+    q, kc, vc, tables, ctx = _case(43, 9, 40, 6000, hq, hkv, d, bs, 8192)
+    out = torch.empty_like(q)
+    lib = _C.load()
+
+    def call():
+        return lib.mvllm_paged_decode_noalloc(
+            out.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), tables.data_ptr(), tables.shape[1],
+            ctx.data_ptr(), int(ctx.dtype == torch.int64), q.shape[0], hq, hkv, d, bs, kc.shape[0], float(scale),
+            _C.dtype_code(q.dtype), _C.current_stream_ptr(q.device))
+
+    assert call() == 0                                             # first call on the device: the symbol lookup
+    torch.cuda.synchronize()
+    want = out.clone()
+    free_before, _ = torch.cuda.mem_get_info()
+    assert call() == 0
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+    assert torch.equal(out, want)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            assert call() == 0
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
