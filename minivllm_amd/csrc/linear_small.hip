@@ -291,26 +291,19 @@ static int launch_linear_w(const LinearArgs& a, hipStream_t stream) {
   }
 }
 
-#ifndef MVLLM_LINEAR_NARROW_COLS
-#define MVLLM_LINEAR_NARROW_COLS 8
-#endif
+constexpr int kLinearNarrowCols = 8;
 // columns per workgroup of the plain product: narrower tiles when 16-column tiles would leave most CUs without
 // a workgroup (what a CU can keep in flight bounds its share of the weight stream)
 static int linear_cols(int N, bool plain) {
-  return plain && N / 16 < 128 ? MVLLM_LINEAR_NARROW_COLS : 16;
+  return plain && N / 16 < 128 ? kLinearNarrowCols : 16;
 }
 
-#ifndef MVLLM_LINEAR_ROW_TILE_FROM
-#define MVLLM_LINEAR_ROW_TILE_FROM 17
-#endif
+constexpr int kLinearRowTileFrom = 17;
 // workgroups per column tile: from this many rows on, every 16 rows of x get a workgroup of their own (the code of
 // the 16-row case, which holds few registers and asks for everything at once) instead of one workgroup that walks
 // all rows; the weights are then read once from HBM and again from L2
 static int linear_row_tiles(int M) {
-#ifdef MVLLM_EXPERIMENT
-  if (const char* e = getenv("MVLLM_LINEAR_ROW_TILE_FROM")) return M >= atoi(e) ? (M + 15) / 16 : 1;
-#endif
-  return M >= MVLLM_LINEAR_ROW_TILE_FROM ? (M + 15) / 16 : 1;
+  return M >= kLinearRowTileFrom ? (M + 15) / 16 : 1;
 }
 
 // waves per workgroup: more of them share a column tile's K when the column tiles alone give too few workgroups to

@@ -23,44 +23,24 @@
 
 namespace mvllm {
 
-// Tuning constants (overridable at compile time for experiments).
-#ifndef MVLLM_DECODE_MAX_PARTS
-#define MVLLM_DECODE_MAX_PARTS 32
-#endif
-#ifndef MVLLM_DECODE_PART_CAP
-#define MVLLM_DECODE_PART_CAP 1024  // partitions grow to this many tokens while the grid stays large
-#endif
-#ifndef MVLLM_DECODE_MIN_PART
-#define MVLLM_DECODE_MIN_PART 256
-#endif
-#ifndef MVLLM_DECODE_WAVES_PER_EU
-#define MVLLM_DECODE_WAVES_PER_EU 2
-#endif
-#ifndef MVLLM_DECODE_SMALL_PAIRS
-#define MVLLM_DECODE_SMALL_PAIRS 1024  // partitions are shortened (to >= 64 tokens) while batch * partitions is below this
-#endif
-#ifndef MVLLM_DECODE_SMALL_GRID
-#define MVLLM_DECODE_SMALL_GRID 1024   // kv heads per workgroup are reduced while the grid has fewer workgroups than this
-#endif
-#ifndef MVLLM_DECODE_I8_WPB
-#define MVLLM_DECODE_I8_WPB 4       // INT8 kernel: 4-wave workgroups, three of which fit a CU (more waves to hide latency)
-#endif
-#ifndef MVLLM_DECODE_I8_THREADS
-#define MVLLM_DECODE_I8_THREADS 256
-#endif
-#ifndef MVLLM_DECODE_I8_WAVES_PER_EU
-#define MVLLM_DECODE_I8_WAVES_PER_EU 3
-#endif
+// Tuning constants.
+constexpr int kDecodeMaxParts = 32;
+constexpr int kDecodePartCap = 1024;       // partitions grow to this many tokens while the grid stays large
+constexpr int kDecodeMinPart = 256;
+constexpr int kDecodeWavesPerEu = 2;
+constexpr int kDecodeSmallPairs = 1024;    // partitions are shortened (to >= 64 tokens) while batch * partitions is below this
+constexpr int kDecodeSmallGrid = 1024;     // kv heads per workgroup are reduced while the grid has fewer workgroups than this
+constexpr int kDecodeI8Wpb = 4;            // INT8 kernel: 4-wave workgroups, three of which fit a CU (more waves to hide latency)
+constexpr int kDecodeI8Threads = 256;
+constexpr int kDecodeI8WavesPerEu = 3;
+constexpr int kDecodeWpb = 4;              // waves (= kv heads) per workgroup, upper bound (8-wave workgroups: -1.5 %)
 #ifndef MVLLM_DECODE_LOADS_ONLY
 #define MVLLM_DECODE_LOADS_ONLY 0   // 1: measurement build for libmvllm_probe.so: the MFMA decode kernels issue their loads and
 #endif                              // fold the loaded registers with xor instead of computing (results are meaningless)
-#ifndef MVLLM_DECODE_WPB
-#define MVLLM_DECODE_WPB 4          // waves (= kv heads) per workgroup, upper bound (8-wave workgroups: -1.5 %)
-#endif
 
 constexpr int kTile = 16;                                 // tokens per MFMA tile
-constexpr int kMaxParts = MVLLM_DECODE_MAX_PARTS;         // split-K partitions per sequence (upper bound)
-constexpr int kMinPartTokens = MVLLM_DECODE_MIN_PART;     // smallest partition
+constexpr int kMaxParts = kDecodeMaxParts;         // split-K partitions per sequence (upper bound)
+constexpr int kMinPartTokens = kDecodeMinPart;     // smallest partition
 constexpr float kLazyRescale = 8.f;  // rescale accumulators only when the max grows by > 2^8
 
 struct DecodeArgs {
@@ -97,8 +77,8 @@ __host__ __device__ inline int partition_tokens_for(int64_t max_ctx, int batch) 
   const int64_t per_part = (max_ctx + kMaxParts - 1) / kMaxParts;
   int64_t part = (per_part + kMinPartTokens - 1) / kMinPartTokens * kMinPartTokens;
   if (part < kMinPartTokens) part = kMinPartTokens;
-  while (part < MVLLM_DECODE_PART_CAP && (int64_t)batch * ((max_ctx + 2 * part - 1) / (2 * part)) >= 1024) part *= 2;
-  while (part > 64 && part / 2 >= per_part && (int64_t)batch * ((max_ctx + part - 1) / part) < MVLLM_DECODE_SMALL_PAIRS) part /= 2;
+  while (part < kDecodePartCap && (int64_t)batch * ((max_ctx + 2 * part - 1) / (2 * part)) >= 1024) part *= 2;
+  while (part > 64 && part / 2 >= per_part && (int64_t)batch * ((max_ctx + part - 1) / part) < kDecodeSmallPairs) part /= 2;
   return (int)part;
 }
 
@@ -122,24 +102,16 @@ inline int largest_divisor_le(int n, int cap) {
 // contexts are long, although up to 2x slower when they are much shorter than the table is wide, which the
 // host cannot know.
 // The partition is never shorter than partition_tokens_for's, so a workspace sized from it is always enough.
-#ifndef MVLLM_DECODE_SPLIT
-#define MVLLM_DECODE_SPLIT 1              // 0: never use the split kernel
-#endif
-#ifndef MVLLM_DECODE_SPLIT_WAVES
-#define MVLLM_DECODE_SPLIT_WAVES 4        // 8 waves: 1-3 us slower per call except at 16 sequences (merge cost, one workgroup per CU)
-#endif
-constexpr int kSplitWaves = MVLLM_DECODE_SPLIT_WAVES;
+constexpr int kSplitWaves = 4;            // 8 waves: 1-3 us slower per call except at 16 sequences (merge cost, one workgroup per CU)
 constexpr int kSplitMinGroups = 512;
 constexpr int kSplitMaxPart = 4096;
 constexpr int kSplitOnePartCtx = 512;
 inline bool split_wanted(int64_t max_ctx, int batch, int num_kv_heads, bool int8) {
-  if (!MVLLM_DECODE_SPLIT) return false;
-  if (MVLLM_DECODE_SPLIT == 2) return true;          // timing builds
   const int part = partition_tokens_for(max_ctx, batch);
   const int64_t parts = (max_ctx + part - 1) / part;
-  const int wpb = largest_divisor_le(num_kv_heads, MVLLM_DECODE_WPB);
+  const int wpb = largest_divisor_le(num_kv_heads, kDecodeWpb);
   const bool few_groups = (int64_t)batch * parts * (num_kv_heads / wpb) < 256;
-  const bool short_parts = part < MVLLM_DECODE_PART_CAP, narrow_table = max_ctx <= kSplitMaxPart;
+  const bool short_parts = part < kDecodePartCap, narrow_table = max_ctx <= kSplitMaxPart;
   // INT8: a workgroup of the split form uses 4 of the 32 bytes of scales that a token's kv heads share, so with
   // many long sequences every head's workgroup fetches the scale lines again (128 sequences x 4096 tokens:
   // 218 -> 268 us, 256: 401 -> 467 us; 64: 123 -> 117 us): only up to 512 (sequence, kv head) pairs
@@ -1236,27 +1208,27 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
 // ---------------------------------------------------------------------------
 template <typename T, int D>
 // head_dim 256 holds twice the accumulators and tiles: one wave per SIMD with up to 512 registers
-__global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : kDecodeWavesPerEu) void decode_mfma_kernel(const DecodeArgs a) {
   int b, p, hg;
   if (!decode_item<false>(a, b, p, hg)) return;
   decode_mfma_item<T, 1, D>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
 }
 // Small batches: one workgroup of W waves per (partition, sequence, kv head), the waves splitting the tiles.
 template <typename T, int W, int D>
-__global__ __launch_bounds__(64 * W, D > 128 ? 1 : MVLLM_DECODE_WAVES_PER_EU) void decode_mfma_split_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(64 * W, D > 128 ? 1 : kDecodeWavesPerEu) void decode_mfma_split_kernel(const DecodeArgs a) {
   // kv head fastest: the workgroups of one (sequence, partition) start together and read the same token rows
   const int g = blockIdx.x, b = blockIdx.z;
   const int p = (int)((blockIdx.y + (unsigned)b) % (unsigned)a.num_parts);
   decode_mfma_item<T, W, D>(a, b, p, g, threadIdx.x >> 6);
 }
 template <typename T, int NCH, int D>
-__global__ __launch_bounds__(MVLLM_DECODE_I8_THREADS, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(kDecodeI8Threads, kDecodeI8WavesPerEu) void decode_mfma_int8_kernel(const DecodeArgs a) {
   int b, p, hg;
   if (!decode_item<true>(a, b, p, hg)) return;
   decode_mfma_int8_item<T, NCH, 1, D>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
 }
 template <typename T, int W, int D>
-__global__ __launch_bounds__(64 * W, MVLLM_DECODE_I8_WAVES_PER_EU) void decode_mfma_int8_split_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(64 * W, kDecodeI8WavesPerEu) void decode_mfma_int8_split_kernel(const DecodeArgs a) {
   const int g = blockIdx.x, b = blockIdx.z;
   const int p = (int)((blockIdx.y + (unsigned)b) % (unsigned)a.num_parts);
   decode_mfma_int8_item<T, 1, W, D>(a, b, p, g, threadIdx.x >> 6);
@@ -1520,8 +1492,8 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
   bool launched = false;
   // kv heads (waves) per workgroup of the one-wave-per-head form: as many as allowed, so that a workgroup streams
   // whole token rows; fewer when the grid would otherwise leave most CUs without a workgroup
-  int wpb = largest_divisor_le(a.num_kv_heads, int8 ? MVLLM_DECODE_I8_WPB : MVLLM_DECODE_WPB);
-  while (wpb > 1 && (int64_t)a.num_parts * a.batch * (a.num_kv_heads / wpb) < MVLLM_DECODE_SMALL_GRID)
+  int wpb = largest_divisor_le(a.num_kv_heads, int8 ? kDecodeI8Wpb : kDecodeWpb);
+  while (wpb > 1 && (int64_t)a.num_parts * a.batch * (a.num_kv_heads / wpb) < kDecodeSmallGrid)
     wpb = largest_divisor_le(a.num_kv_heads, wpb - 1);
   const unsigned groups = (unsigned)(a.num_kv_heads / wpb);
   const dim3 split_grid((unsigned)a.num_kv_heads, (unsigned)a.num_parts, (unsigned)a.batch), split_block(64 * kSplitWaves);

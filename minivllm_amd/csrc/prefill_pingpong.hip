@@ -35,12 +35,7 @@ constexpr int kPpWaves = 8;
 #ifndef MVLLM_PP_TIMELINE
 #define MVLLM_PP_TIMELINE 0            // 1: the timing build of the probe library (per-tile clock stamps)
 #endif
-#ifndef MVLLM_PP_PRIO
-#define MVLLM_PP_PRIO 3
-#endif
-#ifndef MVLLM_PP_LB
-#define MVLLM_PP_LB 512
-#endif
+
 
 template <int D>
 struct PpLds {
@@ -471,7 +466,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     const int n_slot = c_slot == kPpRing - 1 ? 0 : c_slot + 1;
     const bool more = !last || nxt.valid;
     // this wave's MFMAs go in front of the other group's vector instructions on the shared SIMD
-    __builtin_amdgcn_s_setprio(MVLLM_PP_PRIO);
+    __builtin_amdgcn_s_setprio(3);
     uint4 vf2[kTD], vf3[kTD];
     uint4 kf0[2], kf1[2], kf2[2], kf3[2], kf4[2], kf5[2], kf6[2], kf7[2];
     // stage A
@@ -632,7 +627,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 }
 
 template <typename T, int D>
-__global__ __launch_bounds__(MVLLM_PP_LB) void prefill_pp_kernel(const PrefillPpArgs a) {
+__global__ __launch_bounds__(64 * kPpWaves, 1) void prefill_pp_kernel(const PrefillPpArgs a) {
   __shared__ __attribute__((aligned(1024))) PpLds<D> lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   if (wave < 4) pp_run<T, D, 0>(a, lds, wave);

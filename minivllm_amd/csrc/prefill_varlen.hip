@@ -142,26 +142,8 @@ __global__ __launch_bounds__(256) void prefill_generic_kernel(const PrefillArgs 
 // 4*(row%4)) so both access patterns spread over all banks.  Causal tiles past
 // the diagonal are never visited; only the diagonal tile is masked.
 // ---------------------------------------------------------------------------
-#ifndef MVLLM_PF_XCD_CHUNK
-#define MVLLM_PF_XCD_CHUNK 32
-#endif
-constexpr unsigned kXcdChunk = MVLLM_PF_XCD_CHUNK;   // consecutive work items handed to one XCD
-#ifndef MVLLM_PF_BAND_ROWS
-#define MVLLM_PF_BAND_ROWS 256        // rows per band of the heaviest-first item order (a multiple of 128)
-#endif
-#ifndef MVLLM_PF_PIN_KREADS
-#define MVLLM_PF_PIN_KREADS 1
-#endif
-#ifndef MVLLM_PF_INT8_TILED
-#define MVLLM_PF_INT8_TILED 1         // 0: INT8 caches always on the 16-row tile kernel
-#endif
-#ifndef MVLLM_PF_PINGPONG
-#define MVLLM_PF_PINGPONG 1             // 0: every batch on prefill_mfma_kernel
-#endif
-#ifndef MVLLM_PF_WAVES
-#define MVLLM_PF_WAVES 4
-#endif
-constexpr int kPfWaves = MVLLM_PF_WAVES;             // waves per workgroup: 4, so that two workgroups share a CU
+constexpr unsigned kXcdChunk = 32;      // consecutive work items handed to one XCD
+constexpr int kPfWaves = 4;             // waves per workgroup: 4, so that two workgroups share a CU
 constexpr int kBN = 64;                 // K/V rows per LDS tile
 constexpr int kWaveRows = 32;           // query rows per wave
 
@@ -188,7 +170,7 @@ template <typename T> __device__ __forceinline__ uint4 dequant8_biased(uint32_t 
 // neighbouring bands of the same level), which keeps them in one XCD's L2.  Bands past a sequence's last tile are
 // padding: those workgroups return at once (at most R - 1 per sequence and head slice).
 // Every lane of the calling wave must be active; all lanes return the same values.
-constexpr int kBandRows = MVLLM_PF_BAND_ROWS;
+constexpr int kBandRows = 256;          // rows per band of the heaviest-first item order (a multiple of 128)
 template <int BM>
 __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, int num_seqs, unsigned item, int heads_y,
                                               int band_bits, int& seq_start, int& seq_len, int& row0, int& seq_index, int& item_y) {
@@ -553,7 +535,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
 #pragma unroll
           for (int tk = 0; tk < NH; ++tk)
             kf[(ks + 1) & 1][tk] = *reinterpret_cast<const uint4*>(kb + k_off[ks + 1] + tk * 32 * kRowB);
-          if (MVLLM_PF_PIN_KREADS) __builtin_amdgcn_sched_barrier(0);   // keep the reads in front of this step's MFMAs
+          __builtin_amdgcn_sched_barrier(0);   // keep the reads in front of this step's MFMAs
         }
 #pragma unroll
         for (int tk = 0; tk < NH; ++tk) s[tk] = mfma32x32x16<T>(kf[ks & 1][tk], qf[ks], ks == 0 ? neg_m : s[tk]);
@@ -842,7 +824,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   const bool aligned = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out);
   const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, 0, dtype, false, false) : 0;
   const bool mfma_ok = kind == 2;
-  if (MVLLM_PF_PINGPONG && mfma_ok && scale > 0.f && prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype)) {
+  if (mfma_ok && scale > 0.f && prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype)) {
     PrefillPpArgs p;
     p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
     p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
@@ -916,7 +898,7 @@ extern "C" int mvllm_prefill_paged_int8(void* out, const void* q, const int8_t* 
       total_q_tokens > ((int64_t)1 << 30) || (int64_t)num_kv_heads * head_dim * 64 >= ((int64_t)1 << 31))
     return MVLLM_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(out) || !aligned16(k_cache) || !aligned16(v_cache)) return MVLLM_ERR_MISALIGNED;
-  if (prefill_kernel_for(num_heads, num_kv_heads, head_dim, block_size, dtype, true, true) == 2 && MVLLM_PF_INT8_TILED) {
+  if (prefill_kernel_for(num_heads, num_kv_heads, head_dim, block_size, dtype, true, true) == 2) {
     PrefillArgs a;
     a.out = out; a.q = q; a.k = k_cache; a.v = v_cache; a.cu_seqlens = cu_seqlens_q;
     a.total_tokens = total_q_tokens; a.num_seqs = num_seqs; a.num_heads = num_heads;
