@@ -760,7 +760,9 @@ def bench_prefill_timeline(args):
     """Where a workgroup of the two-group prefill kernel spends a tile: the probe library's timing build logs the
     shader clock at the four corners of every tile (softmax begins / done, matrix part begins / done) for the waves of
     one workgroup.  A stamp costs about 100 clocks, so every logged interval is that much longer than in the product
-    build; the shares are what the figures are for."""
+    build; the shares are what the figures are for.  `workgroups`: from a second launch in which every workgroup logs
+    only when it began and ended and what it went through (life in clocks; max over mean is what uneven dealing of
+    the items costs)."""
     import ctypes
     import statistics
     import torch
@@ -802,6 +804,22 @@ def bench_prefill_timeline(args):
             res[grp] = {"tiles_logged": tiles, "softmax": med(seg[0]), "wait_for_matrix_part": med(seg[1]),
                         "matrix_part": med(seg[2]), "wait_for_softmax": med(seg[3]), "tile": med(per_tile),
                         "life": t[-1] - t[0] if t else None}
+        # every workgroup's begin and end (block < 0): how evenly the items were dealt
+        grid = torch.cuda.get_device_properties(0).multi_processor_count // 8 * 8
+        per_wg = torch.zeros(grid, 4, dtype=torch.int64, device=dev)
+        for _ in range(3):
+            per_wg.zero_()
+            st = fn(o.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), cu.data_ptr(), len(lengths), total, hq, hkv, d,
+                    1.0 / math.sqrt(d), _C.dtype_code(q.dtype), per_wg.data_ptr(), 4, -1,
+                    torch.cuda.current_stream().cuda_stream)
+            assert st == 0, st
+        torch.cuda.synchronize()
+        rows = [r for r in per_wg.cpu().tolist() if r[1] > r[0]]
+        life = [r[1] - r[0] for r in rows]
+        res["workgroups"] = {"busy": len(rows), "life_max": max(life), "life_mean": int(sum(life) / len(life)),
+                             "max_over_mean": round(max(life) * len(life) / sum(life), 4),
+                             "items_max": max(r[2] for r in rows), "items_min": min(r[2] for r in rows),
+                             "tiles_max": max(r[3] for r in rows), "tiles_mean": round(sum(r[3] for r in rows) / len(rows), 2)}
         out[name] = res
     return out
 

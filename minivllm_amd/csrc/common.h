@@ -228,6 +228,7 @@ struct PrefillPpArgs {
   int n_teams;      // gcd(8, slices): workgroup teams, each with its own item list
   int team_size;    // workgroups per team
   int level_bits;   // bits that hold the block count of the longest possible sequence
+  unsigned spt_magic, chunks_magic;   // 2^32 / d + 1 for d = slices per team and d = query heads per kv head / 4 (0 for d = 1)
   // timing build only (the probe library): where workgroup `timeline_block` logs its clock stamps; null otherwise
   unsigned long long* timeline;
   int timeline_entries;

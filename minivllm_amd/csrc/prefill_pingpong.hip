@@ -56,6 +56,12 @@ __device__ __forceinline__ void pp_barrier() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// 16 bytes per lane to base + lane_off, streaming; lanes whose 16 bytes do not end inside `bytes` store nothing.
+__device__ __forceinline__ void store16_buffer(void* base, uint32_t bytes, uint32_t lane_off, uint4 v) {
+  const u32x4 w = {v.x, v.y, v.z, v.w};
+  __builtin_amdgcn_raw_buffer_store_b128(w, __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)bytes, 0x00020000), (int)lane_off, 0, 2);
+}
+
 // 16 bytes per lane into LDS at m0_base + 16 * lane, from rsrc + lane_off.
 __device__ __forceinline__ void dma16(v4i rsrc, uint32_t lane_off, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(lane_off), "s"(rsrc) : "m0", "memory");
@@ -67,12 +73,17 @@ __device__ __forceinline__ void dma16(v4i rsrc, uint32_t lane_off, uint32_t lds_
 struct PpItems {
   int level;          // level the walk has reached (-1: past the last item)
   unsigned base;      // rank of that level's first item
-  unsigned taken;     // items this workgroup has asked for
 };
 struct PpItem {
-  int seq_start, seq_len, rb, y;
+  int seq_start, seq_len, rb;
+  int kvh, h0;        // kv head; first of the item's four query heads
   bool valid;
 };
+
+// x / d for x < 2^16 by a multiplication: magic = 2^32 / d + 1 (d > 1; d == 1 has magic 0 and is passed through).
+__device__ __forceinline__ unsigned div_small(unsigned x, unsigned d, unsigned magic) {
+  return d == 1u ? x : __umulhi(x, magic);
+}
 
 template <typename T, int D, int GRP>
 __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, const int wave) {
@@ -95,10 +106,16 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // A stamp costs about a hundred clocks, so the logged intervals are each that much longer than in the product build.
   unsigned long long* tlog = a.timeline + (size_t)wave * a.timeline_entries;
   int tn = 0;
-  const bool tlogging = a.timeline != nullptr && (int)blockIdx.x == a.timeline_block;
-#define TSTAMP() do { if (tlogging && tn < a.timeline_entries) { const unsigned long long t_ = __builtin_amdgcn_s_memtime(); if (lane == 0) tlog[tn] = t_; ++tn; } } while (0)
+  const bool tlogging = MVLLM_PP_TIMELINE == 1 && a.timeline != nullptr && (int)blockIdx.x == a.timeline_block;
+  // timeline_block < 0: instead, wave 4 of every workgroup logs when it began and ended and how many items and tiles
+  // it went through, four entries per workgroup.
+  const unsigned long long t_begin = __builtin_amdgcn_s_memtime();
+  int t_items = 0, t_tiles = 0;
+#define TCOUNT(items, tiles) do { t_items += (items); t_tiles += (tiles); } while (0)
+#define TSTAMP() do { if (MVLLM_PP_TIMELINE == 1 && tlogging && tn < a.timeline_entries) { const unsigned long long t_ = __builtin_amdgcn_s_memtime(); if (lane == 0) tlog[tn] = t_; ++tn; } } while (0)
 #else
 #define TSTAMP() do {} while (0)
+#define TCOUNT(items, tiles) do {} while (0)
 #endif
   // ---- the batch, one sequence per lane ----
   int lo = 0, len = 0;
@@ -120,46 +137,81 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   const unsigned TS = (unsigned)a.team_size;
   const unsigned t = (wg >> 3) * (8u / (unsigned)a.n_teams) + xcd / (unsigned)a.n_teams;   // index inside the team
   const unsigned spt = (unsigned)(a.slices / a.n_teams);                                  // slices per team
-  auto next_item = [&](PpItems& w) {
-    PpItem it;
-    it.seq_start = 0; it.seq_len = 0; it.rb = 0; it.y = 0; it.valid = false;
-    const unsigned round = w.taken++;
-    const unsigned R = round * TS + ((round & 1u) ? TS - 1u - t : t);
+  const int group = a.num_heads / a.num_kv_heads;
+  const int chunks = group / 4;
+  // The workgroup's k-th item is rank k TS + (t or, in odd rounds, TS - 1 - t) of the team's list.  Locating an item
+  // costs a hundred-odd instructions per wave, and two cursors go through the same items (the copies run ahead of the
+  // arithmetic), so every item is located once and kept in lane (k mod 16) of four registers until both have passed.
+  // Ranks are dealt in rounds of TS, forwards and backwards in turn; the serpentine leaves the team's first
+  // workgroups the most tiles (the first rounds, whose costs fall fastest, weigh most), so a last round that is not
+  // full always runs backwards: its items, each worth three to four tiles of fixed cost, go to the workgroups that
+  // have the least.
+  int team_items = nb;
+#pragma unroll
+  for (int step = 1; step < 64; step <<= 1) team_items += __shfl_xor(team_items, step, 64);
+  team_items = __builtin_amdgcn_readfirstlane(team_items) * (int)spt;
+  const unsigned short_round = (unsigned)team_items % TS != 0u ? (unsigned)team_items / TS : 0xffffffffu;
+  PpItems walk = {top - 1, 0u};
+  int produced = 0;
+  int kept_start = 0, kept_len = 0, kept_rb = 0, kept_heads = 0;
+  auto produce = [&]() {
+    const unsigned round = (unsigned)produced;
+    const bool backwards = (round & 1u) != 0u || round == short_round;
+    const unsigned R = round * TS + (backwards ? TS - 1u - t : t);
     unsigned long long mask = 0ull;
     unsigned cnt = 0;
-    while (w.level >= 0) {
-      mask = __ballot(nb > w.level);
+    while (walk.level >= 0) {
+      mask = __ballot(nb > walk.level);
       cnt = (unsigned)__popcll(mask);
       const unsigned items = cnt * spt;
-      if (R - w.base < items) break;
-      w.base += items;
-      --w.level;
+      if (R - walk.base < items) break;
+      walk.base += items;
+      --walk.level;
     }
-    if (w.level < 0) return it;
-    const unsigned idx = R - w.base;
-    const unsigned sl = idx / cnt;
-    const int qth = (int)(idx - sl * cnt);
-    const int below = __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
-    const unsigned long long pick = __ballot(((mask >> lane) & 1ull) != 0ull && below == qth);
-    const int owner = __ffsll((long long)pick) - 1;
-    it.seq_start = __builtin_amdgcn_readfirstlane(__shfl(lo, owner, 64));
-    it.seq_len = __builtin_amdgcn_readfirstlane(__shfl(len, owner, 64));
-    it.rb = __builtin_amdgcn_readfirstlane(w.level);
-    it.y = __builtin_amdgcn_readfirstlane(team + a.n_teams * (int)sl);
-    it.valid = true;
+    int seq_start = 0, seq_len = 0, heads = 0;
+    if (walk.level >= 0) {
+      // inside a level: sequence-major, the team's slices of one sequence side by side
+      const unsigned idx = R - walk.base;
+      const unsigned qth = div_small(idx, spt, a.spt_magic);
+      const unsigned sl = idx - qth * spt;
+      const int below = __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+      const unsigned long long pick = __ballot(((mask >> lane) & 1ull) != 0ull && below == (int)qth);
+      const int owner = __ffsll((long long)pick) - 1;
+      seq_start = __builtin_amdgcn_readlane(lo, owner);
+      seq_len = __builtin_amdgcn_readlane(len, owner);
+      const unsigned y = (unsigned)team + (unsigned)a.n_teams * sl;
+      const unsigned kvh = div_small(y, (unsigned)chunks, a.chunks_magic);
+      heads = (int)((kvh << 16) | (kvh * (unsigned)group + (y - kvh * (unsigned)chunks) * 4u));
+    }
+    const int at = produced & 15;
+    kept_start = lane == at ? seq_start : kept_start;
+    kept_len = lane == at ? seq_len : kept_len;
+    kept_rb = lane == at ? walk.level : kept_rb;     // -1: no such item
+    kept_heads = lane == at ? heads : kept_heads;
+    ++produced;
+  };
+  auto item_at = [&](int k) {
+    while (produced <= k) produce();
+    PpItem it;
+    const int at = k & 15;
+    it.seq_start = __builtin_amdgcn_readlane(kept_start, at);
+    it.seq_len = __builtin_amdgcn_readlane(kept_len, at);
+    it.rb = __builtin_amdgcn_readlane(kept_rb, at);
+    const int heads = __builtin_amdgcn_readlane(kept_heads, at);
+    it.kvh = (int)((unsigned)heads >> 16);
+    it.h0 = heads & 0xffff;
+    it.valid = it.rb >= 0;
     return it;
   };
 
-  PpItems walk_c = {top - 1, 0u, 0u};          // the walk that feeds the compute cursor (runs one item ahead)
-  PpItems walk_d = walk_c;                     // ... and the one of the K/V copy cursor
-  PpItem cur = next_item(walk_c);
+  int ci = 0;                                  // items handed to the arithmetic so far
+  PpItem cur = item_at(ci++);
   if (!cur.valid) return;                      // no item for this workgroup (all waves agree)
-  PpItem nxt = next_item(walk_c);
-  PpItem dit = next_item(walk_d);              // item the copy cursor is in
+  PpItem nxt = item_at(ci++);
+  int di = 0;
+  PpItem dit = cur;                            // item the copy cursor is in
   int dj = 0;                                  // ... and its tile there
 
-  const int group = a.num_heads / a.num_kv_heads;
-  const int chunks = group / 4;
   const T* qg = reinterpret_cast<const T*>(a.q);
   const char* kg = reinterpret_cast<const char*>(a.k);
   const char* vg = reinterpret_cast<const char*>(a.v);
@@ -189,7 +241,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   int d_rows_left = 0;                         // rows from the tile's first to the tensor's last; <= 0: no tile
   int d_head_off = 0;                          // byte offset of the kv head inside a row
   auto enter_item = [&]() {                    // the cursor's tile = first tile of `dit`
-    d_head_off = (dit.y / chunks) * kRowB;
+    d_head_off = dit.kvh * kRowB;
     d_off = (int64_t)dit.seq_start * kv_row_bytes + d_head_off;
     d_rows_left = dit.valid ? total_rows - dit.seq_start : 0;
   };
@@ -206,7 +258,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     d_slot = d_slot == kPpRing - 1 ? 0 : d_slot + 1;
     if (dit.valid) {
       if (++dj > dit.rb) {
-        dit = next_item(walk_d);
+        dit = item_at(++di);
         dj = 0;
         enter_item();
       } else {
@@ -218,7 +270,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // Q rows of an item -> this wave's slot, 4 rows per instruction, chunks swizzled like a K tile's
   const uint32_t lds_q = lds_address(&lds.qo[wave][0]);
   auto copy_q = [&](const PpItem& it) {
-    const int h = (it.y / chunks) * group + (it.y % chunks) * 4 + wq;
+    const int h = it.h0 + wq;
     const int row = it.seq_start + it.rb * 64 + 32 * GRP;
     const int rows_left = total_rows - row;
     const int rows_4g = (int)(0xffffffffu / (uint32_t)q_row_bytes);
@@ -268,17 +320,23 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 
   // slot -> registers, times scale * log2 e (rounded to the element type once), so that the scores leave the matrix
   // unit as exp2 arguments.  The multiplications run in a matrix interval, whose wave has vector slots to spare.
-  auto load_q = [&]() {
+  auto read_q = [&]() {
     const char* qs = &lds.qo[wave][0];
 #pragma unroll
     for (int ks = 0; ks < kKS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(qs + k_off[ks]);
+  };
+  auto scale_q = [&](auto QUARTER) {              // a quarter of the fragments
 #pragma unroll
-    for (int ks = 0; ks < kKS; ++ks) {
+    for (int ks = 2 * decltype(QUARTER)::value; ks < 2 * decltype(QUARTER)::value + 2; ++ks) {
       qf[ks].x = scale_pair<T>(qf[ks].x, a.scale_log2);
       qf[ks].y = scale_pair<T>(qf[ks].y, a.scale_log2);
       qf[ks].z = scale_pair<T>(qf[ks].z, a.scale_log2);
       qf[ks].w = scale_pair<T>(qf[ks].w, a.scale_log2);
     }
+  };
+  auto load_q = [&]() {
+    read_q();
+    static_for<4>([&](auto QUARTER) { scale_q(QUARTER); });
   };
   // Operand fragments from LDS.  K: rows l32 and l32 + 32 of the tile in K ring slot `slot`, dims 16 ks + 8 hi ..;
   // V^T: the transposing reads of the 16 keys of `step` ( = 2 tk + st) of the tile in V ring slot `slot`.
@@ -318,36 +376,48 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       }
     });
   };
-  // normalise, transpose through the wave's slot, store whole rows (rows past the sequence's end are not stored)
+  // An item's output leaves in two steps.  stage_out, in the matrix interval of the item's last tile (once the next
+  // item's Q rows have been read out of the slot): O^T / row sum, rounded, into the wave's slot, transposed.
+  // write_out, in the next softmax interval: whole rows from the slot to memory (rows past the sequence's end are not
+  // stored).
   T* out = reinterpret_cast<T*>(a.out);
-  auto store_item = [&](int seq_start, int seq_len, int rb, int y, float lsum) {
-    char* ot = &lds.qo[wave][0];
-    const float lt = lsum + __shfl_xor(lsum, 32, 64);
-    const float inv = 1.f / lt;
-    int lane_o = lane;
-    asm volatile("" : "+v"(lane_o));              // addresses below are computed per item, not kept in registers between items
-    const int ol32 = lane_o & 31, ohi = lane_o >> 5;
+  auto stage_out = [&](auto TD, float inv) {     // 32 of the 128 dims
+    constexpr int td = decltype(TD)::value;
+    char* orow = &lds.qo[wave][0] + l32 * kRowB + 8 * hi;
+    const int oswz = kswz(l32);
 #pragma unroll
-    for (int td = 0; td < kTD; ++td)
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
+    for (int r4 = 0; r4 < 4; ++r4) {
         uint2 w;
         w.x = pack2<T>(o[td][4 * r4 + 0] * inv, o[td][4 * r4 + 1] * inv);
         w.y = pack2<T>(o[td][4 * r4 + 2] * inv, o[td][4 * r4 + 3] * inv);
-        *reinterpret_cast<uint2*>(ot + ol32 * kRowB + (((4 * td + r4) ^ kswz(ol32)) << 4) + 8 * ohi) = w;
+        *reinterpret_cast<uint2*>(orow + (((4 * td + r4) ^ oswz) << 4)) = w;
       }
-    const int h = (y / chunks) * group + (y % chunks) * 4 + wq;
-    const int r0 = rb * 64 + 32 * GRP;
+  };
+  auto write_out = [&](int seq_start, int seq_len, int rb, int h0) {
+    const char* ot = &lds.qo[wave][0];
+    int lane_o = lane;
+    asm volatile("" : "+v"(lane_o));
     const int orow = lane_o >> 4, ochunk = lane_o & 15;
+    const int r0 = rb * 64 + 32 * GRP;
+    // The descriptor ends with the head's part of the sequence's last row, so the stores of rows past it are dropped
+    // by the bounds check: all eight are always issued, as the wait counts assume.
+    const int rows = seq_len - r0 < 32 ? seq_len - r0 : 32;
+    const uint32_t size = rows > 0 ? (uint32_t)(rows - 1) * (uint32_t)q_row_bytes + (uint32_t)kRowB : 0u;
+    char* base = reinterpret_cast<char*>(out) + (int64_t)(seq_start + r0) * q_row_bytes + (int64_t)(h0 + wq) * kRowB;
+    const uint32_t off0 = (uint32_t)(orow * q_row_bytes + 16 * ochunk);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int row = 4 * i + orow;
       const uint4 w = *reinterpret_cast<const uint4*>(ot + row * kRowB + ((ochunk ^ kswz(row)) << 4));
-      if (r0 + row < seq_len)
-        store16_stream(out + ((int64_t)(seq_start + r0 + row) * a.num_heads + h) * D + 8 * ochunk, w);
+      store16_buffer(base, size, off0 + (uint32_t)(4 * i) * (uint32_t)q_row_bytes, w);
     }
   };
-  auto wait_copies = [&](int later) {            // everything but the `later` newest VMEM instructions has completed
+  // The barrier that ends a softmax interval publishes the copy step issued in the wave's previous softmax interval:
+  // everything but the `later` vector memory instructions issued in this one (its copy step and, in an item's first
+  // tile, the previous item's 8 output stores and the next item's 8 Q copies: the bounds-checked stores are issued
+  // whatever the sequence's length, so the count is exact) must have completed.  (Letting the previous interval's
+  // stores and Q copies stay in flight as well was measured and is slower.)
+  auto wait_copies = [&](int later) {
     if (later == 4) vm_wait<4>();
     else if (later == 12) vm_wait<12>();
     else if (later == 20) vm_wait<20>();
@@ -362,9 +432,8 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   pp_barrier();
   load_q();
   int c_slot = 0;                               // ring slot of the tile whose softmax comes next
-  int p_seq_start = 0, p_seq_len = 0, p_rb = 0, p_y = 0;   // item whose output is still in the accumulators
+  int p_seq_start = 0, p_seq_len = 0, p_rb = 0, p_h0 = 0;   // item whose output waits in the slot
   bool have_prev = false;
-  float l_prev = 0.f;
 
   if (GRP == 1) pp_barrier();                   // group 1 runs one interval behind
   first_scores(c_slot);
@@ -436,13 +505,19 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // A wave issues about one instruction in five clocks, an MFMA keeps the matrix unit for 32: at most five other
   // instructions fit between two MFMAs without a bubble, so each stage's fragment reads and their address
   // arithmetic are dealt out between its four MFMAs instead of standing in front of them.
-  auto stage_end = [&](int reads_per_mfma) {
+  auto stage_end = [&](int reads_per_mfma, int others_per_mfma) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // one MFMA
       if (reads_per_mfma == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // LDS reads
       else if (reads_per_mfma == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (reads_per_mfma > 0) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);    // one vector instruction (an address)
+      // vector instructions (a fragment's address; in an item's last tile the Q scaling and the output's
+      // normalisation) and the output's LDS writes
+      if (others_per_mfma == 1) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
+      else if (others_per_mfma == 8) {
+        __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -458,11 +533,18 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     asm volatile("" : "+v"(s[0]), "+v"(s[1]));
     asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
   };
-  auto matrix_interval = [&](auto FRESH, bool last, uint4 (&vf0)[kTD], uint4 (&vf1)[kTD]) {
+  // LAST (compile time: an item's last tile has a code path of its own, so the others carry none of its branches):
+  // the next item's Q rows are read out of the slot after the P V MFMAs; their scaling, and the normalisation of the
+  // item's output and its way into the slot, are dealt out between the K Q^T MFMAs of the next item's first tile.  When the stream ends here both still run, on whatever the slot and the next ring
+  // tile hold, and nothing uses the results.
+  auto matrix_interval = [&](auto FRESH, auto LAST, bool single, uint4 (&vf0)[kTD], uint4 (&vf1)[kTD]) {
     using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>; using I3 = std::integral_constant<int, 3>;
     using I4 = std::integral_constant<int, 4>; using I5 = std::integral_constant<int, 5>;
     using I6 = std::integral_constant<int, 6>; using I7 = std::integral_constant<int, 7>;
+    constexpr bool kFresh = decltype(FRESH)::value, kLast = decltype(LAST)::value;
+    static_assert(!(kFresh && kLast), "an item's first tile finds out at run time whether it is also the last");
+    const bool last = kFresh ? single : kLast;
     const int n_slot = c_slot == kPpRing - 1 ? 0 : c_slot + 1;
     const bool more = !last || nxt.valid;
     // this wave's MFMAs go in front of the other group's vector instructions on the shared SIMD
@@ -471,7 +553,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     uint4 kf0[2], kf1[2], kf2[2], kf3[2], kf4[2], kf5[2], kf6[2], kf7[2];
     // stage A
     v_frags(c_slot, I2{}, vf2);
-    if constexpr (decltype(FRESH)::value) {
+    if constexpr (kFresh) {
       v16f z;
 #pragma unroll
       for (int r = 0; r < 16; ++r) z[r] = 0.f;
@@ -481,66 +563,79 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 #pragma unroll
       for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf0[td], pf[0], o[td]);
     }
-    stage_end(2);
+    stage_end(2, 1);
     // stage B
     v_frags(c_slot, I3{}, vf3);
 #pragma unroll
     for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf1[td], pf[1], o[td]);
-    stage_end(2);
+    stage_end(2, 1);
     // stage C
     k_frags(n_slot, I0{}, kf0); k_frags(n_slot, I1{}, kf1);      // (read and not used when the stream ends here)
 #pragma unroll
     for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf2[td], pf[2], o[td]);
-    stage_end(1);
+    stage_end(1, 1);
     // stage D
     k_frags(n_slot, I2{}, kf2); k_frags(n_slot, I3{}, kf3);
 #pragma unroll
     for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(vf3[td], pf[3], o[td]);
-    stage_end(1);
-    if (last && nxt.valid) {
-      // the next item's Q rows, copied since this item's first softmax interval; one copy step was issued behind
-      // them unless the item has a single tile
-      if (cur.rb > 0) vm_wait<4>();
-      else vm_wait<0>();
-      load_q();
-    }
-    if (more) {
-      // stage E
-      k_frags(n_slot, I4{}, kf4); k_frags(n_slot, I5{}, kf5);
-      if (last) {
-        // another item's first tile: its maximum is not known yet, the scores arrive as they are
-        v16f z;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) z[r] = 0.f;
-#pragma unroll
-        for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf0[tk], qf[0], z);
-      } else {
-#pragma unroll
-        for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf0[tk], qf[0], neg_m);
+    stage_end(1, 1);
+    float inv = 0.f;
+    if constexpr (kFresh) {
+      if (last) {                                // a single tile: no other work to hide these behind
+        vm_wait<0>();
+        load_q();
+        inv = __builtin_amdgcn_rcpf(sum_with_lane_xor32(l));
+        static_for<4>([&](auto TD) { stage_out(TD, inv); });
       }
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf1[tk], qf[1], s[tk]);
-      stage_end(1);
-      // stage F
-      k_frags(n_slot, I6{}, kf6); k_frags(n_slot, I7{}, kf7);
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf2[tk], qf[2], s[tk]);
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf3[tk], qf[3], s[tk]);
-      stage_end(1);
-      // stage G
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf4[tk], qf[4], s[tk]);
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf5[tk], qf[5], s[tk]);
-      stage_end(0);
-      // stage H
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf6[tk], qf[6], s[tk]);
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf7[tk], qf[7], s[tk]);
-      stage_end(0);
     }
+    if constexpr (kLast) {
+      // the next item's Q rows, copied since this item's first softmax interval; one copy step was issued behind
+      // them
+      vm_wait<4>();
+      read_q();
+      inv = __builtin_amdgcn_rcpf(sum_with_lane_xor32(l));
+      scale_q(I0{});
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // stage E
+    k_frags(n_slot, I4{}, kf4); k_frags(n_slot, I5{}, kf5);
+    if (last) {
+      // another item's first tile: its maximum is not known yet, the scores arrive as they are
+      v16f z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf0[tk], qf[0], z);
+    } else {
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf0[tk], qf[0], neg_m);
+    }
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf1[tk], qf[1], s[tk]);
+    if constexpr (kLast) { scale_q(I1{}); stage_out(I0{}, inv); }
+    stage_end(1, kLast ? 8 : 1);
+    // stage F
+    k_frags(n_slot, I6{}, kf6); k_frags(n_slot, I7{}, kf7);
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf2[tk], qf[2], s[tk]);
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf3[tk], qf[3], s[tk]);
+    if constexpr (kLast) { scale_q(I2{}); stage_out(I1{}, inv); }
+    stage_end(1, kLast ? 8 : 1);
+    // stage G
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf4[tk], qf[4], s[tk]);
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf5[tk], qf[5], s[tk]);
+    if constexpr (kLast) { scale_q(I3{}); stage_out(I2{}, inv); }
+    stage_end(0, kLast ? 8 : 0);
+    // stage H
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf6[tk], qf[6], s[tk]);
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk) s[tk] = mfma32x32x16<T>(kf7[tk], qf[7], s[tk]);
+    if constexpr (kLast) stage_out(I3{}, inv);
+    stage_end(0, kLast ? 8 : 0);
     pin_products();
     __builtin_amdgcn_s_setprio(0);
     TSTAMP();
@@ -549,24 +644,58 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     return more;
   };
 
-  while (true) {
-    // ======== first tile of an item ========
-    bool last = cur.rb == 0;
-    int later = 4;
+  // the softmax interval of tile j > 0 of `cur`, up to the barrier; returns nothing, leaves pf, l, vf0, vf1
+  auto later_tile = [&](auto LAST, uint4 (&vf0)[kTD], uint4 (&vf1)[kTD]) {
     TSTAMP();
     copy_step();
-    if (last) mask_diagonal();
+    if constexpr (decltype(LAST)::value) mask_diagonal();
+    // The scores are relative to the running maximum, which is not looked at again unless it is badly out of
+    // date: the weights are computed first, and only when a lane's share of the tile's row sum passes 2^12 (a
+    // weight above 2^7 at least; 16-bit weights and fp32 sums are far from their limits there) is the tile redone
+    // the long way: true maximum, accumulators and row sum scaled down, weights again from the kept scores.
+    float sum = weights(std::false_type{}, 0.f);
+    if (__any(!(sum <= 4096.f))) {
+      const float mx = tile_max();
+      const float d = mx > 8.f ? mx : 0.f;       // per row (both lanes of a row see the same maximum)
+      if (d != 0.f) {
+        const float alpha = fast_exp2(-d);
+        l *= alpha;
+#pragma unroll
+        for (int td = 0; td < kTD; ++td)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[td][r] *= alpha;
+      }
+      set_neg_m(neg_m[0] - d);
+      sum = weights(std::true_type{}, d);
+    }
+    l += sum;
+    pin_weights();
+    TSTAMP();
+    v_frags(c_slot, std::integral_constant<int, 0>{}, vf0);
+    v_frags(c_slot, std::integral_constant<int, 1>{}, vf1);
+    vm_wait<4>();
+    pp_barrier();
+    TSTAMP();
+  };
+
+  while (true) {
+    // ======== first tile of an item ========
+    const bool single = cur.rb == 0;
+    int trail = 0;                               // vector memory instructions behind this interval's copy step
+    TSTAMP();
+    copy_step();
+    if (single) mask_diagonal();
     const float mx_first = tile_max();           // neg_m is zero here: the tile's maximum itself
-    // the item before this one leaves (its last P V ran in the interval before) ...
+    // the item before this one leaves (its output was staged in the slot during the interval before) ...
     if (have_prev) {
-      store_item(p_seq_start, p_seq_len, p_rb, p_y, l_prev);
-      later += 8;
+      write_out(p_seq_start, p_seq_len, p_rb, p_h0);
+      trail += 8;
     }
     // ... and the next one's Q rows set out
     if (nxt.valid) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slot's last readers are done
       copy_q(nxt);
-      later += 8;
+      trail += 8;
     }
     l = weights(std::true_type{}, mx_first);
     set_neg_m(-mx_first);
@@ -575,55 +704,38 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     TSTAMP();
     v_frags(c_slot, std::integral_constant<int, 0>{}, vf0);   // the tile's first V^T fragments: on their way across the barrier
     v_frags(c_slot, std::integral_constant<int, 1>{}, vf1);
-    wait_copies(later);
+    wait_copies(4 + trail);
     pp_barrier();
     TSTAMP();
-    bool more = matrix_interval(std::true_type{}, last, vf0, vf1);
-    // ======== the item's other tiles ========
-    for (int j = 1; j <= cur.rb; ++j) {
-      last = j == cur.rb;
-      TSTAMP();
-      copy_step();
-      if (last) mask_diagonal();
-      // The scores are relative to the running maximum, which is not looked at again unless it is badly out of
-      // date: the weights are computed first, and only when a lane's share of the tile's row sum passes 2^12 (a
-      // weight above 2^7 at least; 16-bit weights and fp32 sums are far from their limits there) is the tile redone
-      // the long way: true maximum, accumulators and row sum scaled down, weights again from the kept scores.
-      float sum = weights(std::false_type{}, 0.f);
-      if (__any(!(sum <= 4096.f))) {
-        const float mx = tile_max();
-        const float d = mx > 8.f ? mx : 0.f;       // per row (both lanes of a row see the same maximum)
-        if (d != 0.f) {
-          const float alpha = fast_exp2(-d);
-          l *= alpha;
-#pragma unroll
-          for (int td = 0; td < kTD; ++td)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[td][r] *= alpha;
-        }
-        set_neg_m(neg_m[0] - d);
-        sum = weights(std::true_type{}, d);
+    bool more = matrix_interval(std::true_type{}, std::false_type{}, single, vf0, vf1);
+    if (!single) {
+      // ======== the item's other tiles ========
+      for (int j = 1; j < cur.rb; ++j) {
+        later_tile(std::false_type{}, vf0, vf1);
+        matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
       }
-      l += sum;
-      pin_weights();
-      TSTAMP();
-      v_frags(c_slot, std::integral_constant<int, 0>{}, vf0);
-      v_frags(c_slot, std::integral_constant<int, 1>{}, vf1);
-      wait_copies(4);
-      pp_barrier();
-      TSTAMP();
-      more = matrix_interval(std::false_type{}, last, vf0, vf1);
+      later_tile(std::true_type{}, vf0, vf1);
+      more = matrix_interval(std::false_type{}, std::true_type{}, false, vf0, vf1);
     }
-    l_prev = l;
-    p_seq_start = cur.seq_start; p_seq_len = cur.seq_len; p_rb = cur.rb; p_y = cur.y;
+    TCOUNT(1, cur.rb + 1);
+    p_seq_start = cur.seq_start; p_seq_len = cur.seq_len; p_rb = cur.rb; p_h0 = cur.h0;
     have_prev = true;
     if (!more) break;
     cur = nxt;
-    nxt = next_item(walk_c);
+    nxt = item_at(ci++);
   }
   if (GRP == 0) pp_barrier();                   // group 1's last interval
   vm_wait<0>();
-  store_item(p_seq_start, p_seq_len, p_rb, p_y, l_prev);
+  write_out(p_seq_start, p_seq_len, p_rb, p_h0);
+#if MVLLM_PP_TIMELINE
+  if (a.timeline != nullptr && a.timeline_block < 0 && wave == 4 && lane == 0) {
+    unsigned long long* e = a.timeline + 4 * (size_t)blockIdx.x;
+    e[0] = t_begin;
+    e[1] = __builtin_amdgcn_s_memtime();
+    e[2] = (unsigned long long)t_items;
+    e[3] = (unsigned long long)t_tiles;
+  }
+#endif
 }
 
 template <typename T, int D>
@@ -656,6 +768,9 @@ int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) 
   }
   const int grid = cus / 8 * 8 > 0 ? cus / 8 * 8 : 8;
   a.team_size = grid / n_teams;
+  auto magic = [](int d) { return d <= 1 ? 0u : (unsigned)(((uint64_t)1 << 32) / (uint64_t)d + 1u); };
+  a.spt_magic = magic(a.slices / n_teams);
+  a.chunks_magic = magic(group / 4);
   a.level_bits = 1;
   while (((int64_t)1 << a.level_bits) <= a.total_tokens / 64 + 1) ++a.level_bits;
   if (dtype == MVLLM_BF16) prefill_pp_kernel<bf16_t, 128><<<dim3(grid), dim3(64 * kPpWaves), 0, stream>>>(a);
@@ -668,6 +783,8 @@ int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) 
 #if MVLLM_PP_TIMELINE
 // Probe library only: the two-group prefill with the clock stamps of workgroup `block` written to `log`
 // ([8 waves][entries_per_wave] 64-bit shader clocks; entries past a wave's last stamp stay as the caller filled them).
+// block < 0: `log` receives {begin, end, items, tiles} of every workgroup instead (4 entries each, grid x 4 in all;
+// the grid is the CU count rounded down to a multiple of 8).
 extern "C" int mvllm_probe_prefill_timeline(void* out, const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
                                             int num_seqs, int64_t total_tokens, int num_heads, int num_kv_heads, int head_dim,
                                             float scale, int dtype, unsigned long long* log, int entries_per_wave, int block,
@@ -680,7 +797,7 @@ extern "C" int mvllm_probe_prefill_timeline(void* out, const void* q, const void
   PrefillPpArgs p;
   p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
   p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
-  p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0;
+  p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0; p.spt_magic = 0; p.chunks_magic = 0;
   p.timeline = log; p.timeline_entries = entries_per_wave; p.timeline_block = block;
   return launch_prefill_pp(p, dtype, (hipStream_t)stream);
 }

@@ -828,7 +828,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
     PrefillPpArgs p;
     p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
     p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
-    p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0;
+    p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0; p.spt_magic = 0; p.chunks_magic = 0;
     p.timeline = nullptr; p.timeline_entries = 0; p.timeline_block = 0;
     return launch_prefill_pp(p, dtype, (hipStream_t)stream);
   }
