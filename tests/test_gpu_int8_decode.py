@@ -36,7 +36,7 @@ def _quantised_case(seed, batch, ctx_lo, ctx_hi, hq, hkv, d, bs, dtype=torch.bfl
 def _check(case, hq, hkv, d, bs, scale, ctx_dtype=torch.int64):
     """Max-abs 2e-2 / mean-abs 2e-3 against the fp32 oracle on the dequantised cache, with one allowance: the kernel's
     output is 16 bits wide, and these small cases (a handful of keys, 1 % of them 8-sigma outliers) have outputs of
-    magnitude 4 to 10, where half a bf16 step alone (|want| * 2^-9) is 0.008 to 0.02.  One bf16 step of the value is
+    magnitude 4 to 10, where half a bf16 step alone (|want| * 2^-9) is 0.008 to 0.02.  That half step of the value is
     therefore taken off the difference before it is held against 2e-2.  The full-size configuration-4 test, whose
     outputs average thousands of keys, uses the bound as stated."""
     q, ck, cv, sk, sv, tables, ctx = case
@@ -46,7 +46,7 @@ def _check(case, hq, hkv, d, bs, scale, ctx_dtype=torch.int64):
                                      hq, hkv, d, bs)
     mx, mean = error_stats(got, want)
     assert got.dtype == q.dtype and torch.isfinite(got).all()
-    excess = ((got.float() - want).abs() - want.abs() * 2.0 ** -8).max().item()
+    excess = ((got.float() - want).abs() - want.abs() * (2.0 ** -9 if got.dtype == torch.bfloat16 else 2.0 ** -12)).max().item()
     assert excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
     return got
 
@@ -119,7 +119,7 @@ def test_int8_both_grid_forms(hq, hkv, bs, d, form):
     got = paged_attention_decode_int8(q.to(DEV), ck, cv, sk, sv, wide.to(DEV), ctx.to(DEV), scale, hq, hkv, d, bs).cpu()
     want = oracle.decode_int8_oracle(q.float(), ck.cpu(), cv.cpu(), sk.cpu(), sv.cpu(), tables, ctx, scale, hq, hkv, d, bs)
     mx, mean = error_stats(got, want)
-    excess = ((got.float() - want).abs() - want.abs() * 2.0 ** -8).max().item()
+    excess = ((got.float() - want).abs() - want.abs() * (2.0 ** -9 if got.dtype == torch.bfloat16 else 2.0 ** -12)).max().item()
     assert torch.isfinite(got).all() and excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
 
 
