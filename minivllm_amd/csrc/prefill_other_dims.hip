@@ -1,0 +1,28 @@
+// The LDS-tiled MFMA prefill kernel for head dimensions 32, 80, 96 and 112: the same kernel as for 64 and 128, in the
+// tile layout of the next of those two (the reference picks its tile sizes by head_dim and covers every size:
+// src/myvllm/layers/attention.py:249-257).  A translation unit of its own so that its 48 instances compile next to
+// the others.
+#include "prefill_mfma.h"
+
+namespace mvllm {
+
+bool prefill_mfma_other_dim(int head_dim) { return head_dim == 32 || head_dim == 80 || head_dim == 96 || head_dim == 112; }
+
+template <typename T, bool PAGED>
+static int launch_other(const PrefillArgs& a, hipStream_t stream) {
+  switch (a.head_dim) {
+    case 32: return launch_prefill_mfma_as<T, PAGED, false, 64, 32>(a, stream);
+    case 80: return launch_prefill_mfma_as<T, PAGED, false, 128, 80>(a, stream);
+    case 96: return launch_prefill_mfma_as<T, PAGED, false, 128, 96>(a, stream);
+    case 112: return launch_prefill_mfma_as<T, PAGED, false, 128, 112>(a, stream);
+    default: return MVLLM_ERR_UNSUPPORTED;
+  }
+}
+
+int launch_prefill_mfma_other(const PrefillArgs& a, int dtype, bool paged, hipStream_t stream) {
+  if (dtype == MVLLM_BF16) return paged ? launch_other<bf16_t, true>(a, stream) : launch_other<bf16_t, false>(a, stream);
+  if (dtype == MVLLM_F16) return paged ? launch_other<f16_t, true>(a, stream) : launch_other<f16_t, false>(a, stream);
+  return MVLLM_ERR_UNSUPPORTED;
+}
+
+}  // namespace mvllm
