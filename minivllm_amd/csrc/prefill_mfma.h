@@ -125,7 +125,7 @@ __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, in
 // steps and never reads them, the second one carries them through the output columns DD .. 32 ceil(DD / 32) - 1 of
 // its last block, which are not stored.
 template <typename T, int HPW, bool PAGED, int D, bool I8 = false, int DD = D>
-__global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const PrefillArgs a) {
+__global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_kernel(const PrefillArgs a) {
   static_assert(!I8 || PAGED, "INT8 caches are paged");
   static_assert(DD % 16 == 0 && DD <= D && (!I8 || DD == D), "head dims in steps of 16, INT8 only at 64 and 128");
   constexpr int kRowB = D * 2;                  // bytes per tile row
@@ -136,12 +136,12 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   constexpr int kTD = (DD + 31) / 32;           // 32-dim blocks of the output
   // K rows are read 16 at a time with the same logical chunk: the swizzle spreads them over the banks.  With 128-byte
   // rows two rows share a 256-byte bank line, so the row index is halved first.
-  auto kswz = [](int row) __attribute__((always_inline)) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
+  auto kswz = [](int row) __attribute__((always_inline)) { return D >= 128 ? (row & 15) : ((row >> 1) & 7); };
   // V is read by the transposing loads as 4 rows x 64 bytes per 16 lanes: bits 2-3 of the chunk index take the row's
   // low bits so that the four rows land in four 64-byte groups.  Bit 0 (D = 128) swaps the chunks of a pair in odd
   // rows; the reads do not care (the pair stays in its group), and the INT8 conversion's LDS writes, which go two rows
   // x four quarters at a time over 128 bytes of banks, meet 2-way instead of 4-way (32 -> 16 clocks per write).
-  auto vswz = [](int row) __attribute__((always_inline)) { return D == 128 ? (((row & 3) << 2) | (row & 1)) : (((row >> 1) & 1) << 2); };
+  auto vswz = [](int row) __attribute__((always_inline)) { return D >= 128 ? (((row & 3) << 2) | (row & 1)) : (((row >> 1) & 1) << 2); };
   constexpr int ROW_TILES = kPfWaves / HPW;     // 32-row query tiles per workgroup
   constexpr int ROWS_PER_WAVE = kBN / kPfWaves; // K/V tile rows one wave copies (4 per instruction)
   constexpr int BM = kWaveRows * ROW_TILES;     // query rows per workgroup
@@ -393,14 +393,19 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
   //   V: row 4*hi + (lane&15)/4 (+8, +16*st, +32*tk rows), chunk (4*td + 2*half + ...) ^ (4*(row & 3) | (row & 1))
   const int i16 = lane & 15;
   const int half = (lane >> 4) & 1;
-  int k_off[kKS];
+  // (The swizzles are xors on the low four bits of the chunk index, so with 32 chunks per row (head_dim 256) the
+  // offsets of step ks + 8 and block td + 4 are those of ks and td plus 256 bytes: an immediate, not another register.)
+  constexpr int kKOffs = kKS > 8 ? 8 : kKS, kVOffs = kTD > 4 ? 4 : kTD;
+  int k_off_[kKOffs];
 #pragma unroll
-  for (int ks = 0; ks < kKS; ++ks) k_off[ks] = l32 * kRowB + (((2 * ks + hi) ^ kswz(l32)) << 4);
+  for (int ks = 0; ks < kKOffs; ++ks) k_off_[ks] = l32 * kRowB + (((2 * ks + hi) ^ kswz(l32)) << 4);
+  auto k_off = [&](int ks) __attribute__((always_inline)) { return k_off_[ks & 7] + (ks >> 3) * 256; };
   const int v_row = 4 * hi + (i16 >> 2);
-  int v_off[kTD];
+  int v_off_[kVOffs];
 #pragma unroll
-  for (int td = 0; td < kTD; ++td)
-    v_off[td] = v_row * kRowB + (((4 * td + 2 * half + ((i16 & 3) >> 1)) ^ vswz(v_row)) << 4) + ((i16 & 1) << 3);
+  for (int td = 0; td < kVOffs; ++td)
+    v_off_[td] = v_row * kRowB + (((4 * td + 2 * half + ((i16 & 3) >> 1)) ^ vswz(v_row)) << 4) + ((i16 & 1) << 3);
+  auto v_off = [&](int td) __attribute__((always_inline)) { return v_off_[td & 3] + (td >> 2) * 256; };
 
   // One K/V tile: scores, softmax, P.V.  Compile-time parameters: BUF, the buffer index (so that all LDS
   // addresses are register + constant); DIAG, set for the wave's last tile, the one the causal diagonal runs
@@ -426,13 +431,13 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       // across, so reads placed after it would be issued right before their use and wait out the LDS latency.
       uint4 kf[2][NH];
 #pragma unroll
-      for (int tk = 0; tk < NH; ++tk) kf[0][tk] = *reinterpret_cast<const uint4*>(kb + k_off[0] + tk * 32 * kRowB);
+      for (int tk = 0; tk < NH; ++tk) kf[0][tk] = *reinterpret_cast<const uint4*>(kb + k_off(0) + tk * 32 * kRowB);
       static_for<kKS>([&](auto KS) {
         constexpr int ks = decltype(KS)::value;
         if constexpr (ks + 1 < kKS) {
 #pragma unroll
           for (int tk = 0; tk < NH; ++tk)
-            kf[(ks + 1) & 1][tk] = *reinterpret_cast<const uint4*>(kb + k_off[ks + 1] + tk * 32 * kRowB);
+            kf[(ks + 1) & 1][tk] = *reinterpret_cast<const uint4*>(kb + k_off(ks + 1) + tk * 32 * kRowB);
           __builtin_amdgcn_sched_barrier(0);   // keep the reads in front of this step's MFMAs
         }
 #pragma unroll
@@ -516,7 +521,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_mfma_kernel(const Pr
       uint4 af[kTD];
 #pragma unroll
       for (int td = 0; td < kTD; ++td) {
-        const char* p0 = vb + v_off[td] + (32 * tk + 16 * st) * kRowB;
+        const char* p0 = vb + v_off(td) + (32 * tk + 16 * st) * kRowB;
         const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
         const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * kRowB));
         af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;

@@ -6,7 +6,9 @@
 
 namespace mvllm {
 
-bool prefill_mfma_other_dim(int head_dim) { return head_dim == 32 || head_dim == 80 || head_dim == 96 || head_dim == 112; }
+bool prefill_mfma_other_dim(int head_dim) {
+  return head_dim == 32 || head_dim == 80 || head_dim == 96 || head_dim == 112 || head_dim == 256;
+}
 
 template <typename T, bool PAGED>
 static int launch_other(const PrefillArgs& a, hipStream_t stream) {
@@ -15,6 +17,7 @@ static int launch_other(const PrefillArgs& a, hipStream_t stream) {
     case 80: return launch_prefill_mfma_as<T, PAGED, false, 128, 80>(a, stream);
     case 96: return launch_prefill_mfma_as<T, PAGED, false, 128, 96>(a, stream);
     case 112: return launch_prefill_mfma_as<T, PAGED, false, 128, 112>(a, stream);
+    case 256: return launch_prefill_mfma_as<T, PAGED, false, 256, 256>(a, stream);
     default: return MVLLM_ERR_UNSUPPORTED;
   }
 }

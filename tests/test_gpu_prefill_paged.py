@@ -52,6 +52,7 @@ def _check(got, want, dtype):
     (6, 3, 112, 32, [131, 260], [50, 259]),                        # head_dim 112, two query heads per kv head
     (4, 4, 32, 16, [200, 70], [160, 32]),                          # head_dim 32 in the 64 layout
     (8, 2, 80, 16, [140, 23], [16, 8]),                            # head_dim 80, blocks of 16: the tiled kernel
+    (8, 2, 256, 16, [300, 64, 129], [256, 0, 17]),                 # head_dim 256: 512-byte tile rows
     (4, 4, 64, 16, [70], [32]),                                    # head_dim 64: 16-row tiles (fp32: generic kernel)
     (16, 8, 64, 16, [300, 64, 129, 500], [256, 0, 17, 48]),        # head_dim 64, the reference demo's heads
     (12, 1, 64, 256, [700, 30, 257], [512, 29, 0]),                # head_dim 64, one kv head, the engine's block size
