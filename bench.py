@@ -598,7 +598,8 @@ def bench_demo_shape(args):
 
 def bench_other_head_dims(args):
     """bf16 head dims beside 64 and 128 that run on matrix-unit kernels (32, 80, 96, 112, 256: the decode kernels and
-    the LDS-tiled prefill) and one that does not (72: the generic kernels), on the demo leg's batch: decode of 64
+    the LDS-tiled prefill; 72: the decode kernels and the 16-row tile prefill) and one that does not (100: the generic
+    kernels), on the demo leg's batch: decode of 64
     sequences of 1000-3000 tokens, prefill of 16 prompts of 64-2048 tokens, 16 query / 8 kv heads."""
     import torch
     from helpers import make_paged_case_on_device, make_varlen_case
@@ -609,11 +610,11 @@ def bench_other_head_dims(args):
     g = torch.Generator().manual_seed(args.seed)
     lengths = torch.randint(64, 2049, (16,), generator=g).tolist()
     out = {"workload": "bf16, Hq16 Hkv8: decode B64 ctx~U[1000,3000] block_size 16; prefill 16 prompts L~U[64,2048]"}
-    for d in (32, 80, 96, 112, 256, 72):
+    for d in (32, 80, 96, 112, 256, 72, 100):
         q, kc, vc, tables, ctx = make_paged_case_on_device(args.seed, dev, 64, 1000, 3000, hq, hkv, d, bs,
                                                            dtype=torch.bfloat16, log_uniform=False)
         td, cd = tables.to(dev), ctx.to(dev)
-        steps = args.steps if d != 72 else 3                       # the generic kernels are slow
+        steps = args.steps if d != 100 else 3                      # the generic kernels are slow
         _, ms = time_steps(lambda: paged_attention_decode(q, kc, vc, td, cd, 1 / math.sqrt(d), hq, hkv, d, bs),
                            steps, min(args.warmup, steps), 0.0)
         nbytes = int(ctx.sum()) * hkv * d * 2 * kc.element_size()

@@ -1462,11 +1462,32 @@ static size_t workspace_bytes_for(int batch, int num_heads, int head_dim, int ma
   return (size_t)batch * (size_t)np * (size_t)num_heads * (size_t)(head_dim + 2) * sizeof(float);
 }
 
+// Head dims the 16-bit MFMA kernels (decode, 16-row tile prefill) have instances for beside 64 and 128: the multiples
+// of 8 from 32 to 120 (a last 32-dim step that is partial loads nothing past the row's end) and 256.
+static bool other_mfma_dim(int head_dim) { return head_dim == 256 || (head_dim >= 32 && head_dim < 128 && head_dim % 8 == 0 && head_dim != 64); }
+template <typename F>
+static void with_other_mfma_dim(int head_dim, F&& go) {
+  switch (head_dim) {
+    case 32: go(std::integral_constant<int, 32>{}); break;
+    case 40: go(std::integral_constant<int, 40>{}); break;
+    case 48: go(std::integral_constant<int, 48>{}); break;
+    case 56: go(std::integral_constant<int, 56>{}); break;
+    case 72: go(std::integral_constant<int, 72>{}); break;
+    case 80: go(std::integral_constant<int, 80>{}); break;
+    case 88: go(std::integral_constant<int, 88>{}); break;
+    case 96: go(std::integral_constant<int, 96>{}); break;
+    case 104: go(std::integral_constant<int, 104>{}); break;
+    case 112: go(std::integral_constant<int, 112>{}); break;
+    case 120: go(std::integral_constant<int, 120>{}); break;
+    case 256: go(std::integral_constant<int, 256>{}); break;
+    default: break;
+  }
+}
+
 // shapes the MFMA kernels are built for (pointer alignment is checked by the caller)
 static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool int8) {
-  // 16-bit caches: 32, 64, 80, 96, 112, 128 or 256 dims per head; fp32 and INT8 caches: 64 or 128
-  const bool dim_ok = head_dim == 128 || head_dim == 64 ||
-                      (dtype != MVLLM_F32 && !int8 && (head_dim == 256 || head_dim == 112 || head_dim == 96 || head_dim == 80 || head_dim == 32));
+  // 16-bit caches: a multiple of 8 from 32 to 128, or 256, dims per head; fp32 and INT8 caches: 64 or 128
+  const bool dim_ok = head_dim == 128 || head_dim == 64 || (dtype != MVLLM_F32 && !int8 && other_mfma_dim(head_dim));
   return (dtype != MVLLM_F32 || !int8) && dim_ok && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
          (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
 }
@@ -1508,13 +1529,7 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
     };
     if (a.head_dim == 128) go(std::integral_constant<int, 128>{});
     else if (a.head_dim == 64) go(std::integral_constant<int, 64>{});
-    if constexpr (IsSixteenBit<T>::value) {         // 16-bit caches also with 32, 96 and 256 dims per head
-      if (a.head_dim == 256) go(std::integral_constant<int, 256>{});
-      else if (a.head_dim == 96) go(std::integral_constant<int, 96>{});
-      else if (a.head_dim == 80) go(std::integral_constant<int, 80>{});
-      else if (a.head_dim == 112) go(std::integral_constant<int, 112>{});
-      else if (a.head_dim == 32) go(std::integral_constant<int, 32>{});
-    }
+    if constexpr (IsSixteenBit<T>::value) with_other_mfma_dim(a.head_dim, go);    // 16-bit caches only
   }
   if constexpr (IsSixteenBit<T>::value) {           // the INT8 kernels take 16-bit queries
     if (fast_ok && int8) {
@@ -1612,7 +1627,7 @@ static void launch_rows16(const PrefillRowsArgs& a, dim3 grid, int tiles, hipStr
 }
 bool prefill_rows16_takes(int head_dim, int dtype, bool int8_cache) {
   if (head_dim == 64 || head_dim == 128) return true;
-  return (head_dim == 32 || head_dim == 80 || head_dim == 96 || head_dim == 112 || head_dim == 256) && dtype != MVLLM_F32 && !int8_cache;
+  return other_mfma_dim(head_dim) && dtype != MVLLM_F32 && !int8_cache;
 }
 int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hipStream_t stream) {
   if (!prefill_rows16_takes(head_dim, dtype, a.k_scale != nullptr)) return MVLLM_ERR_UNSUPPORTED;
@@ -1631,11 +1646,7 @@ int launch_prefill_rows16(const PrefillRowsArgs& a, int head_dim, int dtype, hip
     };
     if (head_dim == 64) go(std::integral_constant<int, 64>{});
     else if (head_dim == 128) go(std::integral_constant<int, 128>{});
-    else if (head_dim == 32) go(std::integral_constant<int, 32>{});
-    else if (head_dim == 96) go(std::integral_constant<int, 96>{});
-    else if (head_dim == 80) go(std::integral_constant<int, 80>{});
-    else if (head_dim == 112) go(std::integral_constant<int, 112>{});
-    else go(std::integral_constant<int, 256>{});
+    else with_other_mfma_dim(head_dim, go);
   }
   return launch_status();
 }

@@ -1,19 +1,20 @@
-// The LDS-tiled MFMA prefill kernel for head dimensions 32, 80, 96 and 112: the same kernel as for 64 and 128, in the
-// tile layout of the next of those two (the reference picks its tile sizes by head_dim and covers every size:
-// src/myvllm/layers/attention.py:249-257).  A translation unit of its own so that its 48 instances compile next to
-// the others.
+// The LDS-tiled MFMA prefill kernel for head dimensions 32, 48, 80, 96 and 112 (the same kernel as for 64 and 128, in
+// the tile layout of the next of those two) and 256 (a layout of its own).  The reference picks its tile sizes by
+// head_dim and covers every size (src/myvllm/layers/attention.py:249-257).  A translation unit of its own so that
+// its instances compile next to the others.
 #include "prefill_mfma.h"
 
 namespace mvllm {
 
 bool prefill_mfma_other_dim(int head_dim) {
-  return head_dim == 32 || head_dim == 80 || head_dim == 96 || head_dim == 112 || head_dim == 256;
+  return head_dim == 32 || head_dim == 48 || head_dim == 80 || head_dim == 96 || head_dim == 112 || head_dim == 256;
 }
 
 template <typename T, bool PAGED>
 static int launch_other(const PrefillArgs& a, hipStream_t stream) {
   switch (a.head_dim) {
     case 32: return launch_prefill_mfma_as<T, PAGED, false, 64, 32>(a, stream);
+    case 48: return launch_prefill_mfma_as<T, PAGED, false, 64, 48>(a, stream);
     case 80: return launch_prefill_mfma_as<T, PAGED, false, 128, 80>(a, stream);
     case 96: return launch_prefill_mfma_as<T, PAGED, false, 128, 96>(a, stream);
     case 112: return launch_prefill_mfma_as<T, PAGED, false, 128, 112>(a, stream);

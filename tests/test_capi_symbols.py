@@ -58,6 +58,7 @@ def test_host_only_entry_points():
 
 def test_decode_plan_is_host_arithmetic():
     """Which form a decode call takes, and that the split form never needs more workspace than is advertised."""
+    import torch
     from minivllm_amd.layers.attention import paged_decode_plan
     lib = _lib().load()
     # one-wave-per-head form: large batch over a wide table (1024-token partitions)
@@ -76,12 +77,13 @@ def test_decode_plan_is_host_arithmetic():
     assert paged_decode_plan(64, 16, 16, 96, 256, 16, int8_cache=True)[2] == 0
     assert paged_decode_plan(64, 16, 16, 96, 256, 16)[2] == 4                 # 16-bit caches: also 96 dims (three 32-dim steps)
     assert paged_decode_plan(64, 16, 16, 80, 256, 16)[2] == 4 and paged_decode_plan(64, 16, 16, 112, 256, 16)[2] == 4   # ... and a partial last step
-    assert paged_decode_plan(64, 16, 16, 72, 256, 16)[2] == 0                 # other head dims
+    assert paged_decode_plan(64, 16, 16, 72, 256, 16)[2] == 4 and paged_decode_plan(64, 16, 16, 120, 256, 16)[2] == 4   # any multiple of 8 from 32 to 128
+    assert paged_decode_plan(64, 16, 16, 100, 256, 16)[2] == 0 and paged_decode_plan(64, 16, 16, 136, 256, 16)[2] == 0   # other head dims
+    assert paged_decode_plan(64, 16, 16, 72, 256, 16, dtype=torch.float32)[2] == 0
     assert paged_decode_plan(64, 16, 8, 256, 256, 16)[2] == 4                 # 16-bit caches: also 256 and 32 dims
     assert paged_decode_plan(64, 16, 8, 32, 256, 16)[2] == 4
     assert paged_decode_plan(64, 16, 8, 256, 256, 16, int8_cache=True)[2] == 0
     assert paged_decode_plan(64, 16, 8, 256, 256, 16, dtype=__import__("torch").float32)[2] == 0
-    import torch
     assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32)[2] == 4       # fp32 caches: fp32 MFMA
     assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32, int8_cache=True)[2] == 0
     assert paged_decode_plan(8, 34, 2, 128, 64, 16)[2] == 0                   # 17 query heads per kv head
@@ -106,7 +108,7 @@ def test_prefill_plan_is_host_arithmetic():
     assert prefill_plan(8, 8, 256, dtype=torch.float32) == 0
     assert prefill_plan(6, 2, 80) == 2 and prefill_plan(6, 2, 96) == 2 and prefill_plan(6, 2, 96, dtype=torch.float32) == 0
     assert prefill_plan(6, 2, 112, block_size=16) == 2 and prefill_plan(6, 2, 112, block_size=8) == 0
-    assert prefill_plan(6, 2, 72) == 0
+    assert prefill_plan(6, 2, 72) == 1 and prefill_plan(6, 2, 40) == 1 and prefill_plan(6, 2, 48) == 2 and prefill_plan(6, 2, 100) == 0
     assert prefill_plan(32, 8, 128, 16, int8_cache=True) == 2
     assert prefill_plan(32, 8, 96, 16, int8_cache=True) == -1 and prefill_plan(32, 8, 128, 16, torch.float32, True) == -1
     assert prefill_plan(8, 8, 1024) == -1
@@ -119,9 +121,9 @@ def test_generic_kernel_warning_is_raised_once_per_shape():
     attention._shapes_seen.clear()
     with warnings.catch_warnings(record=True) as seen:
         warnings.simplefilter("always")
-        attention._warn_if_generic("decode", 16, 16, 72, 16, torch.bfloat16, False)
-        attention._warn_if_generic("decode", 16, 16, 72, 16, torch.bfloat16, False)      # same shape: silent
-        attention._warn_if_generic("prefill", 6, 2, 72, 0, torch.bfloat16, False)
+        attention._warn_if_generic("decode", 16, 16, 100, 16, torch.bfloat16, False)
+        attention._warn_if_generic("decode", 16, 16, 100, 16, torch.bfloat16, False)      # same shape: silent
+        attention._warn_if_generic("prefill", 6, 2, 100, 0, torch.bfloat16, False)
         attention._warn_if_generic("decode", 32, 8, 128, 16, torch.bfloat16, False)      # MFMA kernel: silent
         attention._warn_if_generic("prefill", 32, 8, 128, 0, torch.bfloat16, False)
     assert len(seen) == 2 and all("generic kernel" in str(w.message) for w in seen)

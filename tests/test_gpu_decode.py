@@ -244,14 +244,15 @@ def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, d, form):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("hq,hkv,bs,d", [(16, 8, 16, 256), (8, 1, 32, 256), (5, 5, 48, 256), (16, 8, 16, 32), (12, 2, 256, 32),
                                          (32, 8, 16, 96), (6, 6, 48, 96), (12, 1, 256, 96), (32, 8, 16, 80), (5, 5, 48, 112),
-                                         (12, 1, 256, 80), (16, 2, 32, 112)])
+                                         (12, 1, 256, 80), (16, 2, 32, 112), (16, 8, 16, 72), (6, 2, 32, 88), (8, 8, 16, 40),
+                                         (12, 3, 48, 104), (16, 4, 16, 120), (8, 2, 16, 48), (10, 2, 16, 56)])
 @pytest.mark.parametrize("form", ["one wave per head", "waves share a head", "waves share a head, one partition"])
 def test_head_dim_256_96_and_32_on_the_mfma_kernels(dtype, hq, hkv, bs, d, form):
     """The other head dims the reference's kernels take (attention.py:249-257, 453) that are a multiple of 32: with 256
     dims a lane owns two sets of eight output dims and the first product has eight 32-dim steps; with 96 there are three
     steps and twelve of the sixteen output columns, with 80 and 112 the last step is partial (the lanes past the row's
-    end load nothing), with 32 one step and four columns.  Both kernel forms, ragged
-    contexts, one empty."""
+    end load nothing), with 32 one step and four columns; every other multiple of 8 between 32 and 128 likewise.  Both
+    kernel forms, ragged contexts, one empty."""
     batch = 7 if form == "waves share a head" else 64
     width = {"one wave per head": 32768, "waves share a head": 8192}.get(form, 4096) // bs * bs
     g = torch.Generator().manual_seed(177)

@@ -31,7 +31,8 @@ def _oracle32(q, k, v, cu, scale, hq, hkv, d):
     (8, 8, 128, [200]),
     (16, 16, 64, [60, 60]),             # the reference demo's head_dim
     (6, 2, 80, [17, 5]),                # 16-bit: the 16-row tile kernel with a partial last step; fp32: generic
-    (6, 2, 72, [17, 5]),                # a head_dim no matrix-unit kernel takes
+    (6, 2, 72, [17, 5]),                # 16-bit: the 16-row tile kernel, the last step half empty; fp32: generic
+    (6, 2, 100, [17, 5]),               # a head_dim no matrix-unit kernel takes
     (6, 2, 128, [300, 17, 64]),         # three query heads per kv head: one head per workgroup
     (10, 2, 128, [33, 129]),            # five
 ])
@@ -53,7 +54,7 @@ def test_prefill_vs_oracle(dtype, hq, hkv, d, lengths):
     (8, 4, 32, [64, 17, 130]), (8, 2, 96, [70, 1, 33, 129]), (6, 6, 96, [200]), (8, 2, 80, [70, 1, 33, 129]),
     (6, 3, 112, [200, 17]),
     (32, 8, 96, [300, 64, 1, 129, 513]), (16, 2, 112, [1000, 17]), (4, 1, 80, [257, 256, 255]), (16, 16, 32, [90, 700]),
-    (8, 2, 256, [70, 1, 33, 129]), (4, 4, 256, [200]), (6, 3, 256, [300, 65, 700]),
+    (8, 2, 256, [70, 1, 33, 129]), (4, 4, 256, [200]), (6, 3, 256, [300, 65, 700]), (4, 4, 48, [200]), (8, 2, 48, [70, 1, 33, 129]),
 ])
 def test_prefill_head_dim_32_80_96_112_256_on_the_lds_tiled_kernel(dtype, hq, hkv, d, lengths):
     """The tiled kernel in the layout of the next larger of 64 / 128 (the reference's kernel takes any head_dim by
@@ -66,6 +67,22 @@ def test_prefill_head_dim_32_80_96_112_256_on_the_lds_tiled_kernel(dtype, hq, hk
     scale = 1 / math.sqrt(d)
     got = _run(*case, scale, hq, hkv, d)
     assert torch.isfinite(got.float()).all()
+    mx, mean = error_stats(got, _oracle32(*case, scale, hq, hkv, d))
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,d,lengths", [(8, 2, 40, [70, 1, 33, 129]), (8, 4, 56, [64, 17, 130]),
+                                              (8, 2, 72, [70, 1, 33, 129]), (6, 3, 88, [200, 17]), (6, 6, 104, [150]),
+                                              (8, 2, 120, [70, 1, 33, 129])])
+def test_prefill_head_dims_that_are_multiples_of_8_on_the_16_row_tile_kernel(dtype, hq, hkv, d, lengths):
+    """Multiples of 8 that are not multiples of 32: the lanes of the last 32-dim step whose dims lie past the head load
+    neither K nor Q (what follows in memory is the next head, not zeros)."""
+    from minivllm_amd.layers.attention import prefill_plan
+    assert prefill_plan(hq, hkv, d, 0, dtype) == 1
+    case = make_varlen_case(57, lengths, hq, hkv, d, dtype=dtype)
+    scale = 1 / math.sqrt(d)
+    got = _run(*case, scale, hq, hkv, d)
     mx, mean = error_stats(got, _oracle32(*case, scale, hq, hkv, d))
     assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
 
