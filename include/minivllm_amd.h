@@ -98,8 +98,8 @@ size_t mvllm_paged_decode_workspace_bytes(int batch, int num_heads, int head_dim
  *   *waves_per_head   1: a workgroup holds up to 4 kv heads, one wave each, and every wave walks its partition;
  *                     >1: small-batch form, a workgroup is that many waves on one kv head that share the
  *                     partition's 16-token tiles and merge in LDS; 0: the generic kernel (head_dim other than
- *                     128 or 64 (bf16 / fp16 caches: also 32, 80, 96, 112 and 256), block_size % 16 != 0, more than 16 query
- *                     heads per kv head, or fp32 queries over an INT8 cache)
+ *                     128 or 64 (bf16 / fp16 caches: also every other multiple of 8 from 32 to 120, and 256),
+ *                     block_size % 16 != 0, more than 16 query heads per kv head, or fp32 queries over an INT8 cache)
  * Returns MVLLM_OK or MVLLM_ERR_BAD_SHAPE / MVLLM_ERR_BAD_DTYPE.
  */
 int mvllm_paged_decode_plan(int batch, int num_heads, int num_kv_heads, int head_dim,
