@@ -155,6 +155,36 @@ def test_prefill_item_order_covers_every_tile(hq, hkv, num_seqs):
     assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
 
 
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (24, 2), (8, 2), (12, 3), (4, 1)])
+@pytest.mark.parametrize("num_seqs", [1, 7, 64])
+def test_two_group_prefill_deals_every_item_once(hq, hkv, num_seqs):
+    """The two-group kernel (head_dim 128, a multiple of 4 query heads per kv head, at most 64 sequences): one to three
+    slices of four query heads per kv head, 1 / 2 / 3 / 6 / 8 / 16 slices in 1 / 2 / 8 teams of workgroups, rounds dealt
+    forwards, backwards and a short last round backwards.  Ragged lengths around the block boundaries, empty sequences and
+    one long prompt; the output starts as NaN, so an item that no workgroup took would show, and an item taken twice or
+    with the wrong heads would be wrong against the oracle."""
+    d = 128
+    g = torch.Generator().manual_seed(900 + 7 * num_seqs + hq)
+    pool = [0, 1, 31, 32, 33, 63, 64, 65, 127, 128, 129, 191, 192, 193, 257, 300, 448]
+    lengths = [pool[i] for i in torch.randint(0, len(pool), (num_seqs,), generator=g).tolist()]
+    lengths[num_seqs // 2] = 2100 if hq <= 32 else 700           # 33 (or 11) blocks of 64 rows
+    q, k, v, cu = make_varlen_case(58, lengths, hq, hkv, d, dtype=torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    from minivllm_amd import _C
+    out = torch.full_like(q, float("nan")).to(DEV)
+    qd, kd, vd, cud = (t.to(DEV) for t in (q, k, v, cu))
+    st = _C.load().mvllm_prefill_varlen(out.data_ptr(), qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), cud.data_ptr(),
+                                        num_seqs, q.shape[0], hq, hkv, d, scale, _C.dtype_code(q.dtype),
+                                        _C.current_stream_ptr(out.device))
+    torch.cuda.synchronize()
+    assert st == 0
+    got = out.cpu()
+    assert torch.isfinite(got).all()
+    want = _oracle32(q, k, v, cu, scale, hq, hkv, d)
+    mx, mean = error_stats(got, want)
+    assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
 def test_config2_full_size():
     """BASELINE.json config 2: 16 prompts L U[64,2048], Hq32/Hkv8/D128 bf16; store into block-256 cache; the last
     row of each prompt must agree with a paged decode of that token over the stored cache."""
