@@ -179,8 +179,8 @@ int mvllm_prefill_varlen(void* out, const void* q, const void* k, const void* v,
  * Which kernel a prefill of these static sizes runs on (no counterpart in the reference, whose Triton kernels take any
  * power-of-two head_dim from a tile-size table, attention.py:249-257).  block_size 0 = the packed entry point,
  * > 0 = the paged ones.  *kernel: 2 an LDS-tiled MFMA kernel (bf16 / fp16 with head_dim 32, 48, 64, 80, 96, 112, 128
- * or 256; over an INT8 cache 64 or 128; the packed entry point runs its two-group form where head_dim is 128, the query
- * heads per kv head are a multiple of 4 and the batch has at most 64 sequences), 1 the 16-row tile MFMA kernel (fp32
+ * or 256; over an INT8 cache 64 or 128; the packed and the 16-bit paged entry point run its two-group form where head_dim
+ * is 128, the query heads per kv head are a multiple of 4 and the batch has at most 64 sequences), 1 the 16-row tile MFMA kernel (fp32
  * with head_dim 128 or 64; bf16 / fp16 with 40, 56, 72, 88, 104 or 120), 0 the generic kernel (any head_dim <= 512; one key per step, a correctness path two orders
  * of magnitude slower), -1 unsupported.
  * Pointers are assumed 16-byte aligned (unaligned ones take the generic kernel).  Pure host arithmetic.
@@ -202,8 +202,7 @@ int mvllm_prefill_plan(int num_heads, int num_kv_heads, int head_dim, int block_
  * c_s + r, c_s = len_k(s) - len_q(s), and attends keys 0 .. c_s + r.  The first ceil(len_k/bs) table
  * entries of a sequence are expected to be valid; an entry < 0 or >= num_blocks there is not followed (no
  * out-of-range access): its keys and values read as zeros.  With c_s = 0 for every s the result equals
- * mvllm_prefill_varlen's: bit for bit where that call runs the same one-group kernel, to within rounding where it
- * runs the two-group form (the row sums are formed in a different order there).
+ * mvllm_prefill_varlen bit for bit (block sizes that are multiples of 16: both calls then run the same kernel).
  */
 int mvllm_prefill_paged(void* out, const void* q, const void* k_cache, const void* v_cache,
                         const int32_t* block_tables, int max_num_blocks,

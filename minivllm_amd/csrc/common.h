@@ -223,7 +223,15 @@ struct PrefillPpArgs {
   int num_heads;
   int num_kv_heads;
   float scale_log2;
+  // paged mode (block_tables != null): k, v are caches [num_blocks, block_size, Hkv, D]; q, out and cu_seqlens cover the
+  // tokens after each sequence's cached prefix, cu_seqlens_k all of its keys
+  const int32_t* cu_seqlens_k;
+  const int32_t* block_tables;
+  int max_num_blocks;
+  int block_size;
+  int64_t num_blocks;
   // filled in by the launcher
+  unsigned block_magic;   // 2^32 / block_size + 1
   int slices;       // head slices: kv heads x (query heads per kv head / 4)
   int n_teams;      // gcd(8, slices): workgroup teams, each with its own item list
   int team_size;    // workgroups per team
@@ -234,7 +242,8 @@ struct PrefillPpArgs {
   int timeline_entries;
   int timeline_block;
 };
-bool prefill_pp_takes(int num_seqs, int num_heads, int num_kv_heads, int head_dim, int dtype);
+// block_size: 0 for the packed entry point
+bool prefill_pp_takes(int num_seqs, int num_heads, int num_kv_heads, int head_dim, int dtype, int block_size);
 int launch_prefill_pp(const PrefillPpArgs& a, int dtype, hipStream_t stream);
 
 }  // namespace mvllm

@@ -75,8 +75,10 @@ struct PpItems {
   unsigned base;      // rank of that level's first item
 };
 struct PpItem {
-  int seq_start, seq_len, rb;
+  int seq_start, seq_len, rb;   // the sequence's query rows; the item's 64-row block of them
+  int nt;             // index of the item's last key tile ( = rb without a cached prefix)
   int kvh, h0;        // kv head; first of the item's four query heads
+  int seq, cached;    // paged mode: the sequence's row in the block table, its cached tokens
   bool valid;
 };
 
@@ -85,7 +87,11 @@ __device__ __forceinline__ unsigned div_small(unsigned x, unsigned d, unsigned m
   return d == 1u ? x : __umulhi(x, magic);
 }
 
-template <typename T, int D, int GRP>
+// PAGED: prefill of the tokens that follow a cached prefix.  Query row r of a sequence sits at key position c + r
+// (c = its cached tokens); every key, cached or new, is read from the paged cache through the block table (the store
+// precedes this call), 16 rows = one piece of one block per wave and tile.  An item's key tiles are 0 ..
+// ceil(c / 64) + rb, and unless c is a multiple of 64 the causal diagonal crosses the last two of them.
+template <typename T, int D, int GRP, bool PAGED>
 __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, const int wave) {
   constexpr int kRowB = D * 2;
   constexpr int kTileBytes = kPpBN * kRowB;
@@ -118,16 +124,24 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 #define TCOUNT(items, tiles) do {} while (0)
 #endif
   // ---- the batch, one sequence per lane ----
-  int lo = 0, len = 0;
+  int lo = 0, len = 0, cached = 0, kv_len = 0;
   if (lane < a.num_seqs) {
     lo = a.cu_seqlens[lane];
     len = a.cu_seqlens[lane + 1] - lo;
+    if (PAGED) {
+      kv_len = a.cu_seqlens_k[lane + 1] - a.cu_seqlens_k[lane];
+      cached = kv_len > len ? kv_len - len : 0;
+    }
   }
   const int nb = (len + 63) >> 6;              // 64-row blocks of the lane's sequence
-  int top = 0;                                 // highest block count in the batch
+  // An item's level is the index of its last key tile: block rb of a sequence with c cached tokens has level
+  // ceil(c / 64) + rb, so the lane's sequence owns the levels lvl0 .. lvl0 + nb - 1.
+  const int lvl0 = PAGED ? (cached + 63) >> 6 : 0;
+  const int lvl_end = nb > 0 ? lvl0 + nb : 0;
+  int top = 0;                                 // one past the highest level in the batch
   for (int bit = a.level_bits - 1; bit >= 0; --bit) {
     const int trial = top | (1 << bit);
-    if (__ballot(nb >= trial) != 0ull) top = trial;
+    if (__ballot(lvl_end >= trial) != 0ull) top = trial;
   }
 
   // ---- which items are this workgroup's ----
@@ -153,7 +167,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   const unsigned short_round = (unsigned)team_items % TS != 0u ? (unsigned)team_items / TS : 0xffffffffu;
   PpItems walk = {top - 1, 0u};
   int produced = 0;
-  int kept_start = 0, kept_len = 0, kept_rb = 0, kept_heads = 0;
+  int kept_start = 0, kept_len = 0, kept_rb = 0, kept_heads = 0, kept_seq = 0;   // kept_rb: the level; kept_seq: paged only
   auto produce = [&]() {
     const unsigned round = (unsigned)produced;
     const bool backwards = (round & 1u) != 0u || round == short_round;
@@ -161,14 +175,14 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     unsigned long long mask = 0ull;
     unsigned cnt = 0;
     while (walk.level >= 0) {
-      mask = __ballot(nb > walk.level);
+      mask = __ballot(walk.level < lvl_end && walk.level >= lvl0);
       cnt = (unsigned)__popcll(mask);
       const unsigned items = cnt * spt;
       if (R - walk.base < items) break;
       walk.base += items;
       --walk.level;
     }
-    int seq_start = 0, seq_len = 0, heads = 0;
+    int seq_start = 0, seq_len = 0, heads = 0, seq = 0;
     if (walk.level >= 0) {
       // inside a level: sequence-major, the team's slices of one sequence side by side
       const unsigned idx = R - walk.base;
@@ -179,6 +193,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       const int owner = __ffsll((long long)pick) - 1;
       seq_start = __builtin_amdgcn_readlane(lo, owner);
       seq_len = __builtin_amdgcn_readlane(len, owner);
+      seq = owner;
       const unsigned y = (unsigned)team + (unsigned)a.n_teams * sl;
       const unsigned kvh = div_small(y, (unsigned)chunks, a.chunks_magic);
       heads = (int)((kvh << 16) | (kvh * (unsigned)group + (y - kvh * (unsigned)chunks) * 4u));
@@ -188,6 +203,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     kept_len = lane == at ? seq_len : kept_len;
     kept_rb = lane == at ? walk.level : kept_rb;     // -1: no such item
     kept_heads = lane == at ? heads : kept_heads;
+    if (PAGED) kept_seq = lane == at ? seq : kept_seq;
     ++produced;
   };
   auto item_at = [&](int k) {
@@ -196,11 +212,17 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     const int at = k & 15;
     it.seq_start = __builtin_amdgcn_readlane(kept_start, at);
     it.seq_len = __builtin_amdgcn_readlane(kept_len, at);
-    it.rb = __builtin_amdgcn_readlane(kept_rb, at);
+    it.nt = __builtin_amdgcn_readlane(kept_rb, at);
     const int heads = __builtin_amdgcn_readlane(kept_heads, at);
     it.kvh = (int)((unsigned)heads >> 16);
     it.h0 = heads & 0xffff;
-    it.valid = it.rb >= 0;
+    it.valid = it.nt >= 0;
+    it.seq = 0; it.cached = 0; it.rb = it.nt;
+    if (PAGED) {
+      it.seq = __builtin_amdgcn_readlane(kept_seq, at);
+      it.cached = __builtin_amdgcn_readlane(cached, it.seq);
+      it.rb = it.nt - ((it.cached + 63) >> 6);
+    }
     return it;
   };
 
@@ -225,11 +247,11 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // intervals before the barrier that publishes it and overwrites the tile three places back in its ring, whose
   // last readers finished an interval before.
   const int ld_row = lane >> 4, ld_chunk = lane & 15;
-  uint32_t src_off[4];
+  uint32_t src_off[4];                         // (paged: relative to the wave's own piece of the tile)
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int row = 16 * wq + 4 * i + ld_row;
-    src_off[i] = (uint32_t)(row * kv_row_bytes + ((ld_chunk ^ (GRP == 0 ? kswz(row) : vswz(row))) << 4));
+    src_off[i] = (uint32_t)((PAGED ? row - 16 * wq : row) * kv_row_bytes + ((ld_chunk ^ (GRP == 0 ? kswz(row) : vswz(row))) << 4));
   }
   const char* copy_src = GRP == 0 ? kg : vg;
   const uint32_t lds_copy0 = (GRP == 0 ? lds_address(&lds.k[0][0]) : lds_address(&lds.v[0][0])) + (uint32_t)(16 * wq * kRowB);
@@ -240,31 +262,68 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   int64_t d_off = 0;                           // byte offset of the cursor's tile in k (and v)
   int d_rows_left = 0;                         // rows from the tile's first to the tensor's last; <= 0: no tile
   int d_head_off = 0;                          // byte offset of the kv head inside a row
+  // Paged: the wave's 16 rows of the cursor's tile are one piece of one cache block (block_size % 16 == 0).  Its
+  // table entry is fetched with a scalar load one copy step ahead (`d_phys`), so that no step waits for it; the
+  // descriptor starts at the piece and ends with the sequence's last key, so rows that were never written, unmapped
+  // blocks and tiles past the stream's end arrive as zeros.
+  int d_phys = -1;                             // table entry of the cursor's piece
+  int d_in_block = 0;                          // ... and its first row inside that block
+  int d_kv_len = 0;                            // keys of the cursor's sequence
+  auto fetch_entry = [&]() {                   // for the cursor's tile (dit, dj)
+    if constexpr (PAGED) {
+      const unsigned pos = (unsigned)(kPpBN * dj + 16 * wq);
+      const unsigned bi = div_small(pos, (unsigned)a.block_size, a.block_magic);
+      d_in_block = (int)(pos - bi * (unsigned)a.block_size);
+      // (read through the constant address space: a scalar load, which the copies' vmcnt accounting does not see; a
+      // vector load here would make the compiler wait for every copy in flight before each use of the entry)
+      typedef const __attribute__((address_space(4))) int32_t* ConstTable;
+      const ConstTable table = reinterpret_cast<ConstTable>(reinterpret_cast<uintptr_t>(a.block_tables));
+      const int64_t at = (int64_t)__builtin_amdgcn_readfirstlane(dit.seq) * a.max_num_blocks + __builtin_amdgcn_readfirstlane((int)bi);
+      d_phys = dit.valid && (int)bi < a.max_num_blocks ? table[at] : -1;
+    }
+  };
   auto enter_item = [&]() {                    // the cursor's tile = first tile of `dit`
     d_head_off = dit.kvh * kRowB;
-    d_off = (int64_t)dit.seq_start * kv_row_bytes + d_head_off;
-    d_rows_left = dit.valid ? total_rows - dit.seq_start : 0;
+    if constexpr (PAGED) {
+      d_kv_len = dit.valid ? __builtin_amdgcn_readlane(kv_len, dit.seq) : 0;
+    } else {
+      d_off = (int64_t)dit.seq_start * kv_row_bytes + d_head_off;
+      d_rows_left = dit.valid ? total_rows - dit.seq_start : 0;
+    }
   };
   enter_item();
+  fetch_entry();
   int d_slot = 0;                              // ring slot of the cursor's tile ( = its stream index % 3)
   auto copy_step = [&]() {
-    const uint32_t size = d_rows_left <= 0        ? 0u
-                          : d_rows_left > rows_4g ? 0xffffffffu
-                                                  : (uint32_t)d_rows_left * (uint32_t)kv_row_bytes - (uint32_t)d_head_off;
-    const v4i r = make_rsrc(copy_src + d_off, size);
+    v4i r;
+    if constexpr (PAGED) {
+      const int pos = kPpBN * dj + 16 * wq;
+      const int valid = d_kv_len - pos < 16 ? d_kv_len - pos : 16;
+      const int in_block = d_in_block;
+      const bool ok = dit.valid && valid > 0 && d_phys >= 0 && (int64_t)d_phys < a.num_blocks;
+      const uint32_t size = ok ? (uint32_t)(valid - 1) * (uint32_t)kv_row_bytes + (uint32_t)kRowB : 0u;
+      const int64_t start = ok ? ((int64_t)d_phys * a.block_size + in_block) * kv_row_bytes + d_head_off : 0;
+      r = make_rsrc(copy_src + start, size);
+    } else {
+      const uint32_t size = d_rows_left <= 0        ? 0u
+                            : d_rows_left > rows_4g ? 0xffffffffu
+                                                    : (uint32_t)d_rows_left * (uint32_t)kv_row_bytes - (uint32_t)d_head_off;
+      r = make_rsrc(copy_src + d_off, size);
+    }
     const uint32_t dst = lds_copy0 + (uint32_t)(d_slot * kTileBytes);
 #pragma unroll
     for (int i = 0; i < 4; ++i) dma16(r, src_off[i], dst + 1024u * i);
     d_slot = d_slot == kPpRing - 1 ? 0 : d_slot + 1;
     if (dit.valid) {
-      if (++dj > dit.rb) {
+      if (++dj > dit.nt) {
         dit = item_at(++di);
         dj = 0;
         enter_item();
-      } else {
+      } else if constexpr (!PAGED) {
         d_off += (int64_t)kPpBN * kv_row_bytes;      // the next 64 rows of the same sequence and head
         d_rows_left -= kPpBN;
       }
+      fetch_entry();
     }
   };
   // Q rows of an item -> this wave's slot, 4 rows per instruction, chunks swizzled like a K tile's
@@ -450,6 +509,17 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       if (8 * (r >> 2) + (r & 3) > lim) s[GRP][r] = -INFINITY;
       if (GRP == 0) s[1][r] = -INFINITY;
     }
+  };
+  // Paged: the diagonal against tile j of `cur` in general position.  Query row l32 of this group sits at key
+  // position cached + 64 rb + 32 GRP + l32; the lane's keys in the tile are 64 j + 32 tk + 8 (r / 4) + r % 4 + 4 hi.
+  auto mask_tile = [&](int j) {
+    int lim = cur.cached + kPpBN * (cur.rb - j) + 32 * GRP + l32 - 4 * hi;
+    asm volatile("" : "+v"(lim));
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (32 * tk + 8 * (r >> 2) + (r & 3) > lim) s[tk][r] = -INFINITY;
   };
   auto tile_max = [&]() {                        // maximum of the lane's row over the tile, relative to the running one
     const float mx0 = fmaxf(s[0][15], s[1][15]);
@@ -645,10 +715,19 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   };
 
   // the softmax interval of tile j > 0 of `cur`, up to the barrier; returns nothing, leaves pf, l, vf0, vf1
-  auto later_tile = [&](auto LAST, uint4 (&vf0)[kTD], uint4 (&vf1)[kTD]) {
+  // MASKED: the tile the diagonal may cross (the last one; paged: also the one before it when the prefix does not end
+  // on a tile boundary, which has a call of its own so that the middle tiles carry no test for it)
+  auto later_tile = [&](auto LAST, auto MASKED, int j, uint4 (&vf0)[kTD], uint4 (&vf1)[kTD]) {
     TSTAMP();
     copy_step();
-    if constexpr (decltype(LAST)::value) mask_diagonal();
+    if constexpr (PAGED) {
+      if constexpr (decltype(LAST)::value) mask_tile(j);
+      else if constexpr (decltype(MASKED)::value) {
+        if ((cur.cached & 63) != 0) mask_tile(j);
+      }
+    } else if constexpr (decltype(LAST)::value) {
+      mask_diagonal();
+    }
     // The scores are relative to the running maximum, which is not looked at again unless it is badly out of
     // date: the weights are computed first, and only when a lane's share of the tile's row sum passes 2^12 (a
     // weight above 2^7 at least; 16-bit weights and fp32 sums are far from their limits there) is the tile redone
@@ -680,11 +759,15 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 
   while (true) {
     // ======== first tile of an item ========
-    const bool single = cur.rb == 0;
+    const bool single = cur.nt == 0;
     int trail = 0;                               // vector memory instructions behind this interval's copy step
     TSTAMP();
     copy_step();
-    if (single) mask_diagonal();
+    if constexpr (PAGED) {
+      if (single || (cur.nt == 1 && (cur.cached & 63) != 0)) mask_tile(0);
+    } else if (single) {
+      mask_diagonal();
+    }
     const float mx_first = tile_max();           // neg_m is zero here: the tile's maximum itself
     // the item before this one leaves (its output was staged in the slot during the interval before) ...
     if (have_prev) {
@@ -710,14 +793,21 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     bool more = matrix_interval(std::true_type{}, std::false_type{}, single, vf0, vf1);
     if (!single) {
       // ======== the item's other tiles ========
-      for (int j = 1; j < cur.rb; ++j) {
-        later_tile(std::false_type{}, vf0, vf1);
+      const int plain_end = PAGED ? cur.nt - 1 : cur.nt;
+      for (int j = 1; j < plain_end; ++j) {
+        later_tile(std::false_type{}, std::false_type{}, j, vf0, vf1);
         matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
       }
-      later_tile(std::true_type{}, vf0, vf1);
+      if constexpr (PAGED) {
+        if (cur.nt >= 2) {
+          later_tile(std::false_type{}, std::true_type{}, cur.nt - 1, vf0, vf1);
+          matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
+        }
+      }
+      later_tile(std::true_type{}, std::true_type{}, cur.nt, vf0, vf1);
       more = matrix_interval(std::false_type{}, std::true_type{}, false, vf0, vf1);
     }
-    TCOUNT(1, cur.rb + 1);
+    TCOUNT(1, cur.nt + 1);
     p_seq_start = cur.seq_start; p_seq_len = cur.seq_len; p_rb = cur.rb; p_h0 = cur.h0;
     have_prev = true;
     if (!more) break;
@@ -738,16 +828,17 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 #endif
 }
 
-template <typename T, int D>
+template <typename T, int D, bool PAGED>
 __global__ __launch_bounds__(64 * kPpWaves, 1) void prefill_pp_kernel(const PrefillPpArgs a) {
   __shared__ __attribute__((aligned(1024))) PpLds<D> lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  if (wave < 4) pp_run<T, D, 0>(a, lds, wave);
-  else pp_run<T, D, 1>(a, lds, wave);
+  if (wave < 4) pp_run<T, D, 0, PAGED>(a, lds, wave);
+  else pp_run<T, D, 1, PAGED>(a, lds, wave);
 }
 
-bool prefill_pp_takes(int num_seqs, int num_heads, int num_kv_heads, int head_dim, int dtype) {
+bool prefill_pp_takes(int num_seqs, int num_heads, int num_kv_heads, int head_dim, int dtype, int block_size) {
   if (dtype == MVLLM_F32 || head_dim != 128 || num_seqs > 64 || num_seqs <= 0) return false;
+  if (block_size != 0 && (block_size < 16 || block_size % 16 != 0)) return false;      // paged: a wave's 16 rows lie in one block
   const int group = num_heads / num_kv_heads;
   return group % 4 == 0 && (int64_t)num_heads * head_dim * 2 * 64 < ((int64_t)1 << 31);
 }
@@ -771,10 +862,20 @@ int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) 
   auto magic = [](int d) { return d <= 1 ? 0u : (unsigned)(((uint64_t)1 << 32) / (uint64_t)d + 1u); };
   a.spt_magic = magic(a.slices / n_teams);
   a.chunks_magic = magic(group / 4);
+  const bool paged = a.block_tables != nullptr;
+  a.block_magic = magic(a.block_size);
+  // levels: the tile count of the longest possible sequence (paged: as wide as its block-table row)
+  const int64_t most_keys = paged ? (int64_t)a.max_num_blocks * a.block_size + a.total_tokens : a.total_tokens;
   a.level_bits = 1;
-  while (((int64_t)1 << a.level_bits) <= a.total_tokens / 64 + 1) ++a.level_bits;
-  if (dtype == MVLLM_BF16) prefill_pp_kernel<bf16_t, 128><<<dim3(grid), dim3(64 * kPpWaves), 0, stream>>>(a);
-  else prefill_pp_kernel<f16_t, 128><<<dim3(grid), dim3(64 * kPpWaves), 0, stream>>>(a);
+  while (((int64_t)1 << a.level_bits) <= most_keys / 64 + 2) ++a.level_bits;
+  const dim3 g(grid), b(64 * kPpWaves);
+  if (dtype == MVLLM_BF16) {
+    if (paged) prefill_pp_kernel<bf16_t, 128, true><<<g, b, 0, stream>>>(a);
+    else prefill_pp_kernel<bf16_t, 128, false><<<g, b, 0, stream>>>(a);
+  } else {
+    if (paged) prefill_pp_kernel<f16_t, 128, true><<<g, b, 0, stream>>>(a);
+    else prefill_pp_kernel<f16_t, 128, false><<<g, b, 0, stream>>>(a);
+  }
   return launch_status();
 }
 
@@ -792,12 +893,13 @@ extern "C" int mvllm_probe_prefill_timeline(void* out, const void* q, const void
   using namespace mvllm;
   if (!out || !q || !k || !v || !cu_seqlens || !log || entries_per_wave <= 0) return MVLLM_ERR_NULL_POINTER;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || !(scale > 0.f) ||
-      !prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype))
+      !prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype, 0))
     return MVLLM_ERR_UNSUPPORTED;
   PrefillPpArgs p;
   p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
   p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
   p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0; p.spt_magic = 0; p.chunks_magic = 0;
+  p.cu_seqlens_k = nullptr; p.block_tables = nullptr; p.max_num_blocks = 0; p.block_size = 0; p.num_blocks = 0; p.block_magic = 0;
   p.timeline = log; p.timeline_entries = entries_per_wave; p.timeline_block = block;
   return launch_prefill_pp(p, dtype, (hipStream_t)stream);
 }

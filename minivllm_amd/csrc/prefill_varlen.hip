@@ -187,11 +187,12 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   const bool aligned = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out);
   const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, 0, dtype, false, false) : 0;
   const bool mfma_ok = kind == 2;
-  if (mfma_ok && scale > 0.f && prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype)) {
+  if (mfma_ok && scale > 0.f && prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype, 0)) {
     PrefillPpArgs p;
     p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
     p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
     p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0; p.spt_magic = 0; p.chunks_magic = 0;
+    p.cu_seqlens_k = nullptr; p.block_tables = nullptr; p.max_num_blocks = 0; p.block_size = 0; p.num_blocks = 0; p.block_magic = 0;
     p.timeline = nullptr; p.timeline_entries = 0; p.timeline_block = 0;
     return launch_prefill_pp(p, dtype, (hipStream_t)stream);
   }
@@ -232,6 +233,16 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
   const bool aligned = aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out);
   const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, block_size, dtype, true, false) : 0;
   const bool mfma_ok = kind == 2;
+  if (mfma_ok && scale > 0.f && prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype, block_size)) {
+    PrefillPpArgs p;
+    p.out = out; p.q = q; p.k = k_cache; p.v = v_cache; p.cu_seqlens = cu_seqlens_q; p.total_tokens = total_q_tokens;
+    p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
+    p.cu_seqlens_k = cu_seqlens_k; p.block_tables = block_tables; p.max_num_blocks = max_num_blocks;
+    p.block_size = block_size; p.num_blocks = num_blocks; p.block_magic = 0;
+    p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0; p.spt_magic = 0; p.chunks_magic = 0;
+    p.timeline = nullptr; p.timeline_entries = 0; p.timeline_block = 0;
+    return launch_prefill_pp(p, dtype, (hipStream_t)stream);
+  }
   if (kind == 1) {
     PrefillRowsArgs r;
     r.out = out; r.q = q; r.k = k_cache; r.v = v_cache; r.cu_seqlens = cu_seqlens_q; r.total_tokens = total_q_tokens;

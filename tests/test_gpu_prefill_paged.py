@@ -82,19 +82,18 @@ def test_paged_prefill_without_prefix_matches_plain_prefill_bitwise():
     assert torch.equal(got, plain)
 
 
-def test_paged_prefill_without_prefix_close_to_two_group_prefill():
-    """Four query heads per kv head: the packed call runs on the two-group kernel, which sums a row's weights before
-    they are rounded to 16 bits; the two results agree to the last bits of the 16-bit outputs."""
-    hq, hkv, d, bs = 32, 8, 128, 16
-    lengths = [257, 64, 31, 400]
-    c = make_paged_prefill_case(62, lengths, [0] * 4, hq, hkv, d, bs, dtype=torch.bfloat16)
+@pytest.mark.parametrize("bs", [16, 48, 256])
+def test_two_group_paged_prefill_without_prefix_matches_packed_bitwise(bs):
+    """Four query heads per kv head: both calls run on the two-group kernel, same tiles, same arithmetic, only the
+    copies' source differs (the paged cache through the block table)."""
+    hq, hkv, d = 32, 8, 128
+    lengths = [257, 64, 31, 400, 1, 1000]
+    c = make_paged_prefill_case(62, lengths, [0] * 6, hq, hkv, d, bs, dtype=torch.bfloat16)
     scale = 1 / math.sqrt(d)
-    got = _run(c, scale, hq, hkv, d, bs).float()
+    got = _run(c, scale, hq, hkv, d, bs)
     plain = flash_attention_prefill(c["q"].to(DEV), c["k"].to(DEV), c["v"].to(DEV), c["cu_k"].to(DEV), scale,
-                                    hq, hkv, d).cpu().float()
-    err = (got - plain).abs()
-    assert (err <= plain.abs() * 2.0 ** -6 + 1e-3).all()      # two bf16 steps of the value
-    assert err.mean() <= 2e-4
+                                    hq, hkv, d).cpu()
+    assert torch.equal(got, plain)
 
 
 def test_paged_prefill_single_new_token_matches_decode():
@@ -199,6 +198,42 @@ def test_paged_prefill_over_an_int8_cache(dtype, hq, hkv, d, bs, lengths, cached
                                       torch.tensor(lengths, device=DEV), scale, hq, hkv, d, bs).cpu()
     mx, mean = error_stats(got[last], dec.float())
     assert mx <= 3e-2 and mean <= 3e-3, (mx, mean)
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (8, 2), (12, 3)])
+@pytest.mark.parametrize("bs", [16, 48, 256])
+@pytest.mark.parametrize("num_seqs", [1, 9, 64])
+def test_two_group_paged_prefill_takes_every_item_once(hq, hkv, bs, num_seqs):
+    """The two-group kernel over cached prefixes (head_dim 128, a multiple of 4 query heads per kv head, at most 64
+    sequences): prefixes of 0, whole tiles and anything in between (the diagonal then crosses the last two key tiles of
+    an item), a single new token behind a long prefix, sequences with nothing new, blocks of 16, 48 and 256 tokens in
+    shuffled physical order with poisoned rows past every sequence's end.  The output starts as NaN, so an item that no
+    workgroup took would show."""
+    d = 128
+    g = torch.Generator().manual_seed(1300 + num_seqs + bs + hq)
+    pool = [1, 2, 31, 63, 64, 65, 100, 128, 129, 191, 192, 257, 300, 448]
+    kv_lengths = [pool[i] for i in torch.randint(0, len(pool), (num_seqs,), generator=g).tolist()]
+    kv_lengths[num_seqs // 2] = 1500 if hq <= 32 else 600
+    cached = []
+    for n in kv_lengths:
+        mode = int(torch.randint(0, 5, (1,), generator=g))
+        c = [0, n - 1, (n // 2) // 64 * 64, n // 2, n][mode]      # nothing, all but one, whole tiles, half, everything
+        cached.append(max(0, min(c, n)))
+    cached[num_seqs // 2] = 333                                    # the long one: a prefix that ends inside a tile
+    if sum(n - c for n, c in zip(kv_lengths, cached)) == 0:
+        cached[0] = 0
+    c = make_paged_prefill_case(70, kv_lengths, cached, hq, hkv, d, bs, dtype=torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    from minivllm_amd import _C
+    q_new = c["q_new"].to(DEV)
+    out = torch.full_like(q_new, float("nan"))
+    kc, vc, bt, cuq, cuk = (c[k].to(DEV) for k in ("k_cache", "v_cache", "block_tables", "cu_q", "cu_k"))
+    st = _C.load().mvllm_prefill_paged(out.data_ptr(), q_new.data_ptr(), kc.data_ptr(), vc.data_ptr(), bt.data_ptr(),
+                                       bt.shape[1], cuq.data_ptr(), cuk.data_ptr(), num_seqs, q_new.shape[0], hq, hkv, d, bs,
+                                       kc.shape[0], scale, _C.dtype_code(q_new.dtype), _C.current_stream_ptr(out.device))
+    torch.cuda.synchronize()
+    assert st == 0
+    _check(out.cpu(), _oracle32(c, scale, hq, hkv, d, bs), torch.bfloat16)
 
 
 def _half_step(dtype):
