@@ -1,11 +1,12 @@
 // Varlen causal flash-attention prefill for gfx950, two-group ("ping-pong") form.
 // Replaces the Triton kernel of src/myvllm/layers/attention.py:111-209 for batches this kernel is built for
-// (16-bit q/k/v, head_dim 128, query heads per kv head a multiple of 4, at most 64 sequences); the launcher in
+// (16-bit q/k/v, head_dim 128, an even number of query heads per kv head, at most 64 sequences); the launcher in
 // prefill_varlen.hip falls back to prefill_mfma_kernel for everything else.
 //
 // One persistent workgroup of 8 waves per CU (two waves per SIMD, 160 KB of LDS).  A work item is one kv head, four
 // of its query heads and a block of 64 consecutive query rows of one sequence; wave w owns query head w % 4 and the
-// 32-row half w / 4 of the block.  Waves 0-3 (group 0) and waves 4-7 (group 1) run the same tile loop one barrier
+// 32-row half w / 4 of the block.  (Where the heads per kv head are not a multiple of 4 an item is two heads and
+// 128 rows: see pp_run.)  Waves 0-3 (group 0) and waves 4-7 (group 1) run the same tile loop one barrier
 // interval apart: while one group feeds the matrix unit (O += V^T P^T of tile n, then S^T = K Q^T of tile n + 1: 32
 // MFMAs, no other vector work) the other does the softmax of its tile on the vector unit, and they swap at every
 // barrier.  The two waves that share a SIMD are then never both in their softmax nor both waiting for the matrix
@@ -91,8 +92,17 @@ __device__ __forceinline__ unsigned div_small(unsigned x, unsigned d, unsigned m
 // (c = its cached tokens); every key, cached or new, is read from the paged cache through the block table (the store
 // precedes this call), 16 rows = one piece of one block per wave and tile.  An item's key tiles are 0 ..
 // ceil(c / 64) + rb, and unless c is a multiple of 64 the causal diagonal crosses the last two of them.
-template <typename T, int D, int GRP, bool PAGED>
+//
+// HPI: query heads per item.  4: the item is a 64-row block, wave w has head w % 4 and rows 32 GRP ...  2 (two or six
+// ... query heads per kv head): the item is a 128-row block of two heads, wave w has head w % 2 and rows
+// 64 GRP + 32 ((w % 4) / 2) ...; the block's last key tile is then the index of its second 64-row step, the
+// diagonal crosses its last two tiles (three over a prefix in general position), and the waves of its first 64 rows
+// compute a last tile they see nothing of.
+template <typename T, int D, int GRP, bool PAGED, int HPI>
 __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, const int wave) {
+  static_assert(HPI == 4 || HPI == 2, "items of four or of two query heads");
+  constexpr int kTPB = 4 / HPI;                // 64-row steps (and diagonal key tiles) per item
+  constexpr int kRPI = 64 * kTPB;              // query rows per item
   constexpr int kRowB = D * 2;
   constexpr int kTileBytes = kPpBN * kRowB;
   constexpr int kKS = D / 16;
@@ -104,7 +114,9 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   const int lane = threadIdx.x & 63;
   const int l32 = lane & 31;
   const int hi = lane >> 5;
-  const int wq = wave & 3;                     // query head inside the slice
+  const int wq = wave & 3;                     // wave inside its group: its piece of the group's copies
+  const int wh = wq & (HPI - 1);               // query head inside the item
+  const int row_off = 32 * kTPB * GRP + 32 * (wq / HPI);   // the wave's 32 query rows inside the item's block
 
 #if MVLLM_PP_TIMELINE
   // Timing build (the probe library): the waves of one workgroup log the shader clock at the four corners of every
@@ -133,11 +145,11 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       cached = kv_len > len ? kv_len - len : 0;
     }
   }
-  const int nb = (len + 63) >> 6;              // 64-row blocks of the lane's sequence
+  const int nb = (len + kRPI - 1) / kRPI;      // item blocks of the lane's sequence
   // An item's level is the index of its last key tile: block rb of a sequence with c cached tokens has level
-  // ceil(c / 64) + rb, so the lane's sequence owns the levels lvl0 .. lvl0 + nb - 1.
-  const int lvl0 = PAGED ? (cached + 63) >> 6 : 0;
-  const int lvl_end = nb > 0 ? lvl0 + nb : 0;
+  // (c + kRPI - 1) / 64 + kTPB rb, so the lane's sequence owns every kTPB-th level from lvl0 to lvl_end - 1.
+  const int lvl0 = (cached + kRPI - 1) >> 6;
+  const int lvl_end = nb > 0 ? lvl0 + kTPB * (nb - 1) + 1 : 0;
   int top = 0;                                 // one past the highest level in the batch
   for (int bit = a.level_bits - 1; bit >= 0; --bit) {
     const int trial = top | (1 << bit);
@@ -152,7 +164,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   const unsigned t = (wg >> 3) * (8u / (unsigned)a.n_teams) + xcd / (unsigned)a.n_teams;   // index inside the team
   const unsigned spt = (unsigned)(a.slices / a.n_teams);                                  // slices per team
   const int group = a.num_heads / a.num_kv_heads;
-  const int chunks = group / 4;
+  const int chunks = group / HPI;
   // The workgroup's k-th item is rank k TS + (t or, in odd rounds, TS - 1 - t) of the team's list.  Locating an item
   // costs a hundred-odd instructions per wave, and two cursors go through the same items (the copies run ahead of the
   // arithmetic), so every item is located once and kept in lane (k mod 16) of four registers until both have passed.
@@ -175,7 +187,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     unsigned long long mask = 0ull;
     unsigned cnt = 0;
     while (walk.level >= 0) {
-      mask = __ballot(walk.level < lvl_end && walk.level >= lvl0);
+      mask = __ballot(walk.level < lvl_end && walk.level >= lvl0 && (kTPB == 1 || ((walk.level - lvl0) & (kTPB - 1)) == 0));
       cnt = (unsigned)__popcll(mask);
       const unsigned items = cnt * spt;
       if (R - walk.base < items) break;
@@ -196,7 +208,7 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       seq = owner;
       const unsigned y = (unsigned)team + (unsigned)a.n_teams * sl;
       const unsigned kvh = div_small(y, (unsigned)chunks, a.chunks_magic);
-      heads = (int)((kvh << 16) | (kvh * (unsigned)group + (y - kvh * (unsigned)chunks) * 4u));
+      heads = (int)((kvh << 16) | (kvh * (unsigned)group + (y - kvh * (unsigned)chunks) * (unsigned)HPI));
     }
     const int at = produced & 15;
     kept_start = lane == at ? seq_start : kept_start;
@@ -217,12 +229,12 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     it.kvh = (int)((unsigned)heads >> 16);
     it.h0 = heads & 0xffff;
     it.valid = it.nt >= 0;
-    it.seq = 0; it.cached = 0; it.rb = it.nt;
+    it.seq = 0; it.cached = 0;
     if (PAGED) {
       it.seq = __builtin_amdgcn_readlane(kept_seq, at);
       it.cached = __builtin_amdgcn_readlane(cached, it.seq);
-      it.rb = it.nt - ((it.cached + 63) >> 6);
     }
+    it.rb = (it.nt - ((it.cached + kRPI - 1) >> 6)) / kTPB;
     return it;
   };
 
@@ -329,8 +341,8 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // Q rows of an item -> this wave's slot, 4 rows per instruction, chunks swizzled like a K tile's
   const uint32_t lds_q = lds_address(&lds.qo[wave][0]);
   auto copy_q = [&](const PpItem& it) {
-    const int h = it.h0 + wq;
-    const int row = it.seq_start + it.rb * 64 + 32 * GRP;
+    const int h = it.h0 + wh;
+    const int row = it.seq_start + it.rb * kRPI + row_off;
     const int rows_left = total_rows - row;
     const int rows_4g = (int)(0xffffffffu / (uint32_t)q_row_bytes);
     const uint32_t size = rows_left <= 0 ? 0u
@@ -457,12 +469,12 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     int lane_o = lane;
     asm volatile("" : "+v"(lane_o));
     const int orow = lane_o >> 4, ochunk = lane_o & 15;
-    const int r0 = rb * 64 + 32 * GRP;
+    const int r0 = rb * kRPI + row_off;
     // The descriptor ends with the head's part of the sequence's last row, so the stores of rows past it are dropped
     // by the bounds check: all eight are always issued, as the wait counts assume.
     const int rows = seq_len - r0 < 32 ? seq_len - r0 : 32;
     const uint32_t size = rows > 0 ? (uint32_t)(rows - 1) * (uint32_t)q_row_bytes + (uint32_t)kRowB : 0u;
-    char* base = reinterpret_cast<char*>(out) + (int64_t)(seq_start + r0) * q_row_bytes + (int64_t)(h0 + wq) * kRowB;
+    char* base = reinterpret_cast<char*>(out) + (int64_t)(seq_start + r0) * q_row_bytes + (int64_t)(h0 + wh) * kRowB;
     const uint32_t off0 = (uint32_t)(orow * q_row_bytes + 16 * ochunk);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -510,10 +522,12 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       if (GRP == 0) s[1][r] = -INFINITY;
     }
   };
-  // Paged: the diagonal against tile j of `cur` in general position.  Query row l32 of this group sits at key
-  // position cached + 64 rb + 32 GRP + l32; the lane's keys in the tile are 64 j + 32 tk + 8 (r / 4) + r % 4 + 4 hi.
+  // The diagonal against tile j of `cur` in general position (over a cached prefix; items of two heads).  Query row
+  // l32 of this wave sits at key position cached + kRPI rb + row_off + l32; the lane's keys in the tile are
+  // 64 j + 32 tk + 8 (r / 4) + r % 4 + 4 hi.  A wave whose rows all lie above the tile masks all of it: its weights
+  // are zeros then, and the running maximum, which only a large row sum moves, stays.
   auto mask_tile = [&](int j) {
-    int lim = cur.cached + kPpBN * (cur.rb - j) + 32 * GRP + l32 - 4 * hi;
+    int lim = cur.cached + kPpBN * (kTPB * cur.rb - j) + row_off + l32 - 4 * hi;
     asm volatile("" : "+v"(lim));
 #pragma unroll
     for (int tk = 0; tk < 2; ++tk)
@@ -720,10 +734,10 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   auto later_tile = [&](auto LAST, auto MASKED, int j, uint4 (&vf0)[kTD], uint4 (&vf1)[kTD]) {
     TSTAMP();
     copy_step();
-    if constexpr (PAGED) {
+    if constexpr (PAGED || HPI != 4) {
       if constexpr (decltype(LAST)::value) mask_tile(j);
       else if constexpr (decltype(MASKED)::value) {
-        if ((cur.cached & 63) != 0) mask_tile(j);
+        if (HPI != 4 || (cur.cached & 63) != 0) mask_tile(j);
       }
     } else if constexpr (decltype(LAST)::value) {
       mask_diagonal();
@@ -763,8 +777,11 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     int trail = 0;                               // vector memory instructions behind this interval's copy step
     TSTAMP();
     copy_step();
-    if constexpr (PAGED) {
-      if (single || (cur.nt == 1 && (cur.cached & 63) != 0)) mask_tile(0);
+    // tiles at the item's end that the diagonal may cross (items of four heads without a prefix: the last one, by
+    // mask_diagonal)
+    const int masked_tail = kTPB + (PAGED && (cur.cached & 63) != 0 ? 1 : 0);
+    if constexpr (PAGED || HPI != 4) {
+      if (cur.nt < masked_tail) mask_tile(0);
     } else if (single) {
       mask_diagonal();
     }
@@ -793,14 +810,26 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
     bool more = matrix_interval(std::true_type{}, std::false_type{}, single, vf0, vf1);
     if (!single) {
       // ======== the item's other tiles ========
-      const int plain_end = PAGED ? cur.nt - 1 : cur.nt;
-      for (int j = 1; j < plain_end; ++j) {
-        later_tile(std::false_type{}, std::false_type{}, j, vf0, vf1);
-        matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
-      }
-      if constexpr (PAGED) {
-        if (cur.nt >= 2) {
-          later_tile(std::false_type{}, std::true_type{}, cur.nt - 1, vf0, vf1);
+      if constexpr (HPI == 4) {
+        const int plain_end = PAGED ? cur.nt - 1 : cur.nt;
+        for (int j = 1; j < plain_end; ++j) {
+          later_tile(std::false_type{}, std::false_type{}, j, vf0, vf1);
+          matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
+        }
+        if constexpr (PAGED) {
+          if (cur.nt >= 2) {
+            later_tile(std::false_type{}, std::true_type{}, cur.nt - 1, vf0, vf1);
+            matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
+          }
+        }
+      } else {
+        int j = 1;
+        for (; j <= cur.nt - masked_tail; ++j) {
+          later_tile(std::false_type{}, std::false_type{}, j, vf0, vf1);
+          matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
+        }
+        for (; j < cur.nt; ++j) {                  // one or two tiles before the last that the diagonal crosses
+          later_tile(std::false_type{}, std::true_type{}, j, vf0, vf1);
           matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
         }
       }
@@ -828,25 +857,37 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 #endif
 }
 
-template <typename T, int D, bool PAGED>
+template <typename T, int D, bool PAGED, int HPI>
 __global__ __launch_bounds__(64 * kPpWaves, 1) void prefill_pp_kernel(const PrefillPpArgs a) {
   __shared__ __attribute__((aligned(1024))) PpLds<D> lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  if (wave < 4) pp_run<T, D, 0, PAGED>(a, lds, wave);
-  else pp_run<T, D, 1, PAGED>(a, lds, wave);
+  if (wave < 4) pp_run<T, D, 0, PAGED, HPI>(a, lds, wave);
+  else pp_run<T, D, 1, PAGED, HPI>(a, lds, wave);
+}
+
+template <typename T>
+static void launch_prefill_pp_as(const PrefillPpArgs& a, bool paged, int hpi, dim3 g, dim3 b, hipStream_t stream) {
+  if (hpi == 4) {
+    if (paged) prefill_pp_kernel<T, 128, true, 4><<<g, b, 0, stream>>>(a);
+    else prefill_pp_kernel<T, 128, false, 4><<<g, b, 0, stream>>>(a);
+  } else {
+    if (paged) prefill_pp_kernel<T, 128, true, 2><<<g, b, 0, stream>>>(a);
+    else prefill_pp_kernel<T, 128, false, 2><<<g, b, 0, stream>>>(a);
+  }
 }
 
 bool prefill_pp_takes(int num_seqs, int num_heads, int num_kv_heads, int head_dim, int dtype, int block_size) {
   if (dtype == MVLLM_F32 || head_dim != 128 || num_seqs > 64 || num_seqs <= 0) return false;
   if (block_size != 0 && (block_size < 16 || block_size % 16 != 0)) return false;      // paged: a wave's 16 rows lie in one block
   const int group = num_heads / num_kv_heads;
-  return group % 4 == 0 && (int64_t)num_heads * head_dim * 2 * 64 < ((int64_t)1 << 31);
+  return group % 2 == 0 && (int64_t)num_heads * head_dim * 2 * 64 < ((int64_t)1 << 31);
 }
 
 int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) {
   PrefillPpArgs a = args;
   const int group = a.num_heads / a.num_kv_heads;
-  a.slices = a.num_kv_heads * (group / 4);
+  const int hpi = group % 4 == 0 ? 4 : 2;             // query heads per item
+  a.slices = a.num_kv_heads * (group / hpi);
   int n_teams = 8;
   while (a.slices % n_teams != 0) n_teams >>= 1;      // gcd(8, slices)
   a.n_teams = n_teams;
@@ -861,7 +902,7 @@ int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) 
   a.team_size = grid / n_teams;
   auto magic = [](int d) { return d <= 1 ? 0u : (unsigned)(((uint64_t)1 << 32) / (uint64_t)d + 1u); };
   a.spt_magic = magic(a.slices / n_teams);
-  a.chunks_magic = magic(group / 4);
+  a.chunks_magic = magic(group / hpi);
   const bool paged = a.block_tables != nullptr;
   a.block_magic = magic(a.block_size);
   // levels: the tile count of the longest possible sequence (paged: as wide as its block-table row)
@@ -869,13 +910,8 @@ int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) 
   a.level_bits = 1;
   while (((int64_t)1 << a.level_bits) <= most_keys / 64 + 2) ++a.level_bits;
   const dim3 g(grid), b(64 * kPpWaves);
-  if (dtype == MVLLM_BF16) {
-    if (paged) prefill_pp_kernel<bf16_t, 128, true><<<g, b, 0, stream>>>(a);
-    else prefill_pp_kernel<bf16_t, 128, false><<<g, b, 0, stream>>>(a);
-  } else {
-    if (paged) prefill_pp_kernel<f16_t, 128, true><<<g, b, 0, stream>>>(a);
-    else prefill_pp_kernel<f16_t, 128, false><<<g, b, 0, stream>>>(a);
-  }
+  if (dtype == MVLLM_BF16) launch_prefill_pp_as<bf16_t>(a, paged, hpi, g, b, stream);
+  else launch_prefill_pp_as<f16_t>(a, paged, hpi, g, b, stream);
   return launch_status();
 }
 

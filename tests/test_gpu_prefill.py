@@ -155,20 +155,25 @@ def test_prefill_item_order_covers_every_tile(hq, hkv, num_seqs):
     assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
 
 
-@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (24, 2), (8, 2), (12, 3), (4, 1)])
+@pytest.mark.parametrize("hq,hkv,dtype", [(32, 8, torch.bfloat16), (64, 8, torch.bfloat16), (24, 2, torch.bfloat16),
+                                          (8, 2, torch.bfloat16), (12, 3, torch.bfloat16), (4, 1, torch.bfloat16),
+                                          (16, 8, torch.bfloat16), (16, 8, torch.float16), (12, 2, torch.bfloat16),
+                                          (2, 1, torch.bfloat16), (20, 2, torch.float16)])
 @pytest.mark.parametrize("num_seqs", [1, 7, 64])
-def test_two_group_prefill_deals_every_item_once(hq, hkv, num_seqs):
-    """The two-group kernel (head_dim 128, a multiple of 4 query heads per kv head, at most 64 sequences): one to three
-    slices of four query heads per kv head, 1 / 2 / 3 / 6 / 8 / 16 slices in 1 / 2 / 8 teams of workgroups, rounds dealt
-    forwards, backwards and a short last round backwards.  Ragged lengths around the block boundaries, empty sequences and
-    one long prompt; the output starts as NaN, so an item that no workgroup took would show, and an item taken twice or
-    with the wrong heads would be wrong against the oracle."""
+def test_two_group_prefill_deals_every_item_once(hq, hkv, dtype, num_seqs):
+    """The two-group kernel (head_dim 128, an even number of query heads per kv head, at most 64 sequences).  Items of
+    four heads and 64 rows: one to three slices of four query heads per kv head, 1 / 2 / 3 / 6 / 8 / 16 slices in
+    1 / 2 / 8 teams of workgroups, rounds dealt forwards, backwards and a short last round backwards.  Items of two heads
+    and 128 rows (2, 6 or 10 query heads per kv head): 1 / 6 / 8 / 10 slices, the diagonal through an item's last two
+    tiles, the waves of the first 64 rows masking all of the last one.  Ragged lengths around the block boundaries,
+    empty sequences and one long prompt; the output starts as NaN, so an item that no workgroup took would show, and an
+    item taken twice or with the wrong heads would be wrong against the oracle."""
     d = 128
     g = torch.Generator().manual_seed(900 + 7 * num_seqs + hq)
     pool = [0, 1, 31, 32, 33, 63, 64, 65, 127, 128, 129, 191, 192, 193, 257, 300, 448]
     lengths = [pool[i] for i in torch.randint(0, len(pool), (num_seqs,), generator=g).tolist()]
     lengths[num_seqs // 2] = 2100 if hq <= 32 else 700           # 33 (or 11) blocks of 64 rows
-    q, k, v, cu = make_varlen_case(58, lengths, hq, hkv, d, dtype=torch.bfloat16)
+    q, k, v, cu = make_varlen_case(58, lengths, hq, hkv, d, dtype=dtype)
     scale = 1 / math.sqrt(d)
     from minivllm_amd import _C
     out = torch.full_like(q, float("nan")).to(DEV)

@@ -70,9 +70,9 @@ def test_paged_prefill_vs_oracle(dtype, hq, hkv, d, bs, lengths, cached):
 
 
 def test_paged_prefill_without_prefix_matches_plain_prefill_bitwise():
-    """No cached prefix: same tiles, same arithmetic as the packed kernel, only the copies' source differs.  (Two query
+    """No cached prefix: same tiles, same arithmetic as the packed kernel, only the copies' source differs.  (Three query
     heads per kv head: both calls run on prefill_mfma_kernel.)"""
-    hq, hkv, d, bs = 16, 8, 128, 16
+    hq, hkv, d, bs = 24, 8, 128, 16
     lengths = [257, 64, 31, 400]
     c = make_paged_prefill_case(62, lengths, [0] * 4, hq, hkv, d, bs, dtype=torch.bfloat16)
     scale = 1 / math.sqrt(d)
@@ -82,11 +82,12 @@ def test_paged_prefill_without_prefix_matches_plain_prefill_bitwise():
     assert torch.equal(got, plain)
 
 
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (16, 8)])
 @pytest.mark.parametrize("bs", [16, 48, 256])
-def test_two_group_paged_prefill_without_prefix_matches_packed_bitwise(bs):
-    """Four query heads per kv head: both calls run on the two-group kernel, same tiles, same arithmetic, only the
-    copies' source differs (the paged cache through the block table)."""
-    hq, hkv, d = 32, 8, 128
+def test_two_group_paged_prefill_without_prefix_matches_packed_bitwise(bs, hq, hkv):
+    """Four (or two) query heads per kv head: both calls run on the two-group kernel, same tiles, same arithmetic, only
+    the copies' source differs (the paged cache through the block table)."""
+    d = 128
     lengths = [257, 64, 31, 400, 1, 1000]
     c = make_paged_prefill_case(62, lengths, [0] * 6, hq, hkv, d, bs, dtype=torch.bfloat16)
     scale = 1 / math.sqrt(d)
@@ -200,15 +201,16 @@ def test_paged_prefill_over_an_int8_cache(dtype, hq, hkv, d, bs, lengths, cached
     assert mx <= 3e-2 and mean <= 3e-3, (mx, mean)
 
 
-@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (8, 2), (12, 3)])
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (8, 2), (12, 3), (16, 8), (12, 2), (2, 1)])
 @pytest.mark.parametrize("bs", [16, 48, 256])
 @pytest.mark.parametrize("num_seqs", [1, 9, 64])
 def test_two_group_paged_prefill_takes_every_item_once(hq, hkv, bs, num_seqs):
-    """The two-group kernel over cached prefixes (head_dim 128, a multiple of 4 query heads per kv head, at most 64
-    sequences): prefixes of 0, whole tiles and anything in between (the diagonal then crosses the last two key tiles of
-    an item), a single new token behind a long prefix, sequences with nothing new, blocks of 16, 48 and 256 tokens in
-    shuffled physical order with poisoned rows past every sequence's end.  The output starts as NaN, so an item that no
-    workgroup took would show."""
+    """The two-group kernel over cached prefixes (head_dim 128, an even number of query heads per kv head, at most 64
+    sequences; items of four heads and 64 rows, or with 2 / 6 heads per kv head of two heads and 128 rows): prefixes of
+    0, whole tiles and anything in between (the diagonal then crosses one tile more at an item's end), a single new
+    token behind a long prefix, sequences with nothing new, blocks of 16, 48 and 256 tokens in shuffled physical order
+    with poisoned rows past every sequence's end.  The output starts as NaN, so an item that no workgroup took would
+    show."""
     d = 128
     g = torch.Generator().manual_seed(1300 + num_seqs + bs + hq)
     pool = [1, 2, 31, 63, 64, 65, 100, 128, 129, 191, 192, 257, 300, 448]
