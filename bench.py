@@ -278,6 +278,20 @@ def bench_prefill_store(args, which, want_cpu=False):
         if want_cpu:
             out["prefill"]["cpu_baseline"] = cpu_prefill_baseline(q, k, v, cu, lengths, scale, hq, hkv, d, flops,
                                                                   flash_attention_prefill)
+    if "prefill" in which:
+        # the same prompts on 16 query / 8 kv heads, the attention shape of the reference's model (Qwen3-0.6B): the
+        # two-group kernel's items of two heads and 128 rows
+        q16 = q[:, :16].contiguous()
+        scale = 1.0 / math.sqrt(d)
+        _, event_ms_16 = time_steps(lambda: flash_attention_prefill(q16, k, v, cu, scale, 16, hkv, d),
+                                    args.steps, args.warmup, EXTRA_WARM_MS)
+        flops_16 = 4 * 16 * d * sum(n * (n + 1) // 2 for n in lengths)
+        out["prefill_hq16"] = {
+            "workload": "the same prompts on Hq16 Hkv8 D128 bf16 (two query heads per kv head)",
+            "algorithmic_flops": flops_16, "event_ms_per_step": event_ms_16, "tflops": flops_16 / (event_ms_16 * 1e-3) / 1e12,
+            "roofline": roofline("mfma", flops_16 / (event_ms_16 * 1e-3) / 1e12, "prefill_pp_kernel, items of two heads"),
+        }
+        del q16
     if "prefill_long" in which:
         # the same kernel away from config 2's short prompts: 4 prompts of 8192 tokens (the start and end of a
         # workgroup's life are a small share of its 128 key tiles)
@@ -322,7 +336,7 @@ def bench_prefill_store(args, which, want_cpu=False):
             "new_tokens": int(cu_q[-1]), "algorithmic_flops": flops, "event_ms_per_step": event_ms,
             "tflops": flops / (event_ms * 1e-3) / 1e12,
             "frac_of_bf16_mfma_peak": flops / (event_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-            "roofline": roofline("mfma", flops / (event_ms * 1e-3) / 1e12, "prefill_mfma_kernel, paged mode"),
+            "roofline": roofline("mfma", flops / (event_ms * 1e-3) / 1e12, "prefill_pp_kernel, paged form"),
         }
         # ... and over an INT8 cache holding the same keys (codes + scales written by the INT8 store)
         from minivllm_amd.layers.attention import flash_attention_prefill_paged_int8, store_kvcache_int8
@@ -879,6 +893,7 @@ def summary_of(line):
     put("prefill_tflops", "prefill", "tflops")
     put("prefill_us", "prefill", "event_ms_per_step")
     put("prefill_vs_oracle_max_abs", "prefill", "cpu_baseline", "gpu_vs_oracle_max_abs")
+    put("prefill_hq16_frac", "prefill_hq16", "roofline", "frac")
     put("prefill_4x8192_frac", "prefill_long_prompts", "roofline", "frac")
     put("prefill_paged_frac", "prefill_cached_prefix", "roofline", "frac")
     put("prefill_paged_int8_frac", "prefill_cached_prefix_int8", "roofline", "frac")
