@@ -232,11 +232,13 @@ struct PrefillPpArgs {
   int64_t num_blocks;
   // filled in by the launcher
   unsigned block_magic;   // 2^32 / block_size + 1
-  int slices;       // head slices: kv heads x (query heads per kv head / 4)
+  int block_bytes;        // bytes of one cache block (all kv heads); filled by the launcher
+  int num_blocks32;       // num_blocks, capped at 2^31 - 1 (table entries are 32-bit); filled by the launcher
+  int slices;       // head slices: kv heads x (query heads per kv head / heads per item)
   int n_teams;      // gcd(8, slices): workgroup teams, each with its own item list
   int team_size;    // workgroups per team
   int level_bits;   // bits that hold the block count of the longest possible sequence
-  unsigned spt_magic, chunks_magic;   // 2^32 / d + 1 for d = slices per team and d = query heads per kv head / 4 (0 for d = 1)
+  unsigned spt_magic, chunks_magic;   // 2^32 / d + 1 for d = slices per team and d = query heads per kv head / heads per item (0 for d = 1)
   // timing build only (the probe library): where workgroup `timeline_block` logs its clock stamps; null otherwise
   unsigned long long* timeline;
   int timeline_entries;

@@ -279,13 +279,13 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // descriptor starts at the piece and ends with the sequence's last key, so rows that were never written, unmapped
   // blocks and tiles past the stream's end arrive as zeros.
   int d_phys = -1;                             // table entry of the cursor's piece
-  int d_in_block = 0;                          // ... and its first row inside that block
+  int d_in_off = 0;                            // ... and the byte offset of its first row (at the item's kv head) inside that block
   int d_kv_len = 0;                            // keys of the cursor's sequence
   auto fetch_entry = [&]() {                   // for the cursor's tile (dit, dj)
     if constexpr (PAGED) {
       const unsigned pos = (unsigned)(kPpBN * dj + 16 * wq);
       const unsigned bi = div_small(pos, (unsigned)a.block_size, a.block_magic);
-      d_in_block = (int)(pos - bi * (unsigned)a.block_size);
+      d_in_off = (int)(pos - bi * (unsigned)a.block_size) * kv_row_bytes + d_head_off;
       // (read through the constant address space: a scalar load, which the copies' vmcnt accounting does not see; a
       // vector load here would make the compiler wait for every copy in flight before each use of the entry)
       typedef const __attribute__((address_space(4))) int32_t* ConstTable;
@@ -306,15 +306,14 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   enter_item();
   fetch_entry();
   int d_slot = 0;                              // ring slot of the cursor's tile ( = its stream index % 3)
-  auto copy_step = [&]() {
+  auto issue_copy = [&]() {                    // the cursor's tile -> its ring slot
     v4i r;
     if constexpr (PAGED) {
       const int pos = kPpBN * dj + 16 * wq;
       const int valid = d_kv_len - pos < 16 ? d_kv_len - pos : 16;
-      const int in_block = d_in_block;
-      const bool ok = dit.valid && valid > 0 && d_phys >= 0 && (int64_t)d_phys < a.num_blocks;
+      const bool ok = dit.valid && valid > 0 && (unsigned)d_phys < (unsigned)a.num_blocks32;   // (-1: not mapped)
       const uint32_t size = ok ? (uint32_t)(valid - 1) * (uint32_t)kv_row_bytes + (uint32_t)kRowB : 0u;
-      const int64_t start = ok ? ((int64_t)d_phys * a.block_size + in_block) * kv_row_bytes + d_head_off : 0;
+      const int64_t start = ok ? (int64_t)d_phys * a.block_bytes + d_in_off : 0;
       r = make_rsrc(copy_src + start, size);
     } else {
       const uint32_t size = d_rows_left <= 0        ? 0u
@@ -326,6 +325,9 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
 #pragma unroll
     for (int i = 0; i < 4; ++i) dma16(r, src_off[i], dst + 1024u * i);
     d_slot = d_slot == kPpRing - 1 ? 0 : d_slot + 1;
+  };
+  auto copy_step = [&]() {
+    issue_copy();
     if (dit.valid) {
       if (++dj > dit.nt) {
         dit = item_at(++di);
@@ -337,6 +339,18 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       }
       fetch_entry();
     }
+  };
+  // The same where the caller knows that the cursor stays inside its item (the cursor is two tiles ahead of the
+  // arithmetic, so this holds in tiles 1 .. nt - 3 of an item): no test, no item located, and none of the register
+  // copies that the merge with that path costs in every tile.
+  auto copy_step_inside = [&]() {
+    issue_copy();
+    ++dj;
+    if constexpr (!PAGED) {
+      d_off += (int64_t)kPpBN * kv_row_bytes;
+      d_rows_left -= kPpBN;
+    }
+    fetch_entry();
   };
   // Q rows of an item -> this wave's slot, 4 rows per instruction, chunks swizzled like a K tile's
   const uint32_t lds_q = lds_address(&lds.qo[wave][0]);
@@ -731,9 +745,10 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
   // the softmax interval of tile j > 0 of `cur`, up to the barrier; returns nothing, leaves pf, l, vf0, vf1
   // MASKED: the tile the diagonal may cross (the last one; paged: also the one before it when the prefix does not end
   // on a tile boundary, which has a call of its own so that the middle tiles carry no test for it)
-  auto later_tile = [&](auto LAST, auto MASKED, int j, uint4 (&vf0)[kTD], uint4 (&vf1)[kTD]) {
+  auto later_tile = [&](auto LAST, auto MASKED, auto INSIDE, int j, uint4 (&vf0)[kTD], uint4 (&vf1)[kTD]) {
     TSTAMP();
-    copy_step();
+    if constexpr (decltype(INSIDE)::value) copy_step_inside();
+    else copy_step();
     if constexpr (PAGED || HPI != 4) {
       if constexpr (decltype(LAST)::value) mask_tile(j);
       else if constexpr (decltype(MASKED)::value) {
@@ -812,28 +827,37 @@ __device__ __forceinline__ void pp_run(const PrefillPpArgs& a, PpLds<D>& lds, co
       // ======== the item's other tiles ========
       if constexpr (HPI == 4) {
         const int plain_end = PAGED ? cur.nt - 1 : cur.nt;
-        for (int j = 1; j < plain_end; ++j) {
-          later_tile(std::false_type{}, std::false_type{}, j, vf0, vf1);
+        int j = 1;
+        for (; j < cur.nt - 2; ++j) {              // the copy cursor stays inside this item
+          later_tile(std::false_type{}, std::false_type{}, std::true_type{}, j, vf0, vf1);
+          matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
+        }
+        for (; j < plain_end; ++j) {
+          later_tile(std::false_type{}, std::false_type{}, std::false_type{}, j, vf0, vf1);
           matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
         }
         if constexpr (PAGED) {
           if (cur.nt >= 2) {
-            later_tile(std::false_type{}, std::true_type{}, cur.nt - 1, vf0, vf1);
+            later_tile(std::false_type{}, std::true_type{}, std::false_type{}, cur.nt - 1, vf0, vf1);
             matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
           }
         }
       } else {
         int j = 1;
+        for (; j < cur.nt - 2; ++j) {              // the copy cursor stays inside this item (masked_tail >= 2)
+          later_tile(std::false_type{}, std::false_type{}, std::true_type{}, j, vf0, vf1);
+          matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
+        }
         for (; j <= cur.nt - masked_tail; ++j) {
-          later_tile(std::false_type{}, std::false_type{}, j, vf0, vf1);
+          later_tile(std::false_type{}, std::false_type{}, std::false_type{}, j, vf0, vf1);
           matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
         }
         for (; j < cur.nt; ++j) {                  // one or two tiles before the last that the diagonal crosses
-          later_tile(std::false_type{}, std::true_type{}, j, vf0, vf1);
+          later_tile(std::false_type{}, std::true_type{}, std::false_type{}, j, vf0, vf1);
           matrix_interval(std::false_type{}, std::false_type{}, false, vf0, vf1);
         }
       }
-      later_tile(std::true_type{}, std::true_type{}, cur.nt, vf0, vf1);
+      later_tile(std::true_type{}, std::true_type{}, std::false_type{}, cur.nt, vf0, vf1);
       more = matrix_interval(std::false_type{}, std::true_type{}, false, vf0, vf1);
     }
     TCOUNT(1, cur.nt + 1);
@@ -879,6 +903,7 @@ static void launch_prefill_pp_as(const PrefillPpArgs& a, bool paged, int hpi, di
 bool prefill_pp_takes(int num_seqs, int num_heads, int num_kv_heads, int head_dim, int dtype, int block_size) {
   if (dtype == MVLLM_F32 || head_dim != 128 || num_seqs > 64 || num_seqs <= 0) return false;
   if (block_size != 0 && (block_size < 16 || block_size % 16 != 0)) return false;      // paged: a wave's 16 rows lie in one block
+  if ((int64_t)block_size * num_kv_heads * head_dim * 2 >= ((int64_t)1 << 31)) return false;   // a block's bytes in 32 bits
   const int group = num_heads / num_kv_heads;
   return group % 2 == 0 && (int64_t)num_heads * head_dim * 2 * 64 < ((int64_t)1 << 31);
 }
@@ -905,6 +930,8 @@ int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) 
   a.chunks_magic = magic(group / hpi);
   const bool paged = a.block_tables != nullptr;
   a.block_magic = magic(a.block_size);
+  a.block_bytes = a.block_size * a.num_kv_heads * 128 * 2;
+  a.num_blocks32 = a.num_blocks > 0x7fffffff ? 0x7fffffff : (int)a.num_blocks;
   // levels: the tile count of the longest possible sequence (paged: as wide as its block-table row)
   const int64_t most_keys = paged ? (int64_t)a.max_num_blocks * a.block_size + a.total_tokens : a.total_tokens;
   a.level_bits = 1;
@@ -935,7 +962,7 @@ extern "C" int mvllm_probe_prefill_timeline(void* out, const void* q, const void
   p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
   p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
   p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0; p.spt_magic = 0; p.chunks_magic = 0;
-  p.cu_seqlens_k = nullptr; p.block_tables = nullptr; p.max_num_blocks = 0; p.block_size = 0; p.num_blocks = 0; p.block_magic = 0;
+  p.cu_seqlens_k = nullptr; p.block_tables = nullptr; p.max_num_blocks = 0; p.block_size = 0; p.num_blocks = 0; p.block_magic = 0; p.block_bytes = 0; p.num_blocks32 = 0;
   p.timeline = log; p.timeline_entries = entries_per_wave; p.timeline_block = block;
   return launch_prefill_pp(p, dtype, (hipStream_t)stream);
 }

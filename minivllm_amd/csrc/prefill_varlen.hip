@@ -192,7 +192,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
     p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
     p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
     p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0; p.spt_magic = 0; p.chunks_magic = 0;
-    p.cu_seqlens_k = nullptr; p.block_tables = nullptr; p.max_num_blocks = 0; p.block_size = 0; p.num_blocks = 0; p.block_magic = 0;
+    p.cu_seqlens_k = nullptr; p.block_tables = nullptr; p.max_num_blocks = 0; p.block_size = 0; p.num_blocks = 0; p.block_magic = 0; p.block_bytes = 0; p.num_blocks32 = 0;
     p.timeline = nullptr; p.timeline_entries = 0; p.timeline_block = 0;
     return launch_prefill_pp(p, dtype, (hipStream_t)stream);
   }
@@ -238,7 +238,7 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
     p.out = out; p.q = q; p.k = k_cache; p.v = v_cache; p.cu_seqlens = cu_seqlens_q; p.total_tokens = total_q_tokens;
     p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;
     p.cu_seqlens_k = cu_seqlens_k; p.block_tables = block_tables; p.max_num_blocks = max_num_blocks;
-    p.block_size = block_size; p.num_blocks = num_blocks; p.block_magic = 0;
+    p.block_size = block_size; p.num_blocks = num_blocks; p.block_magic = 0; p.block_bytes = 0; p.num_blocks32 = 0;
     p.slices = 0; p.n_teams = 0; p.team_size = 0; p.level_bits = 0; p.spt_magic = 0; p.chunks_magic = 0;
     p.timeline = nullptr; p.timeline_entries = 0; p.timeline_block = 0;
     return launch_prefill_pp(p, dtype, (hipStream_t)stream);
