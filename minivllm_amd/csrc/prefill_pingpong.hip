@@ -932,10 +932,12 @@ int launch_prefill_pp(const PrefillPpArgs& args, int dtype, hipStream_t stream) 
   a.block_magic = magic(a.block_size);
   a.block_bytes = a.block_size * a.num_kv_heads * 128 * 2;
   a.num_blocks32 = a.num_blocks > 0x7fffffff ? 0x7fffffff : (int)a.num_blocks;
-  // levels: the tile count of the longest possible sequence (paged: as wide as its block-table row)
+  // levels: one past the last key tile of the longest possible sequence (paged: as wide as its block-table row).  An
+  // item of 128 rows counts its tiles from its block's last row, which may lie up to 127 positions past the
+  // sequence's last key: three tiles of margin.
   const int64_t most_keys = paged ? (int64_t)a.max_num_blocks * a.block_size + a.total_tokens : a.total_tokens;
   a.level_bits = 1;
-  while (((int64_t)1 << a.level_bits) <= most_keys / 64 + 2) ++a.level_bits;
+  while (((int64_t)1 << a.level_bits) <= most_keys / 64 + 4) ++a.level_bits;
   const dim3 g(grid), b(64 * kPpWaves);
   if (dtype == MVLLM_BF16) launch_prefill_pp_as<bf16_t>(a, paged, hpi, g, b, stream);
   else launch_prefill_pp_as<f16_t>(a, paged, hpi, g, b, stream);

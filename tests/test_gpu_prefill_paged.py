@@ -238,6 +238,28 @@ def test_two_group_paged_prefill_takes_every_item_once(hq, hkv, bs, num_seqs):
     _check(out.cpu(), _oracle32(c, scale, hq, hkv, d, bs), torch.bfloat16)
 
 
+@pytest.mark.parametrize("hq,hkv,new,cached", [(16, 8, 4, 846), (10, 1, 5, 1873), (40, 4, 5, 72), (2, 1, 3, 833),
+                                               (32, 8, 4, 846), (16, 8, 1, 0), (16, 8, 129, 1)])
+def test_two_group_paged_prefill_short_tail_behind_a_long_prefix(hq, hkv, new, cached):
+    """One sequence, a few new tokens behind a prefix that ends early in a key tile: an item of 128 rows ranks by the tile
+    of its block's last row, up to two tiles past the sequence's last key, and the walk over the ranks has to start
+    above it (a walk that started at the last key's tile left such an item to no workgroup).  The output starts as
+    NaN."""
+    d, bs = 128, 16
+    c = make_paged_prefill_case(71, [new + cached], [cached], hq, hkv, d, bs, dtype=torch.float16)
+    scale = 1 / math.sqrt(d)
+    from minivllm_amd import _C
+    q_new = c["q_new"].to(DEV)
+    out = torch.full_like(q_new, float("nan"))
+    kc, vc, bt, cuq, cuk = (c[k].to(DEV) for k in ("k_cache", "v_cache", "block_tables", "cu_q", "cu_k"))
+    st = _C.load().mvllm_prefill_paged(out.data_ptr(), q_new.data_ptr(), kc.data_ptr(), vc.data_ptr(), bt.data_ptr(),
+                                       bt.shape[1], cuq.data_ptr(), cuk.data_ptr(), 1, q_new.shape[0], hq, hkv, d, bs,
+                                       kc.shape[0], scale, _C.dtype_code(q_new.dtype), _C.current_stream_ptr(out.device))
+    torch.cuda.synchronize()
+    assert st == 0
+    _check(out.cpu(), _oracle32(c, scale, hq, hkv, d, bs), torch.float16)
+
+
 def _half_step(dtype):
     """Half the spacing of the output type relative to the value: what rounding the result alone may cost."""
     return 2.0 ** -9 if dtype == torch.bfloat16 else 2.0 ** -12
