@@ -99,7 +99,8 @@ size_t mvllm_paged_decode_workspace_bytes(int batch, int num_heads, int head_dim
  *                     >1: small-batch form, a workgroup is that many waves on one kv head that share the
  *                     partition's 16-token tiles and merge in LDS; 0: the generic kernel (head_dim other than
  *                     128 or 64 (bf16 / fp16 caches: also every other multiple of 8 from 32 to 120, and 256),
- *                     block_size % 16 != 0, more than 16 query heads per kv head, or fp32 queries over an INT8 cache)
+ *                     block_size % 16 != 0, or fp32 queries over an INT8 cache).  A kv head with more than 16 query
+ *                     heads is served in slices of 16, each of which streams its keys and values again.
  * Returns MVLLM_OK or MVLLM_ERR_BAD_SHAPE / MVLLM_ERR_BAD_DTYPE.
  */
 int mvllm_paged_decode_plan(int batch, int num_heads, int num_kv_heads, int head_dim,

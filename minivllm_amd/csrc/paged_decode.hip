@@ -2,10 +2,10 @@
 // GQA-shared K/V reads, log-sum-exp merge in a second pass.
 // Replaces the Triton kernel of src/myvllm/layers/attention.py:283-415.
 //
-// Work decomposition (fast path, 16-bit cache, head_dim 128 or 64, block_size % 16 == 0, up to 16 query heads per kv head)
+// Work decomposition (fast path, 16-bit cache, head_dim 128 or 64, block_size % 16 == 0)
 //   workgroup = (partition p, sequence b, group of <= 4 kv heads); wave w of the
-//   workgroup owns kv head g and all Hq/Hkv query heads that share it, so the
-//   waves of one workgroup stream contiguous pieces of the [token, Hkv, D] rows.
+//   workgroup owns kv head g and all Hq/Hkv query heads that share it (16 of them at a time where a kv head has more:
+//   head_slice), so the waves of one workgroup stream contiguous pieces of the [token, Hkv, D] rows.
 //   A wave walks its partition in tiles of 16 tokens, both products on the matrix unit:
 //     S[16 tok x 16 head]  = K_tile (A operand, straight from global in MFMA
 //                            layout) x Q^T (B operand, column n = head n)
@@ -65,7 +65,24 @@ struct DecodeArgs {
   int part_tokens;
   int num_parts;          // partitions per sequence in the grid / workspace
   float scale_log2;       // scale * log2(e)
+  int head_chunks;        // MFMA kernels: slices of up to 16 query heads per kv head (1 unless a kv head has more than 16)
 };
+
+// The query heads one wave of the MFMA kernels works for.  A wave holds up to 16 query heads as the 16 columns of its
+// matrix tiles.  With at most 16 query heads per kv head, slice s is kv head s with all of its query heads; with more, a
+// kv head's query heads are split into head_chunks slices of 16 (the last may hold fewer), each of which streams the
+// kv head's keys and values again.
+struct HeadSlice {
+  int kvh;      // kv head
+  int head0;    // first query head
+  int heads;    // query heads (<= 16)
+};
+__device__ __forceinline__ HeadSlice head_slice(const DecodeArgs& a, int s) {
+  const int group = a.num_heads / a.num_kv_heads;
+  if (a.head_chunks <= 1) return {s, s * group, group};
+  const int kvh = s / a.head_chunks, c = s - kvh * a.head_chunks;
+  return {kvh, kvh * group + 16 * c, min(16, group - 16 * c)};
+}
 
 // Partition length.  Lower bound: the smallest multiple of 256 tokens that covers the widest context with
 // kMaxParts partitions.  Longer partitions amortise the per-workgroup start-up better (1024 tokens measured
@@ -262,14 +279,13 @@ template <> __device__ __forceinline__ v4f mfma16x16x16<f16_t>(uint2 x, uint2 y,
 
 // Shared by the 16-bit and fp32 heads (HEAD has m, l, o[kAcc], write_row, write_partial).
 template <typename HEAD>
-__device__ __forceinline__ void finish_head(HEAD& hd, const DecodeArgs& a, int b, int p, int g, int group, bool direct, int lane) {
+__device__ __forceinline__ void finish_head(HEAD& hd, const DecodeArgs& a, int b, int p, int head0, int group, bool direct, int lane) {
   using T = typename HEAD::Elem;
   constexpr int D = HEAD::kDim;
   const int cls = lane >> 4;
   // denominators: add the four token classes (every lane of a head then holds the head's total)
   hd.l += __shfl_xor(hd.l, 16, 64);
   hd.l += __shfl_xor(hd.l, 32, 64);
-  const int head0 = g * group;
   if (direct) {
     T* out = reinterpret_cast<T*>(a.out);
     const float linv = hd.l > 0.f ? 1.f / hd.l : 0.f;
@@ -333,10 +349,10 @@ struct DecodeHead {
 #pragma unroll
     for (int e = 0; e < kAcc; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
   }
-  __device__ __forceinline__ void start(const DecodeArgs& a, int b, int g, int group, int lane) {
+  __device__ __forceinline__ void start(const DecodeArgs& a, int b, int head0, int group, int lane) {
     const int col = lane & 15;
     const bool live = col < group;
-    load_q(reinterpret_cast<const T*>(a.q) + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D, live, lane);
+    load_q(reinterpret_cast<const T*>(a.q) + ((int64_t)b * a.num_heads + head0 + (live ? col : 0)) * D, live, lane);
   }
   // this lane's dims of accumulator row j (head or query row 4*(lane/16) + j), scaled, into the row of D elements
   __device__ __forceinline__ void write_row(T* row_ptr, int j, float scale, int lane) const {
@@ -489,8 +505,8 @@ struct DecodeHead {
   }
 
   // write the output row (direct) or this partition's partial result
-  __device__ __forceinline__ void finish(const DecodeArgs& a, int b, int p, int g, int group, bool direct, int lane) {
-    finish_head(*this, a, b, p, g, group, direct, lane);
+  __device__ __forceinline__ void finish(const DecodeArgs& a, int b, int p, int head0, int group, bool direct, int lane) {
+    finish_head(*this, a, b, p, head0, group, direct, lane);
   }
 };
 
@@ -525,10 +541,10 @@ struct DecodeHead<float, D> {
 #pragma unroll
     for (int e = 0; e < kAcc; ++e) o[e] = (v4f){0.f, 0.f, 0.f, 0.f};
   }
-  __device__ __forceinline__ void start(const DecodeArgs& a, int b, int g, int group, int lane) {
+  __device__ __forceinline__ void start(const DecodeArgs& a, int b, int head0, int group, int lane) {
     const int col = lane & 15;
     const bool live = col < group;
-    load_q(reinterpret_cast<const float*>(a.q) + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D, live, lane);
+    load_q(reinterpret_cast<const float*>(a.q) + ((int64_t)b * a.num_heads + head0 + (live ? col : 0)) * D, live, lane);
   }
 
   __device__ __forceinline__ void consume(const KVTile<float, D>& t, int part_end, float scale_log2, int lane,
@@ -648,8 +664,8 @@ struct DecodeHead<float, D> {
           make_float4(o[4 * jj][j] * scale, o[4 * jj + 1][j] * scale, o[4 * jj + 2][j] * scale, o[4 * jj + 3][j] * scale);
   }
   __device__ __forceinline__ void write_partial(float* row_ptr, int j, int lane) const { write_row(row_ptr, j, 1.f, lane); }
-  __device__ __forceinline__ void finish(const DecodeArgs& a, int b, int p, int g, int group, bool direct, int lane) {
-    finish_head(*this, a, b, p, g, group, direct, lane);
+  __device__ __forceinline__ void finish(const DecodeArgs& a, int b, int p, int head0, int group, bool direct, int lane) {
+    finish_head(*this, a, b, p, head0, group, direct, lane);
   }
 };
 
@@ -657,9 +673,11 @@ struct DecodeHead<float, D> {
 // tiles w, w + W, ... and the partial results meet in LDS (DecodeHead::merge), so a short context costs a few tiles
 // of latency per wave and no second launch.
 template <typename T, int W, int D>
-__device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int p, int g, int w) {   // g: kv head
+__device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int p, int slice, int w) {
   const int lane = threadIdx.x & 63;
-  const int group = a.num_heads / a.num_kv_heads;      // q heads per kv head (<= 16)
+  const HeadSlice hs = head_slice(a, slice);
+  const int g = hs.kvh;                                // kv head
+  const int group = hs.heads;                          // q heads of this wave (<= 16)
   const int col = lane & 15;                           // head (first product), dim group (second product)
   const int cls = lane >> 4;                           // token class: tokens 4*cls .. 4*cls+3 of a tile
   const int bs = a.block_size;
@@ -676,7 +694,7 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
   int win_base = bi;
   int win;
   auto prologue = [&]() __attribute__((always_inline)) {
-    head.start(a, b, g, group, lane);
+    head.start(a, b, hs.head0, group, lane);
     win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
   };
   if constexpr (W > 1) prologue();
@@ -745,7 +763,7 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
   if constexpr (W > 1) {
     if (!head.template merge<W>(w, lane)) return;
   }
-  head.finish(a, b, p, g, group, direct, lane);
+  head.finish(a, b, p, hs.head0, group, direct, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -885,7 +903,7 @@ __global__ __launch_bounds__(256) void prefill_rows16_kernel(const PrefillRowsAr
 }
 
 // ---------------------------------------------------------------------------
-// Fast path, INT8 cache (head_dim 128, block_size % 16 == 0, up to 16 query heads per kv head).  Same
+// Fast path, INT8 cache (head_dim 128 or 64, block_size % 16 == 0).  Same
 // decomposition as the 16-bit kernel, both products on the matrix unit.
 //   QK^T   v_mfma_i32_16x16x64_i8 with the int8 codes as they lie in memory (lane = token, 16 bytes = 16 dims):
 //          the query row is turned once per wave into 15-bit fixed point q ~ (128*hi + lo) * amax/16256 with
@@ -923,13 +941,15 @@ __device__ __forceinline__ uint2 load8_stream(const void* p) {
 
 // W as in decode_mfma_item: 1 = the wave walks its partition, > 1 = W waves of the workgroup share it.
 template <typename T, int NCH, int W, int D>
-__device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b, int p, int g, int w) {   // g: kv head
+__device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b, int p, int slice, int w) {
   static_assert(NCH == 1, "one chunk of up to 16 heads");
   static_assert(D == 128 || D == 64, "one or two 64-dim steps");
   constexpr int kSteps = D / 64;               // 64-dim steps of the first product
   const bool owns = D == 128 || (threadIdx.x & 15) < D / 8;   // this lane's 8 output dims exist
   const int lane = threadIdx.x & 63;
-  const int group = a.num_heads / a.num_kv_heads;
+  const HeadSlice hs = head_slice(a, slice);
+  const int g = hs.kvh;                // kv head
+  const int group = hs.heads;          // q heads of this wave (<= 16)
   const int q4 = lane >> 4;            // token class: tokens 4*q4 .. 4*q4+3 of a tile
   const int col = lane & 15;           // head (first product), dim group (second product)
   const int bs = a.block_size;
@@ -957,7 +977,7 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
   {
     const T* q = reinterpret_cast<const T*>(a.q);
     const bool live = col < group;
-    const T* src = q + ((int64_t)b * a.num_heads + (int64_t)g * group + (live ? col : 0)) * D;
+    const T* src = q + ((int64_t)b * a.num_heads + hs.head0 + (live ? col : 0)) * D;
     float x[kSteps][16];
     float amax = 0.f;
 #pragma unroll
@@ -1177,7 +1197,7 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
   l += __shfl_xor(l, 32, 64);
   wsum += __shfl_xor(wsum, 16, 64);
   wsum += __shfl_xor(wsum, 32, 64);
-  const int head0 = g * group;
+  const int head0 = hs.head0;
   const float linv = l > 0.f ? 1.f / l : 0.f;
   const int64_t slot = ((int64_t)b * a.num_parts + p) * a.num_heads + head0;
 #pragma unroll
@@ -1488,9 +1508,12 @@ static void with_other_mfma_dim(int head_dim, F&& go) {
 static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool int8) {
   // 16-bit caches: a multiple of 8 from 32 to 128, or 256, dims per head; fp32 and INT8 caches: 64 or 128
   const bool dim_ok = head_dim == 128 || head_dim == 64 || (dtype != MVLLM_F32 && !int8 && other_mfma_dim(head_dim));
-  return (dtype != MVLLM_F32 || !int8) && dim_ok && block_size % kTile == 0 && num_heads / num_kv_heads <= 16 &&
+  return (dtype != MVLLM_F32 || !int8) && dim_ok && block_size % kTile == 0 &&
          (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
 }
+
+// slices of up to 16 query heads per kv head (a wave's matrix tiles have 16 columns for them)
+static int head_chunks_of(int num_heads, int num_kv_heads) { return (num_heads / num_kv_heads + 15) / 16; }
 
 struct DecodePlan {
   int part_tokens, num_parts, waves_per_head;
@@ -1513,11 +1536,13 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
   bool launched = false;
   // kv heads (waves) per workgroup of the one-wave-per-head form: as many as allowed, so that a workgroup streams
   // whole token rows; fewer when the grid would otherwise leave most CUs without a workgroup
-  int wpb = largest_divisor_le(a.num_kv_heads, int8 ? kDecodeI8Wpb : kDecodeWpb);
-  while (wpb > 1 && (int64_t)a.num_parts * a.batch * (a.num_kv_heads / wpb) < kDecodeSmallGrid)
-    wpb = largest_divisor_le(a.num_kv_heads, wpb - 1);
-  const unsigned groups = (unsigned)(a.num_kv_heads / wpb);
-  const dim3 split_grid((unsigned)a.num_kv_heads, (unsigned)a.num_parts, (unsigned)a.batch), split_block(64 * kSplitWaves);
+  // (a wave's unit of work is a head slice: a kv head, or 16 of its query heads where it has more than 16)
+  const int slices = a.num_kv_heads * a.head_chunks;
+  int wpb = largest_divisor_le(slices, int8 ? kDecodeI8Wpb : kDecodeWpb);
+  while (wpb > 1 && (int64_t)a.num_parts * a.batch * (slices / wpb) < kDecodeSmallGrid)
+    wpb = largest_divisor_le(slices, wpb - 1);
+  const unsigned groups = (unsigned)(slices / wpb);
+  const dim3 split_grid((unsigned)slices, (unsigned)a.num_parts, (unsigned)a.batch), split_block(64 * kSplitWaves);
   const dim3 block(64 * wpb);
   if (fast_ok && !int8) {
     const dim3 grid((unsigned)a.num_parts, (unsigned)a.batch, groups);
@@ -1594,7 +1619,8 @@ static int decode_entry(void* out, const void* q, const void* k_cache, const voi
   a.block_size = block_size;
   const bool fast_ok = fast_shape(num_heads, num_kv_heads, head_dim, block_size, dtype, int8) &&
                        aligned16(q) && aligned16(out) && aligned16(k_cache) && aligned16(v_cache);
-  const DecodePlan plan = plan_decode(batch, num_kv_heads, max_num_blocks, block_size, fast_ok, int8);
+  a.head_chunks = head_chunks_of(num_heads, num_kv_heads);
+  const DecodePlan plan = plan_decode(batch, num_kv_heads * a.head_chunks, max_num_blocks, block_size, fast_ok, int8);
   const bool split = plan.waves_per_head > 1;
   a.part_tokens = plan.part_tokens;
   a.num_parts = plan.num_parts;
@@ -1667,7 +1693,7 @@ extern "C" int mvllm_paged_decode_plan(int batch, int num_heads, int num_kv_head
   if (batch <= 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 || max_num_blocks <= 0 ||
       num_heads % num_kv_heads != 0)
     return MVLLM_ERR_BAD_SHAPE;
-  const DecodePlan plan = plan_decode(batch, num_kv_heads, max_num_blocks, block_size,
+  const DecodePlan plan = plan_decode(batch, num_kv_heads * head_chunks_of(num_heads, num_kv_heads), max_num_blocks, block_size,
                                       fast_shape(num_heads, num_kv_heads, head_dim, block_size, dtype, int8_cache != 0), int8_cache != 0);
   if (part_tokens) *part_tokens = plan.part_tokens;
   if (num_parts) *num_parts = plan.num_parts;

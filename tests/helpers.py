@@ -61,6 +61,15 @@ def make_slot_mapping(seed, lengths, block_size, extra_blocks=2):
     return torch.tensor(slots, dtype=torch.int64), tables, num_blocks
 
 
+def half_step(ref, dtype):
+    """Half the spacing of `dtype` (bf16: 8 significant bits, fp16: 11) at each value of `ref`: what rounding a
+    result to that type may cost by itself, 2^(floor(log2 |x|) - 8) or - 11; between |x| 2^-9 and |x| 2^-8 for bf16."""
+    bits = 8 if dtype == torch.bfloat16 else 11
+    mag = ref.to(torch.float32).abs()
+    step = torch.exp2(torch.floor(torch.log2(mag.clamp_min(2.0 ** -100))) - bits)
+    return torch.where(mag > 0, step, torch.zeros_like(step))
+
+
 def error_stats(out, ref):
     diff = (out.to(torch.float32) - ref.to(torch.float32)).abs()
     return diff.max().item(), diff.mean().item()

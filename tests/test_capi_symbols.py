@@ -86,7 +86,7 @@ def test_decode_plan_is_host_arithmetic():
     assert paged_decode_plan(64, 16, 8, 256, 256, 16, dtype=__import__("torch").float32)[2] == 0
     assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32)[2] == 4       # fp32 caches: fp32 MFMA
     assert paged_decode_plan(64, 32, 8, 128, 256, 16, dtype=torch.float32, int8_cache=True)[2] == 0
-    assert paged_decode_plan(8, 34, 2, 128, 64, 16)[2] == 0                   # 17 query heads per kv head
+    assert paged_decode_plan(8, 34, 2, 128, 64, 16)[2] == 4                   # 17 query heads per kv head: two slices each
     # the advertised workspace covers whatever form is chosen
     for batch in (1, 3, 16, 64, 200, 1000):
         for blocks, bs in ((16, 16), (64, 16), (300, 16), (2048, 16), (40, 256), (70000, 16)):

@@ -204,7 +204,8 @@ def _pad_tables(tables, width_tokens, bs):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("hq,hkv,bs,d", [(32, 8, 16, 128), (16, 8, 256, 128), (16, 1, 32, 128), (24, 2, 16, 128),
                                          (5, 1, 64, 128), (8, 8, 48, 128),
-                                         (16, 8, 16, 64), (16, 16, 256, 64), (12, 1, 32, 64), (5, 5, 48, 64)])
+                                         (16, 8, 16, 64), (16, 16, 256, 64), (12, 1, 32, 64), (5, 5, 48, 64),
+                                         (34, 2, 16, 128), (48, 1, 32, 128), (71, 1, 16, 64)])
 @pytest.mark.parametrize("form", ["one wave per head", "waves share a head", "waves share a head, one partition"])
 def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, d, form):
     """A ragged batch (contexts 1..1300, one empty) through both forms of the MFMA kernel: the batch size and the
@@ -212,7 +213,8 @@ def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, d, form):
     one-wave-per-head grid; 7 sequences in a table of 8 K tokens are spread over four waves per head in several
     partitions; 64 sequences x 8 kv heads in a table of 4 K tokens are one partition each, written without the
     merge kernel.  head_dim 64 (the reference demo's model, qwen3.py:338) runs on the same kernels with half of
-    the second product's columns switched off."""
+    the second product's columns switched off.  More than 16 query heads per kv head (17, 48, 71) are served in slices
+    of 16, the last one partial."""
     batch = 7 if form == "waves share a head" else 64
     width = {"one wave per head": 32768, "waves share a head": 8192}.get(form, 4096) // bs * bs
     g = torch.Generator().manual_seed(77)

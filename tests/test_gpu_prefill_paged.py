@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import error_stats, make_paged_prefill_case
+from helpers import error_stats, half_step, make_paged_prefill_case
 from minivllm_amd.layers.attention import (Attention, flash_attention_prefill, flash_attention_prefill_paged,
                                            paged_attention_decode)
 from minivllm_amd.utils import reset_context, set_context
@@ -190,7 +190,7 @@ def test_paged_prefill_over_an_int8_cache(dtype, hq, hkv, d, bs, lengths, cached
                                        hq, hkv, d, bs)
     assert got.dtype == dtype and got.shape == want.shape and torch.isfinite(got.float()).all()
     mx, mean = error_stats(got, want)
-    excess = ((got.float() - want).abs() - want.abs() * _half_step(dtype)).max().item()
+    excess = ((got.float() - want).abs() - half_step(want, dtype)).max().item()
     assert excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
     # one new token per sequence: the same rows as INT8 decode over the same cache
     from minivllm_amd.layers.attention import paged_attention_decode_int8
@@ -260,11 +260,6 @@ def test_two_group_paged_prefill_short_tail_behind_a_long_prefix(hq, hkv, new, c
     _check(out.cpu(), _oracle32(c, scale, hq, hkv, d, bs), torch.float16)
 
 
-def _half_step(dtype):
-    """Half the spacing of the output type relative to the value: what rounding the result alone may cost."""
-    return 2.0 ** -9 if dtype == torch.bfloat16 else 2.0 ** -12
-
-
 @pytest.mark.parametrize("hq,hkv,d,bs", [(16, 8, 64, 16), (32, 8, 128, 16), (6, 2, 64, 48)])
 def test_int8_paged_prefill_short_sequences(hq, hkv, d, bs):
     """Queries with one to a dozen keys over an INT8 cache (head_dim 64 with two keys is the case a long random run
@@ -299,7 +294,7 @@ def test_int8_paged_prefill_short_sequences(hq, hkv, d, bs):
         want = oracle.prefill_paged_oracle(c["q_new"].float(), kd, vd, c["block_tables"], c["cu_q"], c["cu_k"], scale,
                                            hq, hkv, d, bs)
         mx, mean = error_stats(got, want)
-        excess = ((got.float() - want).abs() - want.abs() * _half_step(dtype)).max().item()
+        excess = ((got.float() - want).abs() - half_step(want, dtype)).max().item()
         assert excess <= 2e-2 and mean <= 2e-3, (seed, lengths, cached, str(dtype), mx, excess, mean)
 
 
