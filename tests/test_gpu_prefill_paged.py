@@ -238,6 +238,83 @@ def test_two_group_paged_prefill_takes_every_item_once(hq, hkv, bs, num_seqs):
     _check(out.cpu(), _oracle32(c, scale, hq, hkv, d, bs), torch.bfloat16)
 
 
+def _int8_case(seed, lengths, cached, hq, hkv, d, bs, dtype):
+    from minivllm_amd.layers.attention import store_kvcache_int8
+    c = make_paged_prefill_case(seed, lengths, cached, hq, hkv, d, bs, dtype=dtype, poison=0.0)
+    nb = c["k_cache"].shape[0]
+    ck, cv = (torch.zeros(nb, bs, hkv, d, dtype=torch.int8, device=DEV) for _ in range(2))
+    sk, sv = (torch.zeros(nb, bs, hkv, device=DEV) for _ in range(2))
+    store_kvcache_int8(c["k_cache"].view(-1, hkv, d).to(DEV), c["v_cache"].view(-1, hkv, d).to(DEV), ck, cv, sk, sv,
+                       torch.arange(nb * bs, device=DEV), bs)
+    return c, ck, cv, sk, sv
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,bs,lengths,cached,slack", [
+    (32, 8, 16, [300, 64, 129, 500], [256, 0, 17, 48], 0),
+    (16, 8, 256, [700, 30, 257], [512, 29, 0], 5),                 # two query heads per kv head, the engine's block size
+    (12, 2, 48, [131, 77, 260, 1, 90], [50, 1, 259, 0, 90], 100),  # six heads per kv head; a sequence with nothing new
+    (8, 2, 32, [1500], [1499], 0),                                 # one new token behind a long prefix
+])
+def test_int8_paged_prefill_in_two_steps(dtype, hq, hkv, bs, lengths, cached, slack):
+    """With max_seqlen_k the INT8 prefill stages the batch's keys and values as 16-bit values in a temporary cache of
+    16-token blocks and runs the two-group kernel over it.  The staged values are the oracle's code * scale rounded
+    to the query type, so the result equals, bit for bit, the 16-bit paged prefill over a cache holding exactly those
+    values (whatever its block size), and it meets the INT8 bounds against the fp32 oracle.  max_seqlen_k may be any
+    upper bound of the key counts."""
+    from minivllm_amd.layers.attention import flash_attention_prefill_paged_int8
+    from minivllm_amd import _C
+    d = 128
+    c, ck, cv, sk, sv = _int8_case(72, lengths, cached, hq, hkv, d, bs, dtype)
+    scale = 1 / math.sqrt(d)
+    top = max(lengths) + slack
+    assert _C.load().mvllm_prefill_paged_int8_workspace_bytes(len(lengths), top, hq, hkv, d, bs, _C.dtype_code(dtype)) > 0
+    args = (c["q_new"].to(DEV), ck, cv, sk, sv, c["block_tables"].to(DEV), c["cu_q"].to(DEV), c["cu_k"].to(DEV), scale,
+            hq, hkv, d, bs)
+    got = flash_attention_prefill_paged_int8(*args, max_seqlen_k=top).cpu()
+    kd = oracle.dequantize_cache_oracle(ck.cpu(), sk.cpu())
+    vd = oracle.dequantize_cache_oracle(cv.cpu(), sv.cpu())
+    same = flash_attention_prefill_paged(c["q_new"].to(DEV), kd.to(dtype).to(DEV), vd.to(dtype).to(DEV),
+                                         c["block_tables"].to(DEV), c["cu_q"].to(DEV), c["cu_k"].to(DEV), scale, hq, hkv,
+                                         d, bs).cpu()
+    assert torch.equal(got, same)
+    want = oracle.prefill_paged_oracle(c["q_new"].float(), kd, vd, c["block_tables"], c["cu_q"], c["cu_k"], scale,
+                                       hq, hkv, d, bs)
+    mx, mean = error_stats(got, want)
+    excess = ((got.float() - want).abs() - half_step(want, dtype)).max().item()
+    assert torch.isfinite(got.float()).all() and excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
+    one_step = flash_attention_prefill_paged_int8(*args).cpu()                # the one-step kernel: same values, other order
+    mx, mean = error_stats(got, one_step.float())
+    assert mx <= 2e-2 and mean <= 2e-3, (mx, mean)
+
+
+def test_int8_paged_prefill_in_two_steps_unmapped_block_and_unsupported_shapes():
+    """A table entry outside the pool stages zeros, as the one-step kernel reads them; shapes the two-group kernel does
+    not take report no workspace and the operator falls back to the one-step kernel."""
+    from minivllm_amd.layers.attention import flash_attention_prefill_paged_int8
+    from minivllm_amd import _C
+    hq, hkv, d, bs, dtype = 8, 2, 128, 16, torch.bfloat16
+    lengths, cached = [100, 70], [32, 0]
+    c, ck, cv, sk, sv = _int8_case(73, lengths, cached, hq, hkv, d, bs, dtype)
+    tables = c["block_tables"].clone()
+    tables[0, 1] = 10 ** 6
+    args = (c["q_new"].to(DEV), ck, cv, sk, sv, tables.to(DEV), c["cu_q"].to(DEV), c["cu_k"].to(DEV), 0.09, hq, hkv, d, bs)
+    got = flash_attention_prefill_paged_int8(*args, max_seqlen_k=100).cpu()
+    one_step = flash_attention_prefill_paged_int8(*args).cpu()
+    mx, mean = error_stats(got, one_step.float())
+    assert torch.isfinite(got.float()).all() and mx <= 2e-2 and mean <= 2e-3, (mx, mean)
+    ws = _C.load().mvllm_prefill_paged_int8_workspace_bytes
+    code = _C.dtype_code(dtype)
+    assert ws(2, 100, hq, hkv, d, bs, code) == 2 * (2 * 7 * 16 * hkv * d * 2) + 256
+    assert ws(2, 100, 6, 2, d, bs, code) == 0 and ws(2, 100, hq, hkv, 64, bs, code) == 0      # three heads per kv head; head_dim 64
+    assert ws(65, 100, hq, hkv, d, bs, code) == 0 and ws(2, 100, hq, hkv, d, 8, code) == 0     # 65 sequences; block size 8
+    assert ws(2, 100, hq, hkv, d, bs, _C.dtype_code(torch.float32)) == 0 and ws(2, 0, hq, hkv, d, bs, code) == 0
+    c6, ck6, cv6, sk6, sv6 = _int8_case(74, lengths, cached, 6, 2, d, bs, dtype)
+    args6 = (c6["q_new"].to(DEV), ck6, cv6, sk6, sv6, c6["block_tables"].to(DEV), c6["cu_q"].to(DEV), c6["cu_k"].to(DEV),
+             0.09, 6, 2, d, bs)
+    assert torch.equal(flash_attention_prefill_paged_int8(*args6, max_seqlen_k=100), flash_attention_prefill_paged_int8(*args6))
+
+
 @pytest.mark.parametrize("hq,hkv,new,cached", [(16, 8, 4, 846), (10, 1, 5, 1873), (40, 4, 5, 72), (2, 1, 3, 833),
                                                (32, 8, 4, 846), (16, 8, 1, 0), (16, 8, 129, 1)])
 def test_two_group_paged_prefill_short_tail_behind_a_long_prefix(hq, hkv, new, cached):
