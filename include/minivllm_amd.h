@@ -238,8 +238,9 @@ int mvllm_prefill_paged_int8(void* out, const void* q,
  *   workspace      256-byte aligned, at least mvllm_prefill_paged_int8_workspace_bytes(...) bytes; contents need not
  *                  be kept between calls; calls that share a workspace must not overlap
  * mvllm_prefill_paged_int8_workspace_bytes returns 0 for shapes this form is not built for (it takes bf16 / fp16 with
- * head_dim 128, an even number of query heads per kv head, at most 64 sequences, block_size a multiple of 16); the
- * entry point then returns MVLLM_ERR_UNSUPPORTED and the one-step form is the one to call.
+ * head_dim 128 or 64 and block_size a multiple of 16; shapes the two-group kernel does not take run the one-group
+ * kernel's 16-bit paged form over the workspace); the entry point then returns MVLLM_ERR_UNSUPPORTED and the one-step
+ * form is the one to call.
  * Other arguments and the result's meaning as for mvllm_prefill_paged_int8; MVLLM_ERR_WORKSPACE for a workspace that
  * is null, too small or misaligned.
  */

@@ -1,9 +1,10 @@
 // Prefill over an INT8 paged cache in two steps: the keys and values of every sequence of the batch are dequantised
 // once (code * scale, rounded to the query's 16-bit type: the values the one-step kernel of prefill_mfma.h feeds the
 // matrix unit) into a caller-provided workspace laid out as a 16-bit paged cache with blocks of 16 tokens, then the
-// two-group kernel of prefill_pingpong.hip runs over that cache.  The one-step kernel converts each K/V tile again for
-// every 32-row query tile and head slice that walks it, which is most of its time; here a value is converted once and
-// read back as often as the kernel needs it.  No counterpart in the reference (it has no INT8 cache).
+// two-group kernel of prefill_pingpong.hip (shapes it does not take: the one-group kernel's 16-bit paged form) runs over
+// that cache.  The one-step kernel converts each K/V tile again for every 32-row query tile and head slice that walks
+// it, which is most of its time; here a value is converted once and read back as often as the kernel needs it.  No
+// counterpart in the reference (it has no INT8 cache).
 #include "common.h"
 #include "prefill_mfma.h"
 
@@ -88,11 +89,14 @@ StageLayout stage_layout(int num_seqs, int max_kv_len, int num_kv_heads, int hea
   return l;
 }
 
-bool staged_takes(int num_seqs, int max_kv_len, int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype) {
-  if (num_seqs <= 0 || max_kv_len <= 0 || num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return false;
-  if (block_size <= 0 || block_size % 16 != 0 || num_heads > 65535) return false;
-  if ((int64_t)num_seqs * ((max_kv_len + kStageBlock - 1) / kStageBlock) >= ((int64_t)1 << 31)) return false;
-  return prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype, kStageBlock);
+// 2: the two-group kernel runs over the staged cache, 1: the one-group kernel, 0: this form is not built for the shape
+int staged_kind(int num_seqs, int max_kv_len, int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype) {
+  if (num_seqs <= 0 || max_kv_len <= 0 || num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return 0;
+  if (block_size <= 0 || block_size % 16 != 0 || num_heads > 65535 || dtype == MVLLM_F32) return 0;
+  if (head_dim != 128 && head_dim != 64) return 0;
+  if ((int64_t)num_seqs * ((max_kv_len + kStageBlock - 1) / kStageBlock) >= ((int64_t)1 << 31)) return 0;
+  if ((int64_t)num_kv_heads * head_dim * 64 >= ((int64_t)1 << 31)) return 0;
+  return prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype, kStageBlock) ? 2 : 1;
 }
 
 }  // namespace
@@ -103,7 +107,7 @@ using namespace mvllm;
 
 extern "C" size_t mvllm_prefill_paged_int8_workspace_bytes(int num_seqs, int max_kv_len, int num_heads, int num_kv_heads,
                                                            int head_dim, int block_size, int dtype) {
-  if (!staged_takes(num_seqs, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype)) return 0;
+  if (staged_kind(num_seqs, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype) == 0) return 0;
   return stage_layout(num_seqs, max_kv_len, num_kv_heads, head_dim).total_bytes;
 }
 
@@ -121,8 +125,8 @@ extern "C" int mvllm_prefill_paged_int8_staged(void* out, const void* q, const i
   if (num_seqs == 0 || total_q_tokens == 0) return MVLLM_OK;
   if (!out || !q || !k_cache || !v_cache || !k_scale || !v_scale || !block_tables || !cu_seqlens_q || !cu_seqlens_k)
     return MVLLM_ERR_NULL_POINTER;
-  if (total_q_tokens > ((int64_t)1 << 30) || !staged_takes(num_seqs, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype))
-    return MVLLM_ERR_UNSUPPORTED;
+  const int kind = staged_kind(num_seqs, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype);
+  if (total_q_tokens > ((int64_t)1 << 30) || kind == 0) return MVLLM_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(out) || !aligned16(k_cache) || !aligned16(v_cache)) return MVLLM_ERR_MISALIGNED;
   const StageLayout l = stage_layout(num_seqs, max_kv_len, num_kv_heads, head_dim);
   if (!workspace || workspace_bytes < l.total_bytes || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
@@ -141,6 +145,16 @@ extern "C" int mvllm_prefill_paged_int8_staged(void* out, const void* q, const i
   else stage_int8_blocks_kernel<f16_t><<<grid, dim3(256), 0, s>>>(st);
   const int status = launch_status();
   if (status != MVLLM_OK) return status;
+  if (kind == 1) {
+    PrefillArgs a;
+    a.out = out; a.q = q; a.k = st.ws_k; a.v = st.ws_v; a.cu_seqlens = cu_seqlens_q;
+    a.total_tokens = total_q_tokens; a.num_seqs = num_seqs; a.num_heads = num_heads;
+    a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
+    a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
+    a.cu_seqlens_k = cu_seqlens_k; a.block_tables = st.ws_table; a.max_num_blocks = l.blocks_per_seq;
+    a.block_size = kStageBlock; a.num_blocks = (int64_t)num_seqs * l.blocks_per_seq; a.k_scale = nullptr; a.v_scale = nullptr;
+    return launch_prefill_paged_16bit(a, dtype, s);
+  }
   PrefillPpArgs p;
   p.out = out; p.q = q; p.k = st.ws_k; p.v = st.ws_v; p.cu_seqlens = cu_seqlens_q; p.total_tokens = total_q_tokens;
   p.num_seqs = num_seqs; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.scale_log2 = scale * kLog2e;

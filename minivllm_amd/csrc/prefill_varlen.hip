@@ -137,6 +137,12 @@ static int prefill_dispatch(const PrefillArgs& a, int dtype, bool mfma_ok, hipSt
 
 }  // namespace mvllm
 
+namespace mvllm {
+int launch_prefill_paged_16bit(const PrefillArgs& a, int dtype, hipStream_t stream) {
+  return dtype == MVLLM_BF16 ? launch_prefill_mfma<bf16_t, true, false>(a, stream) : launch_prefill_mfma<f16_t, true, false>(a, stream);
+}
+}  // namespace mvllm
+
 using namespace mvllm;
 
 // Which kernel serves a prefill of these static sizes, pointers assumed 16-byte aligned: 2 = the LDS-tiled MFMA

@@ -234,6 +234,9 @@ def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cach
     return output
 
 
+STAGED_INT8_PREFILL_MAX_BYTES = 4 << 30    # larger temporary caches are not asked for: the call then runs in one step
+
+
 def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                                        k_scale: torch.Tensor, v_scale: torch.Tensor, block_tables: torch.Tensor,
                                        cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, scale: float,
@@ -242,10 +245,10 @@ def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v
     """``flash_attention_prefill_paged`` over an INT8 cache written by ``store_kvcache_int8``: every key, the new
     tokens' included, is read from the cache and dequantised in the kernel, as decode does for the same tokens.
     q bf16 / fp16; caches int8 (num_blocks, block_size, Hkv, D); scales float32 (num_blocks, block_size, Hkv).
-    ``max_seqlen_k`` (the host's upper bound of every sequence's key count, ``Context.max_seqlen_k``) lets shapes the
-    two-group kernel takes run in two steps: the batch's keys and values are dequantised once into a temporary
-    16-bit cache (2 x num_seqs x max_seqlen_k x Hkv x D x 2 bytes from torch's allocator), which is a quarter faster
-    than converting every tile for every query tile that walks it."""
+    ``max_seqlen_k`` (the host's upper bound of every sequence's key count, ``Context.max_seqlen_k``) lets the call
+    run in two steps: the batch's keys and values are dequantised once into a temporary 16-bit cache
+    (2 x num_seqs x max_seqlen_k x Hkv x D x 2 bytes from torch's allocator, at most ``STAGED_INT8_PREFILL_MAX_BYTES``),
+    which is a quarter faster than converting every tile for every query tile that walks it."""
     _C.require_cuda(q, k_cache, v_cache, k_scale, v_scale, block_tables, cu_seqlens_q, cu_seqlens_k)
     if q.dim() != 3 or tuple(q.shape[1:]) != (num_heads, head_dim):
         raise ValueError(f"q must be (total_tokens, {num_heads}, {head_dim}), got {tuple(q.shape)}")
@@ -271,7 +274,7 @@ def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v
     if max_seqlen_k is not None and int(max_seqlen_k) > 0:
         need = _C.load().mvllm_prefill_paged_int8_workspace_bytes(num_seqs, int(max_seqlen_k), num_heads, num_kv_heads,
                                                                   head_dim, block_size, _C.dtype_code(q.dtype))
-        if need > 0:
+        if 0 < need <= STAGED_INT8_PREFILL_MAX_BYTES:
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
             st = _C.load().mvllm_prefill_paged_int8_staged(
                 _ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale), _ptr(block_tables),

@@ -250,21 +250,23 @@ def _int8_case(seed, lengths, cached, hq, hkv, d, bs, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("hq,hkv,bs,lengths,cached,slack", [
-    (32, 8, 16, [300, 64, 129, 500], [256, 0, 17, 48], 0),
-    (16, 8, 256, [700, 30, 257], [512, 29, 0], 5),                 # two query heads per kv head, the engine's block size
-    (12, 2, 48, [131, 77, 260, 1, 90], [50, 1, 259, 0, 90], 100),  # six heads per kv head; a sequence with nothing new
-    (8, 2, 32, [1500], [1499], 0),                                 # one new token behind a long prefix
+@pytest.mark.parametrize("hq,hkv,d,bs,lengths,cached,slack", [
+    (32, 8, 128, 16, [300, 64, 129, 500], [256, 0, 17, 48], 0),
+    (16, 8, 128, 256, [700, 30, 257], [512, 29, 0], 5),                 # two query heads per kv head, the engine's block size
+    (12, 2, 128, 48, [131, 77, 260, 1, 90], [50, 1, 259, 0, 90], 100),  # six heads per kv head; a sequence with nothing new
+    (8, 2, 128, 32, [1500], [1499], 0),                                 # one new token behind a long prefix
+    (6, 2, 128, 16, [131, 77, 260], [50, 1, 259], 3),                   # three heads per kv head: the one-group kernel
+    (16, 8, 64, 16, [200, 90, 33], [160, 80, 0], 0),                    # head_dim 64: the one-group kernel
 ])
-def test_int8_paged_prefill_in_two_steps(dtype, hq, hkv, bs, lengths, cached, slack):
+def test_int8_paged_prefill_in_two_steps(dtype, hq, hkv, d, bs, lengths, cached, slack):
     """With max_seqlen_k the INT8 prefill stages the batch's keys and values as 16-bit values in a temporary cache of
-    16-token blocks and runs the two-group kernel over it.  The staged values are the oracle's code * scale rounded
+    16-token blocks and runs the two-group kernel (shapes it does not take: the one-group kernel) over it.  The staged
+    values are the oracle's code * scale rounded
     to the query type, so the result equals, bit for bit, the 16-bit paged prefill over a cache holding exactly those
     values (whatever its block size), and it meets the INT8 bounds against the fp32 oracle.  max_seqlen_k may be any
     upper bound of the key counts."""
     from minivllm_amd.layers.attention import flash_attention_prefill_paged_int8
     from minivllm_amd import _C
-    d = 128
     c, ck, cv, sk, sv = _int8_case(72, lengths, cached, hq, hkv, d, bs, dtype)
     scale = 1 / math.sqrt(d)
     top = max(lengths) + slack
@@ -289,8 +291,8 @@ def test_int8_paged_prefill_in_two_steps(dtype, hq, hkv, bs, lengths, cached, sl
 
 
 def test_int8_paged_prefill_in_two_steps_unmapped_block_and_unsupported_shapes():
-    """A table entry outside the pool stages zeros, as the one-step kernel reads them; shapes the two-group kernel does
-    not take report no workspace and the operator falls back to the one-step kernel."""
+    """A table entry outside the pool stages zeros, as the one-step kernel reads them; shapes the MFMA kernels do not
+    take report no workspace and the operator runs in one step."""
     from minivllm_amd.layers.attention import flash_attention_prefill_paged_int8
     from minivllm_amd import _C
     hq, hkv, d, bs, dtype = 8, 2, 128, 16, torch.bfloat16
@@ -306,13 +308,14 @@ def test_int8_paged_prefill_in_two_steps_unmapped_block_and_unsupported_shapes()
     ws = _C.load().mvllm_prefill_paged_int8_workspace_bytes
     code = _C.dtype_code(dtype)
     assert ws(2, 100, hq, hkv, d, bs, code) == 2 * (2 * 7 * 16 * hkv * d * 2) + 256
-    assert ws(2, 100, 6, 2, d, bs, code) == 0 and ws(2, 100, hq, hkv, 64, bs, code) == 0      # three heads per kv head; head_dim 64
-    assert ws(65, 100, hq, hkv, d, bs, code) == 0 and ws(2, 100, hq, hkv, d, 8, code) == 0     # 65 sequences; block size 8
+    assert ws(2, 100, 6, 2, d, bs, code) > 0 and ws(2, 100, hq, hkv, 64, bs, code) > 0 and ws(65, 100, hq, hkv, d, bs, code) > 0
+    assert ws(2, 100, hq, hkv, 96, bs, code) == 0 and ws(2, 100, hq, hkv, d, 8, code) == 0      # head_dim 96; block size 8
     assert ws(2, 100, hq, hkv, d, bs, _C.dtype_code(torch.float32)) == 0 and ws(2, 0, hq, hkv, d, bs, code) == 0
-    c6, ck6, cv6, sk6, sv6 = _int8_case(74, lengths, cached, 6, 2, d, bs, dtype)
-    args6 = (c6["q_new"].to(DEV), ck6, cv6, sk6, sv6, c6["block_tables"].to(DEV), c6["cu_q"].to(DEV), c6["cu_k"].to(DEV),
-             0.09, 6, 2, d, bs)
-    assert torch.equal(flash_attention_prefill_paged_int8(*args6, max_seqlen_k=100), flash_attention_prefill_paged_int8(*args6))
+    c8, ck8, cv8, sk8, sv8 = _int8_case(74, lengths, cached, hq, hkv, d, 8, dtype)      # block size 8: no int8 prefill kernel at all
+    args8 = (c8["q_new"].to(DEV), ck8, cv8, sk8, sv8, c8["block_tables"].to(DEV), c8["cu_q"].to(DEV), c8["cu_k"].to(DEV),
+             0.09, hq, hkv, d, 8)
+    with pytest.raises(ValueError):
+        flash_attention_prefill_paged_int8(*args8, max_seqlen_k=100)
 
 
 @pytest.mark.parametrize("hq,hkv,new,cached", [(16, 8, 4, 846), (10, 1, 5, 1873), (40, 4, 5, 72), (2, 1, 3, 833),
