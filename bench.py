@@ -359,7 +359,7 @@ def bench_prefill_store(args, which, want_cpu=False):
             "tflops": flops / (event_ms8 * 1e-3) / 1e12,
             "one_step_event_ms_per_step": event_ms8_one, "one_step_tflops": flops / (event_ms8_one * 1e-3) / 1e12,
             "roofline": roofline("mfma", flops / (event_ms8 * 1e-3) / 1e12,
-                                 "stage_int8_blocks_kernel + prefill_pp_kernel (mvllm_prefill_paged_int8_staged; the workspace comes from torch's allocator inside the timed call)"),
+                                 "stage_blocks_kernel + prefill_pp_kernel (mvllm_prefill_paged_int8_staged; the workspace comes from torch's allocator inside the timed call)"),
         }
     if "store" in which:
         slots, _, nb = make_slot_mapping(args.seed + 2, lengths, bs)

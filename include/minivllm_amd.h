@@ -229,23 +229,32 @@ int mvllm_prefill_paged_int8(void* out, const void* q,
                              int64_t num_blocks, float scale, int dtype, void* stream);
 
 /*
- * mvllm_prefill_paged_int8 in two steps, for callers that can lend device memory: every sequence's keys and values are
- * dequantised once (the same code * scale rounded to `dtype`) into `workspace`, laid out as a 16-bit paged cache of
- * 16-token blocks, and the two-group prefill kernel runs over that; the one-step form converts a K/V tile again for
- * every query tile that walks it.  No counterpart in the reference.
+ * mvllm_prefill_paged and mvllm_prefill_paged_int8 in two steps, for callers that can lend device memory: every
+ * sequence's keys and values are first written into `workspace`, laid out as a 16-bit paged cache of 16-token blocks with
+ * a block table of its own, and the two-group prefill kernel (shapes it does not take: the one-group kernel's 16-bit
+ * paged form) runs over that.  No counterpart in the reference.  Two uses:
+ *   - an INT8 cache: a value is dequantised once (the same code * scale rounded to `dtype`), where the one-step form
+ *     converts a K/V tile again for every query tile that walks it;
+ *   - any block_size >= 1: the one-step forms need a multiple of 16 for their MFMA kernels.
  *   max_kv_len     an upper bound of every sequence's len_k, known to the host (the reference's Context.max_seqlen_k,
  *                  utils/context.py:11); keys of a sequence past it read as zeros
- *   workspace      256-byte aligned, at least mvllm_prefill_paged_int8_workspace_bytes(...) bytes; contents need not
+ *   workspace      256-byte aligned, at least mvllm_prefill_paged_staged_workspace_bytes(...) bytes; contents need not
  *                  be kept between calls; calls that share a workspace must not overlap
- * mvllm_prefill_paged_int8_workspace_bytes returns 0 for shapes this form is not built for (it takes bf16 / fp16 with
- * head_dim 128 or 64 and block_size a multiple of 16; shapes the two-group kernel does not take run the one-group
- * kernel's 16-bit paged form over the workspace); the entry point then returns MVLLM_ERR_UNSUPPORTED and the one-step
- * form is the one to call.
- * Other arguments and the result's meaning as for mvllm_prefill_paged_int8; MVLLM_ERR_WORKSPACE for a workspace that
- * is null, too small or misaligned.
+ * mvllm_prefill_paged_staged_workspace_bytes returns 0 for shapes this form is not built for (it takes bf16 / fp16 with
+ * head_dim 128 or 64, 16-bit caches also 32, 48, 80, 96, 112 and 256); the entry points then return
+ * MVLLM_ERR_UNSUPPORTED and the one-step form is the one to call.
+ * Other arguments and the result's meaning as for the one-step forms; MVLLM_ERR_WORKSPACE for a workspace that is null,
+ * too small or misaligned.
  */
-size_t mvllm_prefill_paged_int8_workspace_bytes(int num_seqs, int max_kv_len, int num_heads, int num_kv_heads,
-                                                int head_dim, int block_size, int dtype);
+size_t mvllm_prefill_paged_staged_workspace_bytes(int num_seqs, int max_kv_len, int num_heads, int num_kv_heads,
+                                                  int head_dim, int dtype, int int8_cache);
+int mvllm_prefill_paged_staged(void* out, const void* q, const void* k_cache, const void* v_cache,
+                               const int32_t* block_tables, int max_num_blocks,
+                               const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                               int num_seqs, int64_t total_q_tokens, int max_kv_len,
+                               int num_heads, int num_kv_heads, int head_dim, int block_size,
+                               int64_t num_blocks, float scale, int dtype,
+                               void* workspace, size_t workspace_bytes, void* stream);
 int mvllm_prefill_paged_int8_staged(void* out, const void* q,
                                     const int8_t* k_cache, const int8_t* v_cache,
                                     const float* k_scale, const float* v_scale,

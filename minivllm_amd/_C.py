@@ -41,7 +41,9 @@ SIGNATURES = {
                                                       c_int, c_int64, c_float, c_int, c_void_p]),
     "mvllm_prefill_paged_int8": (c_int, [c_void_p] * 7 + [c_int, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int,
                                            c_int, c_int64, c_float, c_int, c_void_p]),
-    "mvllm_prefill_paged_int8_workspace_bytes": (c_size_t, [c_int] * 7),
+    "mvllm_prefill_paged_staged_workspace_bytes": (c_size_t, [c_int] * 7),
+    "mvllm_prefill_paged_staged": (c_int, [c_void_p] * 5 + [c_int, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int,
+                                             c_int, c_int64, c_float, c_int, c_void_p, c_size_t, c_void_p]),
     "mvllm_prefill_paged_int8_staged": (c_int, [c_void_p] * 7 + [c_int, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int,
                                                   c_int, c_int64, c_float, c_int, c_void_p, c_size_t, c_void_p]),
     "mvllm_sample_tokens_workspace_bytes": (c_size_t, [c_int, c_int]),

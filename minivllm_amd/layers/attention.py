@@ -194,7 +194,7 @@ def flash_attention_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, c
 def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                                   block_tables: torch.Tensor, cu_seqlens_q: torch.Tensor,
                                   cu_seqlens_k: torch.Tensor, scale: float, num_heads: int, num_kv_heads: int,
-                                  head_dim: int, block_size: int) -> torch.Tensor:
+                                  head_dim: int, block_size: int, max_seqlen_k: int | None = None) -> torch.Tensor:
     """Causal prefill of the tokens that follow each sequence's cached prefix, with every key read from the
     paged cache.  Consumes the metadata ``ModelRunner.prepare_prefill`` builds for prefix-cache hits
     (model_runner.py:192-226), which the reference's ``Attention.forward`` ignores (attention.py:518-523).
@@ -202,6 +202,10 @@ def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cach
     q: (total_new_tokens, num_heads, head_dim) packed by ``cu_seqlens_q``; caches
     (num_blocks, block_size, Hkv, D) already holding all ``cu_seqlens_k`` keys of every sequence;
     block_tables int32 (num_seqs, max_num_blocks).  Returns a tensor like q.
+    A block size that is not a multiple of 16 (8, 1, 24 ...) runs on the generic kernel unless ``max_seqlen_k`` (the
+    host's upper bound of every sequence's key count, ``Context.max_seqlen_k``) is given: the batch's keys and values
+    are then copied into a temporary cache of 16-token blocks (``STAGED_PREFILL_MAX_BYTES`` at most) and the MFMA
+    kernels run over that.
     """
     _C.require_cuda(q, k_cache, v_cache, block_tables, cu_seqlens_q, cu_seqlens_k)
     if q.dim() != 3 or tuple(q.shape[1:]) != (num_heads, head_dim):
@@ -224,8 +228,20 @@ def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cach
     cu_seqlens_q = cu_seqlens_q.to(torch.int32).contiguous()
     cu_seqlens_k = cu_seqlens_k.to(torch.int32).contiguous()
     output = torch.empty_like(q)
-    _warn_if_generic("prefill", num_heads, num_kv_heads, head_dim, block_size, q.dtype, False)
     lib = _C.load()
+    if max_seqlen_k is not None and int(max_seqlen_k) > 0 and block_size % 16 != 0:
+        need = lib.mvllm_prefill_paged_staged_workspace_bytes(num_seqs, int(max_seqlen_k), num_heads, num_kv_heads, head_dim,
+                                                              _C.dtype_code(q.dtype), 0)
+        if 0 < need <= STAGED_PREFILL_MAX_BYTES:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+            st = lib.mvllm_prefill_paged_staged(_ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                                block_tables.shape[1], _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), num_seqs,
+                                                q.shape[0], int(max_seqlen_k), num_heads, num_kv_heads, head_dim, block_size,
+                                                k_cache.shape[0], float(scale), _C.dtype_code(q.dtype), _ptr(workspace), need,
+                                                _C.current_stream_ptr(q.device))
+            _C.check(st, "flash_attention_prefill_paged (staged)")
+            return output
+    _warn_if_generic("prefill", num_heads, num_kv_heads, head_dim, block_size, q.dtype, False)
     st = lib.mvllm_prefill_paged(_ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                  block_tables.shape[1], _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), num_seqs,
                                  q.shape[0], num_heads, num_kv_heads, head_dim, block_size, k_cache.shape[0],
@@ -234,7 +250,7 @@ def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cach
     return output
 
 
-STAGED_INT8_PREFILL_MAX_BYTES = 4 << 30    # larger temporary caches are not asked for: the call then runs in one step
+STAGED_PREFILL_MAX_BYTES = 4 << 30    # larger temporary caches are not asked for: the call then runs in one step
 
 
 def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -247,8 +263,9 @@ def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v
     q bf16 / fp16; caches int8 (num_blocks, block_size, Hkv, D); scales float32 (num_blocks, block_size, Hkv).
     ``max_seqlen_k`` (the host's upper bound of every sequence's key count, ``Context.max_seqlen_k``) lets the call
     run in two steps: the batch's keys and values are dequantised once into a temporary 16-bit cache
-    (2 x num_seqs x max_seqlen_k x Hkv x D x 2 bytes from torch's allocator, at most ``STAGED_INT8_PREFILL_MAX_BYTES``),
-    which is a quarter faster than converting every tile for every query tile that walks it."""
+    (2 x num_seqs x max_seqlen_k x Hkv x D x 2 bytes from torch's allocator, at most ``STAGED_PREFILL_MAX_BYTES``),
+    which is a quarter faster than converting every tile for every query tile that walks it, and the only MFMA path
+    for block sizes that are not a multiple of 16."""
     _C.require_cuda(q, k_cache, v_cache, k_scale, v_scale, block_tables, cu_seqlens_q, cu_seqlens_k)
     if q.dim() != 3 or tuple(q.shape[1:]) != (num_heads, head_dim):
         raise ValueError(f"q must be (total_tokens, {num_heads}, {head_dim}), got {tuple(q.shape)}")
@@ -272,9 +289,9 @@ def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v
     cu_seqlens_k = cu_seqlens_k.to(torch.int32).contiguous()
     output = torch.empty_like(q)
     if max_seqlen_k is not None and int(max_seqlen_k) > 0:
-        need = _C.load().mvllm_prefill_paged_int8_workspace_bytes(num_seqs, int(max_seqlen_k), num_heads, num_kv_heads,
-                                                                  head_dim, block_size, _C.dtype_code(q.dtype))
-        if 0 < need <= STAGED_INT8_PREFILL_MAX_BYTES:
+        need = _C.load().mvllm_prefill_paged_staged_workspace_bytes(num_seqs, int(max_seqlen_k), num_heads, num_kv_heads,
+                                                                    head_dim, _C.dtype_code(q.dtype), 1)
+        if 0 < need <= STAGED_PREFILL_MAX_BYTES:
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
             st = _C.load().mvllm_prefill_paged_int8_staged(
                 _ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale), _ptr(block_tables),
@@ -498,7 +515,8 @@ class Attention(nn.Module):
                     else:
                         o = flash_attention_prefill_paged(q_rows, k_cache, v_cache, context.block_tables, cu,
                                                           context.cu_seqlens_k, scale, self.num_heads,
-                                                          self.num_kv_heads, self.head_dim, self.block_size)
+                                                          self.num_kv_heads, self.head_dim, self.block_size,
+                                                          context.max_seqlen_k or None)
                     return o.reshape(bsz, n, self.num_heads * self.head_dim)
                 o = flash_attention_prefill(q.reshape(bsz * n, self.num_heads, self.head_dim),
                                             k.reshape(bsz * n, self.num_kv_heads, self.head_dim),
@@ -524,7 +542,7 @@ class Attention(nn.Module):
                 else:
                     o = flash_attention_prefill_paged(q, k_cache, v_cache, context.block_tables, cu_seqlens,
                                                       context.cu_seqlens_k, scale, self.num_heads, self.num_kv_heads,
-                                                      self.head_dim, self.block_size)
+                                                      self.head_dim, self.block_size, context.max_seqlen_k or None)
                 return o.reshape(o.shape[0], self.num_heads * self.head_dim)
             o = flash_attention_prefill(q, k, v, cu_seqlens, scale, self.num_heads, self.num_kv_heads,
                                         self.head_dim)

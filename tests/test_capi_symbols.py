@@ -28,7 +28,7 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_noalloc", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_plan", "mvllm_prefill_varlen",
-              "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_prefill_paged_int8_staged", "mvllm_prefill_paged_int8_workspace_bytes", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_dev_offset", "mvllm_decode_advance", "mvllm_sample_tokens_workspace_bytes",
+              "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_prefill_paged_int8_staged", "mvllm_prefill_paged_staged", "mvllm_prefill_paged_staged_workspace_bytes", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_dev_offset", "mvllm_decode_advance", "mvllm_sample_tokens_workspace_bytes",
               "mvllm_add_rms_norm", "mvllm_linear_small_m", "mvllm_norm_linear_small_m", "mvllm_linear_small_m_plan",
               "mvllm_lm_head_sample", "mvllm_lm_head_sample_workspace_bytes",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:

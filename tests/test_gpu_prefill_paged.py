@@ -270,7 +270,7 @@ def test_int8_paged_prefill_in_two_steps(dtype, hq, hkv, d, bs, lengths, cached,
     c, ck, cv, sk, sv = _int8_case(72, lengths, cached, hq, hkv, d, bs, dtype)
     scale = 1 / math.sqrt(d)
     top = max(lengths) + slack
-    assert _C.load().mvllm_prefill_paged_int8_workspace_bytes(len(lengths), top, hq, hkv, d, bs, _C.dtype_code(dtype)) > 0
+    assert _C.load().mvllm_prefill_paged_staged_workspace_bytes(len(lengths), top, hq, hkv, d, _C.dtype_code(dtype), 1) > 0
     args = (c["q_new"].to(DEV), ck, cv, sk, sv, c["block_tables"].to(DEV), c["cu_q"].to(DEV), c["cu_k"].to(DEV), scale,
             hq, hkv, d, bs)
     got = flash_attention_prefill_paged_int8(*args, max_seqlen_k=top).cpu()
@@ -305,17 +305,56 @@ def test_int8_paged_prefill_in_two_steps_unmapped_block_and_unsupported_shapes()
     one_step = flash_attention_prefill_paged_int8(*args).cpu()
     mx, mean = error_stats(got, one_step.float())
     assert torch.isfinite(got.float()).all() and mx <= 2e-2 and mean <= 2e-3, (mx, mean)
-    ws = _C.load().mvllm_prefill_paged_int8_workspace_bytes
+    ws = _C.load().mvllm_prefill_paged_staged_workspace_bytes
     code = _C.dtype_code(dtype)
-    assert ws(2, 100, hq, hkv, d, bs, code) == 2 * (2 * 7 * 16 * hkv * d * 2) + 256
-    assert ws(2, 100, 6, 2, d, bs, code) > 0 and ws(2, 100, hq, hkv, 64, bs, code) > 0 and ws(65, 100, hq, hkv, d, bs, code) > 0
-    assert ws(2, 100, hq, hkv, 96, bs, code) == 0 and ws(2, 100, hq, hkv, d, 8, code) == 0      # head_dim 96; block size 8
-    assert ws(2, 100, hq, hkv, d, bs, _C.dtype_code(torch.float32)) == 0 and ws(2, 0, hq, hkv, d, bs, code) == 0
-    c8, ck8, cv8, sk8, sv8 = _int8_case(74, lengths, cached, hq, hkv, d, 8, dtype)      # block size 8: no int8 prefill kernel at all
+    assert ws(2, 100, hq, hkv, d, code, 1) == 2 * (2 * 7 * 16 * hkv * d * 2) + 256 == ws(2, 100, hq, hkv, d, code, 0)
+    assert ws(2, 100, 6, 2, d, code, 1) > 0 and ws(2, 100, hq, hkv, 64, code, 1) > 0 and ws(65, 100, hq, hkv, d, code, 1) > 0
+    assert ws(2, 100, hq, hkv, 96, code, 1) == 0 and ws(2, 100, hq, hkv, 96, code, 0) > 0      # head_dim 96: 16-bit caches only
+    assert ws(2, 100, hq, hkv, 72, code, 0) == 0 and ws(2, 100, hq, hkv, 100, code, 0) == 0    # no LDS-tiled kernel for these
+    assert ws(2, 100, hq, hkv, d, _C.dtype_code(torch.float32), 1) == 0 and ws(2, 0, hq, hkv, d, code, 1) == 0
+    # block size 8: the one-step INT8 kernels do not take it, the two-step form does
+    c8, ck8, cv8, sk8, sv8 = _int8_case(74, lengths, cached, hq, hkv, d, 8, dtype)
     args8 = (c8["q_new"].to(DEV), ck8, cv8, sk8, sv8, c8["block_tables"].to(DEV), c8["cu_q"].to(DEV), c8["cu_k"].to(DEV),
              0.09, hq, hkv, d, 8)
     with pytest.raises(ValueError):
-        flash_attention_prefill_paged_int8(*args8, max_seqlen_k=100)
+        flash_attention_prefill_paged_int8(*args8)
+    got8 = flash_attention_prefill_paged_int8(*args8, max_seqlen_k=100).cpu()
+    kd = oracle.dequantize_cache_oracle(ck8.cpu(), sk8.cpu())
+    vd = oracle.dequantize_cache_oracle(cv8.cpu(), sv8.cpu())
+    want8 = oracle.prefill_paged_oracle(c8["q_new"].float(), kd, vd, c8["block_tables"], c8["cu_q"], c8["cu_k"], 0.09,
+                                        hq, hkv, d, 8)
+    mx, mean = error_stats(got8, want8)
+    excess = ((got8.float() - want8).abs() - half_step(want8, dtype)).max().item()
+    assert excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,d,bs,lengths,cached", [
+    (32, 8, 128, 8, [300, 64, 129, 500], [256, 0, 17, 48]),        # block size 8: the two-group kernel over the staged cache
+    (16, 8, 128, 1, [200, 90, 33], [160, 80, 0]),                  # a block per token
+    (6, 2, 128, 24, [131, 77, 260], [50, 1, 259]),                 # 24 tokens per block, three query heads per kv head
+    (16, 8, 64, 8, [200, 90, 33, 5], [160, 80, 0, 5]),             # head_dim 64; a sequence with nothing new
+    (6, 2, 96, 3, [131, 77], [50, 1]),                             # head_dim 96, 3 tokens per block
+])
+def test_paged_prefill_with_other_block_sizes_in_two_steps(dtype, hq, hkv, d, bs, lengths, cached):
+    """A 16-bit cache whose block size is not a multiple of 16: with max_seqlen_k the operator copies the batch's keys
+    and values into a temporary cache of 16-token blocks and runs the MFMA kernels over it.  The copy is exact, so the
+    result equals the one-step prefill over the same keys in a cache of 16-token blocks bit for bit, and it meets the
+    bounds against the oracle; without max_seqlen_k the call runs on the generic kernel (same bounds)."""
+    c = make_paged_prefill_case(75, lengths, cached, hq, hkv, d, bs, dtype=dtype)
+    scale = 1 / math.sqrt(d)
+    args = (c["q_new"].to(DEV), c["k_cache"].to(DEV), c["v_cache"].to(DEV), c["block_tables"].to(DEV), c["cu_q"].to(DEV),
+            c["cu_k"].to(DEV), scale, hq, hkv, d, bs)
+    got = flash_attention_prefill_paged(*args, max_seqlen_k=max(lengths) + 7).cpu()
+    want = _oracle32(c, scale, hq, hkv, d, bs)
+    _check(got, want, dtype)
+    c16 = make_paged_prefill_case(75, lengths, cached, hq, hkv, d, 16, dtype=dtype)       # same seed: the same q, k, v
+    assert torch.equal(c16["q_new"], c["q_new"])
+    assert torch.equal(got, _run(c16, scale, hq, hkv, d, 16))
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _check(flash_attention_prefill_paged(*args).cpu(), want, dtype)
 
 
 @pytest.mark.parametrize("hq,hkv,new,cached", [(16, 8, 4, 846), (10, 1, 5, 1873), (40, 4, 5, 72), (2, 1, 3, 833),
