@@ -99,7 +99,8 @@ size_t mvllm_paged_decode_workspace_bytes(int batch, int num_heads, int head_dim
  *                     >1: small-batch form, a workgroup is that many waves on one kv head that share the
  *                     partition's 16-token tiles and merge in LDS; 0: the generic kernel (head_dim other than
  *                     128 or 64 (bf16 / fp16 caches: also every other multiple of 8 from 32 to 120, and 256),
- *                     block_size % 16 != 0, or fp32 queries over an INT8 cache).  A kv head with more than 16 query
+ *                     a block_size that is neither a multiple of 16 nor, for 16-bit and fp32 caches with head_dim 128 or
+ *                     64, one of 1, 2, 4, 8; or fp32 queries over an INT8 cache).  A kv head with more than 16 query
  *                     heads is served in slices of 16, each of which streams its keys and values again.
  * Returns MVLLM_OK or MVLLM_ERR_BAD_SHAPE / MVLLM_ERR_BAD_DTYPE.
  */

@@ -672,7 +672,9 @@ struct DecodeHead<float, D> {
 // W = 1: the wave walks all tiles of its partition.  W > 1 (the workgroup is W waves on one kv head): wave w takes
 // tiles w, w + W, ... and the partial results meet in LDS (DecodeHead::merge), so a short context costs a few tiles
 // of latency per wave and no second launch.
-template <typename T, int W, int D>
+// SUB: blocks of 1, 2, 4 or 8 tokens.  A 16-token tile then spans several blocks, and every lane looks up the blocks
+// of its own tokens (one for its K row, up to four for its V rows) in the block-table window.
+template <typename T, int W, int D, bool SUB = false>
 __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int p, int slice, int w) {
   const int lane = threadIdx.x & 63;
   const HeadSlice hs = head_slice(a, slice);
@@ -718,6 +720,40 @@ __device__ __forceinline__ void decode_mfma_item(const DecodeArgs& a, int b, int
 
   auto load_tile = [&](KVTile<T, D>& t, int tile) {
     t.t0 = first + tile * (W * kTile);
+    if constexpr (SUB) {
+      const int lb = __builtin_ctz((unsigned)bs);              // block_size is a power of two below 16
+      const int bpt = kTile >> lb;                             // blocks per tile
+      if (bi + bpt - win_base > 64) {
+        win_base = bi;
+        win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
+      }
+      // A token past the partition's end (the tile is the last one) has no block of its own: the lane loads the
+      // last live token's row instead, and consume() masks it by position.
+      const int live = part_end - 1 - t.t0;                    // index of the tile's last live token (>= 0)
+      const int kt = col < live ? col : live;
+      const int kb = bi + (kt >> lb);
+      const int kphys = __shfl(win, kb - win_base, 64);
+      bool ok = kb < a.max_num_blocks && kphys >= 0 && (int64_t)kphys < a.num_blocks;
+      int vphys[4], vt[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        vt[i] = 4 * cls + i < live ? 4 * cls + i : live;
+        const int vb = bi + (vt[i] >> lb);
+        vphys[i] = __shfl(win, vb - win_base, 64);
+        ok = ok && vb < a.max_num_blocks && vphys[i] >= 0 && (int64_t)vphys[i] < a.num_blocks;
+      }
+      t.ok = __all(ok);                                        // a tile with an unmapped block is left out as a whole
+      if (t.ok) {
+        IO::load_k(t, kc + ((int64_t)kphys * bs + (kt & (bs - 1))) * row + cls * IO::kKLane, lane >> 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          IO::template load_v<true>(t, i, vc + ((int64_t)vphys[i] * bs + (vt[i] & (bs - 1))) * row + col * IO::kVLane, IO::owns(col));
+      } else {
+        IO::zero(t);
+      }
+      bi += W * bpt;
+      return;
+    }
     if (bi - win_base >= 64) {
       win_base = bi;
       win = (win_base + lane < a.max_num_blocks) ? table[win_base + lane] : -1;
@@ -1226,20 +1262,20 @@ __device__ __forceinline__ void decode_mfma_int8_item(const DecodeArgs& a, int b
 // Kernels of the fast path: one workgroup per (partition, sequence, group of kv heads); the partition index is
 // an upper bound, and a workgroup whose partition lies past its sequence's context returns at once.
 // ---------------------------------------------------------------------------
-template <typename T, int D>
+template <typename T, int D, bool SUB = false>
 // head_dim 256 holds twice the accumulators and tiles: one wave per SIMD with up to 512 registers
 __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : kDecodeWavesPerEu) void decode_mfma_kernel(const DecodeArgs a) {
   int b, p, hg;
   if (!decode_item<false>(a, b, p, hg)) return;
-  decode_mfma_item<T, 1, D>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
+  decode_mfma_item<T, 1, D, SUB>(a, b, p, hg * (blockDim.x >> 6) + (threadIdx.x >> 6), 0);
 }
 // Small batches: one workgroup of W waves per (partition, sequence, kv head), the waves splitting the tiles.
-template <typename T, int W, int D>
+template <typename T, int W, int D, bool SUB = false>
 __global__ __launch_bounds__(64 * W, D > 128 ? 1 : kDecodeWavesPerEu) void decode_mfma_split_kernel(const DecodeArgs a) {
   // kv head fastest: the workgroups of one (sequence, partition) start together and read the same token rows
   const int g = blockIdx.x, b = blockIdx.z;
   const int p = (int)((blockIdx.y + (unsigned)b) % (unsigned)a.num_parts);
-  decode_mfma_item<T, W, D>(a, b, p, g, threadIdx.x >> 6);
+  decode_mfma_item<T, W, D, SUB>(a, b, p, g, threadIdx.x >> 6);
 }
 template <typename T, int NCH, int D>
 __global__ __launch_bounds__(kDecodeI8Threads, kDecodeI8WavesPerEu) void decode_mfma_int8_kernel(const DecodeArgs a) {
@@ -1508,7 +1544,10 @@ static void with_other_mfma_dim(int head_dim, F&& go) {
 static bool fast_shape(int num_heads, int num_kv_heads, int head_dim, int block_size, int dtype, bool int8) {
   // 16-bit caches: a multiple of 8 from 32 to 128, or 256, dims per head; fp32 and INT8 caches: 64 or 128
   const bool dim_ok = head_dim == 128 || head_dim == 64 || (dtype != MVLLM_F32 && !int8 && other_mfma_dim(head_dim));
-  return (dtype != MVLLM_F32 || !int8) && dim_ok && block_size % kTile == 0 &&
+  // blocks: whole tiles; 16-bit and fp32 caches with head_dim 128 or 64 also 1, 2, 4 or 8 tokens
+  const bool blocks_ok = block_size % kTile == 0 ||
+                         (kTile % block_size == 0 && !int8 && (head_dim == 128 || head_dim == 64));
+  return (dtype != MVLLM_F32 || !int8) && dim_ok && blocks_ok &&
          (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31);
 }
 
@@ -1552,9 +1591,20 @@ static int launch_decode(DecodeArgs a, bool int8, bool fast_ok, bool split, hipS
       else decode_mfma_kernel<T, D><<<grid, block, 0, stream>>>(a);
       launched = true;
     };
-    if (a.head_dim == 128) go(std::integral_constant<int, 128>{});
-    else if (a.head_dim == 64) go(std::integral_constant<int, 64>{});
-    if constexpr (IsSixteenBit<T>::value) with_other_mfma_dim(a.head_dim, go);    // 16-bit caches only
+    auto go_small_blocks = [&](auto DIM) {          // blocks of 1, 2, 4 or 8 tokens (head_dim 128 or 64)
+      constexpr int D = decltype(DIM)::value;
+      if (split) decode_mfma_split_kernel<T, kSplitWaves, D, true><<<split_grid, split_block, 0, stream>>>(a);
+      else decode_mfma_kernel<T, D, true><<<grid, block, 0, stream>>>(a);
+      launched = true;
+    };
+    if (a.block_size < kTile) {
+      if (a.head_dim == 128) go_small_blocks(std::integral_constant<int, 128>{});
+      else if (a.head_dim == 64) go_small_blocks(std::integral_constant<int, 64>{});
+    } else {
+      if (a.head_dim == 128) go(std::integral_constant<int, 128>{});
+      else if (a.head_dim == 64) go(std::integral_constant<int, 64>{});
+      if constexpr (IsSixteenBit<T>::value) with_other_mfma_dim(a.head_dim, go);    // 16-bit caches only
+    }
   }
   if constexpr (IsSixteenBit<T>::value) {           // the INT8 kernels take 16-bit queries
     if (fast_ok && int8) {

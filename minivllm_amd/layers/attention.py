@@ -65,8 +65,9 @@ def _warn_if_generic(op: str, num_heads: int, num_kv_heads: int, head_dim: int, 
     """One warning per shape when a call runs on a generic kernel (a correctness path, about two orders of magnitude
     slower than the MFMA kernels).  The reference's Triton kernels tile any power-of-two head_dim
     (attention.py:249-257, 453); here the fast kernels cover head_dim 128 and 64 (bf16 / fp16 also 32, 80, 96, 112 and 256),
-    blocks of a multiple of 16 tokens and any number of query heads per kv head (decode streams a kv head once per 16
-    of them)."""
+    blocks of a multiple of 16 tokens (decode at head_dim 128 / 64 also 1, 2, 4 and 8; prefill any size when the
+    caller passes max_seqlen_k) and any number of query heads per kv head (decode streams a kv head once per 16 of
+    them)."""
     key = (op, num_heads, num_kv_heads, head_dim, block_size, dtype, int8)
     if key in _shapes_seen:
         return

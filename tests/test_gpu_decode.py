@@ -63,9 +63,10 @@ def test_fast_path_vs_oracle(dtype, hq, hkv, bs, ctx_hi):
     assert got.dtype == dtype and mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
 
 
+@pytest.mark.parametrize("bs", [16, 8, 1])
 @pytest.mark.parametrize("ctx_list", [[1, 2, 15, 16, 17], [255, 256, 257, 511, 512, 513], [31, 32, 33, 1024, 1025]])
-def test_context_length_boundaries(ctx_list):
-    hq, hkv, d, bs = 8, 2, 128, 16
+def test_context_length_boundaries(ctx_list, bs):
+    hq, hkv, d = 8, 2, 128
     case = make_paged_case(33, 0, 0, 0, hq, hkv, d, bs, dtype=torch.bfloat16, ctx_list=ctx_list)
     got = _run(*case, 0.1, hq, hkv, d, bs)
     want = _oracle32(*case, 0.1, hq, hkv, d, bs)
@@ -76,7 +77,8 @@ def test_context_length_boundaries(ctx_list):
 @pytest.mark.parametrize("dtype,hq,hkv,d,bs", [
     (torch.float32, 4, 2, 64, 4),       # generic kernel: fp32 with a block size of 4
     (torch.float32, 6, 2, 96, 16),      # fp32, head_dim 96
-    (torch.bfloat16, 16, 16, 64, 8),    # head_dim 64 with a block size the MFMA kernel is not built for
+    (torch.bfloat16, 16, 16, 64, 8),    # head_dim 64, blocks of 8 tokens (the MFMA kernel's small-block form)
+    (torch.bfloat16, 4, 2, 128, 12),    # a block size that neither divides 16 nor is a multiple of it
     (torch.float32, 16, 8, 64, 16),     # the reference demo's shape and dtype (main.py)
     (torch.float16, 6, 3, 80, 3),       # odd head_dim and block size
     (torch.bfloat16, 4, 1, 256, 16),
@@ -205,7 +207,8 @@ def _pad_tables(tables, width_tokens, bs):
 @pytest.mark.parametrize("hq,hkv,bs,d", [(32, 8, 16, 128), (16, 8, 256, 128), (16, 1, 32, 128), (24, 2, 16, 128),
                                          (5, 1, 64, 128), (8, 8, 48, 128),
                                          (16, 8, 16, 64), (16, 16, 256, 64), (12, 1, 32, 64), (5, 5, 48, 64),
-                                         (34, 2, 16, 128), (48, 1, 32, 128), (71, 1, 16, 64)])
+                                         (34, 2, 16, 128), (48, 1, 32, 128), (71, 1, 16, 64),
+                                         (32, 8, 8, 128), (16, 8, 1, 128), (16, 16, 4, 64), (5, 1, 2, 128)])
 @pytest.mark.parametrize("form", ["one wave per head", "waves share a head", "waves share a head, one partition"])
 def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, d, form):
     """A ragged batch (contexts 1..1300, one empty) through both forms of the MFMA kernel: the batch size and the
@@ -214,7 +217,7 @@ def test_both_grid_forms_vs_oracle(dtype, hq, hkv, bs, d, form):
     partitions; 64 sequences x 8 kv heads in a table of 4 K tokens are one partition each, written without the
     merge kernel.  head_dim 64 (the reference demo's model, qwen3.py:338) runs on the same kernels with half of
     the second product's columns switched off.  More than 16 query heads per kv head (17, 48, 71) are served in slices
-    of 16, the last one partial."""
+    of 16, the last one partial.  Blocks of 8, 4, 2 and 1 tokens: every lane looks up the blocks of its own tokens."""
     batch = 7 if form == "waves share a head" else 64
     width = {"one wave per head": 32768, "waves share a head": 8192}.get(form, 4096) // bs * bs
     g = torch.Generator().manual_seed(77)
