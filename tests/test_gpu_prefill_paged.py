@@ -131,10 +131,12 @@ def test_paged_prefill_unmapped_blocks_and_empty_sequences():
         assert int(c["cu_q"][2] - c["cu_q"][1]) == 0 and got.shape[0] == 68 + 70
 
 
-def test_attention_module_uses_the_paged_prefill_when_block_tables_are_set():
+@pytest.mark.parametrize("bs", [16, 8])
+def test_attention_module_uses_the_paged_prefill_when_block_tables_are_set(bs):
     """Store the new tokens, then prefill over (cached prefix + new tokens) through ``Attention.forward``, as the
-    engine does on a prefix-cache hit."""
-    hq, hkv, d, bs = 16, 8, 128, 16
+    engine does on a prefix-cache hit.  With 8 tokens per block the module's max_seqlen_k sends the call through the
+    two-step form (a temporary cache of 16-token blocks)."""
+    hq, hkv, d = 16, 8, 128
     lengths, cached = [120, 50], [64, 16]
     c = make_paged_prefill_case(65, lengths, cached, hq, hkv, d, bs, dtype=torch.bfloat16, poison=0.0)
     att = Attention(hq, d, 1.0, hkv, bs)
