@@ -157,6 +157,11 @@ static int prefill_kernel_for(int num_heads, int num_kv_heads, int head_dim, int
   if (dtype != MVLLM_F32 && (head_dim == 128 || head_dim == 64 || prefill_mfma_other_dim(head_dim)) && blocks_ok &&
       (!paged || (int64_t)block_size * num_kv_heads * head_dim * 2 < ((int64_t)1 << 31)))
     return 2;
+  // fp32, head_dim 128 or 64: prefill_f32_kernel (a token row's bytes times 32 tile rows fit 32-bit copy offsets)
+  if (dtype == MVLLM_F32 && (head_dim == 128 || head_dim == 64) && blocks_ok &&
+      (int64_t)num_kv_heads * head_dim * 4 * 64 < ((int64_t)1 << 31) &&
+      (!paged || (int64_t)block_size * num_kv_heads * head_dim * 4 < ((int64_t)1 << 31)))
+    return 2;
   if (prefill_rows16_takes(head_dim, dtype, false) && blocks_ok && (int64_t)num_kv_heads * head_dim * 64 < ((int64_t)1 << 31))
     return 1;
   return head_dim <= 64 * kGenMaxR ? 0 : -1;
@@ -193,6 +198,7 @@ extern "C" int mvllm_prefill_varlen(void* out, const void* q, const void* k, con
   const bool aligned = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out);
   const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, 0, dtype, false, false) : 0;
   const bool mfma_ok = kind == 2;
+  if (mfma_ok && dtype == MVLLM_F32) return launch_prefill_f32(a, false, (hipStream_t)stream);
   if (mfma_ok && scale > 0.f && prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype, 0)) {
     PrefillPpArgs p;
     p.out = out; p.q = q; p.k = k; p.v = v; p.cu_seqlens = cu_seqlens; p.total_tokens = total_tokens;
@@ -239,6 +245,7 @@ extern "C" int mvllm_prefill_paged(void* out, const void* q, const void* k_cache
   const bool aligned = aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out);
   const int kind = aligned ? prefill_kernel_for(num_heads, num_kv_heads, head_dim, block_size, dtype, true, false) : 0;
   const bool mfma_ok = kind == 2;
+  if (mfma_ok && dtype == MVLLM_F32) return launch_prefill_f32(a, true, (hipStream_t)stream);
   if (mfma_ok && scale > 0.f && prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype, block_size)) {
     PrefillPpArgs p;
     p.out = out; p.q = q; p.k = k_cache; p.v = v_cache; p.cu_seqlens = cu_seqlens_q; p.total_tokens = total_q_tokens;

@@ -103,7 +103,8 @@ def test_prefill_plan_is_host_arithmetic():
     from minivllm_amd.layers.attention import prefill_plan
     assert prefill_plan(32, 8, 128) == 2 and prefill_plan(16, 8, 64, dtype=torch.float16) == 2
     assert prefill_plan(32, 8, 128, block_size=16) == 2 and prefill_plan(32, 8, 128, block_size=8) == 0
-    assert prefill_plan(32, 8, 128, dtype=torch.float32) == 1 and prefill_plan(16, 8, 64, 16, torch.float32) == 1
+    assert prefill_plan(32, 8, 128, dtype=torch.float32) == 2 and prefill_plan(16, 8, 64, 16, torch.float32) == 2     # fp32: its own LDS-tiled kernel
+    assert prefill_plan(16, 8, 64, 8, torch.float32) == 0
     assert prefill_plan(8, 8, 256) == 2 and prefill_plan(8, 8, 32, block_size=32) == 2      # bf16 / fp16 only
     assert prefill_plan(8, 8, 256, dtype=torch.float32) == 0
     assert prefill_plan(6, 2, 80) == 2 and prefill_plan(6, 2, 96) == 2 and prefill_plan(6, 2, 96, dtype=torch.float32) == 0

@@ -233,8 +233,7 @@ def test_config2_full_size():
     (6, 2, [17, 0, 5, 0, 48]),               # heads not a multiple of the four waves; empty sequences
 ])
 def test_prefill_head_dim_64_vs_oracle(dtype, hq, hkv, lengths):
-    """head_dim 64 runs on the LDS-tiled kernel in 16 bit and on 16-row tiles of the decode kernel's arithmetic in fp32
-    (not on the generic kernel)."""
+    """head_dim 64 runs on the LDS-tiled kernels, 16-bit and fp32 (not on the generic kernel)."""
     d = 64
     case = make_varlen_case(56, lengths, hq, hkv, d, dtype=dtype)
     scale = 1 / math.sqrt(d)
