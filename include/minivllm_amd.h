@@ -267,6 +267,31 @@ int mvllm_prefill_paged_int8_staged(void* out, const void* q,
                                     void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * mvllm_prefill_paged with every sequence's keys cut into `splits` ranges that are walked side by side and merged: for
+ * batches of few new tokens behind long cached prefixes (a follow-up turn, the last chunk of a chunked prefill), whose
+ * few query tiles would each walk a whole prefix while most of the chip idles.  No counterpart in the reference (its
+ * prefill never reads the paged cache, src/myvllm/layers/attention.py:111-209, and the prefix-hit metadata that
+ * model_runner.py:192-226 builds goes unused, attention.py:518-523).
+ * 16-bit caches, head_dim 64 or 128, block_size a multiple of 16, num_seqs * splits <= 64.
+ *   _split_plan: the number of ranges the library would use for a batch of these sizes; 0 = run mvllm_prefill_paged.
+ *   _split_workspace_bytes: 256-byte aligned device memory the call needs for `splits` ranges (range tables, partial
+ *     results [splits, total_q_tokens, Hq, D] and their softmax denominators); 0 = shape not taken.
+ * max_kv_len: the host's upper bound of every sequence's key count, as in the staged forms.  Results differ from the
+ * one-step form's by the rounding of the partial results to the element type (within the same tolerance).
+ */
+int mvllm_prefill_paged_split_plan(int num_seqs, int64_t total_q_tokens, int max_kv_len, int num_heads,
+                                   int num_kv_heads, int head_dim, int block_size, int dtype, int int8_cache);
+size_t mvllm_prefill_paged_split_workspace_bytes(int num_seqs, int64_t total_q_tokens, int max_kv_len, int num_heads,
+                                                 int num_kv_heads, int head_dim, int block_size, int dtype, int splits);
+int mvllm_prefill_paged_split(void* out, const void* q, const void* k_cache, const void* v_cache,
+                              const int32_t* block_tables, int max_num_blocks,
+                              const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                              int num_seqs, int64_t total_q_tokens, int max_kv_len,
+                              int num_heads, int num_kv_heads, int head_dim, int block_size,
+                              int64_t num_blocks, float scale, int dtype, int splits,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * The caller's per-layer chain between the QKV projection and the attention kernels, fused:
  *   q = rms_norm(q); k = rms_norm(k)      src/myvllm/models/qwen3.py:104-106, layers/layernorm.py:9-17
  *   q, k = rotary_emb(positions, q, k)    qwen3.py:108, layers/rotary_embedding.py:4-23, 77-83

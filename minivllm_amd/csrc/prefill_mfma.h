@@ -32,6 +32,16 @@ struct PrefillArgs {
   // [num_blocks, block_size, Hkv], else null
   const float* k_scale;
   const float* v_scale;
+  // Paged mode, optional (prefill_split.hip, where one sequence's keys are cut into ranges that are walked as
+  // sequences of their own): q_pos = position of each sequence's first query row among its keys where it is not
+  // len_k - len_q (a query block that sees all of a key range has q_pos >= len_k); lse = where to write, per (query
+  // row, head), log2 of the softmax denominator counted in powers of two (m + log2 l), with which the partial
+  // results of the ranges are merged; q_period > 0 = the query tensor holds that many rows and row t of the
+  // cu_seqlens numbering reads row t mod q_period (the ranges of a sequence share its queries).  A sequence
+  // without keys is skipped.
+  const int32_t* q_pos = nullptr;
+  float* lse = nullptr;
+  int64_t q_period = 0;
 };
 
 constexpr unsigned kXcdChunk = 32;      // consecutive work items handed to one XCD
@@ -178,7 +188,8 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
   // Keys of the sequence: its own rows, or in paged mode the cached prefix plus them (query row r sits at
   // position cached + r and sees keys 0 .. cached + r).
   const int kv_len = PAGED ? a.cu_seqlens_k[seq_index + 1] - a.cu_seqlens_k[seq_index] : seq_len;
-  const int cached = PAGED ? max(kv_len - seq_len, 0) : 0;
+  const int cached = !PAGED ? 0 : a.q_pos != nullptr ? a.q_pos[seq_index] : max(kv_len - seq_len, 0);
+  if (PAGED && a.q_pos != nullptr && kv_len <= 0) return;   // a key range that is empty (uniform over the workgroup)
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -189,10 +200,11 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
   const int r0 = row0 + kWaveRows * (wave / HPW);    // first query row of this wave (inside the sequence)
   const bool active = r0 < seq_len;
   const int pos0 = cached + r0;                      // position of that row among the keys
-  const int n_full = (pos0 + 1) / kBN;               // tiles every row of the wave sees completely
+  // tiles every row of the wave sees completely (a row sees keys up to its position, and never past the last key)
+  const int n_full = min((pos0 + 1) / kBN, kv_len / kBN);
   const int j_last = min(pos0 + kWaveRows - 1, kv_len - 1) / kBN;   // last tile any row of the wave sees
   const int wg_last = min(row0 + BM, seq_len) - 1;
-  const int ntiles = (cached + wg_last) / kBN + 1;
+  const int ntiles = min((cached + wg_last) / kBN, (kv_len - 1) / kBN) + 1;
   const int l32 = lane & 31;
   const int hi = lane >> 5;                          // 0/1: which half of the k-slots / rows
   const int qrow = r0 + l32;                         // query row of this lane
@@ -353,6 +365,7 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
   {
     int64_t tok = (int64_t)seq_start + qrow;
     if (tok > last_token) tok = last_token;
+    if (PAGED && a.q_period > 0) tok = (int64_t)((uint32_t)tok % (uint32_t)a.q_period);   // both below 2^31
     const T* src = q + (tok * a.num_heads + h) * DD + 8 * hi;
 #pragma unroll
     for (int ks = 0; ks < kKS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
@@ -452,7 +465,7 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
     // ---- online softmax, one query row per lane (scores stay unscaled; the scale is folded
     //      into the exp2 argument) ----
     if constexpr (diag) {
-      const int thr = cached + qrow - j * kBN - 4 * hi;   // kv offset inside the tile must be <= thr
+      const int thr = min(cached + qrow, kv_len - 1) - j * kBN - 4 * hi;   // kv offset inside the tile must be <= thr
 #pragma unroll
       for (int tk = 0; tk < NH; ++tk)
 #pragma unroll
@@ -608,6 +621,8 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
   {
     const float lt = l + __shfl_xor(l, 32, 64);
     const float inv = 1.f / lt;
+    if (PAGED && a.lse != nullptr && hi == 0 && qrow < seq_len)
+      a.lse[(int64_t)(seq_start + qrow) * a.num_heads + h] = __log2f(lt) - neg_m[0];
 #pragma unroll
     for (int td = 0; td < kTD; ++td)
 #pragma unroll

@@ -195,7 +195,8 @@ def flash_attention_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, c
 def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                                   block_tables: torch.Tensor, cu_seqlens_q: torch.Tensor,
                                   cu_seqlens_k: torch.Tensor, scale: float, num_heads: int, num_kv_heads: int,
-                                  head_dim: int, block_size: int, max_seqlen_k: int | None = None) -> torch.Tensor:
+                                  head_dim: int, block_size: int, max_seqlen_k: int | None = None,
+                                  key_splits: int | None = None) -> torch.Tensor:
     """Causal prefill of the tokens that follow each sequence's cached prefix, with every key read from the
     paged cache.  Consumes the metadata ``ModelRunner.prepare_prefill`` builds for prefix-cache hits
     (model_runner.py:192-226), which the reference's ``Attention.forward`` ignores (attention.py:518-523).
@@ -207,6 +208,9 @@ def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cach
     host's upper bound of every sequence's key count, ``Context.max_seqlen_k``) is given: the batch's keys and values
     are then copied into a temporary cache of 16-token blocks (``STAGED_PREFILL_MAX_BYTES`` at most) and the MFMA
     kernels run over that.
+    With ``max_seqlen_k`` given, a batch of few new tokens behind long prefixes (too few query tiles to occupy the
+    chip) has every sequence's keys cut into ranges that are walked side by side and merged; ``key_splits`` forces the
+    number of ranges (0 or 1: never split; None: the library's ``mvllm_prefill_paged_split_plan`` decides).
     """
     _C.require_cuda(q, k_cache, v_cache, block_tables, cu_seqlens_q, cu_seqlens_k)
     if q.dim() != 3 or tuple(q.shape[1:]) != (num_heads, head_dim):
@@ -241,6 +245,27 @@ def flash_attention_prefill_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cach
                                                 k_cache.shape[0], float(scale), _C.dtype_code(q.dtype), _ptr(workspace), need,
                                                 _C.current_stream_ptr(q.device))
             _C.check(st, "flash_attention_prefill_paged (staged)")
+            return output
+    if max_seqlen_k is not None and int(max_seqlen_k) > 0 and q.dtype != torch.float32:
+        code = _C.dtype_code(q.dtype)
+        splits = key_splits
+        if splits is None:
+            splits = lib.mvllm_prefill_paged_split_plan(num_seqs, q.shape[0], int(max_seqlen_k), num_heads, num_kv_heads,
+                                                        head_dim, block_size, code, 0)
+        need = 0
+        if splits >= 2:
+            need = lib.mvllm_prefill_paged_split_workspace_bytes(num_seqs, q.shape[0], int(max_seqlen_k), num_heads,
+                                                                 num_kv_heads, head_dim, block_size, code, splits)
+            if key_splits is not None and need == 0:
+                raise ValueError(f"key_splits={key_splits}: the split form is not built for this shape")
+        if 0 < need <= STAGED_PREFILL_MAX_BYTES:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+            st = lib.mvllm_prefill_paged_split(_ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                               block_tables.shape[1], _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), num_seqs,
+                                               q.shape[0], int(max_seqlen_k), num_heads, num_kv_heads, head_dim, block_size,
+                                               k_cache.shape[0], float(scale), code, splits, _ptr(workspace), need,
+                                               _C.current_stream_ptr(q.device))
+            _C.check(st, "flash_attention_prefill_paged (split over keys)")
             return output
     _warn_if_generic("prefill", num_heads, num_kv_heads, head_dim, block_size, q.dtype, False)
     st = lib.mvllm_prefill_paged(_ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),

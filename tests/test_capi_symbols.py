@@ -28,7 +28,7 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_noalloc", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_plan", "mvllm_prefill_varlen",
-              "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_prefill_paged_int8_staged", "mvllm_prefill_paged_staged", "mvllm_prefill_paged_staged_workspace_bytes", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_dev_offset", "mvllm_decode_advance", "mvllm_sample_tokens_workspace_bytes",
+              "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_prefill_paged_int8_staged", "mvllm_prefill_paged_staged", "mvllm_prefill_paged_staged_workspace_bytes", "mvllm_prefill_paged_split", "mvllm_prefill_paged_split_plan", "mvllm_prefill_paged_split_workspace_bytes", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_dev_offset", "mvllm_decode_advance", "mvllm_sample_tokens_workspace_bytes",
               "mvllm_add_rms_norm", "mvllm_linear_small_m", "mvllm_norm_linear_small_m", "mvllm_linear_small_m_plan",
               "mvllm_lm_head_sample", "mvllm_lm_head_sample_workspace_bytes",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
@@ -54,6 +54,28 @@ def test_host_only_entry_points():
     assert lib.mvllm_paged_decode_workspace_bytes(8, 16, 128, 16, 16) == 8 * 4 * 16 * 130 * 4     # 4 x 64 tokens
     assert lib.mvllm_paged_decode_workspace_bytes(2, 4, 128, 64, 16) == 2 * 16 * 4 * 130 * 4      # 16 x 64 tokens
     assert lib.mvllm_paged_decode_workspace_bytes(256, 32, 128, 2048, 16) == 256 * 32 * 32 * 130 * 4
+
+
+def test_prefill_split_plan_is_host_arithmetic():
+    """When a paged prefill is cut over its keys: few query tiles, at least 4096 keys, a shape the split form takes;
+    and the workspace holds the ranges' tables, partial results and denominators."""
+    _C = _lib()
+    lib = _C.load()
+    bf16, f32 = 1, 0
+    plan = lib.mvllm_prefill_paged_split_plan
+    assert plan(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 0) == 12          # 40 workgroups a range: 11 prefix ranges
+    assert plan(1, 16, 32768 + 16, 32, 8, 128, 256, bf16, 0) == 17            # never more than 16 prefix ranges
+    assert plan(2, 256, 4096 + 128, 32, 8, 128, 16, bf16, 0) == 5             # 1024 keys a range at least
+    assert plan(2, 1024, 16384 + 512, 32, 8, 128, 256, bf16, 0) == 5          # a small batch is cut in 4 at least
+    assert plan(16, 512, 4096 + 32, 32, 8, 128, 256, bf16, 0) == 0            # enough query tiles
+    assert plan(1, 128, 4095, 32, 8, 128, 256, bf16, 0) == 0                  # too few keys
+    assert plan(1, 128, 32768, 32, 8, 128, 256, f32, 0) == 0                  # fp32
+    assert plan(1, 128, 32768, 32, 8, 128, 8, bf16, 0) == 0                   # blocks of 8 tokens
+    assert plan(1, 128, 32768, 32, 8, 128, 256, bf16, 1) == 0                 # INT8 cache
+    need = lib.mvllm_prefill_paged_split_workspace_bytes(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 12)
+    partial = 12 * 128 * 32 * 128 * 2 + 12 * 128 * 32 * 4
+    assert partial < need < partial + 16384
+    assert lib.mvllm_prefill_paged_split_workspace_bytes(8, 128, 32768, 32, 8, 128, 256, bf16, 9) == 0   # 72 ranges
 
 
 def test_decode_plan_is_host_arithmetic():
