@@ -309,6 +309,33 @@ def bench_prefill_store(args, which, want_cpu=False):
             "roofline": roofline("mfma", flops_l / (event_ms_l * 1e-3) / 1e12, "prefill_pp_kernel"),
         }
         del ql, kl, vl
+        # few new tokens behind a long cached prefix (a follow-up turn): 128 tokens behind 32768 in a block-256 cache.
+        # Given the host's bound on the key count the operator cuts the keys into ranges (mvllm_prefill_paged_split);
+        # without it the call runs in one step, on 16 of the chip's 256 compute units.
+        from minivllm_amd.layers.attention import flash_attention_prefill_paged
+        new_s, prefix_s = 128, 32768
+        kv_s = new_s + prefix_s
+        nb_s = (kv_s + bs - 1) // bs
+        kcs = torch.randn(nb_s, bs, hkv, d, generator=dg, device=dev).to(torch.bfloat16)
+        vcs = torch.randn(nb_s, bs, hkv, d, generator=dg, device=dev).to(torch.bfloat16)
+        qs = torch.randn(new_s, hq, d, generator=dg, device=dev).to(torch.bfloat16)
+        bts = torch.randperm(nb_s, generator=torch.Generator().manual_seed(args.seed + 5)).to(torch.int32).view(1, nb_s).to(dev)
+        cu_qs = torch.tensor([0, new_s], dtype=torch.int32, device=dev)
+        cu_ks = torch.tensor([0, kv_s], dtype=torch.int32, device=dev)
+        _, ms_split = time_steps(lambda: flash_attention_prefill_paged(qs, kcs, vcs, bts, cu_qs, cu_ks, scale, hq, hkv, d, bs,
+                                                                       max_seqlen_k=kv_s),
+                                 args.steps, args.warmup, EXTRA_WARM_MS)
+        _, ms_one = time_steps(lambda: flash_attention_prefill_paged(qs, kcs, vcs, bts, cu_qs, cu_ks, scale, hq, hkv, d, bs),
+                               max(3, args.steps // 4), 2, EXTRA_WARM_MS)
+        flops_s = 4 * hq * d * (new_s * prefix_s + new_s * (new_s + 1) // 2)
+        out["prefill_short_suffix"] = {
+            "workload": "paged prefill of 128 new tokens behind a 32768-token cached prefix, one sequence, block_size 256, Hq32 Hkv8 D128 bf16",
+            "algorithmic_flops": flops_s, "event_ms_per_step": ms_split, "tflops": flops_s / (ms_split * 1e-3) / 1e12,
+            "one_step_event_ms_per_step": ms_one, "one_step_tflops": flops_s / (ms_one * 1e-3) / 1e12,
+            "roofline": roofline("mfma", flops_s / (ms_split * 1e-3) / 1e12,
+                                 "split_plan_kernel + prefill_mfma_kernel over key ranges + split_merge_kernel (the workspace comes from torch's allocator inside the timed call)"),
+        }
+        del kcs, vcs, qs
     if "prefill" in which:
         # the same prompts with the first half (whole 16-token blocks) already cached: only the second half is
         # computed, every key comes from a block-16 paged cache
@@ -902,6 +929,7 @@ def summary_of(line):
     put("prefill_vs_oracle_max_abs", "prefill", "cpu_baseline", "gpu_vs_oracle_max_abs")
     put("prefill_hq16_frac", "prefill_hq16", "roofline", "frac")
     put("prefill_4x8192_frac", "prefill_long_prompts", "roofline", "frac")
+    put("prefill_suffix128_behind_32k_us", "prefill_short_suffix", "event_ms_per_step")
     put("prefill_paged_frac", "prefill_cached_prefix", "roofline", "frac")
     put("prefill_paged_int8_frac", "prefill_cached_prefix_int8", "roofline", "frac")
     put("store_frac_hbm", "store", "roofline", "frac")
@@ -915,8 +943,9 @@ def summary_of(line):
                 if name in node:
                     out[key] = round(node[name])
                     break
-    if "prefill_us" in out:
-        out["prefill_us"] = round(out["prefill_us"] * 1e3, 1)
+    for key in ("prefill_us", "prefill_suffix128_behind_32k_us"):
+        if key in out:
+            out[key] = round(out[key] * 1e3, 1)
     return out
 
 
