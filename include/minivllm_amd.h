@@ -272,7 +272,9 @@ int mvllm_prefill_paged_int8_staged(void* out, const void* q,
  * few query tiles would each walk a whole prefix while most of the chip idles.  No counterpart in the reference (its
  * prefill never reads the paged cache, src/myvllm/layers/attention.py:111-209, and the prefix-hit metadata that
  * model_runner.py:192-226 builds goes unused, attention.py:518-523).
- * 16-bit caches, head_dim 64 or 128, block_size a multiple of 16, num_seqs * splits <= 64.
+ * 16-bit caches at the head dims of the LDS-tiled kernel (64, 128; 32, 48, 80, 96, 112, 256), INT8 caches
+ * (mvllm_prefill_paged_int8_split: codes + scales as for mvllm_prefill_paged_int8) at head_dim 64 and 128; block_size a
+ * multiple of 16, num_seqs * splits <= 64.
  *   _split_plan: the number of ranges the library would use for a batch of these sizes; 0 = run mvllm_prefill_paged.
  *   _split_workspace_bytes: 256-byte aligned device memory the call needs for `splits` ranges (range tables, partial
  *     results [splits, total_q_tokens, Hq, D] and their softmax denominators); 0 = shape not taken.
@@ -290,6 +292,15 @@ int mvllm_prefill_paged_split(void* out, const void* q, const void* k_cache, con
                               int num_heads, int num_kv_heads, int head_dim, int block_size,
                               int64_t num_blocks, float scale, int dtype, int splits,
                               void* workspace, size_t workspace_bytes, void* stream);
+int mvllm_prefill_paged_int8_split(void* out, const void* q,
+                                   const int8_t* k_cache, const int8_t* v_cache,
+                                   const float* k_scale, const float* v_scale,
+                                   const int32_t* block_tables, int max_num_blocks,
+                                   const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                   int num_seqs, int64_t total_q_tokens, int max_kv_len,
+                                   int num_heads, int num_kv_heads, int head_dim, int block_size,
+                                   int64_t num_blocks, float scale, int dtype, int splits,
+                                   void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * The caller's per-layer chain between the QKV projection and the attention kernels, fused:

@@ -50,6 +50,8 @@ SIGNATURES = {
     "mvllm_prefill_paged_split_workspace_bytes": (c_size_t, [c_int, c_int64] + [c_int] * 7),
     "mvllm_prefill_paged_split": (c_int, [c_void_p] * 5 + [c_int, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int,
                                             c_int, c_int64, c_float, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "mvllm_prefill_paged_int8_split": (c_int, [c_void_p] * 7 + [c_int, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int,
+                                                 c_int, c_int64, c_float, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "mvllm_sample_tokens_workspace_bytes": (c_size_t, [c_int, c_int]),
     "mvllm_sample_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_uint64, c_uint64, c_int, c_int,
                                     c_int, c_void_p, c_size_t, c_void_p]),

@@ -1,7 +1,7 @@
 // Version and status text of the C ABI declared in include/minivllm_amd.h.
 #include "common.h"
 
-extern "C" int mvllm_version(void) { return 1 * 1000 + 5; }
+extern "C" int mvllm_version(void) { return 1 * 1000 + 6; }
 
 extern "C" const char* mvllm_status_string(int status) {
   switch (status) {

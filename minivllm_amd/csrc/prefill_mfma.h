@@ -678,6 +678,8 @@ static int launch_prefill_mfma(const PrefillArgs& a, hipStream_t stream) {
 
 // the paged form over a 16-bit cache, head_dim 64 or 128, bf16 / fp16 (prefill_varlen.hip)
 int launch_prefill_paged_16bit(const PrefillArgs& a, int dtype, hipStream_t stream);
+// the paged form over an INT8 cache (codes + fp32 scales), head_dim 64 or 128, bf16 / fp16 queries (prefill_varlen.hip)
+int launch_prefill_paged_int8(const PrefillArgs& a, int dtype, hipStream_t stream);
 // fp32 tensors, head_dim 128 or 64, packed or over a paged fp32 cache (prefill_f32.hip)
 int launch_prefill_f32(const PrefillArgs& a, bool paged, hipStream_t stream);
 // head_dim 32, 80, 96, 112 (prefill_other_dims.hip); 16-bit element types only

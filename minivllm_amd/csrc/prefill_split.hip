@@ -1,4 +1,4 @@
-// Prefill over a paged 16-bit cache with the keys of every sequence cut into ranges: a batch of few new tokens behind
+// Prefill over a paged cache (16-bit, or INT8 codes with fp32 scales) with the keys of every sequence cut into ranges: a batch of few new tokens behind
 // long cached prefixes (a follow-up turn of a chat, the last chunk of a chunked prefill) has too few query tiles to
 // occupy the chip, and every one of them walks the whole prefix.  Here a sequence's prefix is cut into `splits - 1`
 // ranges of whole key tiles and whole cache blocks plus one last range that holds the rest of the prefix and the new
@@ -106,17 +106,17 @@ struct MergeArgs {
   int head_dim;
 };
 
-// One workgroup per (query row, slice of 256 / (D / 8) heads); a thread merges 8 output elements of one head.  out =
+// One workgroup per (query row, slice of floor(256 / (D / 8)) heads); a thread merges 8 output elements of one head.  out =
 // sum_i 2^(lse_i - M) o_i / sum_i 2^(lse_i - M) over the ranges that hold keys, M their largest lse: o_i is range i's
 // normalised result and 2^lse_i its softmax denominator, so the weights restore the numerators.  The denominators of
 // the slice are fetched into LDS first, all at once (an empty range's as -inf, which weighs it out), so that the loop
 // over the ranges has nothing to wait for but its own independent loads.
 template <typename T>
 __global__ __launch_bounds__(256) void split_merge_kernel(const MergeArgs a) {
-  __shared__ float lse_s[kMaxRanges][32];
+  __shared__ float lse_s[kMaxRanges][64];
   const int t = blockIdx.x;
-  const int chunks = a.head_dim / 8;               // 16 or 8
-  const int heads_here = 256 / chunks;             // 16 or 32
+  const int chunks = a.head_dim / 8;               // 4 .. 32
+  const int heads_here = 256 / chunks;             // 64 .. 8
   const int head0 = blockIdx.y * heads_here;
   int s = 0;
   while (s + 1 < a.num_seqs && a.cu_seqlens_q[s + 1] <= t) ++s;
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(256) void split_merge_kernel(const MergeArgs a) {
   __syncthreads();
   const int hh = threadIdx.x / chunks, c = threadIdx.x - hh * chunks;
   const int h = head0 + hh;
-  if (h >= a.num_heads) return;
+  if (hh >= heads_here || h >= a.num_heads) return;
   float top = -INFINITY;
   for (int i = 0; i < a.splits; ++i) top = fmaxf(top, lse_s[i][hh]);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -195,13 +195,15 @@ SplitLayout split_layout(int num_seqs, int64_t total_q, int max_kv_len, int num_
   return l;
 }
 
+// int8: an INT8 cache (head_dim 64 and 128 only; a 16-bit cache also the other head dims of the LDS-tiled kernel)
 bool split_shape_ok(int num_seqs, int64_t total_q, int max_kv_len, int num_heads, int num_kv_heads, int head_dim,
-                    int block_size, int dtype, int splits) {
+                    int block_size, int dtype, int splits, bool int8) {
   if (num_seqs <= 0 || total_q <= 0 || max_kv_len <= 0 || num_heads <= 0 || num_kv_heads <= 0 || block_size <= 0) return false;
   if (num_heads % num_kv_heads != 0 || num_heads > 65535) return false;
   if (dtype != MVLLM_BF16 && dtype != MVLLM_F16) return false;
-  if ((head_dim != 128 && head_dim != 64) || block_size % 16 != 0 || block_size > (1 << 20)) return false;
-  if ((int64_t)block_size * num_kv_heads * head_dim * 2 >= ((int64_t)1 << 31)) return false;
+  const bool dim_ok = head_dim == 128 || head_dim == 64 || (!int8 && prefill_mfma_other_dim(head_dim));
+  if (!dim_ok || block_size % 16 != 0 || block_size > (1 << 20)) return false;
+  if ((int64_t)block_size * num_kv_heads * head_dim * (int8 ? 1 : 2) >= ((int64_t)1 << 31)) return false;
   if (splits < 2 || (int64_t)num_seqs * splits > kMaxRanges) return false;
   if ((int64_t)splits * total_q > ((int64_t)1 << 30)) return false;
   return true;
@@ -217,20 +219,31 @@ using namespace mvllm;
 // sequences, the longest of max_kv_len keys): 0 = do not split (enough query tiles to fill the chip, keys too few to be
 // worth the two extra launches, or a shape the split form is not built for).  The numbers: the two-group kernel deals
 // items of 64 rows x 4 heads to 256 compute units, and a launch of fewer than 192 of them leaves a quarter of the chip
-// idle from the start; the one-group kernel that walks the ranges runs two workgroups per compute unit, so the ranges
+// idle from the start (shapes it does not take: fewer than three quarters of the one-group kernel's 512 places, 256 at head_dim 256);
+// the one-group kernel that walks the ranges runs two workgroups per compute unit, so the ranges
 // aim at 512 workgroups in all (but at 4 prefix ranges at least), each prefix range at least 1024 keys long, at most 16
 // of them (more only lengthen the merge).
 extern "C" int mvllm_prefill_paged_split_plan(int num_seqs, int64_t total_q_tokens, int max_kv_len, int num_heads,
                                               int num_kv_heads, int head_dim, int block_size, int dtype, int int8_cache) {
-  if (int8_cache != 0 || !split_shape_ok(num_seqs, total_q_tokens, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype, 2))
+  if (!split_shape_ok(num_seqs, total_q_tokens, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype, 2, int8_cache != 0))
     return 0;
   if (max_kv_len < 4096) return 0;
   const int group = num_heads / num_kv_heads;
-  const int64_t wide_items = (total_q_tokens / 64 + num_seqs) * std::max(num_heads / 4, 1);
-  if (wide_items >= 192) return 0;
   const int hpw = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
-  const int64_t items = (total_q_tokens / (32 * (4 / hpw)) + num_seqs) * (num_heads / hpw);
-  int64_t prefix_ranges = std::max<int64_t>(512 / items - 1, 4);   // 4: a batch this small gains from any cut (measured)
+  const int64_t items = (total_q_tokens / (32 * (4 / hpw)) + num_seqs) * (num_heads / hpw);   // one-group workgroups of one range
+  const int places = head_dim == 256 ? 256 : 512;     // workgroups of the one-group kernel the chip holds at a time
+  // what the call would run on otherwise: the two-group kernel (for an INT8 cache behind the staging step), or the
+  // one-group kernel with its 512 places
+  if (prefill_pp_takes(num_seqs, num_heads, num_kv_heads, head_dim, dtype, 16)) {
+    const int64_t wide_items = (total_q_tokens / 64 + num_seqs) * std::max(num_heads / 4, 1);
+    // INT8: the ranges run on the one-step kernel, which converts every tile for every query tile (two thirds of the
+    // two-step form's rate), so the chip has to be emptier for the cut to pay (2 x 512 tokens behind 16384: 362 us in
+    // two steps, 406 us cut)
+    if (wide_items >= (int8_cache != 0 ? 96 : 192)) return 0;
+  } else if (items >= 3 * places / 4) {
+    return 0;
+  }
+  int64_t prefix_ranges = std::max<int64_t>(places / items - 1, 4);   // 4: a batch this small gains from any cut (measured)
   prefix_ranges = std::min<int64_t>(prefix_ranges, max_kv_len / 1024);
   prefix_ranges = std::min<int64_t>(prefix_ranges, kMaxRanges / num_seqs - 1);
   prefix_ranges = std::min<int64_t>(prefix_ranges, 16);
@@ -239,23 +252,23 @@ extern "C" int mvllm_prefill_paged_split_plan(int num_seqs, int64_t total_q_toke
 
 extern "C" size_t mvllm_prefill_paged_split_workspace_bytes(int num_seqs, int64_t total_q_tokens, int max_kv_len, int num_heads,
                                                             int num_kv_heads, int head_dim, int block_size, int dtype, int splits) {
-  if (!split_shape_ok(num_seqs, total_q_tokens, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype, splits)) return 0;
+  if (!split_shape_ok(num_seqs, total_q_tokens, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype, splits, false)) return 0;
   return split_layout(num_seqs, total_q_tokens, max_kv_len, num_heads, head_dim, block_size, splits).total_bytes;
 }
 
-extern "C" int mvllm_prefill_paged_split(void* out, const void* q, const void* k_cache, const void* v_cache,
-                                         const int32_t* block_tables, int max_num_blocks, const int32_t* cu_seqlens_q,
-                                         const int32_t* cu_seqlens_k, int num_seqs, int64_t total_q_tokens, int max_kv_len,
-                                         int num_heads, int num_kv_heads, int head_dim, int block_size, int64_t num_blocks,
-                                         float scale, int dtype, int splits, void* workspace, size_t workspace_bytes,
-                                         void* stream) {
+static int run_split(void* out, const void* q, const void* k_cache, const void* v_cache, const float* k_scale,
+                     const float* v_scale, bool int8, const int32_t* block_tables, int max_num_blocks,
+                     const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int num_seqs, int64_t total_q_tokens,
+                     int max_kv_len, int num_heads, int num_kv_heads, int head_dim, int block_size, int64_t num_blocks,
+                     float scale, int dtype, int splits, void* workspace, size_t workspace_bytes, void* stream) {
   if (dtype_size(dtype) == 0) return MVLLM_ERR_BAD_DTYPE;
   if (num_seqs < 0 || total_q_tokens < 0 || max_kv_len < 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 ||
       block_size <= 0 || num_blocks < 0 || max_num_blocks < 0 || num_heads % num_kv_heads != 0 || !(scale > 0.f))
     return MVLLM_ERR_BAD_SHAPE;
   if (num_seqs == 0 || total_q_tokens == 0) return MVLLM_OK;
-  if (!out || !q || !k_cache || !v_cache || !block_tables || !cu_seqlens_q || !cu_seqlens_k) return MVLLM_ERR_NULL_POINTER;
-  if (!split_shape_ok(num_seqs, total_q_tokens, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype, splits))
+  if (!out || !q || !k_cache || !v_cache || (int8 && (!k_scale || !v_scale)) || !block_tables || !cu_seqlens_q || !cu_seqlens_k)
+    return MVLLM_ERR_NULL_POINTER;
+  if (!split_shape_ok(num_seqs, total_q_tokens, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, dtype, splits, int8))
     return MVLLM_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(out) || !aligned16(k_cache) || !aligned16(v_cache)) return MVLLM_ERR_MISALIGNED;
   const SplitLayout l = split_layout(num_seqs, total_q_tokens, max_kv_len, num_heads, head_dim, block_size, splits);
@@ -284,9 +297,11 @@ extern "C" int mvllm_prefill_paged_split(void* out, const void* q, const void* k
   a.num_kv_heads = num_kv_heads; a.head_dim = head_dim; a.scale_log2 = scale * kLog2e;
   a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
   a.cu_seqlens_k = sp.ws_cu_k; a.block_tables = sp.ws_table; a.max_num_blocks = l.table_width;
-  a.block_size = block_size; a.num_blocks = num_blocks; a.k_scale = nullptr; a.v_scale = nullptr;
+  a.block_size = block_size; a.num_blocks = num_blocks; a.k_scale = k_scale; a.v_scale = v_scale;
   a.q_pos = sp.ws_q_pos; a.lse = lse; a.q_period = total_q_tokens;
-  status = launch_prefill_paged_16bit(a, dtype, s);
+  status = int8                               ? launch_prefill_paged_int8(a, dtype, s)
+           : prefill_mfma_other_dim(head_dim) ? launch_prefill_mfma_other(a, dtype, true, s)
+                                              : launch_prefill_paged_16bit(a, dtype, s);
   if (status != MVLLM_OK) return status;
 
   MergeArgs m;
@@ -297,4 +312,26 @@ extern "C" int mvllm_prefill_paged_split(void* out, const void* q, const void* k
   if (dtype == MVLLM_BF16) split_merge_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(m);
   else split_merge_kernel<f16_t><<<grid, dim3(256), 0, s>>>(m);
   return launch_status();
+}
+
+extern "C" int mvllm_prefill_paged_split(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                         const int32_t* block_tables, int max_num_blocks, const int32_t* cu_seqlens_q,
+                                         const int32_t* cu_seqlens_k, int num_seqs, int64_t total_q_tokens, int max_kv_len,
+                                         int num_heads, int num_kv_heads, int head_dim, int block_size, int64_t num_blocks,
+                                         float scale, int dtype, int splits, void* workspace, size_t workspace_bytes,
+                                         void* stream) {
+  return run_split(out, q, k_cache, v_cache, nullptr, nullptr, false, block_tables, max_num_blocks, cu_seqlens_q, cu_seqlens_k,
+                   num_seqs, total_q_tokens, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, dtype,
+                   splits, workspace, workspace_bytes, stream);
+}
+
+extern "C" int mvllm_prefill_paged_int8_split(void* out, const void* q, const int8_t* k_cache, const int8_t* v_cache,
+                                              const float* k_scale, const float* v_scale, const int32_t* block_tables,
+                                              int max_num_blocks, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                              int num_seqs, int64_t total_q_tokens, int max_kv_len, int num_heads,
+                                              int num_kv_heads, int head_dim, int block_size, int64_t num_blocks, float scale,
+                                              int dtype, int splits, void* workspace, size_t workspace_bytes, void* stream) {
+  return run_split(out, q, k_cache, v_cache, k_scale, v_scale, true, block_tables, max_num_blocks, cu_seqlens_q, cu_seqlens_k,
+                   num_seqs, total_q_tokens, max_kv_len, num_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, dtype,
+                   splits, workspace, workspace_bytes, stream);
 }

@@ -141,6 +141,9 @@ namespace mvllm {
 int launch_prefill_paged_16bit(const PrefillArgs& a, int dtype, hipStream_t stream) {
   return dtype == MVLLM_BF16 ? launch_prefill_mfma<bf16_t, true, false>(a, stream) : launch_prefill_mfma<f16_t, true, false>(a, stream);
 }
+int launch_prefill_paged_int8(const PrefillArgs& a, int dtype, hipStream_t stream) {
+  return dtype == MVLLM_BF16 ? launch_prefill_mfma<bf16_t, true, true>(a, stream) : launch_prefill_mfma<f16_t, true, true>(a, stream);
+}
 }  // namespace mvllm
 
 using namespace mvllm;
@@ -293,8 +296,7 @@ extern "C" int mvllm_prefill_paged_int8(void* out, const void* q, const int8_t* 
     a.tiles_x = 0; a.heads_y = 0; a.band_bits = 0;
     a.cu_seqlens_k = cu_seqlens_k; a.block_tables = block_tables; a.max_num_blocks = max_num_blocks;
     a.block_size = block_size; a.num_blocks = num_blocks; a.k_scale = k_scale; a.v_scale = v_scale;
-    return dtype == MVLLM_BF16 ? launch_prefill_mfma<bf16_t, true, true>(a, (hipStream_t)stream)
-                               : launch_prefill_mfma<f16_t, true, true>(a, (hipStream_t)stream);
+    return launch_prefill_paged_int8(a, dtype, (hipStream_t)stream);
   }
   PrefillRowsArgs r;
   r.out = out; r.q = q; r.k = k_cache; r.v = v_cache; r.cu_seqlens = cu_seqlens_q; r.total_tokens = total_q_tokens;

@@ -283,7 +283,7 @@ def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v
                                        k_scale: torch.Tensor, v_scale: torch.Tensor, block_tables: torch.Tensor,
                                        cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, scale: float,
                                        num_heads: int, num_kv_heads: int, head_dim: int, block_size: int,
-                                       max_seqlen_k: int | None = None) -> torch.Tensor:
+                                       max_seqlen_k: int | None = None, key_splits: int | None = None) -> torch.Tensor:
     """``flash_attention_prefill_paged`` over an INT8 cache written by ``store_kvcache_int8``: every key, the new
     tokens' included, is read from the cache and dequantised in the kernel, as decode does for the same tokens.
     q bf16 / fp16; caches int8 (num_blocks, block_size, Hkv, D); scales float32 (num_blocks, block_size, Hkv).
@@ -291,7 +291,8 @@ def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v
     run in two steps: the batch's keys and values are dequantised once into a temporary 16-bit cache
     (2 x num_seqs x max_seqlen_k x Hkv x D x 2 bytes from torch's allocator, at most ``STAGED_PREFILL_MAX_BYTES``),
     which is a quarter faster than converting every tile for every query tile that walks it, and the only MFMA path
-    for block sizes that are not a multiple of 16."""
+    for block sizes that are not a multiple of 16.  Few new tokens behind long prefixes are instead cut over the keys
+    as in ``flash_attention_prefill_paged`` (``key_splits`` as there)."""
     _C.require_cuda(q, k_cache, v_cache, k_scale, v_scale, block_tables, cu_seqlens_q, cu_seqlens_k)
     if q.dim() != 3 or tuple(q.shape[1:]) != (num_heads, head_dim):
         raise ValueError(f"q must be (total_tokens, {num_heads}, {head_dim}), got {tuple(q.shape)}")
@@ -315,6 +316,26 @@ def flash_attention_prefill_paged_int8(q: torch.Tensor, k_cache: torch.Tensor, v
     cu_seqlens_k = cu_seqlens_k.to(torch.int32).contiguous()
     output = torch.empty_like(q)
     if max_seqlen_k is not None and int(max_seqlen_k) > 0:
+        lib, code = _C.load(), _C.dtype_code(q.dtype)
+        splits = key_splits
+        if splits is None:
+            splits = lib.mvllm_prefill_paged_split_plan(num_seqs, q.shape[0], int(max_seqlen_k), num_heads, num_kv_heads,
+                                                        head_dim, block_size, code, 1)
+        need = 0
+        if splits >= 2:
+            need = lib.mvllm_prefill_paged_split_workspace_bytes(num_seqs, q.shape[0], int(max_seqlen_k), num_heads,
+                                                                 num_kv_heads, head_dim, block_size, code, splits)
+            if key_splits is not None and need == 0:
+                raise ValueError(f"key_splits={key_splits}: the split form is not built for this shape")
+        if 0 < need <= STAGED_PREFILL_MAX_BYTES:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+            st = lib.mvllm_prefill_paged_int8_split(
+                _ptr(output), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale), _ptr(block_tables),
+                block_tables.shape[1], _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), num_seqs, q.shape[0], int(max_seqlen_k),
+                num_heads, num_kv_heads, head_dim, block_size, k_cache.shape[0], float(scale), code, splits,
+                _ptr(workspace), need, _C.current_stream_ptr(q.device))
+            _C.check(st, "flash_attention_prefill_paged_int8 (split over keys)")
+            return output
         need = _C.load().mvllm_prefill_paged_staged_workspace_bytes(num_seqs, int(max_seqlen_k), num_heads, num_kv_heads,
                                                                     head_dim, _C.dtype_code(q.dtype), 1)
         if 0 < need <= STAGED_PREFILL_MAX_BYTES:

@@ -28,7 +28,7 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for n in ["mvllm_store_kvcache", "mvllm_store_kvcache_int8", "mvllm_paged_decode",
               "mvllm_paged_decode_int8", "mvllm_paged_decode_noalloc", "mvllm_paged_decode_workspace_bytes", "mvllm_paged_decode_plan", "mvllm_prefill_plan", "mvllm_prefill_varlen",
-              "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_prefill_paged_int8_staged", "mvllm_prefill_paged_staged", "mvllm_prefill_paged_staged_workspace_bytes", "mvllm_prefill_paged_split", "mvllm_prefill_paged_split_plan", "mvllm_prefill_paged_split_workspace_bytes", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_dev_offset", "mvllm_decode_advance", "mvllm_sample_tokens_workspace_bytes",
+              "mvllm_prefill_paged", "mvllm_prefill_paged_int8", "mvllm_prefill_paged_int8_staged", "mvllm_prefill_paged_staged", "mvllm_prefill_paged_staged_workspace_bytes", "mvllm_prefill_paged_split", "mvllm_prefill_paged_int8_split", "mvllm_prefill_paged_split_plan", "mvllm_prefill_paged_split_workspace_bytes", "mvllm_qk_norm_rope_store", "mvllm_sample_tokens", "mvllm_sample_tokens_dev_offset", "mvllm_decode_advance", "mvllm_sample_tokens_workspace_bytes",
               "mvllm_add_rms_norm", "mvllm_linear_small_m", "mvllm_norm_linear_small_m", "mvllm_linear_small_m_plan",
               "mvllm_lm_head_sample", "mvllm_lm_head_sample_workspace_bytes",
               "mvllm_silu_and_mul", "mvllm_version", "mvllm_status_string"]:
@@ -71,7 +71,11 @@ def test_prefill_split_plan_is_host_arithmetic():
     assert plan(1, 128, 4095, 32, 8, 128, 256, bf16, 0) == 0                  # too few keys
     assert plan(1, 128, 32768, 32, 8, 128, 256, f32, 0) == 0                  # fp32
     assert plan(1, 128, 32768, 32, 8, 128, 8, bf16, 0) == 0                   # blocks of 8 tokens
-    assert plan(1, 128, 32768, 32, 8, 128, 256, bf16, 1) == 0                 # INT8 cache
+    assert plan(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 1) == 12          # INT8 cache: as the 16-bit one
+    assert plan(1, 128, 32768, 32, 8, 80, 256, bf16, 1) == 0                  # ... but at head_dim 64 / 128 only
+    assert plan(1, 128, 32768, 16, 8, 80, 256, bf16, 0) == 17                 # head_dim 80: 24 workgroups a range
+    assert plan(8, 4096, 32768, 16, 8, 80, 256, bf16, 0) == 0                 # ... 576 of them fill the chip
+    assert plan(1, 128, 32768, 16, 8, 72, 256, bf16, 0) == 0                  # head_dim 72: not an LDS-tiled shape
     need = lib.mvllm_prefill_paged_split_workspace_bytes(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 12)
     partial = 12 * 128 * 32 * 128 * 2 + 12 * 128 * 32 * 4
     assert partial < need < partial + 16384

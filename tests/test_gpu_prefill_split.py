@@ -1,5 +1,5 @@
-"""Paged prefill with every sequence's keys cut into ranges (mvllm_prefill_paged_split) against the CPU oracle and
-against the one-step form."""
+"""Paged prefill with every sequence's keys cut into ranges (mvllm_prefill_paged_split, mvllm_prefill_paged_int8_split)
+against the CPU oracle and against the one-step form."""
 import math
 
 import pytest
@@ -29,6 +29,9 @@ def _run(c, hq, hkv, d, bs, scale, splits, max_k):
     (5, 5, 128, 32, [600, 130], [500, 100], 2),                    # no grouping: one head per workgroup
     (32, 8, 128, 16, [200, 100], [100, 40], 8),                    # more ranges than the prefixes have tiles
     (8, 1, 64, 64, [3000], [2990], 16),                            # one kv head, ten new tokens
+    (16, 8, 80, 16, [900, 300], [800, 299], 4),                    # head_dim 80 in the layout of 128
+    (6, 2, 32, 32, [700], [650], 3),                               # head_dim 32 in the layout of 64; three heads per kv head
+    (8, 4, 256, 16, [600, 200], [520, 130], 3),                    # head_dim 256: one workgroup per compute unit
 ])
 def test_paged_prefill_split_over_keys(hq, hkv, d, bs, lengths, cached, splits, dtype):
     c = make_paged_prefill_case(83, lengths, cached, hq, hkv, d, bs, dtype=dtype)
@@ -43,6 +46,39 @@ def test_paged_prefill_split_over_keys(hq, hkv, d, bs, lengths, cached, splits, 
     one_step = _run(c, hq, hkv, d, bs, scale, 0, max(lengths))
     mx, mean = error_stats(got, one_step.float())
     assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,d,bs,lengths,cached,splits", [
+    (32, 8, 128, 16, [1300, 90, 700], [1237, 0, 699], 4),
+    (16, 8, 64, 256, [2100, 800], [2000, 512], 5),
+    (6, 2, 128, 48, [1000, 30], [900, 7], 3),
+])
+def test_int8_paged_prefill_split_over_keys(hq, hkv, d, bs, lengths, cached, splits, dtype):
+    """The split form over an INT8 cache: against the fp32 oracle over the dequantised cache with the INT8 bounds (2e-2
+    beyond the output's half step, mean 2e-3), and against the one-step kernel."""
+    from helpers import half_step
+    from minivllm_amd.layers.attention import flash_attention_prefill_paged_int8, store_kvcache_int8
+    c = make_paged_prefill_case(97, lengths, cached, hq, hkv, d, bs, dtype=dtype, poison=0.0)
+    nb = c["k_cache"].shape[0]
+    ck, cv = (torch.zeros(nb, bs, hkv, d, dtype=torch.int8, device=DEV) for _ in range(2))
+    sk, sv = (torch.zeros(nb, bs, hkv, device=DEV) for _ in range(2))
+    store_kvcache_int8(c["k_cache"].view(-1, hkv, d).to(DEV), c["v_cache"].view(-1, hkv, d).to(DEV), ck, cv, sk, sv,
+                       torch.arange(nb * bs, device=DEV), bs)
+    scale = 1 / math.sqrt(d)
+    args = (c["q_new"].to(DEV), ck, cv, sk, sv, c["block_tables"].to(DEV), c["cu_q"].to(DEV), c["cu_k"].to(DEV), scale,
+            hq, hkv, d, bs)
+    got = flash_attention_prefill_paged_int8(*args, max_seqlen_k=max(lengths), key_splits=splits).cpu()
+    kd = oracle.dequantize_cache_oracle(ck.cpu(), sk.cpu())
+    vd = oracle.dequantize_cache_oracle(cv.cpu(), sv.cpu())
+    want = oracle.prefill_paged_oracle(c["q_new"].float(), kd, vd, c["block_tables"], c["cu_q"], c["cu_k"], scale,
+                                       hq, hkv, d, bs)
+    mx, mean = error_stats(got, want)
+    excess = ((got.float() - want).abs() - half_step(want, dtype)).max().item()
+    assert torch.isfinite(got.float()).all() and excess <= 2e-2 and mean <= 2e-3, (mx, excess, mean)
+    one_step = flash_attention_prefill_paged_int8(*args).cpu()
+    mx, mean = error_stats(got, one_step.float())
+    assert mx <= 2e-2 and mean <= 2e-3, (mx, mean)
 
 
 def test_paged_prefill_splits_by_itself_behind_a_long_prefix():
@@ -73,8 +109,9 @@ def test_split_plan_and_rejections():
     assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 128, 256, bf, 0) >= 3
     assert lib.mvllm_prefill_paged_split_plan(16, 16384, 2048, 32, 8, 128, 256, bf, 0) == 0      # the chip is full
     assert lib.mvllm_prefill_paged_split_plan(1, 128, 2048, 32, 8, 128, 256, bf, 0) == 0         # too few keys to cut
-    assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 128, 256, bf, 1) == 0        # INT8 cache
-    assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 80, 256, bf, 0) == 0         # head_dim 80
+    assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 128, 256, bf, 1) >= 3        # INT8 cache
+    assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 80, 256, bf, 1) == 0         # ... not at head_dim 80
+    assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 72, 256, bf, 0) == 0         # head_dim 72
     assert lib.mvllm_prefill_paged_split_workspace_bytes(40, 128, 32768, 32, 8, 128, 256, bf, 2) == 0   # 80 ranges
     c = make_paged_prefill_case(5, [300], [200], 8, 8, 128, 16, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
