@@ -230,7 +230,9 @@ extern "C" int mvllm_prefill_paged_split_plan(int num_seqs, int64_t total_q_toke
   if (max_kv_len < 4096) return 0;
   const int group = num_heads / num_kv_heads;
   const int hpw = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
-  const int64_t items = (total_q_tokens / (32 * (4 / hpw)) + num_seqs) * (num_heads / hpw);   // one-group workgroups of one range
+  const int rows = 32 * (4 / hpw);                    // query rows of a one-group workgroup
+  // one-group workgroups of one range (every sequence but one may add a partial row tile)
+  const int64_t items = ((total_q_tokens + rows - 1) / rows + num_seqs - 1) * (num_heads / hpw);
   const int places = head_dim == 256 ? 256 : 512;     // workgroups of the one-group kernel the chip holds at a time
   // what the call would run on otherwise: the two-group kernel (for an INT8 cache behind the staging step), or the
   // one-group kernel with its 512 places

@@ -63,7 +63,7 @@ def test_prefill_split_plan_is_host_arithmetic():
     lib = _C.load()
     bf16, f32 = 1, 0
     plan = lib.mvllm_prefill_paged_split_plan
-    assert plan(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 0) == 12          # 40 workgroups a range: 11 prefix ranges
+    assert plan(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 0) == 16          # 32 workgroups a range: 15 prefix ranges
     assert plan(1, 16, 32768 + 16, 32, 8, 128, 256, bf16, 0) == 17            # never more than 16 prefix ranges
     assert plan(2, 256, 4096 + 128, 32, 8, 128, 16, bf16, 0) == 5             # 1024 keys a range at least
     assert plan(2, 1024, 16384 + 512, 32, 8, 128, 256, bf16, 0) == 5          # a small batch is cut in 4 at least
@@ -71,13 +71,13 @@ def test_prefill_split_plan_is_host_arithmetic():
     assert plan(1, 128, 4095, 32, 8, 128, 256, bf16, 0) == 0                  # too few keys
     assert plan(1, 128, 32768, 32, 8, 128, 256, f32, 0) == 0                  # fp32
     assert plan(1, 128, 32768, 32, 8, 128, 8, bf16, 0) == 0                   # blocks of 8 tokens
-    assert plan(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 1) == 12          # INT8 cache: as the 16-bit one
+    assert plan(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 1) == 16          # INT8 cache: as the 16-bit one
     assert plan(1, 128, 32768, 32, 8, 80, 256, bf16, 1) == 0                  # ... but at head_dim 64 / 128 only
-    assert plan(1, 128, 32768, 16, 8, 80, 256, bf16, 0) == 17                 # head_dim 80: 24 workgroups a range
+    assert plan(1, 128, 32768, 16, 8, 80, 256, bf16, 0) == 17                 # head_dim 80: 16 workgroups a range
     assert plan(8, 4096, 32768, 16, 8, 80, 256, bf16, 0) == 0                 # ... 576 of them fill the chip
     assert plan(1, 128, 32768, 16, 8, 72, 256, bf16, 0) == 0                  # head_dim 72: not an LDS-tiled shape
-    need = lib.mvllm_prefill_paged_split_workspace_bytes(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 12)
-    partial = 12 * 128 * 32 * 128 * 2 + 12 * 128 * 32 * 4
+    need = lib.mvllm_prefill_paged_split_workspace_bytes(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 16)
+    partial = 16 * 128 * 32 * 128 * 2 + 16 * 128 * 32 * 4
     assert partial < need < partial + 16384
     assert lib.mvllm_prefill_paged_split_workspace_bytes(8, 128, 32768, 32, 8, 128, 256, bf16, 9) == 0   # 72 ranges
 
