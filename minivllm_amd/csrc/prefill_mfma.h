@@ -442,6 +442,27 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
       // K fragments are read one step ahead of the MFMAs that use them.  The reads of step ks + 1 stand in front
       // of step ks's copy instruction on purpose: the copy is an asm statement, which no LDS read is moved
       // across, so reads placed after it would be issued right before their use and wait out the LDS latency.
+      if constexpr (D == 256) {
+        // One wave per SIMD: nothing else covers an LDS round trip, so the fragments are requested two steps (four
+        // MFMAs) ahead.
+        uint4 kf[3][NH];
+#pragma unroll
+        for (int pre = 0; pre < 2; ++pre)
+#pragma unroll
+          for (int tk = 0; tk < NH; ++tk) kf[pre][tk] = *reinterpret_cast<const uint4*>(kb + k_off(pre) + tk * 32 * kRowB);
+        static_for<kKS>([&](auto KS) {
+          constexpr int ks = decltype(KS)::value;
+          if constexpr (ks + 2 < kKS) {
+#pragma unroll
+            for (int tk = 0; tk < NH; ++tk)
+              kf[(ks + 2) % 3][tk] = *reinterpret_cast<const uint4*>(kb + k_off(ks + 2) + tk * 32 * kRowB);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+#pragma unroll
+          for (int tk = 0; tk < NH; ++tk) s[tk] = mfma32x32x16<T>(kf[ks % 3][tk], qf[ks], ks == 0 ? neg_m : s[tk]);
+          if constexpr (!I8 && ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);
+        });
+      } else {
       uint4 kf[2][NH];
 #pragma unroll
       for (int tk = 0; tk < NH; ++tk) kf[0][tk] = *reinterpret_cast<const uint4*>(kb + k_off(0) + tk * 32 * kRowB);
@@ -460,6 +481,24 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
       // fewer steps than copy instructions (head dims below the layout's): the rest of the copies follow here
       if constexpr (!I8 && kKS < 2 * kCopies)
         static_for<2 * kCopies - kKS>([&](auto C) { issue_copy(next, NEXT_BUF{}, std::integral_constant<int, kKS + decltype(C)::value>{}); });
+      }
+    }
+    // head_dim 256: the V^T fragments of the tile's first 16 keys set out now and arrive during the softmax
+    const char* vb = &lds.v[buf][0];
+    auto v_frags = [&](int step, uint4 (&af)[kTD]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int td = 0; td < kTD; ++td) {
+        const char* p0 = vb + v_off(td) + 16 * step * kRowB;
+        const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
+        const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * kRowB));
+        af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;
+        af[td].z = __builtin_bit_cast(uint2, a1).x; af[td].w = __builtin_bit_cast(uint2, a1).y;
+      }
+    };
+    uint4 afr[2][kTD];
+    if constexpr (D == 256) {
+      v_frags(0, afr[0]);
+      __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- online softmax, one query row per lane (scores stay unscaled; the scale is folded
@@ -497,14 +536,29 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
     // no wait behind the fragment reads queued there)
     mx = max_with_lane_xor32(mx);                      // tile maximum of the row, relative to the running one
     const bool grow = first || mx > 8.f;
-    if (__any(grow)) {
+    if (__builtin_expect(__any(grow), 0)) {
       const float d = grow ? mx : 0.f;                 // the running maximum moves up by d (any finite d on the first tile)
       const float alpha = first ? 1.f : fast_exp2(-d); // nothing is accumulated yet on the first tile
       l *= alpha;
+      if constexpr (D == 256) {
 #pragma unroll
-      for (int td = 0; td < kTD; ++td)
+        for (int td = 0; td < kTD; ++td)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[td][r] *= alpha;
+          for (int r = 0; r < 16; ++r) {
+            const float x = o[td][r];
+            float t, y;
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(x));
+            t *= alpha;
+            asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(y) : "v"(t));
+            o[td][r] = y;
+          }
+        asm volatile("s_nop 7");
+      } else {
+#pragma unroll
+        for (int td = 0; td < kTD; ++td)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[td][r] *= alpha;
+      }
       const float nm = neg_m[0] - d;
 #pragma unroll
       for (int r = 0; r < 16; ++r) neg_m[r] = nm;
@@ -520,7 +574,21 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
       for (int r = 0; r < 16; ++r) s[tk][r] = fast_exp2(s[tk][r]);
 
     // ---- O^T += V^T P^T ----
-    const char* vb = &lds.v[buf][0];
+    if constexpr (D == 256) {
+      static_for<2 * NH>([&](auto STEP) {              // 16 kv rows per step; the next step's fragments set out first
+        constexpr int step = decltype(STEP)::value, tk = step / 2, st = step % 2;
+        uint4 pf;
+        pf.x = pack2<T>(s[tk][8 * st + 0], s[tk][8 * st + 1]);
+        pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
+        pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
+        pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
+        l = add_pair<T>(pf.w, add_pair<T>(pf.z, add_pair<T>(pf.y, add_pair<T>(pf.x, l))));
+        if constexpr (step + 1 < 2 * NH) v_frags(step + 1, afr[(step + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(afr[step & 1][td], pf, o[td]);
+      });
+    } else
     static_for<2 * NH>([&](auto STEP) {                // 16 kv rows per step
       constexpr int tk = decltype(STEP)::value / 2, st = decltype(STEP)::value % 2;
       uint4 pf;

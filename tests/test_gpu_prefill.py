@@ -87,6 +87,31 @@ def test_prefill_head_dims_that_are_multiples_of_8_on_the_16_row_tile_kernel(dty
     assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,d", [(4, 2, 256), (8, 2, 128), (4, 1, 96), (4, 2, 64), (16, 8, 128)])
+def test_prefill_running_maximum_moves_in_later_tiles(dtype, hq, hkv, d):
+    """Keys whose norm grows with their position (and queries five times the usual size) make the row maxima jump by
+    more than the lazy-rescale threshold in tile after tile, so the accumulators that already hold several tiles are
+    scaled down again and again (head_dim 256 does this on the accumulator half of the register file directly).
+    fp16 meets the usual bounds.  bf16 does not at logits this large, in any kernel and for a reason that has nothing
+    to do with the rescaling: the queries enter the matrix unit as q * scale * log2 e rounded to 8 bits of mantissa,
+    and an error of 2^-9 of a logit near 40 is 8 % of a weight (measured: 0.06-0.11 max, 0.0021-0.0022 mean for every
+    head_dim), so bf16 gets bounds that a lost or doubled rescale (errors of order one) still fails by far."""
+    lengths = [700, 130, 333]
+    q, k, v, cu = make_varlen_case(57, lengths, hq, hkv, d, dtype=dtype)
+    ramp = torch.cat([torch.linspace(0.5, 3.0, n) for n in lengths]).to(k.device)
+    q = (q.float() * 5).to(dtype)
+    k = (k.float() * ramp[:, None, None]).to(dtype)
+    scale = 1 / math.sqrt(d)
+    got = _run(q, k, v, cu, scale, hq, hkv, d)
+    assert torch.isfinite(got.float()).all()
+    mx, mean = error_stats(got, _oracle32(q, k, v, cu, scale, hq, hkv, d))
+    if dtype == torch.float16:
+        assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16, (mx, mean)
+    else:
+        assert mx <= 0.2 and mean <= 4e-3, (mx, mean)
+
+
 def test_prefill_other_head_dims_ignore_what_follows_the_head():
     """head_dim 96: the last two chunks of each 256-byte tile row are copied from whatever follows the head in memory.
     With the next head (and for the last head the next token) poisoned by huge values and NaNs in one run, the outputs
