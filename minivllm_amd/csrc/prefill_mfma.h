@@ -541,6 +541,10 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
       const float alpha = first ? 1.f : fast_exp2(-d); // nothing is accumulated yet on the first tile
       l *= alpha;
       if constexpr (D == 256) {
+        // The accumulators live in the accumulator half of the register file, which only the matrix unit and these
+        // moves reach: each is fetched, scaled and put back where it was, so the tile loop never holds a second copy
+        // of all 128 in ordinary registers.  (Nothing is accumulated yet in a wave's first tile.)
+        if (!first) {
 #pragma unroll
         for (int td = 0; td < kTD; ++td)
 #pragma unroll
@@ -552,7 +556,8 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
             asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(y) : "v"(t));
             o[td][r] = y;
           }
-        asm volatile("s_nop 7");
+        asm volatile("s_nop 7");                       // the moves' results are final before the matrix unit reads them
+        }
       } else {
 #pragma unroll
         for (int td = 0; td < kTD; ++td)
