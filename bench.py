@@ -657,7 +657,8 @@ def bench_other_head_dims(args):
     hq, hkv, bs = 16, 8, 16
     g = torch.Generator().manual_seed(args.seed)
     lengths = torch.randint(64, 2049, (16,), generator=g).tolist()
-    out = {"workload": "bf16, Hq16 Hkv8: decode B64 ctx~U[1000,3000] block_size 16; prefill 16 prompts L~U[64,2048]"}
+    out = {"workload": "bf16, Hq16 Hkv8: decode B64 ctx~U[1000,3000] block_size 16; prefill 16 prompts L~U[64,2048] "
+                       f"(prefill timed after {EXTRA_WARM_MS:.0f} ms of warm-up launches, like the other prefill legs)"}
     for d in (32, 80, 96, 112, 256, 72, 100):
         q, kc, vc, tables, ctx = make_paged_case_on_device(args.seed, dev, 64, 1000, 3000, hq, hkv, d, bs,
                                                            dtype=torch.bfloat16, log_uniform=False)
@@ -668,7 +669,7 @@ def bench_other_head_dims(args):
         nbytes = int(ctx.sum()) * hkv * d * 2 * kc.element_size()
         qq, kk, vv, cu = (t.to(dev) for t in make_varlen_case(args.seed + 1, lengths, hq, hkv, d, dtype=torch.bfloat16))
         _, pms = time_steps(lambda: flash_attention_prefill(qq, kk, vv, cu, 1 / math.sqrt(d), hq, hkv, d),
-                            steps, min(args.warmup, steps), 0.0)
+                            steps, min(args.warmup, steps), EXTRA_WARM_MS if d != 100 else 0.0)
         flops = 4 * hq * d * sum(n * (n + 1) // 2 for n in lengths)
         out[f"head_dim_{d}"] = {
             "decode_kernel": "generic" if paged_decode_plan(64, hq, hkv, d, tables.shape[1], bs, torch.bfloat16)[2] == 0 else "mfma",
@@ -932,6 +933,8 @@ def summary_of(line):
     put("prefill_suffix128_behind_32k_us", "prefill_short_suffix", "event_ms_per_step")
     put("prefill_paged_frac", "prefill_cached_prefix", "roofline", "frac")
     put("prefill_paged_int8_frac", "prefill_cached_prefix_int8", "roofline", "frac")
+    put("prefill_d256_tflops", "other_head_dims", "head_dim_256", "prefill_tflops")
+    put("prefill_d96_tflops", "other_head_dims", "head_dim_96", "prefill_tflops")
     put("store_frac_hbm", "store", "roofline", "frac")
     put("int8_decode_frac_hbm", "int8", "roofline", "frac")
     put("int8_store_frac_hbm", "int8", "store_roofline", "frac")
@@ -943,6 +946,9 @@ def summary_of(line):
                 if name in node:
                     out[key] = round(node[name])
                     break
+    for key in ("prefill_d256_tflops", "prefill_d96_tflops"):
+        if key in out:
+            out[key] = round(out[key])
     for key in ("prefill_us", "prefill_suffix128_behind_32k_us"):
         if key in out:
             out[key] = round(out[key] * 1e3, 1)
