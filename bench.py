@@ -646,7 +646,7 @@ def bench_demo_shape(args):
 
 def bench_other_head_dims(args):
     """bf16 head dims beside 64 and 128 that run on matrix-unit kernels (32, 80, 96, 112, 256: the decode kernels and
-    the LDS-tiled prefill; 72: the decode kernels and the 16-row tile prefill) and one that does not (100: the generic
+    the LDS-tiled prefill; 72: the same, with the first product's last step half empty) and one that does not (100: the generic
     kernels), on the demo leg's batch: decode of 64
     sequences of 1000-3000 tokens, prefill of 16 prompts of 64-2048 tokens, 16 query / 8 kv heads."""
     import torch

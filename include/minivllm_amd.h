@@ -180,10 +180,10 @@ int mvllm_prefill_varlen(void* out, const void* q, const void* k, const void* v,
 /*
  * Which kernel a prefill of these static sizes runs on (no counterpart in the reference, whose Triton kernels take any
  * power-of-two head_dim from a tile-size table, attention.py:249-257).  block_size 0 = the packed entry point,
- * > 0 = the paged ones.  *kernel: 2 an LDS-tiled MFMA kernel (bf16 / fp16 with head_dim 32, 48, 64, 80, 96, 112, 128
- * or 256; fp32 with 128 or 64; over an INT8 cache 64 or 128; the packed and the 16-bit paged entry point run its
+ * > 0 = the paged ones.  *kernel: 2 an LDS-tiled MFMA kernel (bf16 / fp16 with a head_dim that is a multiple of 8 from
+ * 32 to 128, or 256; fp32 with 128 or 64; over an INT8 cache 64 or 128; the packed and the 16-bit paged entry point run its
  * two-group form where head_dim is 128, the query heads per kv head are an even number and the batch has at most 64
- * sequences), 1 the 16-row tile MFMA kernel (bf16 / fp16 with 40, 56, 72, 88, 104 or 120), 0 the generic kernel (any
+ * sequences), 1 the 16-row tile MFMA kernel (a paged cache whose blocks hold 2^31 bytes or more), 0 the generic kernel (any
  * head_dim <= 512; one key per step, a correctness path two orders of magnitude slower), -1 unsupported.
  * Pointers are assumed 16-byte aligned (unaligned ones take the generic kernel).  Pure host arithmetic.
  */

@@ -16,7 +16,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libminivllm_amd.so")
 PROBE_LIB_PATH = os.path.join(PKG_DIR, "libmvllm_probe.so")      # measurement support for bench.py, not an operator
 PROBE_SOURCES = ["mfma_probe.hip"]
-SOURCES = ["capi.hip", "store_kvcache.hip", "paged_decode.hip", "prefill_varlen.hip", "prefill_other_dims.hip", "prefill_pingpong.hip", "prefill_staged.hip", "prefill_split.hip", "prefill_f32.hip", "qk_norm_rope_store.hip", "sampler.hip",
+SOURCES = ["capi.hip", "store_kvcache.hip", "paged_decode.hip", "prefill_varlen.hip", "prefill_other_dims.hip", "prefill_half_step_dims.hip", "prefill_pingpong.hip", "prefill_staged.hip", "prefill_split.hip", "prefill_f32.hip", "qk_norm_rope_store.hip", "sampler.hip",
            "rms_norm.hip", "activation.hip", "linear_small.hip"]
 
 HIPCC_FLAGS = [

@@ -137,12 +137,16 @@ __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, in
 template <typename T, int HPW, bool PAGED, int D, bool I8 = false, int DD = D>
 __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_kernel(const PrefillArgs a) {
   static_assert(!I8 || PAGED, "INT8 caches are paged");
-  static_assert(DD % 16 == 0 && DD <= D && (!I8 || DD == D), "head dims in steps of 16, INT8 only at 64 and 128");
+  static_assert(DD % 8 == 0 && DD <= D && (!I8 || DD == D), "head dims in steps of 8, INT8 only at 64 and 128");
   constexpr int kRowB = D * 2;                  // bytes per tile row
   constexpr int kChunks = kRowB / 16;           // 16-byte chunks per row: 16 or 8
   constexpr int kCopyRows = 1024 / kRowB;       // rows per copy instruction: 4 or 8
   constexpr int kTileBytes = kBN * kRowB;       // one K (or V) tile
-  constexpr int kKS = DD / 16;                  // 16-dim steps of the first product
+  constexpr int kKS = (DD + 15) / 16;           // 16-dim steps of the first product
+  // DD = 16 n + 8: the last step holds 8 dims.  Its upper lanes (hi = 1, dims 8 .. 15 of the step) carry zeros as Q and
+  // read the row's first chunk as K (data of the same row and head, so the products are exact zeros and nothing of the
+  // neighbouring head is touched).
+  constexpr bool kHalfStep = DD % 16 == 8;
   constexpr int kTD = (DD + 31) / 32;           // 32-dim blocks of the output
   // K rows are read 16 at a time with the same logical chunk: the swizzle spreads them over the banks.  With 128-byte
   // rows two rows share a 256-byte bank line, so the row index is halved first.
@@ -368,7 +372,11 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
     if (PAGED && a.q_period > 0) tok = (int64_t)((uint32_t)tok % (uint32_t)a.q_period);   // both below 2^31
     const T* src = q + (tok * a.num_heads + h) * DD + 8 * hi;
 #pragma unroll
-    for (int ks = 0; ks < kKS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
+    for (int ks = 0; ks < DD / 16; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
+    if constexpr (kHalfStep) {
+      qf[kKS - 1] = make_uint4(0u, 0u, 0u, 0u);
+      if (hi == 0) qf[kKS - 1] = *reinterpret_cast<const uint4*>(src + 16 * (kKS - 1));
+    }
     // The softmax scale (times log2 e) goes into Q once, rounded to the element type, so that the scores leave
     // the matrix unit as exp2 arguments: the tile loop has no multiply per score.  This runs while the first K/V
     // tile is still on its way.
@@ -412,6 +420,7 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
   int k_off_[kKOffs];
 #pragma unroll
   for (int ks = 0; ks < kKOffs; ++ks) k_off_[ks] = l32 * kRowB + (((2 * ks + hi) ^ kswz(l32)) << 4);
+  if constexpr (kHalfStep) k_off_[kKS - 1] = l32 * kRowB + (((hi ? 0 : 2 * (kKS - 1)) ^ kswz(l32)) << 4);
   auto k_off = [&](int ks) __attribute__((always_inline)) { return k_off_[ks & 7] + (ks >> 3) * 256; };
   const int v_row = 4 * hi + (i16 >> 2);
   int v_off_[kVOffs];
@@ -536,7 +545,9 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
     // no wait behind the fragment reads queued there)
     mx = max_with_lane_xor32(mx);                      // tile maximum of the row, relative to the running one
     const bool grow = first || mx > 8.f;
-    if (__builtin_expect(__any(grow), 0)) {
+    // head_dim 256: marked unlikely, so that the rescale sits out of line and the register allocator does not plan the
+    // tile loop around it (for the other head dims the hint only moves blocks about: measured, no gain)
+    if (D == 256 ? __builtin_expect(__any(grow), 0) : __any(grow)) {
       const float d = grow ? mx : 0.f;                 // the running maximum moves up by d (any finite d on the first tile)
       const float alpha = first ? 1.f : fast_exp2(-d); // nothing is accumulated yet on the first tile
       l *= alpha;
@@ -718,7 +729,7 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
   }
 }
 
-// D: the LDS layout (64 or 128), DD: the data's head dimension.
+// D: the LDS layout (64, 128 or 256), DD: the data's head dimension.
 template <typename T, bool PAGED, bool I8, int D, int DD>
 static int launch_prefill_mfma_as(const PrefillArgs& a, hipStream_t stream) {
   const int group = a.num_heads / a.num_kv_heads;
@@ -755,7 +766,7 @@ int launch_prefill_paged_16bit(const PrefillArgs& a, int dtype, hipStream_t stre
 int launch_prefill_paged_int8(const PrefillArgs& a, int dtype, hipStream_t stream);
 // fp32 tensors, head_dim 128 or 64, packed or over a paged fp32 cache (prefill_f32.hip)
 int launch_prefill_f32(const PrefillArgs& a, bool paged, hipStream_t stream);
-// head_dim 32, 80, 96, 112 (prefill_other_dims.hip); 16-bit element types only
+// every other multiple of 8 from 32 to 120, and 256 (prefill_other_dims.hip, prefill_half_step_dims.hip); 16-bit element types only
 bool prefill_mfma_other_dim(int head_dim);
 int launch_prefill_mfma_other(const PrefillArgs& a, int dtype, bool paged, hipStream_t stream);
 

@@ -75,7 +75,8 @@ def test_prefill_split_plan_is_host_arithmetic():
     assert plan(1, 128, 32768, 32, 8, 80, 256, bf16, 1) == 0                  # ... but at head_dim 64 / 128 only
     assert plan(1, 128, 32768, 16, 8, 80, 256, bf16, 0) == 17                 # head_dim 80: 16 workgroups a range
     assert plan(8, 4096, 32768, 16, 8, 80, 256, bf16, 0) == 0                 # ... 576 of them fill the chip
-    assert plan(1, 128, 32768, 16, 8, 72, 256, bf16, 0) == 0                  # head_dim 72: not an LDS-tiled shape
+    assert plan(1, 128, 32768, 16, 8, 72, 256, bf16, 0) == 17                 # head_dim 72: as 80
+    assert plan(1, 128, 32768, 16, 8, 136, 256, bf16, 0) == 0                 # head_dim 136: not an LDS-tiled shape
     need = lib.mvllm_prefill_paged_split_workspace_bytes(1, 128, 32768 + 128, 32, 8, 128, 256, bf16, 16)
     partial = 16 * 128 * 32 * 128 * 2 + 16 * 128 * 32 * 4
     assert partial < need < partial + 16384
@@ -135,7 +136,9 @@ def test_prefill_plan_is_host_arithmetic():
     assert prefill_plan(8, 8, 256, dtype=torch.float32) == 0
     assert prefill_plan(6, 2, 80) == 2 and prefill_plan(6, 2, 96) == 2 and prefill_plan(6, 2, 96, dtype=torch.float32) == 0
     assert prefill_plan(6, 2, 112, block_size=16) == 2 and prefill_plan(6, 2, 112, block_size=8) == 0
-    assert prefill_plan(6, 2, 72) == 1 and prefill_plan(6, 2, 40) == 1 and prefill_plan(6, 2, 48) == 2 and prefill_plan(6, 2, 100) == 0
+    assert prefill_plan(6, 2, 72) == 2 and prefill_plan(6, 2, 40) == 2 and prefill_plan(6, 2, 48) == 2 and prefill_plan(6, 2, 100) == 0
+    assert prefill_plan(6, 2, 120, block_size=32) == 2 and prefill_plan(6, 2, 72, dtype=torch.float32) == 0
+    assert prefill_plan(6, 2, 136) == 0 and prefill_plan(6, 2, 24) == 0
     assert prefill_plan(32, 8, 128, 16, int8_cache=True) == 2
     assert prefill_plan(32, 8, 96, 16, int8_cache=True) == -1 and prefill_plan(32, 8, 128, 16, torch.float32, True) == -1
     assert prefill_plan(8, 8, 1024) == -1

@@ -74,12 +74,14 @@ def test_prefill_head_dim_32_80_96_112_256_on_the_lds_tiled_kernel(dtype, hq, hk
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("hq,hkv,d,lengths", [(8, 2, 40, [70, 1, 33, 129]), (8, 4, 56, [64, 17, 130]),
                                               (8, 2, 72, [70, 1, 33, 129]), (6, 3, 88, [200, 17]), (6, 6, 104, [150]),
-                                              (8, 2, 120, [70, 1, 33, 129])])
-def test_prefill_head_dims_that_are_multiples_of_8_on_the_16_row_tile_kernel(dtype, hq, hkv, d, lengths):
-    """Multiples of 8 that are not multiples of 32: the lanes of the last 32-dim step whose dims lie past the head load
-    neither K nor Q (what follows in memory is the next head, not zeros)."""
+                                              (8, 2, 120, [70, 1, 33, 129]), (16, 8, 72, [700, 300]), (5, 5, 40, [257, 64]),
+                                              (12, 4, 104, [513, 1, 90])])
+def test_prefill_head_dims_that_are_multiples_of_8_on_the_lds_tiled_kernel(dtype, hq, hkv, d, lengths):
+    """Multiples of 8 that are not multiples of 16: the last 16-dim step of the first product holds 8 dims; its upper
+    lanes carry zeros as Q and the row's first chunk as K (what follows the head in memory is the next head, not
+    zeros)."""
     from minivllm_amd.layers.attention import prefill_plan
-    assert prefill_plan(hq, hkv, d, 0, dtype) == 1
+    assert prefill_plan(hq, hkv, d, 0, dtype) == 2
     case = make_varlen_case(57, lengths, hq, hkv, d, dtype=dtype)
     scale = 1 / math.sqrt(d)
     got = _run(*case, scale, hq, hkv, d)
@@ -112,11 +114,13 @@ def test_prefill_running_maximum_moves_in_later_tiles(dtype, hq, hkv, d):
         assert mx <= 0.2 and mean <= 4e-3, (mx, mean)
 
 
-def test_prefill_other_head_dims_ignore_what_follows_the_head():
-    """head_dim 96: the last two chunks of each 256-byte tile row are copied from whatever follows the head in memory.
+@pytest.mark.parametrize("d", [96, 72, 40, 120])
+def test_prefill_other_head_dims_ignore_what_follows_the_head(d):
+    """head_dim 96: the last two chunks of each 256-byte tile row are copied from whatever follows the head in memory
+    (72, 40, 120: the same, and the last step of the first product is half empty).
     With the next head (and for the last head the next token) poisoned by huge values and NaNs in one run, the outputs
     of every head must equal those of the clean run bit for bit."""
-    hq, hkv, d = 8, 2, 96
+    hq, hkv = 8, 2
     q, k, v, cu = make_varlen_case(56, [150, 31, 64], hq, hkv, d, dtype=torch.bfloat16)
     scale = 1 / math.sqrt(d)
     clean = _run(q, k, v, cu, scale, hq, hkv, d)

@@ -53,6 +53,9 @@ def _check(got, want, dtype):
     (4, 4, 32, 16, [200, 70], [160, 32]),                          # head_dim 32 in the 64 layout
     (8, 2, 80, 16, [140, 23], [16, 8]),                            # head_dim 80, blocks of 16: the tiled kernel
     (8, 2, 256, 16, [300, 64, 129], [256, 0, 17]),                 # head_dim 256: 512-byte tile rows
+    (8, 2, 72, 16, [300, 64, 129], [256, 0, 17]),                  # head_dim 72: the first product's last step half empty (fp32: generic)
+    (6, 3, 120, 32, [131, 260], [50, 259]),                        # head_dim 120
+    (4, 4, 40, 16, [200, 70], [160, 32]),                          # head_dim 40 in the 64 layout
     (4, 4, 64, 16, [70], [32]),                                    # head_dim 64: 16-row tiles (fp32: generic kernel)
     (16, 8, 64, 16, [300, 64, 129, 500], [256, 0, 17, 48]),        # head_dim 64, the reference demo's heads
     (12, 1, 64, 256, [700, 30, 257], [512, 29, 0]),                # head_dim 64, one kv head, the engine's block size
@@ -312,7 +315,8 @@ def test_int8_paged_prefill_in_two_steps_unmapped_block_and_unsupported_shapes()
     assert ws(2, 100, hq, hkv, d, code, 1) == 2 * (2 * 7 * 16 * hkv * d * 2) + 256 == ws(2, 100, hq, hkv, d, code, 0)
     assert ws(2, 100, 6, 2, d, code, 1) > 0 and ws(2, 100, hq, hkv, 64, code, 1) > 0 and ws(65, 100, hq, hkv, d, code, 1) > 0
     assert ws(2, 100, hq, hkv, 96, code, 1) == 0 and ws(2, 100, hq, hkv, 96, code, 0) > 0      # head_dim 96: 16-bit caches only
-    assert ws(2, 100, hq, hkv, 72, code, 0) == 0 and ws(2, 100, hq, hkv, 100, code, 0) == 0    # no LDS-tiled kernel for these
+    assert ws(2, 100, hq, hkv, 136, code, 0) == 0 and ws(2, 100, hq, hkv, 100, code, 0) == 0    # no LDS-tiled kernel for these
+    assert ws(2, 100, hq, hkv, 72, code, 0) > 0                                                  # 16-bit cache, any multiple of 8 from 32 to 128
     assert ws(2, 100, hq, hkv, d, _C.dtype_code(torch.float32), 1) == 0 and ws(2, 0, hq, hkv, d, code, 1) == 0
     # block size 8: the one-step INT8 kernels do not take it, the two-step form does
     c8, ck8, cv8, sk8, sv8 = _int8_case(74, lengths, cached, hq, hkv, d, 8, dtype)

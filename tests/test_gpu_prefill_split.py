@@ -32,6 +32,8 @@ def _run(c, hq, hkv, d, bs, scale, splits, max_k):
     (16, 8, 80, 16, [900, 300], [800, 299], 4),                    # head_dim 80 in the layout of 128
     (6, 2, 32, 32, [700], [650], 3),                               # head_dim 32 in the layout of 64; three heads per kv head
     (8, 4, 256, 16, [600, 200], [520, 130], 3),                    # head_dim 256: one workgroup per compute unit
+    (8, 2, 72, 16, [900, 300], [800, 299], 4),                     # head_dim 72: the first product's last step half empty
+    (6, 2, 40, 32, [700], [650], 3),                               # head_dim 40 in the layout of 64
 ])
 def test_paged_prefill_split_over_keys(hq, hkv, d, bs, lengths, cached, splits, dtype):
     c = make_paged_prefill_case(83, lengths, cached, hq, hkv, d, bs, dtype=dtype)
@@ -138,7 +140,8 @@ def test_split_plan_and_rejections():
     assert lib.mvllm_prefill_paged_split_plan(1, 128, 2048, 32, 8, 128, 256, bf, 0) == 0         # too few keys to cut
     assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 128, 256, bf, 1) >= 3        # INT8 cache
     assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 80, 256, bf, 1) == 0         # ... not at head_dim 80
-    assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 72, 256, bf, 0) == 0         # head_dim 72
+    assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 136, 256, bf, 0) == 0        # head_dim 136: no LDS-tiled kernel
+    assert lib.mvllm_prefill_paged_split_plan(1, 128, 32768, 32, 8, 72, 256, bf, 0) > 0          # every multiple of 8 from 32 to 128 has one
     assert lib.mvllm_prefill_paged_split_workspace_bytes(40, 128, 32768, 32, 8, 128, 256, bf, 2) == 0   # 80 ranges
     c = make_paged_prefill_case(5, [300], [200], 8, 8, 128, 16, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
