@@ -121,7 +121,7 @@ __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, in
   return true;
 }
 
-// D = 128 or 64.  A row of a tile is D*2 bytes = kChunks 16-byte chunks; one copy instruction moves 1 KB = kCopyRows
+// D = 256, 128 or 64.  A row of a tile is D*2 bytes = kChunks 16-byte chunks; one copy instruction moves 1 KB = kCopyRows
 // rows.  The chunk swizzles (kswz for K, vswz for V) must not change when 8, 16 or 32 rows are added, because the
 // per-lane LDS offsets are computed once and the tile rows are reached through immediates.
 // I8 (paged only): the cache holds int8 codes and fp32 scales per (token, kv head).  The codes of a tile are copied
@@ -129,11 +129,11 @@ __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, in
 // 16 rows into the one 16-bit K and V tile (code * scale rounded once to the element type, exactly what the 16-row
 // tile kernel and decode see), after which the tile is an ordinary tile: two barriers per tile instead of one, the
 // conversion (about 180 vector instructions per lane and tile) in front of the products.
-// DD (default D): the head dimension of the data where it is not 64 or 128 itself: 32 in the layout of 64, 80 / 96 /
-// 112 in that of 128.  A tile row is still copied as D * 2 bytes, so its last chunks hold whatever follows the head
-// in memory (the next head, the next token, zeros past the descriptor's end); the first product runs over DD / 16
-// steps and never reads them, the second one carries them through the output columns DD .. 32 ceil(DD / 32) - 1 of
-// its last block, which are not stored.
+// DD (default D): the head dimension of the data where it is not 64, 128 or 256 itself: 32 to 56 in the layout of 64,
+// 72 to 120 in that of 128, in steps of 8.  A tile row is still copied as D * 2 bytes, so its last chunks hold whatever
+// follows the head in memory (the next head, the next token, zeros past the descriptor's end); the first product runs
+// over ceil(DD / 16) steps and never reads them (kHalfStep below: the last step of DD = 16 n + 8), the second one
+// carries them through the output columns DD .. 32 ceil(DD / 32) - 1 of its last block, which are not stored.
 template <typename T, int HPW, bool PAGED, int D, bool I8 = false, int DD = D>
 __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_kernel(const PrefillArgs a) {
   static_assert(!I8 || PAGED, "INT8 caches are paged");
