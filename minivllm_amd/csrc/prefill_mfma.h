@@ -472,25 +472,25 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
           if constexpr (!I8 && ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);
         });
       } else {
-      uint4 kf[2][NH];
+        uint4 kf[2][NH];
 #pragma unroll
-      for (int tk = 0; tk < NH; ++tk) kf[0][tk] = *reinterpret_cast<const uint4*>(kb + k_off(0) + tk * 32 * kRowB);
-      static_for<kKS>([&](auto KS) {
-        constexpr int ks = decltype(KS)::value;
-        if constexpr (ks + 1 < kKS) {
+        for (int tk = 0; tk < NH; ++tk) kf[0][tk] = *reinterpret_cast<const uint4*>(kb + k_off(0) + tk * 32 * kRowB);
+        static_for<kKS>([&](auto KS) {
+          constexpr int ks = decltype(KS)::value;
+          if constexpr (ks + 1 < kKS) {
 #pragma unroll
-          for (int tk = 0; tk < NH; ++tk)
-            kf[(ks + 1) & 1][tk] = *reinterpret_cast<const uint4*>(kb + k_off(ks + 1) + tk * 32 * kRowB);
-          __builtin_amdgcn_sched_barrier(0);   // keep the reads in front of this step's MFMAs
-        }
+            for (int tk = 0; tk < NH; ++tk)
+              kf[(ks + 1) & 1][tk] = *reinterpret_cast<const uint4*>(kb + k_off(ks + 1) + tk * 32 * kRowB);
+            __builtin_amdgcn_sched_barrier(0);   // keep the reads in front of this step's MFMAs
+          }
 #pragma unroll
-        for (int tk = 0; tk < NH; ++tk) s[tk] = mfma32x32x16<T>(kf[ks & 1][tk], qf[ks], ks == 0 ? neg_m : s[tk]);
-        if constexpr (!I8 && ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);    // copies of the next tile, K first
-      });
+          for (int tk = 0; tk < NH; ++tk) s[tk] = mfma32x32x16<T>(kf[ks & 1][tk], qf[ks], ks == 0 ? neg_m : s[tk]);
+          if constexpr (!I8 && ks < 2 * kCopies) issue_copy(next, NEXT_BUF{}, KS);    // copies of the next tile, K first
+        });
+      }
       // fewer steps than copy instructions (head dims below the layout's): the rest of the copies follow here
       if constexpr (!I8 && kKS < 2 * kCopies)
         static_for<2 * kCopies - kKS>([&](auto C) { issue_copy(next, NEXT_BUF{}, std::integral_constant<int, kKS + decltype(C)::value>{}); });
-      }
     }
     // head_dim 256: the V^T fragments of the tile's first 16 keys set out now and arrive during the softmax
     const char* vb = &lds.v[buf][0];
@@ -604,29 +604,23 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
 #pragma unroll
         for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(afr[step & 1][td], pf, o[td]);
       });
-    } else
-    static_for<2 * NH>([&](auto STEP) {                // 16 kv rows per step
-      constexpr int tk = decltype(STEP)::value / 2, st = decltype(STEP)::value % 2;
-      uint4 pf;
-      pf.x = pack2<T>(s[tk][8 * st + 0], s[tk][8 * st + 1]);
-      pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
-      pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
-      pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
-      // row sum from the rounded weights, the ones the numerator uses; partial: this lane's kv rows only
-      // (lanes l and l^32 are added at the end)
-      l = add_pair<T>(pf.w, add_pair<T>(pf.z, add_pair<T>(pf.y, add_pair<T>(pf.x, l))));
-      uint4 af[kTD];
+    } else {
+      static_for<2 * NH>([&](auto STEP) {              // 16 kv rows per step
+        constexpr int tk = decltype(STEP)::value / 2, st = decltype(STEP)::value % 2;
+        uint4 pf;
+        pf.x = pack2<T>(s[tk][8 * st + 0], s[tk][8 * st + 1]);
+        pf.y = pack2<T>(s[tk][8 * st + 2], s[tk][8 * st + 3]);
+        pf.z = pack2<T>(s[tk][8 * st + 4], s[tk][8 * st + 5]);
+        pf.w = pack2<T>(s[tk][8 * st + 6], s[tk][8 * st + 7]);
+        // row sum from the rounded weights, the ones the numerator uses; partial: this lane's kv rows only
+        // (lanes l and l^32 are added at the end)
+        l = add_pair<T>(pf.w, add_pair<T>(pf.z, add_pair<T>(pf.y, add_pair<T>(pf.x, l))));
+        uint4 af[kTD];
+        v_frags(decltype(STEP)::value, af);
 #pragma unroll
-      for (int td = 0; td < kTD; ++td) {
-        const char* p0 = vb + v_off(td) + (32 * tk + 16 * st) * kRowB;
-        const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
-        const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0 + 8 * kRowB));
-        af[td].x = __builtin_bit_cast(uint2, a0).x; af[td].y = __builtin_bit_cast(uint2, a0).y;
-        af[td].z = __builtin_bit_cast(uint2, a1).x; af[td].w = __builtin_bit_cast(uint2, a1).y;
-      }
-#pragma unroll
-      for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(af[td], pf, o[td]);
-    });
+        for (int td = 0; td < kTD; ++td) o[td] = mfma32x32x16<T>(af[td], pf, o[td]);
+      });
+    }
   };
 
   // Tile j lives in buffer j % 2.  The main loop is unrolled by two so that the buffer index is a compile-time
