@@ -160,8 +160,10 @@ def test_attention_module_uses_the_paged_prefill_when_block_tables_are_set(bs):
     assert mx <= MAX_ABS_16 and mean <= MEAN_ABS_16
 
 
-def test_paged_prefill_head_dim_64_without_prefix_matches_plain_prefill_bitwise():
-    hq, hkv, d, bs = 16, 8, 64, 16
+@pytest.mark.parametrize("hq,hkv,d,bs", [(16, 8, 64, 16), (8, 2, 72, 16), (6, 6, 40, 32), (8, 4, 256, 16), (6, 2, 120, 64)])
+def test_paged_prefill_other_head_dims_without_prefix_match_plain_prefill_bitwise(hq, hkv, d, bs):
+    """The one-group kernel's paged and packed forms at head_dim 64, at head dims whose last 16-dim step is half empty
+    (72, 40, 120) and at 256: same tiles, same arithmetic, only the copies' source differs."""
     c = make_paged_prefill_case(66, [90, 1, 257, 33], [0, 0, 0, 0], hq, hkv, d, bs, dtype=torch.bfloat16)
     scale = 1 / math.sqrt(d)
     plain = flash_attention_prefill(c["q"].to(DEV), c["k"].to(DEV), c["v"].to(DEV), c["cu_k"].to(DEV), scale, hq, hkv, d).cpu()
