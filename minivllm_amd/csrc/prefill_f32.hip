@@ -52,7 +52,7 @@ __global__ __launch_bounds__(64 * kPfWaves, 2) void prefill_f32_kernel(const Pre
   const unsigned item = (round * 8 + ((xcd + round) & 7)) * kXcdChunk + slot % kXcdChunk;
   int item_y, seq_start, seq_len, row0, seq_index;
   if (a.num_seqs <= 64) {
-    if (!locate_banded<BM>(a.cu_seqlens, a.num_seqs, item, a.heads_y, a.band_bits, seq_start, seq_len, row0, seq_index, item_y)) return;
+    if (!locate_banded<BM>(a.cu_seqlens, a.num_seqs, item, a.heads_y, a.band_bits, a.band_shift, seq_start, seq_len, row0, seq_index, item_y)) return;
   } else {
     if (item >= (unsigned)tiles_x * (unsigned)a.heads_y) return;
     item_y = (int)(item / (unsigned)tiles_x);
@@ -249,11 +249,12 @@ int launch_f32_as(const PrefillArgs& a, hipStream_t stream) {
   const int hpw = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
   const int bm = kWaveRows * (kPfWaves / hpw);
   PrefillArgs b = a;
-  b.tiles_x = a.num_seqs <= 64 ? (int)(a.total_tokens / bm + (int64_t)a.num_seqs * (kBandRows / bm))
+  b.band_shift = band_shift_for(a.total_tokens, a.num_seqs, bm);
+  b.tiles_x = a.num_seqs <= 64 ? (int)(a.total_tokens / bm + ((int64_t)a.num_seqs << b.band_shift))
                                : (int)(a.total_tokens / bm + a.num_seqs);
   b.heads_y = a.num_kv_heads * (group / hpw);
   b.band_bits = 1;
-  while (((int64_t)1 << b.band_bits) <= a.total_tokens / kBandRows + 1) ++b.band_bits;
+  while (((int64_t)1 << b.band_bits) <= a.total_tokens / (bm << b.band_shift) + 1) ++b.band_bits;
   const int64_t items = (int64_t)b.tiles_x * b.heads_y;
   const int64_t span = 8 * (int64_t)kXcdChunk;
   const dim3 grid((unsigned)((items + span - 1) / span * span)), block(64 * kPfWaves);

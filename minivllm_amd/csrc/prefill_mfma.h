@@ -42,6 +42,7 @@ struct PrefillArgs {
   const int32_t* q_pos = nullptr;
   float* lse = nullptr;
   int64_t q_period = 0;
+  int band_shift = 0;   // MFMA path: log2 of the row tiles per band of the item order (locate_banded)
 };
 
 constexpr unsigned kXcdChunk = 32;      // consecutive work items handed to one XCD
@@ -70,13 +71,25 @@ template <typename T> __device__ __forceinline__ uint4 dequant8_biased(uint32_t 
 // sequence in memory order has: with 16 prompts of 64-2048 tokens the launch used to end with a single prompt's
 // 60-tile items running alone.  Consecutive items still share a sequence's keys (R tiles of one band, and
 // neighbouring bands of the same level), which keeps them in one XCD's L2.  Bands past a sequence's last tile are
-// padding: those workgroups return at once (at most R - 1 per sequence and head slice).
+// padding: those workgroups return at once (at most R - 1 per sequence and head slice), which still costs each of
+// them a place on a CU for the two microseconds of this function: a batch of short prompts (at most 192 rows on
+// average) is dealt in bands of one tile (band_shift 0), which have no padding, and whose loss of L2 sharing between
+// a sequence's tiles costs such prompts nothing.
 // Every lane of the calling wave must be active; all lanes return the same values.
 constexpr int kBandRows = 256;          // rows per band of the heaviest-first item order (a multiple of 128)
+constexpr int kShortPromptRows = 192;   // mean rows per sequence up to which bands are single tiles
+// log2 of the row tiles per band for a batch of these static sizes (bm: rows per workgroup, a power of two <= kBandRows)
+inline int band_shift_for(int64_t total_tokens, int num_seqs, int bm) {
+  if (total_tokens <= (int64_t)num_seqs * kShortPromptRows) return 0;
+  int shift = 0;
+  while ((bm << shift) < kBandRows) ++shift;
+  return shift;
+}
 template <int BM>
 __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, int num_seqs, unsigned item, int heads_y,
-                                              int band_bits, int& seq_start, int& seq_len, int& row0, int& seq_index, int& item_y) {
-  constexpr int R = kBandRows / BM;
+                                              int band_bits, int band_shift, int& seq_start, int& seq_len, int& row0, int& seq_index,
+                                              int& item_y) {
+  const int R = 1 << band_shift;
   const int lane = threadIdx.x & 63;
   int lo = 0, len = 0;
   if (lane < num_seqs) {
@@ -84,7 +97,7 @@ __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, in
     len = cu[lane + 1] - lo;
   }
   const int n = (len + BM - 1) / BM;            // row tiles of the lane's sequence
-  const int nb = (n + R - 1) / R;               // ... and bands
+  const int nb = (n + R - 1) >> band_shift;     // ... and bands
   // highest band level in the batch: bit by bit from the top (band_bits: the host's bound from the token count)
   int top = 0;
   for (int bit = band_bits - 1; bit >= 0; --bit) {
@@ -98,7 +111,7 @@ __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, in
   unsigned per_y = 0;
   for (; b >= 0; --b) {
     mask = __ballot(nb > b);
-    per_y = (unsigned)__popcll(mask) * (unsigned)R;
+    per_y = (unsigned)__popcll(mask) << band_shift;
     const unsigned items = per_y * (unsigned)heads_y;
     if (item - base < items) break;
     base += items;
@@ -107,12 +120,12 @@ __device__ __forceinline__ bool locate_banded(const int32_t* __restrict__ cu, in
   const unsigned idx = item - base;
   item_y = (int)(idx / per_y);
   const unsigned rem = idx - (unsigned)item_y * per_y;
-  const int q = (int)(rem / (unsigned)R), r = (int)(rem % (unsigned)R);
+  const int q = (int)(rem >> band_shift), r = (int)(rem & (unsigned)(R - 1));
   // the q-th sequence of this level = the lane whose bit is set with q set bits below it
   const int below = __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
   const unsigned long long pick = __ballot(((mask >> lane) & 1ull) != 0ull && below == q);
   const int owner = __ffsll((long long)pick) - 1;
-  const int t = b * R + (R - 1 - r);            // row tile inside the sequence, last tile of the band first
+  const int t = (b << band_shift) + (R - 1 - r);   // row tile inside the sequence, last tile of the band first
   if (t >= __shfl(n, owner, 64)) return false;  // the band's padding
   seq_start = __shfl(lo, owner, 64);
   seq_len = __shfl(len, owner, 64);
@@ -174,7 +187,7 @@ __global__ __launch_bounds__(64 * kPfWaves, D == 256 ? 1 : 2) void prefill_mfma_
   const unsigned item = (round * 8 + ((xcd + round) & 7)) * kXcdChunk + slot % kXcdChunk;
   int item_y, seq_start, seq_len, row0, seq_index;
   if (a.num_seqs <= 64) {
-    if (!locate_banded<BM>(a.cu_seqlens, a.num_seqs, item, a.heads_y, a.band_bits, seq_start, seq_len, row0, seq_index, item_y)) return;
+    if (!locate_banded<BM>(a.cu_seqlens, a.num_seqs, item, a.heads_y, a.band_bits, a.band_shift, seq_start, seq_len, row0, seq_index, item_y)) return;
   } else {
     // more sequences than one wave holds: memory order, inside a sequence the latest (heaviest) tiles first
     if (item >= (unsigned)tiles_x * (unsigned)a.heads_y) return;
@@ -734,11 +747,12 @@ static int launch_prefill_mfma_as(const PrefillArgs& a, hipStream_t stream) {
   PrefillArgs b = a;
   // upper bound on the query tiles: every sequence may end with a partial tile; in the banded order (at most 64
   // sequences) every sequence may also end with a partial band of kBandRows / bm tiles
-  b.tiles_x = a.num_seqs <= 64 ? (int)(a.total_tokens / bm + (int64_t)a.num_seqs * (kBandRows / bm))
+  b.band_shift = band_shift_for(a.total_tokens, a.num_seqs, bm);
+  b.tiles_x = a.num_seqs <= 64 ? (int)(a.total_tokens / bm + ((int64_t)a.num_seqs << b.band_shift))
                                : (int)(a.total_tokens / bm + a.num_seqs);
   b.heads_y = a.num_kv_heads * (group / hpw);
   b.band_bits = 1;
-  while (((int64_t)1 << b.band_bits) <= a.total_tokens / kBandRows + 1) ++b.band_bits;
+  while (((int64_t)1 << b.band_bits) <= a.total_tokens / (bm << b.band_shift) + 1) ++b.band_bits;
   const int64_t items = (int64_t)b.tiles_x * b.heads_y;
   const int64_t span = 8 * (int64_t)kXcdChunk;
   dim3 grid((unsigned)((items + span - 1) / span * span));
