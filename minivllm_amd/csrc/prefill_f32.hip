@@ -249,7 +249,7 @@ int launch_f32_as(const PrefillArgs& a, hipStream_t stream) {
   const int hpw = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
   const int bm = kWaveRows * (kPfWaves / hpw);
   PrefillArgs b = a;
-  b.band_shift = band_shift_for(a.total_tokens, a.num_seqs, bm);
+  b.band_shift = band_shift_for(a.total_tokens, a.num_seqs, bm, PAGED);
   b.tiles_x = a.num_seqs <= 64 ? (int)(a.total_tokens / bm + ((int64_t)a.num_seqs << b.band_shift))
                                : (int)(a.total_tokens / bm + a.num_seqs);
   b.heads_y = a.num_kv_heads * (group / hpw);

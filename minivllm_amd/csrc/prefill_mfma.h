@@ -72,15 +72,17 @@ template <typename T> __device__ __forceinline__ uint4 dequant8_biased(uint32_t 
 // 60-tile items running alone.  Consecutive items still share a sequence's keys (R tiles of one band, and
 // neighbouring bands of the same level), which keeps them in one XCD's L2.  Bands past a sequence's last tile are
 // padding: those workgroups return at once (at most R - 1 per sequence and head slice), which still costs each of
-// them a place on a CU for the two microseconds of this function: a batch of short prompts (at most 192 rows on
+// them a place on a CU for the two microseconds of this function: a packed batch of short prompts (at most 192 rows on
 // average) is dealt in bands of one tile (band_shift 0), which have no padding, and whose loss of L2 sharing between
 // a sequence's tiles costs such prompts nothing.
 // Every lane of the calling wave must be active; all lanes return the same values.
 constexpr int kBandRows = 256;          // rows per band of the heaviest-first item order (a multiple of 128)
 constexpr int kShortPromptRows = 192;   // mean rows per sequence up to which bands are single tiles
 // log2 of the row tiles per band for a batch of these static sizes (bm: rows per workgroup, a power of two <= kBandRows)
-inline int band_shift_for(int64_t total_tokens, int num_seqs, int bm) {
-  if (total_tokens <= (int64_t)num_seqs * kShortPromptRows) return 0;
+// (packed: the rows are also the keys.  Over a cached prefix few rows may stand behind many keys, which the tiles of a
+// band share in one XCD's L2: 128 rows behind 32768 keys cut into ranges ran 100 us in single tiles against 88.)
+inline int band_shift_for(int64_t total_tokens, int num_seqs, int bm, bool paged) {
+  if (!paged && total_tokens <= (int64_t)num_seqs * kShortPromptRows) return 0;
   int shift = 0;
   while ((bm << shift) < kBandRows) ++shift;
   return shift;
@@ -747,7 +749,7 @@ static int launch_prefill_mfma_as(const PrefillArgs& a, hipStream_t stream) {
   PrefillArgs b = a;
   // upper bound on the query tiles: every sequence may end with a partial tile; in the banded order (at most 64
   // sequences) every sequence may also end with a partial band of kBandRows / bm tiles
-  b.band_shift = band_shift_for(a.total_tokens, a.num_seqs, bm);
+  b.band_shift = band_shift_for(a.total_tokens, a.num_seqs, bm, PAGED);
   b.tiles_x = a.num_seqs <= 64 ? (int)(a.total_tokens / bm + ((int64_t)a.num_seqs << b.band_shift))
                                : (int)(a.total_tokens / bm + a.num_seqs);
   b.heads_y = a.num_kv_heads * (group / hpw);
